@@ -1,0 +1,146 @@
+/* rg_lru.h -- C ABI of the MI355X (gfx950) Conv1D + RG-LRU recurrent-block core.
+ *
+ * The reference (google-deepmind/recurrentgemma, torch path) has no FFI: its
+ * boundary for this path is the Python module surface of
+ * recurrentgemma/torch/layers.py (Conv1D, BlockDiagonalLinear, RGLRU, rnn_scan).
+ * Each entry point below names the reference function it stands in for.
+ *
+ * Conventions
+ *  - All pointers are DEVICE pointers to dense row-major tensors, channel
+ *    fastest: activations [B,T,W], segment positions [B,T], RG-LRU state [B,W]
+ *    (always float32), conv state [B,K-1,W].
+ *  - `dtype` is the activation/parameter element type (RG_DTYPE_*): the
+ *    reference requires parameters and activations to share one dtype.
+ *  - `stream` is a hipStream_t passed as void*.  Calls only enqueue work on it:
+ *    no synchronisation, no allocation, no use of any other stream.
+ *  - The library never keeps a pointer after a call returns and never frees or
+ *    allocates caller-visible memory.
+ *  - Return value: RG_OK or a negative RG_ERR_* code; rg_last_error() then
+ *    gives a thread-local, human-readable reason.  No C++ exception crosses
+ *    this boundary.  Arguments are validated before anything is launched.
+ *  - Inputs are never modified (the reference's Conv1D multiplies its input by
+ *    the document mask in place, layers.py:497-508; that side effect is NOT
+ *    reproduced, the masked conv state it leads to is).
+ */
+#ifndef RG_LRU_H_
+#define RG_LRU_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RG_ABI_VERSION 1
+
+enum {
+  RG_OK = 0,
+  RG_ERR_BAD_ARG = -1,     /* null pointer, non-positive size, misalignment  */
+  RG_ERR_UNSUPPORTED = -2, /* shape or dtype this build has no kernel for     */
+  RG_ERR_LAUNCH = -3,      /* hipLaunch / runtime error                       */
+  RG_ERR_WORKSPACE = -4    /* workspace missing or too small                  */
+};
+
+enum { RG_DTYPE_F32 = 0, RG_DTYPE_BF16 = 1 };
+
+#define RG_MAX_CONV_WIDTH 16
+
+/* Library identification. */
+int rg_abi_version(void);
+const char* rg_last_error(void);
+
+/* Conv1D.forward, prefill branch (cache is None):
+ * recurrentgemma/torch/layers.py:447-529 (mask :575-607, cache :526-527).
+ *   out[b,t,c] = bias[c] + sum_{s=0..min(K-1,t)} w[K-1-s,c] * x[b,t-s,c] * keep
+ *   keep = 0 iff some segpos[b,t-s+1..t] == 0.
+ * cache_out (nullable, [B,K-1,W]) receives the reference's masked tail
+ *   x[b,t,c] * prod_{j=1..min(K-1,T-1-t)} (segpos[b,t+j] != 0), t = T-K+1..T-1,
+ * zero-filled on the left when T < K-1.  2 <= K <= RG_MAX_CONV_WIDTH. */
+int rg_conv1d_prefill(const void* x, const void* segpos, int segpos_is_i64,
+                      const void* w, const void* bias, void* out,
+                      void* cache_out, int B, int T, int W, int K, int dtype,
+                      void* stream);
+
+/* Conv1D.forward, decode branch (cache given, exactly one token):
+ * recurrentgemma/torch/layers.py:469-474,491-529,531-550.  No document mask.
+ *   out[b,c] = bias[c] + sum_k w[k,c] * concat(cache_in, x)[b,k,c]
+ *   cache_out = concat(cache_in, x)[:,1:]      (may alias cache_in)
+ * x,out [B,1,W]; cache_in/out [B,K-1,W] in the activation dtype. */
+int rg_conv1d_step(const void* x, const void* cache_in, const void* w,
+                   const void* bias, void* out, void* cache_out, int B, int W,
+                   int K, int dtype, void* stream);
+
+/* BlockDiagonalLinear.forward: recurrentgemma/torch/layers.py:127-137.
+ *   y[m, h*bw + j] = b[h,j] + sum_i x[m, h*bw + i] * w[h,i,j]
+ * x,y [M, H*bw]; w [H,bw,bw] laid out [head, in, out]; b [H,bw]. */
+int rg_block_diag_linear(const void* x, const void* w, const void* b, void* y,
+                         int64_t M, int H, int bw, int dtype, void* stream);
+
+/* The two gate projections of RGLRU.forward (layers.py:338-339, before the
+ * sigmoid) in one pass over x:
+ *   gx_pre = input_gate(xc), ga_pre = a_gate(xc), both [B,T,W] in `dtype`.
+ * apply_conv == 0: xc = x (x is already the conv output).
+ * apply_conv != 0: xc = Conv1D(x) computed on load with the width-4 kernel
+ *   conv_w [4,W], conv_b [W] and the segpos mask (prefill semantics of
+ *   rg_conv1d_prefill, rounded to `dtype` like the reference's module output);
+ *   segpos must then be given.
+ * bw = W / H.  bf16 with bw == 256 runs on the MFMA kernel (weights held in
+ * registers, x tiles staged through LDS); any other combination runs on a
+ * plain FMA kernel with fp32 accumulation. */
+int rg_gates_gemm(const void* x, int apply_conv, const void* segpos,
+                  int segpos_is_i64, const void* conv_w, const void* conv_b,
+                  const void* w_x, const void* b_x, const void* w_a,
+                  const void* b_a, void* gx_pre, void* ga_pre, int B, int T,
+                  int W, int H, int dtype, void* stream);
+
+/* RGLRU.forward after the gate projections + rnn_scan, optionally with the
+ * width-4 Conv1D fused in front: recurrentgemma/torch/layers.py:335-365 and
+ * :140-191 (+ :447-529 when apply_conv).
+ *   xc      = apply_conv ? Conv1D(x) : x
+ *   r       = segpos == 0
+ *   gx, ga  = sigmoid(gx_pre), sigmoid(ga_pre)
+ *   a       = r ? 0 : exp(-8 * ga * softplus(a_param))
+ *   xn      = xc * gx * (r ? 1 : sqrt(1 - a^2))
+ *   h_t     = a_t * h_{t-1} + xn_t     (float32 state, h_{-1} = h0 or 0)
+ *   y_t     = h_t rounded to `dtype`
+ * h0 (nullable) and h_last (nullable) are float32 [B,W]; h_last may alias h0.
+ * conv_cache_out (nullable, only with apply_conv) is the [B,3,W] masked tail
+ * described at rg_conv1d_prefill.  The recurrence over T runs as a chunked
+ * parallel scan (per-wave local scans of (a, xn) pairs, carries combined
+ * across the waves of a workgroup). */
+int rg_lru_scan_fused(const void* x, int apply_conv, const void* conv_w,
+                      const void* conv_b, const void* gx_pre,
+                      const void* ga_pre, const void* a_param,
+                      const void* segpos, int segpos_is_i64, const void* h0,
+                      void* y, void* h_last, void* conv_cache_out, int B, int T,
+                      int W, int dtype, void* stream);
+
+/* rnn_scan: recurrentgemma/torch/layers.py:140-191.
+ *   h_t = (reset_t ? 0 : a_t) * h_{t-1} + x_t,  y_t = h_t rounded to `dtype`
+ * x, a, y [B,T,W] in `dtype`; reset [B,T] bytes (non-zero = reset, the memory
+ * of a torch.bool tensor); h0 (nullable) / h_last (nullable) float32 [B,W].
+ * Same chunked scan kernel as rg_lru_scan_fused without the gating. */
+int rg_linear_scan(const void* x, const void* a, const void* reset,
+                   const void* h0, void* y, void* h_last, int B, int T, int W,
+                   int dtype, void* stream);
+
+/* One decode step of the conv -> RG-LRU core, as RecurrentBlock.forward chains
+ * them with a cache (recurrentgemma/torch/modules.py:632-643 with
+ * layers.py:469-474 and :170-177): x [B,1,W], segpos [B,1],
+ * conv_cache_in/out [B,3,W] (`dtype`), h_in/h_out [B,W] float32 (outputs may
+ * alias inputs), y [B,1,W].  `workspace` must hold at least
+ * rg_recurrent_step_workspace_bytes(B, W, dtype) bytes of device memory. */
+size_t rg_recurrent_step_workspace_bytes(int B, int W, int dtype);
+int rg_recurrent_step(const void* x, const void* segpos, int segpos_is_i64,
+                      const void* conv_cache_in, void* conv_cache_out,
+                      const void* h_in, void* h_out, const void* conv_w,
+                      const void* conv_b, const void* w_x, const void* b_x,
+                      const void* w_a, const void* b_a, const void* a_param,
+                      void* y, void* workspace, size_t workspace_bytes, int B,
+                      int W, int H, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RG_LRU_H_ */

@@ -1,0 +1,85 @@
+"""Loads librg_lru.so (the gfx950 HIP kernels behind a C ABI) with ctypes.
+
+There is no CPU or eager-torch fallback: if the library is missing or a kernel
+call fails, the caller gets an exception.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "librg_lru.so")
+CSRC = os.path.join(_HERE, "csrc")
+
+RG_OK = 0
+RG_DTYPE_F32 = 0
+RG_DTYPE_BF16 = 1
+ABI_VERSION = 1
+
+_vp = ctypes.c_void_p
+_i = ctypes.c_int
+_i64 = ctypes.c_int64
+_sz = ctypes.c_size_t
+
+# name -> (restype, argtypes); mirrors include/rg_lru.h declaration by declaration
+SIGNATURES = {
+    "rg_abi_version": (_i, []),
+    "rg_last_error": (ctypes.c_char_p, []),
+    "rg_conv1d_prefill": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i,
+                               _i, _vp]),
+    "rg_conv1d_step": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "rg_block_diag_linear": (_i, [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp]),
+    "rg_gates_gemm": (_i, [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                           _vp, _i, _i, _i, _i, _i, _vp]),
+    "rg_lru_scan_fused": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp,
+                               _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "rg_linear_scan": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "rg_recurrent_step_workspace_bytes": (_sz, [_i, _i, _i]),
+    "rg_recurrent_step": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                               _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i,
+                               _vp]),
+}
+
+_lib = None
+
+
+class KernelError(RuntimeError):
+  """A C-ABI call returned a non-zero status."""
+
+
+def build(force: bool = True) -> str:
+  """Compiles the HIP sources for gfx950 into librg_lru.so (in-tree)."""
+  cmd = ["make", "-C", CSRC, "-j4"]
+  if force:
+    cmd.append("-B")
+  subprocess.check_call(cmd)
+  return LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+  global _lib
+  if _lib is None:
+    if not os.path.exists(LIB_PATH):
+      raise RuntimeError(
+          f"{LIB_PATH} is missing: build it with `make -C {CSRC}` "
+          "(or __graft_entry__.build()). recurrentgemma_amd has no fallback "
+          "path without its HIP library.")
+    handle = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+      fn = getattr(handle, name)
+      fn.restype = res
+      fn.argtypes = args
+    got = handle.rg_abi_version()
+    if got != ABI_VERSION:
+      raise RuntimeError(f"librg_lru.so has ABI {got}, expected {ABI_VERSION}")
+    _lib = handle
+  return _lib
+
+
+def check(status: int) -> None:
+  if status != RG_OK:
+    msg = lib().rg_last_error().decode("utf-8", "replace")
+    raise KernelError(f"librg_lru status {status}: {msg}")

@@ -1,0 +1,298 @@
+// extern "C" boundary of librg_lru.so: argument checks, dispatch, errors.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "../../include/rg_lru.h"
+#include "rg_internal.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int launch_status(const char* what, hipError_t e) {
+  if (e == hipSuccess) return RG_OK;
+  return fail(RG_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+size_t esize(int dtype) { return dtype == RG_DTYPE_F32 ? 4 : 2; }
+
+#define RG_REQUIRE(cond, ...) \
+  do {                        \
+    if (!(cond)) return fail(RG_ERR_BAD_ARG, __VA_ARGS__); \
+  } while (0)
+
+#define RG_CHECK_DTYPE(dtype)                                            \
+  do {                                                                   \
+    if ((dtype) != RG_DTYPE_F32 && (dtype) != RG_DTYPE_BF16)             \
+      return fail(RG_ERR_UNSUPPORTED, "%s: dtype %d is not f32/bf16",    \
+                  __func__, (dtype));                                    \
+  } while (0)
+
+#define RG_CHECK_PTR(p)                                                     \
+  do {                                                                      \
+    RG_REQUIRE((p) != nullptr, "%s: %s is null", __func__, #p);             \
+    RG_REQUIRE(aligned16(p), "%s: %s is not 16-byte aligned", __func__, #p); \
+  } while (0)
+
+#define RG_CHECK_OPT_PTR(p) \
+  RG_REQUIRE(aligned16(p), "%s: %s is not 16-byte aligned", __func__, #p)
+
+}  // namespace
+
+extern "C" {
+
+int rg_abi_version(void) { return RG_ABI_VERSION; }
+
+const char* rg_last_error(void) { return g_err; }
+
+int rg_conv1d_prefill(const void* x, const void* segpos, int segpos_is_i64,
+                      const void* w, const void* bias, void* out,
+                      void* cache_out, int B, int T, int W, int K, int dtype,
+                      void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(B > 0 && T > 0 && W > 0, "%s: B=%d T=%d W=%d must be positive",
+             __func__, B, T, W);
+  if (K < 2 || K > RG_MAX_CONV_WIDTH)
+    return fail(RG_ERR_UNSUPPORTED, "%s: temporal width %d outside [2,%d]",
+                __func__, K, RG_MAX_CONV_WIDTH);
+  RG_CHECK_PTR(x);
+  RG_CHECK_PTR(segpos);
+  RG_CHECK_PTR(w);
+  RG_CHECK_PTR(bias);
+  RG_CHECK_PTR(out);
+  RG_CHECK_OPT_PTR(cache_out);
+  RG_REQUIRE(out != x, "%s: out must not alias x", __func__);
+  rg::ConvArgs a{x, segpos, segpos_is_i64 ? 1 : 0, w, bias, out, cache_out,
+                 B, T, W, K};
+  return launch_status(__func__,
+                       rg::launch_conv1d_prefill(a, dtype, (hipStream_t)stream));
+}
+
+int rg_conv1d_step(const void* x, const void* cache_in, const void* w,
+                   const void* bias, void* out, void* cache_out, int B, int W,
+                   int K, int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(B > 0 && W > 0, "%s: B=%d W=%d must be positive", __func__, B, W);
+  if (K < 2 || K > RG_MAX_CONV_WIDTH)
+    return fail(RG_ERR_UNSUPPORTED, "%s: temporal width %d outside [2,%d]",
+                __func__, K, RG_MAX_CONV_WIDTH);
+  RG_CHECK_PTR(x);
+  RG_CHECK_PTR(cache_in);
+  RG_CHECK_PTR(w);
+  RG_CHECK_PTR(bias);
+  RG_CHECK_PTR(out);
+  RG_CHECK_OPT_PTR(cache_out);
+  RG_REQUIRE(out != x, "%s: out must not alias x", __func__);
+  rg::ConvStepArgs a{x, cache_in, w, bias, out, cache_out, B, W, K};
+  return launch_status(__func__,
+                       rg::launch_conv1d_step(a, dtype, (hipStream_t)stream));
+}
+
+int rg_block_diag_linear(const void* x, const void* w, const void* b, void* y,
+                         int64_t M, int H, int bw, int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(M > 0 && H > 0 && bw > 0, "%s: M=%lld H=%d bw=%d must be positive",
+             __func__, (long long)M, H, bw);
+  RG_REQUIRE((int64_t)H * bw <= 0x7fffffff, "%s: width overflows", __func__);
+  RG_CHECK_PTR(x);
+  RG_CHECK_PTR(w);
+  RG_CHECK_PTR(b);
+  RG_CHECK_PTR(y);
+  RG_REQUIRE(y != x, "%s: y must not alias x", __func__);
+  rg::GemmArgs a{};
+  a.x = x;
+  a.w[0] = w;
+  a.b[0] = b;
+  a.out[0] = y;
+  a.ngates = 1;
+  a.M = M;
+  a.T = 1;
+  a.W = H * bw;
+  a.H = H;
+  a.bw = bw;
+  return launch_status(__func__,
+                       rg::launch_gemm_generic(a, dtype, (hipStream_t)stream));
+}
+
+int rg_gates_gemm(const void* x, int apply_conv, const void* segpos,
+                  int segpos_is_i64, const void* conv_w, const void* conv_b,
+                  const void* w_x, const void* b_x, const void* w_a,
+                  const void* b_a, void* gx_pre, void* ga_pre, int B, int T,
+                  int W, int H, int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(B > 0 && T > 0 && W > 0 && H > 0,
+             "%s: B=%d T=%d W=%d H=%d must be positive", __func__, B, T, W, H);
+  RG_REQUIRE(W % H == 0, "%s: W=%d is not a multiple of H=%d", __func__, W, H);
+  RG_CHECK_PTR(x);
+  RG_CHECK_PTR(w_x);
+  RG_CHECK_PTR(b_x);
+  RG_CHECK_PTR(w_a);
+  RG_CHECK_PTR(b_a);
+  RG_CHECK_PTR(gx_pre);
+  RG_CHECK_PTR(ga_pre);
+  RG_REQUIRE(gx_pre != x && ga_pre != x && gx_pre != ga_pre,
+             "%s: outputs must not alias x or each other", __func__);
+  if (apply_conv) {
+    RG_CHECK_PTR(segpos);
+    RG_CHECK_PTR(conv_w);
+    RG_CHECK_PTR(conv_b);
+  }
+  rg::GemmArgs a{};
+  a.x = x;
+  a.apply_conv = apply_conv != 0;
+  a.segpos = segpos;
+  a.seg_kind = segpos_is_i64 ? 1 : 0;
+  a.conv_w = conv_w;
+  a.conv_b = conv_b;
+  a.w[0] = w_x;
+  a.b[0] = b_x;
+  a.w[1] = w_a;
+  a.b[1] = b_a;
+  a.out[0] = gx_pre;
+  a.out[1] = ga_pre;
+  a.ngates = 2;
+  a.M = (int64_t)B * T;
+  a.T = T;
+  a.W = W;
+  a.H = H;
+  a.bw = W / H;
+  hipError_t e;
+  if (dtype == RG_DTYPE_BF16 && a.bw == 256)
+    e = rg::launch_gemm_mfma_bf16(a, (hipStream_t)stream);
+  else
+    e = rg::launch_gemm_generic(a, dtype, (hipStream_t)stream);
+  return launch_status(__func__, e);
+}
+
+int rg_lru_scan_fused(const void* x, int apply_conv, const void* conv_w,
+                      const void* conv_b, const void* gx_pre,
+                      const void* ga_pre, const void* a_param,
+                      const void* segpos, int segpos_is_i64, const void* h0,
+                      void* y, void* h_last, void* conv_cache_out, int B, int T,
+                      int W, int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(B > 0 && T > 0 && W > 0, "%s: B=%d T=%d W=%d must be positive",
+             __func__, B, T, W);
+  RG_CHECK_PTR(x);
+  RG_CHECK_PTR(gx_pre);
+  RG_CHECK_PTR(ga_pre);
+  RG_CHECK_PTR(a_param);
+  RG_CHECK_PTR(segpos);
+  RG_CHECK_PTR(y);
+  RG_CHECK_OPT_PTR(h0);
+  RG_CHECK_OPT_PTR(h_last);
+  RG_CHECK_OPT_PTR(conv_cache_out);
+  RG_REQUIRE(y != x && y != gx_pre && y != ga_pre,
+             "%s: y must not alias an input", __func__);
+  if (apply_conv) {
+    RG_CHECK_PTR(conv_w);
+    RG_CHECK_PTR(conv_b);
+  } else {
+    RG_REQUIRE(conv_cache_out == nullptr,
+               "%s: conv_cache_out needs apply_conv", __func__);
+  }
+  rg::ScanArgs a{};
+  a.x = x;
+  a.apply_conv = apply_conv != 0;
+  a.conv_w = conv_w;
+  a.conv_b = conv_b;
+  a.gx = gx_pre;
+  a.ga = ga_pre;
+  a.a_param = a_param;
+  a.segpos = segpos;
+  a.seg_kind = segpos_is_i64 ? 1 : 0;
+  a.h0 = (const float*)h0;
+  a.y = y;
+  a.h_last = (float*)h_last;
+  a.cache_out = conv_cache_out;
+  a.B = B;
+  a.T = T;
+  a.W = W;
+  return launch_status(__func__,
+                       rg::launch_lru_scan(a, dtype, (hipStream_t)stream));
+}
+
+int rg_linear_scan(const void* x, const void* a, const void* reset,
+                   const void* h0, void* y, void* h_last, int B, int T, int W,
+                   int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(B > 0 && T > 0 && W > 0, "%s: B=%d T=%d W=%d must be positive",
+             __func__, B, T, W);
+  RG_CHECK_PTR(x);
+  RG_CHECK_PTR(a);
+  RG_CHECK_PTR(reset);
+  RG_CHECK_PTR(y);
+  RG_CHECK_OPT_PTR(h0);
+  RG_CHECK_OPT_PTR(h_last);
+  RG_REQUIRE(y != x && y != a, "%s: y must not alias an input", __func__);
+  rg::ScanArgs s{};
+  s.plain = 1;
+  s.x = x;
+  s.gx = x;  // unused in this mode
+  s.ga = a;
+  s.segpos = reset;
+  s.seg_kind = 2;
+  s.h0 = (const float*)h0;
+  s.y = y;
+  s.h_last = (float*)h_last;
+  s.B = B;
+  s.T = T;
+  s.W = W;
+  return launch_status(__func__,
+                       rg::launch_lru_scan(s, dtype, (hipStream_t)stream));
+}
+
+size_t rg_recurrent_step_workspace_bytes(int B, int W, int dtype) {
+  if (B <= 0 || W <= 0) return 0;
+  // conv output + two gate pre-activations, each [B,W], 256-byte aligned
+  size_t one = ((size_t)B * W * esize(dtype) + 255) & ~(size_t)255;
+  return 3 * one;
+}
+
+int rg_recurrent_step(const void* x, const void* segpos, int segpos_is_i64,
+                      const void* conv_cache_in, void* conv_cache_out,
+                      const void* h_in, void* h_out, const void* conv_w,
+                      const void* conv_b, const void* w_x, const void* b_x,
+                      const void* w_a, const void* b_a, const void* a_param,
+                      void* y, void* workspace, size_t workspace_bytes, int B,
+                      int W, int H, int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(B > 0 && W > 0 && H > 0, "%s: B=%d W=%d H=%d must be positive",
+             __func__, B, W, H);
+  RG_REQUIRE(W % H == 0, "%s: W=%d is not a multiple of H=%d", __func__, W, H);
+  RG_CHECK_PTR(conv_cache_in);
+  RG_CHECK_PTR(conv_cache_out);
+  RG_CHECK_PTR(h_in);
+  RG_CHECK_PTR(h_out);
+  const size_t need = rg_recurrent_step_workspace_bytes(B, W, dtype);
+  if (workspace == nullptr || workspace_bytes < need || !aligned16(workspace))
+    return fail(RG_ERR_WORKSPACE,
+                "%s: workspace of %zu bytes (16-byte aligned) required, got %zu",
+                __func__, need, workspace ? workspace_bytes : (size_t)0);
+  const size_t one = need / 3;
+  char* ws = (char*)workspace;
+  void* xc = ws;
+  void* gx = ws + one;
+  void* ga = ws + 2 * one;
+  int rc = rg_conv1d_step(x, conv_cache_in, conv_w, conv_b, xc, conv_cache_out,
+                          B, W, 4, dtype, stream);
+  if (rc != RG_OK) return rc;
+  rc = rg_gates_gemm(xc, 0, nullptr, 0, nullptr, nullptr, w_x, b_x, w_a, b_a, gx,
+                     ga, B, 1, W, H, dtype, stream);
+  if (rc != RG_OK) return rc;
+  return rg_lru_scan_fused(xc, 0, nullptr, nullptr, gx, ga, a_param, segpos,
+                           segpos_is_i64, h_in, y, h_out, nullptr, B, 1, W,
+                           dtype, stream);
+}
+
+}  // extern "C"

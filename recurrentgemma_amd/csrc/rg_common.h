@@ -1,0 +1,179 @@
+// Shared device helpers for the gfx950 Conv1D + RG-LRU kernels.
+#ifndef RG_COMMON_H_
+#define RG_COMMON_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace rg {
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int kWave = 64;
+
+// ---------------------------------------------------------------- bf16 ----
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) {
+  return __uint_as_float(bits16 << 16);
+}
+// Round-to-nearest-even float -> bf16 (v_cvt_pk_bf16_f32 on gfx950).
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  f32x2 v = {lo, hi};
+  bf16x2 p = __builtin_convertvector(v, bf16x2);
+  return *reinterpret_cast<uint32_t*>(&p);
+}
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float v) {
+  return (uint16_t)(pack_bf16x2(v, 0.0f) & 0xffffu);
+}
+__device__ __forceinline__ float round_to_bf16(float v) {
+  return bf16_bits_to_f32(f32_to_bf16_bits(v));
+}
+
+// ------------------------------------------------------- element traits ----
+// Act<T>: how CH adjacent channels of an activation tensor are read into
+// floats and written back.  T is float or uint16_t (bf16 bit pattern).
+template <typename T, int CH>
+struct Act;
+
+template <>
+struct Act<float, 1> {
+  static constexpr bool kIsBf16 = false;
+  __device__ static void load(const float* p, float (&v)[1]) { v[0] = *p; }
+  __device__ static void store(float* p, const float (&v)[1]) { *p = v[0]; }
+  __device__ static float round(float v) { return v; }
+};
+template <>
+struct Act<float, 2> {
+  static constexpr bool kIsBf16 = false;
+  __device__ static void load(const float* p, float (&v)[2]) {
+    f32x2 t = *reinterpret_cast<const f32x2*>(p);
+    v[0] = t.x;
+    v[1] = t.y;
+  }
+  __device__ static void store(float* p, const float (&v)[2]) {
+    f32x2 t = {v[0], v[1]};
+    *reinterpret_cast<f32x2*>(p) = t;
+  }
+  __device__ static float round(float v) { return v; }
+};
+template <>
+struct Act<uint16_t, 1> {
+  static constexpr bool kIsBf16 = true;
+  __device__ static void load(const uint16_t* p, float (&v)[1]) {
+    v[0] = bf16_bits_to_f32(*p);
+  }
+  __device__ static void store(uint16_t* p, const float (&v)[1]) {
+    *p = f32_to_bf16_bits(v[0]);
+  }
+  __device__ static float round(float v) { return round_to_bf16(v); }
+};
+template <>
+struct Act<uint16_t, 2> {
+  static constexpr bool kIsBf16 = true;
+  __device__ static void load(const uint16_t* p, float (&v)[2]) {
+    uint32_t u = *reinterpret_cast<const uint32_t*>(p);
+    v[0] = __uint_as_float(u << 16);
+    v[1] = __uint_as_float(u & 0xffff0000u);
+  }
+  __device__ static void store(uint16_t* p, const float (&v)[2]) {
+    *reinterpret_cast<uint32_t*>(p) = pack_bf16x2(v[0], v[1]);
+  }
+  __device__ static float round(float v) { return round_to_bf16(v); }
+};
+
+template <typename T>
+__device__ __forceinline__ float load_scalar(const T* p);
+template <>
+__device__ __forceinline__ float load_scalar<float>(const float* p) {
+  return *p;
+}
+template <>
+__device__ __forceinline__ float load_scalar<uint16_t>(const uint16_t* p) {
+  return bf16_bits_to_f32(*p);
+}
+template <typename T>
+__device__ __forceinline__ void store_scalar(T* p, float v);
+template <>
+__device__ __forceinline__ void store_scalar<float>(float* p, float v) {
+  *p = v;
+}
+template <>
+__device__ __forceinline__ void store_scalar<uint16_t>(uint16_t* p, float v) {
+  *p = f32_to_bf16_bits(v);
+}
+template <typename T>
+__device__ __forceinline__ float round_act(float v);
+template <>
+__device__ __forceinline__ float round_act<float>(float v) {
+  return v;
+}
+template <>
+__device__ __forceinline__ float round_act<uint16_t>(float v) {
+  return round_to_bf16(v);
+}
+
+// ------------------------------------------------------ segment_pos ----
+// How document starts are encoded: int32 / int64 positions (start == 0), or a
+// byte mask (start != 0) as rnn_scan's `reset` argument.
+enum SegKind { kSegI32 = 0, kSegI64 = 1, kSegMaskU8 = 2 };
+
+__device__ __forceinline__ bool is_doc_start(const void* segpos, int kind,
+                                             int64_t idx) {
+  if (kind == kSegI64) return reinterpret_cast<const int64_t*>(segpos)[idx] == 0;
+  if (kind == kSegMaskU8) return reinterpret_cast<const uint8_t*>(segpos)[idx] != 0;
+  return reinterpret_cast<const int32_t*>(segpos)[idx] == 0;
+}
+
+// ------------------------------------------------------------- conv ----
+// Width-4 tap chain in the one fixed order every kernel uses, so that the gate
+// GEMM (conv on load) and the scan kernel see bit-identical conv outputs:
+// newest tap first, bias as the starting value, fused multiply-adds.
+// x0 = x[t], x1 = x[t-1], ... ; w3 multiplies x[t] (layers.py:514).
+__device__ __forceinline__ float conv4(float x0, float x1, float x2, float x3,
+                                       float w0, float w1, float w2, float w3,
+                                       float bias) {
+  float acc = __builtin_fmaf(x0, w3, bias);
+  acc = __builtin_fmaf(x1, w2, acc);
+  acc = __builtin_fmaf(x2, w1, acc);
+  acc = __builtin_fmaf(x3, w0, acc);
+  return acc;
+}
+
+// Generic-width conv output at flattened row m = b*T + t, channel c, straight
+// from the definition (same accumulation order as conv4 for K == 4).
+template <typename T>
+__device__ __forceinline__ float conv_point(const T* x, const void* segpos,
+                                            int seg_kind, const T* w,
+                                            const T* bias, int T_len, int W,
+                                            int K, int64_t m, int c) {
+  int t = (int)(m % T_len);
+  float acc = load_scalar(bias + c);
+  bool alive = true;
+  for (int s = 0; s < K && s <= t; ++s) {
+    if (s > 0 && is_doc_start(segpos, seg_kind, m - s + 1)) alive = false;
+    float v = alive ? load_scalar(x + (m - s) * W + c) : 0.0f;
+    acc = __builtin_fmaf(v, load_scalar(w + (int64_t)(K - 1 - s) * W + c), acc);
+  }
+  return round_act<T>(acc);
+}
+
+// ------------------------------------------------------------- math ----
+constexpr float kLog2e = 1.4426950408889634f;
+
+__device__ __forceinline__ float softplus_precise(float v) {
+  return v > 20.0f ? v : log1pf(expf(v));
+}
+__device__ __forceinline__ float sigmoid_precise(float v) {
+  return 1.0f / (1.0f + expf(-v));
+}
+// Hardware exp2/rcp (about 1 ulp each): used on the bf16 path.
+__device__ __forceinline__ float sigmoid_fast(float v) {
+  float e = __builtin_amdgcn_exp2f(-kLog2e * v);
+  return __builtin_amdgcn_rcpf(1.0f + e);
+}
+
+}  // namespace rg
+#endif  // RG_COMMON_H_

@@ -1,0 +1,348 @@
+// Block-diagonal gate projections (BlockDiagonalLinear) for gfx950.
+//
+// Two kernels:
+//  * gates_mfma_bf16_kernel: bf16, block width 256.  Weight-stationary: each of
+//    the 8 waves of a workgroup keeps a 256(K) x 64(N) slice of the two gates'
+//    weights ([W_x | W_a], N = 512) in registers as MFMA B fragments for the
+//    whole kernel and the group walks over 64-row tiles of x, staged (and
+//    optionally convolved) through double-buffered LDS.  fp32 accumulation on
+//    v_mfma_f32_32x32x16_bf16, bias added in fp32, one rounding to bf16.
+//  * bdl_generic_kernel: any dtype / block width, LDS-tiled FMA with fp32
+//    accumulation (used for fp32 and for block widths other than 256).
+#include "rg_common.h"
+#include "rg_internal.h"
+
+namespace rg {
+namespace {
+
+// ===================================================== generic FMA kernel ==
+
+constexpr int kGT = 64;  // output tile edge
+constexpr int kGK = 16;  // K chunk
+
+template <typename T, bool CONV>
+__global__ void __launch_bounds__(256) bdl_generic_kernel(GemmArgs p) {
+  __shared__ float As[kGK][kGT + 4];
+  __shared__ float Bs[kGK][kGT + 4];
+  const int tid = threadIdx.x;
+  const int tx = tid & 15, ty = tid >> 4;
+  const int z = blockIdx.z;
+  const int gate = z / p.H;
+  const int h = z - gate * p.H;
+  const int bw = p.bw;
+  const int64_t m0 = (int64_t)blockIdx.x * kGT;
+  const int n0 = blockIdx.y * kGT;
+  const T* x = (const T*)p.x;
+  const T* w = (const T*)p.w[gate] + (int64_t)h * bw * bw;
+  const T* bias = (const T*)p.b[gate] + (int64_t)h * bw;
+  T* out = (T*)p.out[gate];
+
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.0f;
+
+  for (int k0 = 0; k0 < bw; k0 += kGK) {
+#pragma unroll
+    for (int e = tid; e < kGT * kGK; e += 256) {
+      const int r = e / kGK, kk = e % kGK;
+      const int64_t m = m0 + r;
+      float v = 0.0f;
+      if (m < p.M && k0 + kk < bw) {
+        const int c = h * bw + k0 + kk;
+        if (CONV)
+          v = conv_point<T>(x, p.segpos, p.seg_kind, (const T*)p.conv_w,
+                            (const T*)p.conv_b, p.T, p.W, 4, m, c);
+        else
+          v = load_scalar(x + m * p.W + c);
+      }
+      As[kk][r] = v;
+    }
+#pragma unroll
+    for (int e = tid; e < kGT * kGK; e += 256) {
+      const int kk = e / kGT, n = e % kGT;
+      float v = 0.0f;
+      if (k0 + kk < bw && n0 + n < bw)
+        v = load_scalar(w + (int64_t)(k0 + kk) * bw + n0 + n);
+      Bs[kk][n] = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < kGK; ++kk) {
+      float av[4], bv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) av[i] = As[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) bv[j] = Bs[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_fmaf(av[i], bv[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t m = m0 + ty * 4 + i;
+    if (m >= p.M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n < bw)
+        store_scalar(out + m * p.W + h * bw + n,
+                     acc[i][j] + load_scalar(bias + n));
+    }
+  }
+}
+
+// ======================================================= bf16 MFMA kernel ==
+
+constexpr int kBW = 256;          // block width (K and per-gate N)
+constexpr int kTM = 64;           // rows of x per tile
+constexpr int kLdsStride = 264;   // bf16 elements per LDS row (256 + 8 pad)
+constexpr int kRowsPerGroup = 16; // rows each thread converts per tile
+constexpr size_t kMfmaLdsBytes = 2ull * kTM * kLdsStride * sizeof(uint16_t);
+
+union Frag {
+  bf16x8 v;
+  uint16_t u[8];
+  f32x4 q;
+};
+
+template <bool CONV>
+__global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  uint16_t* lds = reinterpret_cast<uint16_t*>(lds_raw);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int h = blockIdx.y;
+  const int64_t M = p.M;
+  const int64_t W = p.W;
+  const int T_len = p.T;
+  const int64_t ntiles = (M + kTM - 1) / kTM;
+
+  // ---- this wave's weight slice, resident in registers -----------------
+  const int gate = wave >> 2;         // waves 0-3: input gate, 4-7: a gate
+  const int n0 = (wave & 3) * 64;     // first output column inside the gate
+  // The weights are [k][n] with n contiguous, the MFMA B operand wants 8
+  // consecutive k per lane: transpose through LDS, 128 k-rows of one gate at
+  // a time (coalesced 16-byte global reads, 2-byte LDS reads).
+  Frag bfrag[16][2];
+#pragma unroll
+  for (int g = 0; g < 2; ++g) {
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh) {
+      const uint16_t* src =
+          (const uint16_t*)p.w[g] + ((int64_t)h * kBW + kh * 128) * kBW;
+      for (int e = tid; e < 128 * 32; e += 512) {
+        const int r = e >> 5, q = e & 31;
+        *reinterpret_cast<f32x4*>(lds + (size_t)r * kLdsStride + q * 8) =
+            *reinterpret_cast<const f32x4*>(src + (size_t)r * kBW + q * 8);
+      }
+      __syncthreads();
+      if (gate == g) {
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+          for (int nt = 0; nt < 2; ++nt) {
+            const int n = n0 + nt * 32 + (lane & 31);
+            const int kb = ks * 16 + 8 * (lane >> 5);
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              bfrag[kh * 8 + ks][nt].u[e] = lds[(size_t)(kb + e) * kLdsStride + n];
+          }
+      }
+      __syncthreads();
+    }
+  }
+  float biasv[2];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt)
+    biasv[nt] = bf16_bits_to_f32(
+        ((const uint16_t*)p.b[gate])[h * kBW + n0 + nt * 32 + (lane & 31)]);
+  uint16_t* outp = (uint16_t*)p.out[gate] + h * kBW + n0 + (lane & 31);
+
+  // ---- x staging: thread -> (channel pair, group of 16 rows) -----------
+  const int cp = tid & 127;
+  const int rg = __builtin_amdgcn_readfirstlane(tid >> 7);
+  const int c = h * kBW + cp * 2;
+  const uint16_t* xcol = (const uint16_t*)p.x + c;
+  float cw0[2], cw1[2], cw2[2], cw3[2], cb[2];
+  if (CONV) {
+    const uint16_t* cw = (const uint16_t*)p.conv_w;
+#pragma unroll
+    for (int ch = 0; ch < 2; ++ch) {
+      cw0[ch] = bf16_bits_to_f32(cw[c + ch]);
+      cw1[ch] = bf16_bits_to_f32(cw[W + c + ch]);
+      cw2[ch] = bf16_bits_to_f32(cw[2 * W + c + ch]);
+      cw3[ch] = bf16_bits_to_f32(cw[3 * W + c + ch]);
+      cb[ch] = bf16_bits_to_f32(((const uint16_t*)p.conv_b)[c + ch]);
+    }
+  }
+  constexpr int kHalo = CONV ? 3 : 0;
+  constexpr int kRaw = kRowsPerGroup + kHalo;
+  uint32_t raw[kRaw];
+
+  auto fetch = [&](int64_t tile) {
+    const int64_t mbase = tile * kTM + rg * kRowsPerGroup - kHalo;
+#pragma unroll
+    for (int j = 0; j < kRaw; ++j) {
+      int64_t m = mbase + j;
+      m = m < 0 ? 0 : (m >= M ? M - 1 : m);
+      raw[j] = *reinterpret_cast<const uint32_t*>(xcol + m * W);
+    }
+  };
+
+  auto stage = [&](int64_t tile, int buf) {
+    uint16_t* dst = lds + (size_t)buf * kTM * kLdsStride +
+                    (size_t)(rg * kRowsPerGroup) * kLdsStride + cp * 2;
+    if (!CONV) {
+#pragma unroll
+      for (int i = 0; i < kRowsPerGroup; ++i)
+        *reinterpret_cast<uint32_t*>(dst + (size_t)i * kLdsStride) = raw[i];
+      return;
+    }
+    const int64_t mbase = tile * kTM + rg * kRowsPerGroup - kHalo;
+    // bit j: row mbase+j begins a sequence row (t == 0) or a document; the
+    // conv must not look past it.
+    uint32_t cut = 0;
+    int t = (int)(((mbase % T_len) + T_len) % T_len);  // token index of row 0
+#pragma unroll
+    for (int j = 0; j < kRaw; ++j) {
+      const int64_t m = mbase + j;
+      if (m >= 0 && m < M) {
+        const bool st = (t == 0) || is_doc_start(p.segpos, p.seg_kind, m);
+        if (st) cut |= 1u << j;
+      }
+      t = (t + 1 == T_len) ? 0 : t + 1;
+    }
+    float h0[2] = {0.f, 0.f}, h1[2] = {0.f, 0.f}, h2[2] = {0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < kRaw; ++j) {
+      float xv[2];
+      xv[0] = __uint_as_float(raw[j] << 16);
+      xv[1] = __uint_as_float(raw[j] & 0xffff0000u);
+      if ((cut >> j) & 1u) {
+        h0[0] = h0[1] = h1[0] = h1[1] = h2[0] = h2[1] = 0.0f;
+      }
+      if (j >= kHalo) {
+        const float o0 = conv4(xv[0], h0[0], h1[0], h2[0], cw0[0], cw1[0],
+                               cw2[0], cw3[0], cb[0]);
+        const float o1 = conv4(xv[1], h0[1], h1[1], h2[1], cw0[1], cw1[1],
+                               cw2[1], cw3[1], cb[1]);
+        *reinterpret_cast<uint32_t*>(dst + (size_t)(j - kHalo) * kLdsStride) =
+            pack_bf16x2(o0, o1);
+      }
+#pragma unroll
+      for (int ch = 0; ch < 2; ++ch) {
+        h2[ch] = h1[ch];
+        h1[ch] = h0[ch];
+        h0[ch] = xv[ch];
+      }
+    }
+  };
+
+  int64_t tile = blockIdx.x;
+  if (tile < ntiles) {
+    fetch(tile);
+    stage(tile, 0);
+  }
+  __syncthreads();
+
+  int buf = 0;
+  for (; tile < ntiles; tile += gridDim.x, buf ^= 1) {
+    const int64_t next = tile + gridDim.x;
+    const bool has_next = next < ntiles;
+    if (has_next) fetch(next);
+
+    // One 32-row half of the tile at a time keeps only 32 accumulator
+    // registers live next to the 128 registers of resident weights.
+    const uint16_t* abase = lds + (size_t)buf * kTM * kLdsStride +
+                            (size_t)(lane & 31) * kLdsStride + 8 * (lane >> 5);
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) {
+      f32x16 acc0, acc1;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        acc0[r] = 0.0f;
+        acc1[r] = 0.0f;
+      }
+      const uint16_t* arow = abase + (size_t)mt * 32 * kLdsStride;
+#pragma unroll
+      for (int ks = 0; ks < 16; ++ks) {
+        Frag a;
+        a.q = *reinterpret_cast<const f32x4*>(arow + ks * 16);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, bfrag[ks][0].v,
+                                                       acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, bfrag[ks][1].v,
+                                                       acc1, 0, 0, 0);
+      }
+      // epilogue: D[i][j], i = 8*(r/4) + 4*(lane/32) + r%4, j = lane%32
+      const int64_t mrow0 = tile * kTM + mt * 32 + 4 * (lane >> 5);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int64_t m = mrow0 + 8 * (r >> 2) + (r & 3);
+        if (m < M) {
+          outp[m * W] = f32_to_bf16_bits(acc0[r] + biasv[0]);
+          outp[m * W + 32] = f32_to_bf16_bits(acc1[r] + biasv[1]);
+        }
+      }
+    }
+
+    if (has_next) stage(next, buf ^ 1);
+    __syncthreads();
+  }
+}
+
+}  // namespace
+
+hipError_t launch_gemm_generic(const GemmArgs& a, int dtype, hipStream_t s) {
+  const int64_t mt = (a.M + kGT - 1) / kGT;
+  const int ntl = (a.bw + kGT - 1) / kGT;
+  if (mt > 0x7fffffff || (int64_t)a.H * a.ngates > 65535 || ntl > 65535)
+    return hipErrorInvalidValue;
+  dim3 grid((unsigned)mt, (unsigned)ntl, (unsigned)(a.H * a.ngates));
+  if (dtype == 0) {
+    if (a.apply_conv)
+      bdl_generic_kernel<float, true><<<grid, 256, 0, s>>>(a);
+    else
+      bdl_generic_kernel<float, false><<<grid, 256, 0, s>>>(a);
+  } else {
+    if (a.apply_conv)
+      bdl_generic_kernel<uint16_t, true><<<grid, 256, 0, s>>>(a);
+    else
+      bdl_generic_kernel<uint16_t, false><<<grid, 256, 0, s>>>(a);
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_gemm_mfma_bf16(const GemmArgs& a, hipStream_t s) {
+  // needs both gates, bw == 256 (checked by the caller)
+  const int64_t ntiles = (a.M + kTM - 1) / kTM;
+  int per_head = 256 / a.H;  // about one resident workgroup per CU
+  if (per_head < 1) per_head = 1;
+  if (per_head > ntiles) per_head = (int)ntiles;
+  if (a.H > 65535) return hipErrorInvalidValue;
+  dim3 grid((unsigned)per_head, (unsigned)a.H);
+  hipError_t e;
+  if (a.apply_conv) {
+    e = hipFuncSetAttribute((const void*)gates_mfma_bf16_kernel<true>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)kMfmaLdsBytes);
+    if (e != hipSuccess) return e;
+    gates_mfma_bf16_kernel<true><<<grid, 512, kMfmaLdsBytes, s>>>(a);
+  } else {
+    e = hipFuncSetAttribute((const void*)gates_mfma_bf16_kernel<false>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)kMfmaLdsBytes);
+    if (e != hipSuccess) return e;
+    gates_mfma_bf16_kernel<false><<<grid, 512, kMfmaLdsBytes, s>>>(a);
+  }
+  return hipGetLastError();
+}
+
+}  // namespace rg

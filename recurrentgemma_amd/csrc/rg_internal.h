@@ -1,0 +1,74 @@
+// Launcher declarations shared by the kernel files and the C-ABI file.
+#ifndef RG_INTERNAL_H_
+#define RG_INTERNAL_H_
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace rg {
+
+struct ConvArgs {
+  const void* x;
+  const void* segpos;
+  int seg_kind;  // 0: int32 positions, 1: int64 positions, 2: byte mask
+  const void* w;
+  const void* bias;
+  void* out;
+  void* cache_out;
+  int B, T, W, K;
+};
+
+struct ConvStepArgs {
+  const void* x;
+  const void* cache_in;
+  const void* w;
+  const void* bias;
+  void* out;
+  void* cache_out;
+  int B, W, K;
+};
+
+struct GemmArgs {
+  const void* x;       // [M, W]
+  int apply_conv;      // width-4 conv on load
+  const void* segpos;  // [M] (only with apply_conv)
+  int seg_kind;
+  const void* conv_w;  // [4, W]
+  const void* conv_b;  // [W]
+  const void* w[2];    // [H, bw, bw] per gate
+  const void* b[2];    // [H, bw] per gate
+  void* out[2];        // [M, W] per gate
+  int ngates;          // 1 or 2
+  int64_t M;           // rows = B*T
+  int T;               // sequence length (row m is token m % T of its row)
+  int W, H, bw;
+};
+
+struct ScanArgs {
+  int plain;  // 1: rnn_scan only (x is the recurrence input, ga holds a)
+  const void* x;
+  int apply_conv;
+  const void* conv_w;
+  const void* conv_b;
+  const void* gx;
+  const void* ga;
+  const void* a_param;
+  const void* segpos;
+  int seg_kind;
+  const float* h0;
+  void* y;
+  float* h_last;
+  void* cache_out;
+  int B, T, W;
+};
+
+// Each returns hipSuccess or the launch error.  dtype: 0 = f32, 1 = bf16.
+hipError_t launch_conv1d_prefill(const ConvArgs& a, int dtype, hipStream_t s);
+hipError_t launch_conv1d_step(const ConvStepArgs& a, int dtype, hipStream_t s);
+hipError_t launch_gemm_generic(const GemmArgs& a, int dtype, hipStream_t s);
+hipError_t launch_gemm_mfma_bf16(const GemmArgs& a, hipStream_t s);
+hipError_t launch_lru_scan(const ScanArgs& a, int dtype, hipStream_t s);
+
+}  // namespace rg
+#endif  // RG_INTERNAL_H_

@@ -1,0 +1,172 @@
+"""Drop-in modules for the reference's recurrent-block layers, on HIP kernels.
+
+Same constructor arguments, parameter names/shapes (so reference state-dicts
+load unchanged), forward signatures and cache conventions as
+recurrentgemma/torch/layers.py:
+  BlockDiagonalLinear  layers.py:76-137
+  rnn_scan             layers.py:140-191
+  rnn_param_init       layers.py:194-213
+  RGLRU                layers.py:233-376
+  Conv1D               layers.py:379-650
+Forward only (inference); the kernels are not differentiable.
+
+Differences from the reference, on purpose:
+  * Conv1D.forward does not modify its input (the reference multiplies slices
+    of `x` by the document mask in place); the returned cache is the same
+    masked tail the reference returns.
+  * In bfloat16 the kernels compute in float32 and round once per module output
+    (gate pre-activations are also held in bfloat16), where the reference rounds
+    after every elementwise op.
+  * Tensors must live on a GPU; there is no CPU path.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+from torch import nn
+
+from recurrentgemma_amd import ops
+
+
+class BlockDiagonalLinear(nn.Module):
+  """Block-diagonal linear layer: y[..., h, :] = x[..., h, :] @ w[h] + b[h]."""
+
+  def __init__(self, width, num_blocks, w_init_variance_scale=1.0, device=None,
+               dtype=None):
+    super().__init__()
+    self.width = width
+    self.num_blocks = num_blocks
+    self.w_init_variance_scale = w_init_variance_scale
+    self.block_width = self.width // self.num_blocks
+    self.w = nn.Parameter(torch.empty(
+        [self.num_blocks, self.block_width, self.block_width], device=device,
+        dtype=dtype))
+    self.b = nn.Parameter(torch.empty(
+        [self.num_blocks, self.block_width], device=device, dtype=dtype))
+    self.reset_parameters()
+
+  def reset_parameters(self) -> None:
+    self.w_init_(self.w)
+    torch.nn.init.zeros_(self.b)
+
+  def w_init_(self, w: torch.Tensor) -> None:
+    std = math.sqrt(self.w_init_variance_scale / self.block_width)
+    torch.nn.init.normal_(w, mean=0.0, std=std)
+
+  @torch.no_grad()
+  def forward(self, x: torch.Tensor) -> torch.Tensor:
+    return ops.block_diag_linear(x, self.w, self.b)
+
+
+@torch.no_grad()
+def rnn_scan(x, a, reset, h0, acc_dtype=torch.float32):
+  """h_t = a_t h_{t-1} + x_t with a zeroed at resets; float32 state."""
+  assert x.ndim == 3
+  assert a.shape == x.shape[-a.ndim:]
+  assert a.dtype == x.dtype
+  assert type(a) is type(x)
+  assert h0 is None or h0.dtype == acc_dtype
+  if acc_dtype != torch.float32:
+    raise NotImplementedError("the scan kernel keeps its state in float32")
+  if a.shape != x.shape:
+    a = a.expand_as(x)
+  return ops.linear_scan(x, a, reset, h0)
+
+
+def rnn_param_init(tensor, min_rad, max_rad, transform="softplus", eps=1e-8):
+  """Initialises Lambda so that exp(-softplus(Lambda)) lies on a ring."""
+  with torch.no_grad():
+    tensor.uniform_(min_rad ** 2 + eps, max_rad ** 2 + eps)
+    tensor.log_().mul_(0.5)
+    if transform == "softplus":
+      return tensor.neg_().exp_().sub_(1.0).log_()
+    raise NotImplementedError()
+
+
+class RGLRU(nn.Module):
+  """Real-Gated Linear Recurrent Unit."""
+
+  def __init__(self, width, num_heads, w_init_variance_scale=1.0, device=None,
+               dtype=None):
+    super().__init__()
+    self.width = width
+    self.num_heads = num_heads
+    self.w_init_variance_scale = w_init_variance_scale
+    self.a_param = nn.Parameter(torch.empty([self.width], device=device,
+                                            dtype=dtype))
+    self.input_gate = BlockDiagonalLinear(
+        width=self.width, num_blocks=self.num_heads,
+        w_init_variance_scale=w_init_variance_scale, device=device, dtype=dtype)
+    self.a_gate = BlockDiagonalLinear(
+        width=self.width, num_blocks=self.num_heads,
+        w_init_variance_scale=self.w_init_variance_scale, device=device,
+        dtype=dtype)
+    self.reset_parameters()
+
+  def reset_parameters(self) -> None:
+    self.input_gate.reset_parameters()
+    self.a_gate.reset_parameters()
+    self.a_param_init(self.a_param)
+
+  def a_param_init(self, w: torch.Tensor) -> torch.Tensor:
+    return rnn_param_init(w, min_rad=0.9, max_rad=0.999)
+
+  @torch.no_grad()
+  def forward(self, x, segment_pos, cache=None, return_cache=True):
+    """x [B,T,W] (the conv output), cache: previous state [B,W] float32."""
+    bs, l, _ = x.shape
+    assert segment_pos.shape == (bs, l)
+    gx_pre, ga_pre = ops.gates_gemm(x, self.input_gate.w, self.input_gate.b,
+                                    self.a_gate.w, self.a_gate.b)
+    y, last_h, _ = ops.lru_scan_fused(x, gx_pre, ga_pre, self.a_param,
+                                      segment_pos, h0=cache,
+                                      return_h=return_cache)
+    if not return_cache:
+      return y, None
+    return y, last_h
+
+  @classmethod
+  def init_cache(cls, batch_size, width, device=None):
+    # The RG-LRU state is always float32.
+    return torch.zeros((batch_size, width), dtype=torch.float32, device=device)
+
+
+class Conv1D(nn.Module):
+  """Causal depthwise temporal convolution with document masking."""
+
+  def __init__(self, width, temporal_width, w_init_variance_scale=0.01,
+               device=None, dtype=None):
+    super().__init__()
+    self.width = width
+    self.temporal_width = temporal_width
+    self.w_init_variance_scale = w_init_variance_scale
+    self.w = nn.Parameter(torch.empty([self.temporal_width, self.width],
+                                      device=device, dtype=dtype))
+    self.b = nn.Parameter(torch.empty([width], device=device, dtype=dtype))
+    self.reset_parameters()
+
+  def reset_parameters(self) -> None:
+    self.w_init_(self.w)
+    torch.nn.init.zeros_(self.b)
+
+  def w_init_(self, w: torch.Tensor) -> None:
+    std = math.sqrt(self.w_init_variance_scale / self.temporal_width)
+    torch.nn.init.normal_(w, mean=0.0, std=std)
+
+  @torch.no_grad()
+  def forward(self, x, segment_pos, cache=None, return_cache=True):
+    """cache None: prefill over [B,T,W]; cache [B,K-1,W]: one decode token."""
+    if cache is not None:
+      b, num_tokens, d = x.shape
+      assert cache.shape == (b, self.temporal_width - 1, d)
+      assert num_tokens == 1
+      return ops.conv1d_step(x, cache, self.w, self.b, return_cache)
+    return ops.conv1d_prefill(x, segment_pos, self.w, self.b, return_cache)
+
+  @classmethod
+  def init_cache(cls, *, batch_size, width, dtype, conv1d_temporal_width=4,
+                 device=None):
+    shape = (batch_size, conv1d_temporal_width - 1, width)
+    return torch.zeros(shape, dtype=dtype, device=device)

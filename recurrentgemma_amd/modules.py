@@ -1,0 +1,135 @@
+"""The caller of the hot path: Griffin's recurrent block, on the fused kernels.
+
+RecurrentBlock / RecurrentBlockCache mirror
+recurrentgemma/torch/modules.py:32-37 and :496-680 (same constructor,
+parameter names, forward signature and cache tuple).  linear_x / linear_y /
+linear_out stay torch.nn.Linear (hipBLASLt); conv_1d -> rg_lru runs as
+  prefill: rg_gates_gemm (conv on load) + rg_lru_scan_fused (conv fused)
+  decode : rg_recurrent_step
+unless the conv width is not 4, where the stand-alone conv kernel is used.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import NamedTuple
+
+import torch
+from torch import nn
+
+from recurrentgemma_amd import layers
+from recurrentgemma_amd import ops
+
+
+class RecurrentBlockCache(NamedTuple):
+  rg_lru_state: torch.Tensor  # [B, lru_width] float32
+  conv1d_state: torch.Tensor  # [B, temporal_width-1, lru_width]
+
+
+def gelu(x: torch.Tensor) -> torch.Tensor:
+  return nn.functional.gelu(x, approximate="tanh")
+
+
+@torch.no_grad()
+def recurrent_core(conv_1d: layers.Conv1D, rg_lru: layers.RGLRU, x,
+                   segment_pos, cache: RecurrentBlockCache | None = None,
+                   return_cache: bool = True):
+  """conv_1d -> rg_lru exactly as RecurrentBlock.forward chains them
+  (modules.py:632-643), fused.  Returns (y, RecurrentBlockCache | None)."""
+  bs, l, _ = x.shape
+  assert segment_pos.shape == (bs, l)
+  fused = conv_1d.temporal_width == 4
+  if cache is not None:
+    b, num_tokens, d = x.shape
+    assert cache.conv1d_state.shape == (b, conv_1d.temporal_width - 1, d)
+    assert num_tokens == 1
+    if fused:
+      y, h, conv_state = ops.recurrent_step(
+          x, segment_pos, cache.conv1d_state, cache.rg_lru_state, conv_1d.w,
+          conv_1d.b, rg_lru.input_gate.w, rg_lru.input_gate.b, rg_lru.a_gate.w,
+          rg_lru.a_gate.b, rg_lru.a_param)
+      if not return_cache:
+        return y, None
+      return y, RecurrentBlockCache(rg_lru_state=h, conv1d_state=conv_state)
+  if not fused or cache is not None:
+    xc, conv_state = conv_1d(x, segment_pos,
+                             None if cache is None else cache.conv1d_state,
+                             return_cache)
+    y, h = rg_lru(xc, segment_pos,
+                  None if cache is None else cache.rg_lru_state, return_cache)
+  else:
+    gx_pre, ga_pre = ops.gates_gemm(
+        x, rg_lru.input_gate.w, rg_lru.input_gate.b, rg_lru.a_gate.w,
+        rg_lru.a_gate.b, conv=(segment_pos, conv_1d.w, conv_1d.b))
+    y, h, conv_state = ops.lru_scan_fused(
+        x, gx_pre, ga_pre, rg_lru.a_param, segment_pos, h0=None,
+        conv=(conv_1d.w, conv_1d.b), return_h=return_cache,
+        return_conv_cache=return_cache)
+  if not return_cache:
+    return y, None
+  return y, RecurrentBlockCache(rg_lru_state=h, conv1d_state=conv_state)
+
+
+class RecurrentBlock(nn.Module):
+  """Griffin and Hawk's recurrent block."""
+
+  def __init__(self, width, num_heads, lru_width=None, conv1d_temporal_width=4,
+               final_w_init_variance_scale=1.0, device=None, dtype=None):
+    super().__init__()
+    self.width = width
+    self.num_heads = num_heads
+    self.lru_width = lru_width or width
+    self.conv1d_temporal_width = conv1d_temporal_width
+    self.final_w_init_variance_scale = final_w_init_variance_scale
+    self.linear_y = nn.Linear(self.width, self.lru_width, device=device,
+                              dtype=dtype)
+    self.linear_x = nn.Linear(self.width, self.lru_width, device=device,
+                              dtype=dtype)
+    self.linear_out = nn.Linear(self.lru_width, self.width, device=device,
+                                dtype=dtype)
+    self.conv_1d = layers.Conv1D(width=self.lru_width,
+                                 temporal_width=self.conv1d_temporal_width,
+                                 device=device, dtype=dtype)
+    self.rg_lru = layers.RGLRU(width=self.lru_width, num_heads=self.num_heads,
+                               device=device, dtype=dtype)
+    self.reset_parameters()
+
+  def reset_parameters(self) -> None:
+    self.w_init_(self.linear_x.weight)
+    torch.nn.init.zeros_(self.linear_x.bias)
+    self.w_init_(self.linear_y.weight)
+    torch.nn.init.zeros_(self.linear_y.bias)
+    self.out_w_init_(self.linear_out.weight)
+    torch.nn.init.zeros_(self.linear_out.bias)
+    self.conv_1d.reset_parameters()
+    self.rg_lru.reset_parameters()
+
+  def w_init_(self, w: torch.Tensor) -> None:
+    torch.nn.init.normal_(w, mean=0.0, std=math.sqrt(1.0 / self.width))
+
+  def out_w_init_(self, w: torch.Tensor) -> None:
+    std = math.sqrt(self.final_w_init_variance_scale / self.lru_width)
+    torch.nn.init.normal_(w, mean=0.0, std=std)
+
+  @torch.no_grad()
+  def forward(self, x, segment_pos, cache=None, return_cache=True):
+    y = gelu(self.linear_y(x))
+    x = self.linear_x(x)
+    x, new_cache = recurrent_core(self.conv_1d, self.rg_lru, x, segment_pos,
+                                  cache, return_cache)
+    x = x * y
+    x = self.linear_out(x)
+    if not return_cache:
+      return x, None
+    return x, new_cache
+
+  @classmethod
+  def init_cache(cls, batch_size, lru_width, dtype, conv1d_temporal_width=4,
+                 device=None):
+    return RecurrentBlockCache(
+        rg_lru_state=layers.RGLRU.init_cache(batch_size=batch_size,
+                                             width=lru_width, device=device),
+        conv1d_state=layers.Conv1D.init_cache(
+            batch_size=batch_size, width=lru_width, dtype=dtype,
+            conv1d_temporal_width=conv1d_temporal_width, device=device),
+    )

@@ -1,0 +1,248 @@
+"""Functional front-end of the C ABI on torch tensors (device memory + stream).
+
+Every function checks shapes/dtypes/devices on the host, allocates the outputs
+with torch's caching allocator, and enqueues the kernels on torch's current
+HIP stream.  Nothing here computes on the CPU.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from recurrentgemma_amd import _lib
+
+_DTYPES = {torch.float32: _lib.RG_DTYPE_F32, torch.bfloat16: _lib.RG_DTYPE_BF16}
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+  if t.dtype not in _DTYPES:
+    raise TypeError(
+        f"recurrentgemma_amd kernels support float32 and bfloat16, got {t.dtype}")
+  return _DTYPES[t.dtype]
+
+
+def _dev(t: torch.Tensor, name: str) -> torch.Tensor:
+  """Contiguous, 16-byte aligned, on a GPU; raises instead of computing on CPU."""
+  if not t.is_cuda:
+    raise RuntimeError(
+        f"{name} is on {t.device}: recurrentgemma_amd runs on the GPU only "
+        "(there is no CPU fallback)")
+  t = t.contiguous()
+  if t.data_ptr() % 16:
+    t = t.clone(memory_format=torch.contiguous_format)
+  return t
+
+
+def _same(dtype, device, **tensors):
+  for name, t in tensors.items():
+    if t is None:
+      continue
+    if t.dtype != dtype:
+      raise TypeError(f"{name} has dtype {t.dtype}, expected {dtype} "
+                      "(parameters and activations must share one dtype)")
+    if t.device != device:
+      raise RuntimeError(f"{name} is on {t.device}, expected {device}")
+
+
+def _segpos(segment_pos: torch.Tensor, B: int, T: int):
+  assert segment_pos.shape == (B, T), (
+      f"segment_pos has shape {tuple(segment_pos.shape)}, expected {(B, T)}")
+  if segment_pos.dtype not in (torch.int32, torch.int64):
+    if segment_pos.dtype.is_floating_point or segment_pos.dtype == torch.bool:
+      raise TypeError(f"segment_pos must be an integer tensor, got "
+                      f"{segment_pos.dtype}")
+    segment_pos = segment_pos.to(torch.int64)
+  return _dev(segment_pos, "segment_pos"), int(segment_pos.dtype == torch.int64)
+
+
+def _stream(t: torch.Tensor) -> int:
+  return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _p(t):
+  return None if t is None else t.data_ptr()
+
+
+def conv1d_prefill(x, segment_pos, w, b, return_cache=True):
+  assert x.ndim == 3, f"x must be [B,T,W], got {tuple(x.shape)}"
+  B, T, W = x.shape
+  K = w.shape[0]
+  assert w.shape == (K, W) and b.shape == (W,)
+  x = _dev(x, "x")
+  _same(x.dtype, x.device, w=w, b=b)
+  w, b = _dev(w, "w"), _dev(b, "b")
+  seg, is64 = _segpos(segment_pos, B, T)
+  out = torch.empty_like(x)
+  cache = x.new_empty((B, K - 1, W)) if return_cache else None
+  with torch.cuda.device(x.device):
+    _lib.check(_lib.lib().rg_conv1d_prefill(
+        _p(x), _p(seg), is64, _p(w), _p(b), _p(out), _p(cache), B, T, W, K,
+        _dtype_code(x), _stream(x)))
+  return out, cache
+
+
+def conv1d_step(x, cache, w, b, return_cache=True):
+  B, n_tok, W = x.shape
+  K = w.shape[0]
+  assert cache.shape == (B, K - 1, W)
+  assert n_tok == 1
+  x = _dev(x, "x")
+  _same(x.dtype, x.device, w=w, b=b)
+  w, b = _dev(w, "w"), _dev(b, "b")
+  cache_in = _dev(cache.to(x.dtype), "cache")
+  out = torch.empty_like(x)
+  new_cache = torch.empty_like(cache_in) if return_cache else None
+  with torch.cuda.device(x.device):
+    _lib.check(_lib.lib().rg_conv1d_step(
+        _p(x), _p(cache_in), _p(w), _p(b), _p(out), _p(new_cache), B, W, K,
+        _dtype_code(x), _stream(x)))
+  if new_cache is not None and new_cache.dtype != cache.dtype:
+    new_cache = new_cache.to(cache.dtype)
+  return out, new_cache
+
+
+def block_diag_linear(x, w, b):
+  H, bw, bw2 = w.shape
+  assert bw == bw2 and b.shape == (H, bw)
+  assert x.shape[-1] == H * bw, (
+      f"last dim {x.shape[-1]} != num_blocks*block_width {H * bw}")
+  x = _dev(x, "x")
+  _same(x.dtype, x.device, w=w, b=b)
+  w, b = _dev(w, "w"), _dev(b, "b")
+  y = torch.empty_like(x)
+  M = x.numel() // (H * bw)
+  if M == 0:
+    return y
+  with torch.cuda.device(x.device):
+    _lib.check(_lib.lib().rg_block_diag_linear(
+        _p(x), _p(w), _p(b), _p(y), M, H, bw, _dtype_code(x), _stream(x)))
+  return y
+
+
+def gates_gemm(x, w_x, b_x, w_a, b_a, conv=None):
+  """conv = None or (segment_pos, conv_w, conv_b) for conv-on-load."""
+  B, T, W = x.shape
+  H, bw, _ = w_x.shape
+  assert H * bw == W and w_a.shape == w_x.shape
+  assert b_x.shape == (H, bw) and b_a.shape == (H, bw)
+  x = _dev(x, "x")
+  _same(x.dtype, x.device, w_x=w_x, b_x=b_x, w_a=w_a, b_a=b_a)
+  w_x, b_x, w_a, b_a = (_dev(w_x, "w_x"), _dev(b_x, "b_x"), _dev(w_a, "w_a"),
+                        _dev(b_a, "b_a"))
+  seg = cw = cb = None
+  is64 = 0
+  if conv is not None:
+    segment_pos, cw, cb = conv
+    assert cw.shape == (4, W) and cb.shape == (W,)
+    _same(x.dtype, x.device, conv_w=cw, conv_b=cb)
+    cw, cb = _dev(cw, "conv_w"), _dev(cb, "conv_b")
+    seg, is64 = _segpos(segment_pos, B, T)
+  gx = torch.empty_like(x)
+  ga = torch.empty_like(x)
+  with torch.cuda.device(x.device):
+    _lib.check(_lib.lib().rg_gates_gemm(
+        _p(x), int(conv is not None), _p(seg), is64, _p(cw), _p(cb), _p(w_x),
+        _p(b_x), _p(w_a), _p(b_a), _p(gx), _p(ga), B, T, W, H, _dtype_code(x),
+        _stream(x)))
+  return gx, ga
+
+
+def lru_scan_fused(x, gx_pre, ga_pre, a_param, segment_pos, h0=None, conv=None,
+                   return_h=True, return_conv_cache=False):
+  """conv = None or (conv_w, conv_b): apply the width-4 conv to x first."""
+  B, T, W = x.shape
+  assert gx_pre.shape == x.shape and ga_pre.shape == x.shape
+  assert a_param.shape == (W,)
+  x = _dev(x, "x")
+  _same(x.dtype, x.device, gx_pre=gx_pre, ga_pre=ga_pre, a_param=a_param)
+  gx_pre, ga_pre, a_param = (_dev(gx_pre, "gx_pre"), _dev(ga_pre, "ga_pre"),
+                             _dev(a_param, "a_param"))
+  seg, is64 = _segpos(segment_pos, B, T)
+  if h0 is not None:
+    assert h0.dtype == torch.float32, "the RG-LRU state is always float32"
+    assert h0.shape == (B, W)
+    h0 = _dev(h0, "h0")
+  cw = cb = None
+  if conv is not None:
+    cw, cb = conv
+    assert cw.shape == (4, W) and cb.shape == (W,)
+    _same(x.dtype, x.device, conv_w=cw, conv_b=cb)
+    cw, cb = _dev(cw, "conv_w"), _dev(cb, "conv_b")
+  y = torch.empty_like(x)
+  h_last = (torch.empty((B, W), dtype=torch.float32, device=x.device)
+            if return_h else None)
+  cache = None
+  if return_conv_cache:
+    assert conv is not None
+    cache = x.new_empty((B, 3, W))
+  with torch.cuda.device(x.device):
+    _lib.check(_lib.lib().rg_lru_scan_fused(
+        _p(x), int(conv is not None), _p(cw), _p(cb), _p(gx_pre), _p(ga_pre),
+        _p(a_param), _p(seg), is64, _p(h0), _p(y), _p(h_last), _p(cache), B, T,
+        W, _dtype_code(x), _stream(x)))
+  return y, h_last, cache
+
+
+def linear_scan(x, a, reset, h0=None):
+  B, T, W = x.shape
+  x = _dev(x, "x")
+  _same(x.dtype, x.device, a=a)
+  a = _dev(a, "a")
+  assert reset.shape == (B, T) and reset.dtype == torch.bool
+  reset = _dev(reset, "reset")
+  if h0 is not None:
+    h0 = _dev(h0, "h0")
+  y = torch.empty_like(x)
+  h_last = torch.empty((B, W), dtype=torch.float32, device=x.device)
+  with torch.cuda.device(x.device):
+    _lib.check(_lib.lib().rg_linear_scan(
+        _p(x), _p(a), _p(reset), _p(h0), _p(y), _p(h_last), B, T, W,
+        _dtype_code(x), _stream(x)))
+  return y, h_last
+
+
+_workspaces = {}
+
+
+def _workspace(B, W, dtype, device):
+  key = (B, W, dtype, device)
+  ws = _workspaces.get(key)
+  if ws is None:
+    n = _lib.lib().rg_recurrent_step_workspace_bytes(B, W, _DTYPES[dtype])
+    ws = torch.empty(n, dtype=torch.uint8, device=device)
+    _workspaces.clear()  # keep one workspace alive at a time
+    _workspaces[key] = ws
+  return ws
+
+
+def recurrent_step(x, segment_pos, conv_cache, h, conv_w, conv_b, w_x, b_x, w_a,
+                   b_a, a_param, in_place=False):
+  """One decode step of conv -> RG-LRU.  Returns (y, h_new, conv_cache_new)."""
+  B, n_tok, W = x.shape
+  assert n_tok == 1
+  assert conv_cache.shape == (B, 3, W)
+  assert h.shape == (B, W) and h.dtype == torch.float32
+  H = w_x.shape[0]
+  x = _dev(x, "x")
+  _same(x.dtype, x.device, conv_w=conv_w, conv_b=conv_b, w_x=w_x, b_x=b_x,
+        w_a=w_a, b_a=b_a, a_param=a_param)
+  cache_in = _dev(conv_cache.to(x.dtype), "conv_cache")
+  h_in = _dev(h, "h")
+  seg, is64 = _segpos(segment_pos, B, 1)
+  args = [_dev(t, n) for t, n in ((conv_w, "conv_w"), (conv_b, "conv_b"),
+                                  (w_x, "w_x"), (b_x, "b_x"), (w_a, "w_a"),
+                                  (b_a, "b_a"), (a_param, "a_param"))]
+  if in_place:
+    cache_out, h_out = cache_in, h_in
+  else:
+    cache_out, h_out = torch.empty_like(cache_in), torch.empty_like(h_in)
+  y = torch.empty_like(x)
+  ws = _workspace(B, W, x.dtype, x.device)
+  with torch.cuda.device(x.device):
+    _lib.check(_lib.lib().rg_recurrent_step(
+        _p(x), _p(seg), is64, _p(cache_in), _p(cache_out), _p(h_in), _p(h_out),
+        *[_p(t) for t in args], _p(y), _p(ws), ws.numel(), B, W, H,
+        _dtype_code(x), _stream(x)))
+  if cache_out.dtype != conv_cache.dtype:
+    cache_out = cache_out.to(conv_cache.dtype)
+  return y, h_out, cache_out

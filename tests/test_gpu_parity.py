@@ -1,0 +1,438 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle.
+
+Tolerances (BASELINE north_star): float32 max|d|/max|ref| <= 1e-5 on y and h;
+bfloat16-in / float32-state <= 1e-2 against the widened oracle (reference
+semantics evaluated in float32 on the bfloat16 values, outputs rounded once).
+"""
+
+import numpy as np
+import pytest
+import torch
+
+import recurrentgemma_amd as rg
+from oracle import torch_ref as R
+from recurrentgemma_amd import ops
+from tests import helpers
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+F32_TOL = 1e-5
+BF16_TOL = 1e-2
+
+
+def _dev(t):
+  return None if t is None else t.to(DEV)
+
+
+def _announce(*what):
+  print("[case]", *what, flush=True)
+
+
+def _mk_conv(w, b):
+  m = rg.Conv1D(width=w.shape[1], temporal_width=w.shape[0], dtype=w.dtype)
+  m.load_state_dict({"w": w, "b": b})
+  return m.to(DEV)
+
+
+def _mk_lru(prm, H):
+  a_param, w_x, b_x, w_a, b_a = prm
+  m = rg.RGLRU(width=a_param.shape[0], num_heads=H, dtype=a_param.dtype)
+  m.load_state_dict({"a_param": a_param, "input_gate.w": w_x,
+                     "input_gate.b": b_x, "a_gate.w": w_a, "a_gate.b": b_a})
+  return m.to(DEV)
+
+
+def _block(params, width, heads, dtype, K=4):
+  blk = rg.RecurrentBlock(width=width, num_heads=heads, lru_width=width,
+                          conv1d_temporal_width=K, dtype=dtype)
+  blk.conv_1d.load_state_dict({"w": params["conv_w"], "b": params["conv_b"]})
+  blk.rg_lru.load_state_dict({
+      "a_param": params["a_param"], "input_gate.w": params["w_x"],
+      "input_gate.b": params["b_x"], "a_gate.w": params["w_a"],
+      "a_gate.b": params["b_a"]})
+  return blk.to(DEV)
+
+
+def test_library_loaded():
+  from recurrentgemma_amd import _lib
+  assert _lib.lib().rg_abi_version() == 1
+  assert torch.cuda.is_available()
+  print(torch.cuda.get_device_name(0))
+
+
+# ------------------------------------------------------------- Conv1D ------
+
+
+def test_conv1d_golden(golden):
+  keys = golden.cases("conv/")
+  assert len(keys) == 80
+  for key in keys:
+    _announce(key)
+    x, seg = golden.get(key + "/x"), golden.get(key + "/seg")
+    conv = _mk_conv(golden.get(key + "/w"), golden.get(key + "/b"))
+    xd = _dev(x)
+    y, cache = conv(xd, _dev(seg))
+    assert torch.equal(xd.cpu(), x), "input must not be modified"
+    want = golden.get(key + "/y")
+    if x.dtype == torch.float32:
+      assert helpers.max_rel(y, want) < F32_TOL, key
+    else:
+      # one rounding instead of the reference's one per tap: <= 2 bf16 ulp
+      torch.testing.assert_close(y.cpu(), want, rtol=1.6e-2, atol=1e-2)
+    assert torch.equal(cache.cpu(), golden.get(key + "/cache")), key
+    y_nc, none = conv(xd, _dev(seg), return_cache=False)
+    assert none is None and torch.equal(y_nc, y)
+    # int32 positions give the same result
+    y32, cache32 = conv(xd, _dev(seg.to(torch.int32)))
+    assert torch.equal(y32, y) and torch.equal(cache32, cache)
+    xs = golden.get(key + "/step_x")
+    for i in range(2):
+      ys, cache = conv(_dev(xs[:, i:i + 1]), _dev(seg[:, -1:] + 1 + i), cache)
+      want = golden.get(key + f"/step{i}_y")
+      if x.dtype == torch.float32:
+        assert helpers.max_rel(ys, want) < F32_TOL, key
+      else:
+        torch.testing.assert_close(ys.cpu(), want, rtol=1.6e-2, atol=1e-2)
+      assert torch.equal(cache.cpu(), golden.get(key + f"/step{i}_cache")), key
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("K", [2, 4, 8])
+def test_conv1d_vs_oracle(dtype, K):
+  g = torch.Generator().manual_seed(200 + K)
+  B, T, W = 3, 211, 130
+  x = torch.randn(B, T, W, generator=g).to(dtype)
+  w = (torch.randn(K, W, generator=g) * 0.3).to(dtype)
+  b = (torch.randn(W, generator=g) * 0.1).to(dtype)
+  seg = helpers.document_positions(B, T, 9, seed=K)
+  _announce("conv", dtype, K)
+  y, cache = _mk_conv(w, b)(_dev(x), _dev(seg))
+  yo, co = R.widened_conv1d_forward(x, seg, w, b)
+  tol = F32_TOL if dtype == torch.float32 else BF16_TOL
+  assert helpers.max_rel(y, yo) < tol
+  assert torch.equal(cache.cpu(), co)
+
+
+# ------------------------------------------------- BlockDiagonalLinear -----
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width,blocks", [(128, 1), (128, 16), (1024, 1),
+                                          (1024, 16), (512, 2), (60, 3)])
+def test_block_diagonal_linear(dtype, width, blocks):
+  g = torch.Generator().manual_seed(width + blocks)
+  bw = width // blocks
+  x = torch.randn(1, 2, width, generator=g).to(dtype)
+  x2 = torch.randn(3, 37, width, generator=g).to(dtype)
+  w = (torch.randn(blocks, bw, bw, generator=g) / bw ** 0.5).to(dtype)
+  b = (torch.randn(blocks, bw, generator=g) * 0.2).to(dtype)
+  m = rg.BlockDiagonalLinear(width, blocks, dtype=dtype)
+  m.load_state_dict({"w": w, "b": b})
+  m = m.to(DEV)
+  tol = F32_TOL if dtype == torch.float32 else BF16_TOL
+  for xi in (x, x2):
+    _announce("bdl", dtype, width, blocks, tuple(xi.shape))
+    want = R.block_diagonal_linear(xi.float(), w.float(), b.float())
+    assert helpers.max_rel(m(_dev(xi)), want) < tol
+
+
+# --------------------------------------------------------------- scan ------
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T", [1, 2, 15, 16, 17, 128, 129, 1000])
+def test_rnn_scan(dtype, T):
+  g = torch.Generator().manual_seed(300 + T)
+  B, W = 2, 200
+  x = torch.randn(B, T, W, generator=g).to(dtype)
+  a = torch.rand(B, T, W, generator=g).to(dtype)
+  reset = torch.rand(B, T, generator=g) < 0.05
+  for h0 in (None, torch.randn(B, W, generator=g)):
+    _announce("rnn_scan", dtype, T, h0 is not None)
+    y, h = rg.rnn_scan(_dev(x), _dev(a), _dev(reset), _dev(h0))
+    yo, ho = R.rnn_scan(x, a, reset, h0)
+    tol = F32_TOL if dtype == torch.float32 else BF16_TOL
+    assert helpers.max_rel(y, yo) < tol
+    assert helpers.max_rel(h, ho) < F32_TOL
+    assert h.dtype == torch.float32
+
+
+def test_rnn_scan_closed_forms():
+  T, W = 3000, 64
+  one = torch.ones(1, T, W, device=DEV)
+  noreset = torch.zeros(1, T, dtype=torch.bool, device=DEV)
+  y, h = rg.rnn_scan(one, torch.full_like(one, 0.9), noreset, None)
+  t = torch.arange(1, T + 1, dtype=torch.float64)
+  want = (1 - 0.9 ** t) / 0.1
+  assert helpers.max_rel(y[0, :, 0], want) < F32_TOL
+  y, h = rg.rnn_scan(one, torch.ones_like(one), noreset, None)
+  assert torch.equal(y[0, :, 5].cpu(), torch.arange(1, T + 1).float())
+  y, h = rg.rnn_scan(one, torch.zeros_like(one), noreset, None)
+  assert torch.equal(y, one)
+
+
+# -------------------------------------------------------------- RGLRU ------
+
+
+def test_rglru_golden(golden):
+  keys = golden.cases("rglru/")
+  assert len(keys) == 72
+  worst = {torch.float32: 0.0, torch.bfloat16: 0.0}
+  for key in keys:
+    _announce(key)
+    pkey = "/".join(key.split("/")[:3])
+    prm = [golden.get(pkey + "/" + n)
+           for n in ("a_param", "w_x", "b_x", "w_a", "b_a")]
+    H = prm[1].shape[0]
+    lru = _mk_lru(prm, H)
+    x, seg = golden.get(key + "/x"), golden.get(key + "/seg")
+    h0 = golden.get(key + "/h0") if golden.has(key + "/h0") else None
+    y, h = lru(_dev(x), _dev(seg), _dev(h0))
+    assert h.dtype == torch.float32 and y.dtype == x.dtype
+    f32 = x.dtype == torch.float32
+    # fp32: the reference itself.  bf16: the reference's all-bf16 arithmetic is
+    # only loosely comparable (checked with its own tolerance form); the tight
+    # bf16 check is against the widened oracle.
+    if f32:
+      e = max(helpers.max_rel(y, golden.get(key + "/y")),
+              helpers.max_rel(h, golden.get(key + "/h")))
+      assert e < F32_TOL, (key, e)
+    else:
+      torch.testing.assert_close(y.cpu().float(),
+                                 golden.get(key + "/y").float(), rtol=1e-2,
+                                 atol=6e-2)
+      yo, ho = R.widened_rglru_forward(x, seg, *prm, cache=h0)
+      e = max(helpers.max_rel(y, yo), helpers.max_rel(h, ho))
+      assert e < BF16_TOL, (key, e)
+    worst[x.dtype] = max(worst[x.dtype], e)
+    xs = golden.get(key + "/step_x")
+    for i in range(2):
+      segi = seg[:, -1:] + 1 + i
+      ys, h_new = lru(_dev(xs[:, i:i + 1]), _dev(segi), h)
+      if f32:
+        e = max(helpers.max_rel(ys, golden.get(key + f"/step{i}_y")),
+                helpers.max_rel(h_new, golden.get(key + f"/step{i}_h")))
+        assert e < F32_TOL, (key, i, e)
+      else:
+        yo, ho = R.widened_rglru_forward(xs[:, i:i + 1], segi, *prm,
+                                         cache=h.cpu())
+        e = max(helpers.max_rel(ys, yo), helpers.max_rel(h_new, ho))
+        assert e < BF16_TOL, (key, i, e)
+      h = h_new
+    y_nc, none = lru(_dev(x), _dev(seg), _dev(h0), return_cache=False)
+    assert none is None and torch.equal(y_nc, y)
+  print("worst max-rel error", worst)
+
+
+# ------------------------------------------------- fused conv -> rg_lru ----
+
+
+def _core_case(dtype, B, T, W, H, seg, seed, bias_std=0.2):
+  p = R.make_params(W, H, dtype, seed=seed, gate_bias_std=bias_std)
+  g = torch.Generator().manual_seed(seed + 1)
+  x = torch.randn(B, T, W, generator=g).to(dtype)
+  blk = _block(p, W, H, dtype)
+  y, cache = rg.recurrent_core(blk.conv_1d, blk.rg_lru, _dev(x), _dev(seg))
+  if dtype == torch.float32:
+    yo, co = R.recurrent_core(x, seg, p)
+  else:
+    yo, co = R.widened_recurrent_core(x, seg, p)
+  return p, x, blk, (y, cache), (yo, co)
+
+
+def test_config1_fp32_parity():
+  """BASELINE config 1: B1 T512 W2560 H10 fp32, segment_pos = arange."""
+  B, T, W, H = 1, 512, 2560, 10
+  seg = torch.arange(T)[None]
+  p = R.make_params(W, H, torch.float32, seed=1101)
+  g = torch.Generator().manual_seed(1001)
+  x = torch.randn(B, T, W, generator=g)
+  blk = _block(p, W, H, torch.float32)
+  _announce("config1")
+  y, cache = rg.recurrent_core(blk.conv_1d, blk.rg_lru, _dev(x), _dev(seg))
+  yo, co = R.recurrent_core(x, seg, p)
+  ey, eh = helpers.max_rel(y, yo), helpers.max_rel(cache.rg_lru_state,
+                                                   co.rg_lru_state)
+  print("config1 max-rel y", ey, "h", eh)
+  assert ey < F32_TOL and eh < F32_TOL
+  assert torch.equal(cache.conv1d_state.cpu(), co.conv1d_state)
+  # module-by-module path gives the same numbers as the fused path
+  xc, cstate = blk.conv_1d(_dev(x), _dev(seg))
+  y2, h2 = blk.rg_lru(xc, _dev(seg))
+  assert helpers.max_rel(y2, yo) < F32_TOL
+  assert torch.equal(cstate, cache.conv1d_state)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,T,W,H,mean_doc", [
+    (2, 700, 512, 2, 60),     # bw 256: MFMA path in bf16, ragged T
+    (3, 129, 768, 3, 7),      # dense document starts
+    (1, 2050, 256, 1, 500),   # long row, many steps
+    (2, 33, 384, 6, 5),       # bw 64: generic GEMM
+    (2, 3, 256, 1, 2),        # shorter than the conv
+    (5, 1, 256, 1, 1),        # single token, every row starts a document
+    (2, 64, 130, 1, 16),      # width not a multiple of the slab
+    (2, 40, 65, 1, 16),       # odd width: one channel per lane
+])
+def test_core_vs_oracle(dtype, B, T, W, H, mean_doc):
+  seg = helpers.document_positions(B, T, mean_doc, seed=T + W)
+  if T > 4:
+    seg[0, -1] = 0   # document start in the last position
+    seg[-1, -2] = 0  # ... and in the one before
+  _announce("core", dtype, B, T, W, H)
+  p, x, blk, (y, cache), (yo, co) = _core_case(dtype, B, T, W, H, seg, seed=T)
+  tol = F32_TOL if dtype == torch.float32 else BF16_TOL
+  ey = helpers.max_rel(y, yo)
+  eh = helpers.max_rel(cache.rg_lru_state, co.rg_lru_state)
+  print("max-rel y", ey, "h", eh)
+  assert ey < tol and eh < tol
+  assert torch.equal(cache.conv1d_state.cpu(), co.conv1d_state)
+  assert cache.rg_lru_state.dtype == torch.float32
+  assert cache.conv1d_state.dtype == dtype
+  # sampler-style positions: left padding is -1, int32
+  seg32 = torch.cat([torch.full((B, T // 3), -1), torch.arange(T - T // 3)
+                     .expand(B, -1)], 1).to(torch.int32)
+  y, cache = rg.recurrent_core(blk.conv_1d, blk.rg_lru, _dev(x), _dev(seg32))
+  ref = R.recurrent_core if dtype == torch.float32 else R.widened_recurrent_core
+  yo, co = ref(x, seg32, p)
+  assert helpers.max_rel(y, yo) < tol
+  assert helpers.max_rel(cache.rg_lru_state, co.rg_lru_state) < tol
+  assert torch.equal(cache.conv1d_state.cpu(), co.conv1d_state)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_prefill_then_decode(dtype):
+  """Prefill, then 6 single-token steps with the carried cache (config 4 in
+  small), and the reference's own invariant prefill(T) == prefill(T-1) o step."""
+  B, T, W, H, steps = 4, 77, 512, 2, 6
+  seg = torch.arange(T).expand(B, T).clone()
+  p = R.make_params(W, H, dtype, seed=77, gate_bias_std=0.2)
+  g = torch.Generator().manual_seed(78)
+  x = torch.randn(B, T + steps, W, generator=g).to(dtype)
+  blk = _block(p, W, H, dtype)
+  ref = R.recurrent_core if dtype == torch.float32 else R.widened_recurrent_core
+  tol = F32_TOL if dtype == torch.float32 else BF16_TOL
+  _announce("decode", dtype)
+  y, cache = rg.recurrent_core(blk.conv_1d, blk.rg_lru, _dev(x[:, :T]),
+                               _dev(seg))
+  yo, co = ref(x[:, :T], seg, p)
+  for i in range(steps):
+    pos = torch.full((B, 1), T + i)
+    xi = x[:, T + i:T + i + 1]
+    y, cache = rg.recurrent_core(blk.conv_1d, blk.rg_lru, _dev(xi), _dev(pos),
+                                 cache)
+    yo, co = ref(xi, pos, p, co)
+    assert helpers.max_rel(y, yo) < tol, i
+    assert helpers.max_rel(cache.rg_lru_state, co.rg_lru_state) < tol, i
+    assert torch.equal(cache.conv1d_state.cpu(), co.conv1d_state), i
+  # invariant
+  full = torch.arange(T + steps).expand(B, -1)
+  y_full, c_full = rg.recurrent_core(blk.conv_1d, blk.rg_lru, _dev(x),
+                                     _dev(full))
+  assert helpers.max_rel(y, y_full[:, -1:]) < tol
+  assert helpers.max_rel(cache.rg_lru_state, c_full.rg_lru_state) < tol
+  assert torch.equal(cache.conv1d_state, c_full.conv1d_state)
+
+
+def test_recurrent_block_module():
+  """RecurrentBlock end to end (linear_x/y/out in torch) against the oracle
+  core wrapped in the same torch linears on the CPU, fp32."""
+  B, T, width, H = 2, 50, 256, 1
+  torch.manual_seed(5)
+  blk = rg.RecurrentBlock(width=width, num_heads=H, dtype=torch.float32)
+  sd = {k: v.clone() for k, v in blk.state_dict().items()}
+  x = torch.randn(B, T, width)
+  seg = helpers.document_positions(B, T, 20, seed=3)
+  p = {"conv_w": sd["conv_1d.w"], "conv_b": sd["conv_1d.b"],
+       "a_param": sd["rg_lru.a_param"], "w_x": sd["rg_lru.input_gate.w"],
+       "b_x": sd["rg_lru.input_gate.b"], "w_a": sd["rg_lru.a_gate.w"],
+       "b_a": sd["rg_lru.a_gate.b"]}
+  lin = torch.nn.functional.linear
+  yb = torch.nn.functional.gelu(lin(x, sd["linear_y.weight"],
+                                    sd["linear_y.bias"]), approximate="tanh")
+  xb = lin(x, sd["linear_x.weight"], sd["linear_x.bias"])
+  core, cache_o = R.recurrent_core(xb, seg, p)
+  want = lin(core * yb, sd["linear_out.weight"], sd["linear_out.bias"])
+  blk = blk.to(DEV)
+  got, cache = blk(_dev(x), _dev(seg))
+  assert helpers.max_rel(got, want) < 1e-4  # torch GPU vs CPU linears
+  assert isinstance(cache, rg.RecurrentBlockCache)
+  assert helpers.max_rel(cache.rg_lru_state, cache_o.rg_lru_state) < 1e-4
+  init = rg.RecurrentBlock.init_cache(B, width, torch.float32, device=DEV)
+  assert init.rg_lru_state.dtype == torch.float32
+  assert init.conv1d_state.shape == (B, 3, width)
+  got1, c1 = blk(_dev(x[:, :1]), _dev(seg[:, :1]), init)
+  assert helpers.max_rel(got1, want[:, :1]) < 1e-4
+
+
+# --------------------------------- full-size, size-independent properties --
+
+
+def _full_size_properties(B, T, W, H, seg, seed):
+  dtype = torch.bfloat16
+  p = R.make_params(W, H, dtype, seed=seed)
+  p["conv_b"].zero_()  # so that the conv is exactly linear
+  g = torch.Generator().manual_seed(seed - 100)
+  x = torch.randn(B, T, W, generator=g).to(dtype).to(DEV)
+  blk = _block(p, W, H, dtype)
+  segd = seg.to(DEV)
+  y, cache = rg.recurrent_core(blk.conv_1d, blk.rg_lru, x, segd)
+  torch.cuda.synchronize()
+  assert torch.isfinite(y.float()).all()
+  # (1) module-by-module equals fused, bit for bit
+  xc, cstate = blk.conv_1d(x, segd)
+  y2, h2 = blk.rg_lru(xc, segd)
+  assert torch.equal(y2, y) and torch.equal(h2, cache.rg_lru_state)
+  assert torch.equal(cstate, cache.conv1d_state)
+  # (2) splitting the sequence and carrying the state changes nothing beyond
+  #     fp32 re-association of the carry
+  cut = T // 2 + 5
+  ya, ha = blk.rg_lru(xc[:, :cut].contiguous(), segd[:, :cut].contiguous())
+  yb, hb = blk.rg_lru(xc[:, cut:].contiguous(), segd[:, cut:].contiguous(), ha)
+  assert torch.equal(ya, y[:, :cut])
+  assert helpers.max_rel(hb, cache.rg_lru_state) < 1e-5
+  assert (yb.float() - y[:, cut:].float()).abs().max().item() <= 0.0625
+  mism = (yb != y[:, cut:]).float().mean().item()
+  assert mism < 1e-3, mism
+  # (3) with the gate pre-activations held fixed the path is linear in x:
+  #     doubling x doubles y and h exactly (powers of two are exact)
+  gx, ga = ops.gates_gemm(x, blk.rg_lru.input_gate.w, blk.rg_lru.input_gate.b,
+                          blk.rg_lru.a_gate.w, blk.rg_lru.a_gate.b,
+                          conv=(segd, blk.conv_1d.w, blk.conv_1d.b))
+  y1, h1, _ = ops.lru_scan_fused(x, gx, ga, blk.rg_lru.a_param, segd,
+                                 conv=(blk.conv_1d.w, blk.conv_1d.b))
+  yd, hd, _ = ops.lru_scan_fused(x * 2, gx, ga, blk.rg_lru.a_param, segd,
+                                 conv=(blk.conv_1d.w, blk.conv_1d.b))
+  assert torch.equal(y1, y)
+  assert torch.equal(yd.float(), y1.float() * 2) and torch.equal(hd, h1 * 2)
+  # (4) at every document start y == conv(x) * sigmoid(gx_pre)
+  starts = segd == 0
+  want = (xc.float() * torch.sigmoid(gx.float()))[starts]
+  got = y[starts].float()
+  assert ((got - want).abs() <= 0.01 * want.abs() + 1e-3).all()
+  # (5) a row's result does not depend on its neighbours (first row alone)
+  y_row, c_row = rg.recurrent_core(blk.conv_1d, blk.rg_lru, x[:1].contiguous(),
+                                   segd[:1].contiguous())
+  assert torch.equal(y_row, y[:1])
+  assert torch.equal(c_row.rg_lru_state, cache.rg_lru_state[:1])
+  # (6) spot parity against the oracle on one row's first tokens
+  n = 300
+  yo, _ = R.widened_recurrent_core(x[:1, :n].cpu(), seg[:1, :n], p)
+  assert helpers.max_rel(y[:1, :n], yo) < BF16_TOL
+
+
+def test_config2_full_size_properties():
+  """BASELINE config 2: B8 T4096 W2560 H10 bf16, documents ~ Geometric(1024)."""
+  B, T, W, H = 8, 4096, 2560, 10
+  seg = helpers.document_positions(B, T, 1024, seed=1002)
+  _announce("config2 full size")
+  _full_size_properties(B, T, W, H, seg, seed=1102)
+
+
+def test_config3_full_size_properties():
+  """BASELINE config 3: B16 T8192 W4096 H16 bf16, one document per row."""
+  B, T, W, H = 16, 8192, 4096, 16
+  seg = torch.arange(T).expand(B, T).contiguous()
+  _announce("config3 full size")
+  _full_size_properties(B, T, W, H, seg, seed=1103)

@@ -1,0 +1,129 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports what
+include/rg_lru.h declares, argument validation happens before any launch, and
+the drop-in modules keep the reference's surface (names, shapes, caches)."""
+
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import recurrentgemma_amd as rg
+from oracle import torch_ref as R
+from recurrentgemma_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+  text = open(os.path.join(ROOT, "include", "rg_lru.h")).read()
+  text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+  return sorted(set(re.findall(r"\b(rg_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+  names = _declared_symbols()
+  assert len(names) == 10, names
+  lib = ctypes.CDLL(_lib.LIB_PATH)
+  for n in names:
+    assert hasattr(lib, n), n
+  assert set(names) == set(_lib.SIGNATURES)
+  assert _lib.lib().rg_abi_version() == 1
+
+
+def test_c_side_validation_without_launch():
+  lib = _lib.lib()
+  ok = ctypes.c_void_p(256)  # aligned, never dereferenced: checks fail first
+  rc = lib.rg_conv1d_prefill(None, ok, 1, ok, ok, ok, None, 1, 1, 8, 4, 0, None)
+  assert rc == -1 and b"x is null" in lib.rg_last_error()
+  rc = lib.rg_conv1d_prefill(ok, ok, 1, ok, ok, ok, None, 1, 1, 8, 1, 0, None)
+  assert rc == -2 and b"temporal width" in lib.rg_last_error()
+  rc = lib.rg_conv1d_prefill(ok, ok, 1, ok, ok, ok, None, 1, 0, 8, 4, 0, None)
+  assert rc == -1 and b"positive" in lib.rg_last_error()
+  rc = lib.rg_conv1d_prefill(ok, ok, 1, ok, ok, ok, None, 1, 1, 8, 4, 7, None)
+  assert rc == -2 and b"dtype" in lib.rg_last_error()
+  odd = ctypes.c_void_p(257)
+  rc = lib.rg_gates_gemm(odd, 0, None, 0, None, None, ok, ok, ok, ok, ok, ok, 1,
+                         1, 256, 1, 1, None)
+  assert rc == -1 and b"aligned" in lib.rg_last_error()
+  rc = lib.rg_gates_gemm(ok, 0, None, 0, None, None, ok, ok, ok, ok, ok, ok, 1,
+                         1, 250, 3, 1, None)
+  assert rc == -1 and b"multiple" in lib.rg_last_error()
+  y = ctypes.c_void_p(512)
+  rc = lib.rg_lru_scan_fused(ok, 0, None, None, ok, ok, ok, ok, 1, None, y,
+                             None, ok, 1, 1, 8, 1, None)
+  assert rc == -1 and b"apply_conv" in lib.rg_last_error()
+  assert lib.rg_recurrent_step_workspace_bytes(256, 4096, 1) == 3 * 256 * 4096 * 2
+  rc = lib.rg_recurrent_step(ok, ok, 1, ok, ok, ok, ok, ok, ok, ok, ok, ok, ok,
+                             ok, ok, None, 0, 2, 256, 1, 1, None)
+  assert rc == -4 and b"workspace" in lib.rg_last_error()
+
+
+def test_no_cpu_fallback():
+  conv = rg.Conv1D(width=8, temporal_width=4)
+  with pytest.raises(RuntimeError, match="GPU only"):
+    conv(torch.randn(1, 5, 8), torch.arange(5)[None])
+  lru = rg.RGLRU(width=8, num_heads=2)
+  with pytest.raises(RuntimeError, match="GPU only"):
+    lru(torch.randn(1, 5, 8), torch.arange(5)[None])
+  with pytest.raises(AssertionError):
+    lru(torch.randn(1, 5, 8), torch.arange(4)[None])  # layers.py:334
+  with pytest.raises(AssertionError):
+    conv(torch.randn(1, 2, 8), torch.arange(2)[None],
+         cache=torch.zeros(1, 3, 8))  # layers.py:549: one token with a cache
+  with pytest.raises(AssertionError):
+    rg.rnn_scan(torch.zeros(1, 2, 4), torch.zeros(1, 2, 4, dtype=torch.bfloat16),
+                torch.zeros(1, 2, dtype=torch.bool), None)  # layers.py:163
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+  monkeypatch.setattr(_lib, "_lib", None)
+  monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/librg_lru.so")
+  with pytest.raises(RuntimeError, match="no fallback"):
+    _lib.lib()
+
+
+def test_module_surface_matches_reference():
+  blk = rg.RecurrentBlock(width=64, num_heads=4, lru_width=128)
+  # recurrentgemma/torch/modules.py:549-580, layers.py:105-112,262-278,409-412
+  want = {
+      "linear_y.weight": (128, 64), "linear_y.bias": (128,),
+      "linear_x.weight": (128, 64), "linear_x.bias": (128,),
+      "linear_out.weight": (64, 128), "linear_out.bias": (64,),
+      "conv_1d.w": (4, 128), "conv_1d.b": (128,),
+      "rg_lru.a_param": (128,),
+      "rg_lru.input_gate.w": (4, 32, 32), "rg_lru.input_gate.b": (4, 32),
+      "rg_lru.a_gate.w": (4, 32, 32), "rg_lru.a_gate.b": (4, 32),
+  }
+  got = {k: tuple(v.shape) for k, v in blk.state_dict().items()}
+  assert got == want
+  assert rg.RecurrentBlockCache._fields == ("rg_lru_state", "conv1d_state")
+  c = rg.RecurrentBlock.init_cache(batch_size=3, lru_width=128,
+                                   dtype=torch.bfloat16)
+  assert c.rg_lru_state.dtype == torch.float32
+  assert c.rg_lru_state.shape == (3, 128)
+  assert c.conv1d_state.dtype == torch.bfloat16
+  assert c.conv1d_state.shape == (3, 3, 128)
+  assert rg.Conv1D.init_cache(batch_size=2, width=8, dtype=torch.float32,
+                              conv1d_temporal_width=8).shape == (2, 7, 8)
+  assert rg.RGLRU.init_cache(2, 8).dtype == torch.float32
+  # initial distributions (layers.py:122-125, 422-425, 289-291)
+  torch.manual_seed(0)
+  big = rg.RGLRU(width=4096, num_heads=16)
+  assert abs(big.input_gate.w.std().item() - 1 / 16) < 1e-3
+  assert torch.all(big.input_gate.b == 0)
+  r = torch.exp(-torch.nn.functional.softplus(big.a_param.double()))
+  assert r.min() >= 0.9 - 1e-4 and r.max() <= 0.999 + 1e-4
+  conv = rg.Conv1D(width=4096, temporal_width=4)
+  assert abs(conv.w.std().item() - 0.05) < 2e-3
+
+
+def test_param_init_same_draws_as_oracle():
+  torch.manual_seed(7)
+  a = torch.empty(100)
+  rg.rnn_param_init(a, 0.9, 0.999)
+  torch.manual_seed(7)
+  b = torch.empty(100)
+  R.rnn_param_init(b, 0.9, 0.999)
+  assert torch.equal(a, b)
