@@ -1,0 +1,212 @@
+"""Benchmark of the Conv1D + RG-LRU recurrent-block core on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A "step" is one pass of the hot path over one synthetic batch that is already
+resident in HBM: rg_gates_gemm (width-4 conv on load, both gate projections on
+bf16 MFMA) followed by rg_lru_scan_fused (conv + gates + chunked scan), called
+through the C ABI on torch's current stream.  Prints ONE JSON line.
+
+Workloads (BASELINE.json configs):
+  9b_prefill  B16 T8192 W4096 H16 bf16 / fp32 state, one document per row
+              (the configuration the >= 70 % HBM-roofline target is stated on;
+              default)
+  2b_prefill  B8 T4096 W2560 H10 bf16, documents ~ Geometric(mean 1024)
+
+`roofline` describes the scan kernel: algorithmic bytes per launch (read x,
+read both gate pre-activations, write y, plus the small terms) over the mean
+launch duration measured with HIP events inside the timed region.
+`cpu_baseline` times the CPU oracle (an op-for-op torch restatement of the
+reference's path, bf16 like the reference would run it) on a bounded sample of
+the same workload on this machine's host cores.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+  sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+WORKLOADS = {
+    "9b_prefill": dict(B=16, T=8192, W=4096, H=16, mean_doc=None, seed=1003),
+    "2b_prefill": dict(B=8, T=4096, W=2560, H=10, mean_doc=1024, seed=1002),
+}
+
+# HBM bytes per scan launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# (scaled by a copy kernel of known size); None until measured for a workload.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def scan_algorithmic_bytes(B, T, W, esize, seg_bytes, has_h0):
+  n = B * T * W
+  return (4 * esize * n            # x, gx_pre, ga_pre in; y out
+          + B * T * seg_bytes      # segment positions
+          + B * W * 4 * (int(has_h0) + 1)   # h0 in, h_last out (fp32)
+          + B * 3 * W * esize      # conv state out
+          + W * esize * 8)         # conv w (4), conv b, a_param (+ gate biases)
+
+
+def make_segment_pos(torch, B, T, mean_doc, seed):
+  if mean_doc is None:
+    return torch.arange(T).expand(B, T).contiguous()
+  import numpy as np
+  rng = np.random.default_rng(seed)
+  out = np.zeros((B, T), np.int64)
+  for b in range(B):
+    t = 0
+    while t < T:
+      n = min(int(rng.geometric(1.0 / mean_doc)), T - t)
+      out[b, t:t + n] = np.arange(n)
+      t += n
+  return torch.from_numpy(out)
+
+
+def cpu_baseline(torch, R, wl, params, seconds_target=20.0):
+  """Oracle (port of the reference torch path) on the host cores, on a slice
+  of the workload: the first Bs batch rows at full sequence length (about
+  10-30 s of CPU work in total)."""
+  cores = os.cpu_count() or 1
+  torch.set_num_threads(cores)
+  Bs, Ts = min(wl["B"], 4), wl["T"]
+  g = torch.Generator().manual_seed(wl["seed"])
+  x = torch.randn(Bs, Ts, wl["W"], generator=g).to(torch.bfloat16)
+  seg = make_segment_pos(torch, Bs, Ts, wl["mean_doc"], wl["seed"])
+  R.recurrent_core(x[:, :64], seg[:, :64], params)  # warm-up
+  times = []
+  t_all = time.perf_counter()
+  while len(times) < 3 and (not times or
+                            time.perf_counter() - t_all < seconds_target):
+    t0 = time.perf_counter()
+    R.recurrent_core(x, seg, params)
+    times.append(time.perf_counter() - t0)
+  best = sorted(times)[len(times) // 2]
+  return {
+      "value": Bs * Ts / best, "unit": "tokens/s", "cores": cores,
+      "kind": "port",
+      "sample": (f"oracle/torch_ref.recurrent_core, bf16, {Bs}x{Ts} tokens of "
+                 f"the workload (W={wl['W']}, H={wl['H']}), median of "
+                 f"{len(times)} runs, torch threads={torch.get_num_threads()}"),
+  }
+
+
+def main():
+  ap = argparse.ArgumentParser()
+  ap.add_argument("--gpus", type=int, default=1)
+  ap.add_argument("--steps", type=int, default=50)
+  ap.add_argument("--warmup", type=int, default=10)
+  ap.add_argument("--workload", default="9b_prefill", choices=sorted(WORKLOADS))
+  ap.add_argument("--no-cpu-baseline", action="store_true")
+  args = ap.parse_args()
+  if args.gpus != 1:
+    sys.exit("bench.py measures one GPU: this build has no multi-GPU path "
+             "(run with --gpus 1)")
+
+  import torch
+
+  import recurrentgemma_amd as rg
+  from oracle import torch_ref as R
+  from recurrentgemma_amd import ops
+
+  wl = WORKLOADS[args.workload]
+  B, T, W, H = wl["B"], wl["T"], wl["W"], wl["H"]
+  dev = torch.device("cuda:0")
+  dtype = torch.bfloat16
+
+  params = R.make_params(W, H, dtype, seed=wl["seed"] + 100)
+  g = torch.Generator().manual_seed(wl["seed"])
+  x = torch.randn(B, T, W, generator=g).to(dtype).to(dev)
+  seg = make_segment_pos(torch, B, T, wl["mean_doc"], wl["seed"]).to(dev)
+  blk = rg.RecurrentBlock(width=W, num_heads=H, dtype=dtype)
+  blk.conv_1d.load_state_dict({"w": params["conv_w"], "b": params["conv_b"]})
+  blk.rg_lru.load_state_dict({
+      "a_param": params["a_param"], "input_gate.w": params["w_x"],
+      "input_gate.b": params["b_x"], "a_gate.w": params["w_a"],
+      "a_gate.b": params["b_a"]})
+  blk = blk.to(dev)
+  conv, lru = blk.conv_1d, blk.rg_lru
+
+  def step(events=None):
+    if events:
+      events[0].record()
+    gx, ga = ops.gates_gemm(x, lru.input_gate.w, lru.input_gate.b,
+                            lru.a_gate.w, lru.a_gate.b,
+                            conv=(seg, conv.w, conv.b))
+    if events:
+      events[1].record()
+    y, h, cache = ops.lru_scan_fused(x, gx, ga, lru.a_param, seg,
+                                     conv=(conv.w, conv.b),
+                                     return_conv_cache=True)
+    if events:
+      events[2].record()
+    return y, h, cache
+
+  for _ in range(args.warmup):
+    out = step()
+  torch.cuda.synchronize()
+
+  evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)]
+         for _ in range(args.steps)]
+  torch.cuda.synchronize()
+  t0 = time.perf_counter()
+  for i in range(args.steps):
+    out = step(evs[i])
+  torch.cuda.synchronize()
+  elapsed = time.perf_counter() - t0
+
+  gemm_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / args.steps
+  scan_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / args.steps
+  ms_per_step = elapsed * 1e3 / args.steps
+  tokens = B * T
+
+  seg_bytes = seg.element_size()
+  algo = scan_algorithmic_bytes(B, T, W, 2, seg_bytes, has_h0=False)
+  achieved = algo / (scan_ms * 1e-3) / 1e9
+  gemm_flops = 1024.0 * W * tokens
+  gemm_bytes = 3 * 2 * B * T * W
+
+  result = {
+      "metric": "RG-LRU block tokens/s + scan HBM GB/s (% of roofline)",
+      "value": tokens / (elapsed / args.steps),
+      "unit": "tokens/s",
+      "n_gpus": 1,
+      "steps": args.steps,
+      "warmup": args.warmup,
+      "ms_per_step": ms_per_step,
+      "higher_is_better": True,
+      "scaling": "weak",
+      "vs_baseline": None,
+      "dtype": "bf16",
+      "data": "synthetic",
+      "config": {
+          "workload": args.workload, "batch": B, "seq_len": T, "lru_width": W,
+          "heads": H, "activations": "bf16", "state": "f32",
+          "documents": ("one per row" if wl["mean_doc"] is None
+                        else f"geometric mean {wl['mean_doc']}"),
+          "path": "rg_gates_gemm(conv on load) + rg_lru_scan_fused(conv)"},
+      "roofline": {
+          "kernel": "lru_scan_kernel (conv + gates + scan)",
+          "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
+          "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+          "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+          "algorithmic_bytes": algo, "avg_launch_ms": scan_ms},
+      "gate_gemm": {
+          "kernel": "gates_mfma_bf16_kernel", "avg_launch_ms": gemm_ms,
+          "tflops": gemm_flops / (gemm_ms * 1e-3) / 1e12,
+          "frac_of_bf16_mfma_peak": gemm_flops / (gemm_ms * 1e-3) / 2.5e15,
+          "gbs": gemm_bytes / (gemm_ms * 1e-3) / 1e9,
+          "frac_of_hbm_peak": gemm_bytes / (gemm_ms * 1e-3) / 1e9
+                              / HBM_PEAK_GBS},
+  }
+  if not args.no_cpu_baseline:
+    result["cpu_baseline"] = cpu_baseline(torch, R, wl, params)
+  print(json.dumps(result))
+
+
+if __name__ == "__main__":
+  main()

@@ -58,7 +58,13 @@ def test_library_loaded():
   from recurrentgemma_amd import _lib
   assert _lib.lib().rg_abi_version() == 1
   assert torch.cuda.is_available()
-  print(torch.cuda.get_device_name(0))
+  name = torch.cuda.get_device_name(0)
+  arch = torch.cuda.get_device_properties(0).gcnArchName
+  print("device:", name, arch, "lib:", _lib.LIB_PATH)
+  assert "gfx950" in arch, arch
+  # the library this process mapped is the in-tree one
+  maps = open("/proc/self/maps").read()
+  assert _lib.LIB_PATH in maps or "librg_lru.so" in maps
 
 
 # ------------------------------------------------------------- Conv1D ------
@@ -78,8 +84,9 @@ def test_conv1d_golden(golden):
     if x.dtype == torch.float32:
       assert helpers.max_rel(y, want) < F32_TOL, key
     else:
-      # one rounding instead of the reference's one per tap: <= 2 bf16 ulp
-      torch.testing.assert_close(y.cpu(), want, rtol=1.6e-2, atol=1e-2)
+      # the reference's own bf16 tolerance for Conv1D (layers_test.py:170)
+      torch.testing.assert_close(y.cpu(), want, rtol=1e-2, atol=3e-2)
+      assert helpers.max_rel(y, want) < BF16_TOL, key
     assert torch.equal(cache.cpu(), golden.get(key + "/cache")), key
     y_nc, none = conv(xd, _dev(seg), return_cache=False)
     assert none is None and torch.equal(y_nc, y)
@@ -93,7 +100,8 @@ def test_conv1d_golden(golden):
       if x.dtype == torch.float32:
         assert helpers.max_rel(ys, want) < F32_TOL, key
       else:
-        torch.testing.assert_close(ys.cpu(), want, rtol=1.6e-2, atol=1e-2)
+        torch.testing.assert_close(ys.cpu(), want, rtol=1e-2, atol=3e-2)
+        assert helpers.max_rel(ys, want) < BF16_TOL, key
       assert torch.equal(cache.cpu(), golden.get(key + f"/step{i}_cache")), key
 
 
@@ -179,6 +187,8 @@ def test_rglru_golden(golden):
   keys = golden.cases("rglru/")
   assert len(keys) == 72
   worst = {torch.float32: 0.0, torch.bfloat16: 0.0}
+  worst_ref_form = [-1e9]  # max of |d| - (atol + rtol*|ref|); <= 0 passes
+  worst_ref_rel = [0.0]
   for key in keys:
     _announce(key)
     pkey = "/".join(key.split("/")[:3])
@@ -199,9 +209,12 @@ def test_rglru_golden(golden):
               helpers.max_rel(h, golden.get(key + "/h")))
       assert e < F32_TOL, (key, e)
     else:
-      torch.testing.assert_close(y.cpu().float(),
-                                 golden.get(key + "/y").float(), rtol=1e-2,
-                                 atol=6e-2)
+      # the reference's own bf16 tolerance form (layers_test.py:131)
+      gold = golden.get(key + "/y").float()
+      d = (y.cpu().float() - gold).abs()
+      excess = (d - (3e-2 + 1e-2 * gold.abs())).max().item()
+      worst_ref_form[0] = max(worst_ref_form[0], excess)
+      worst_ref_rel[0] = max(worst_ref_rel[0], helpers.max_rel(y, gold))
       yo, ho = R.widened_rglru_forward(x, seg, *prm, cache=h0)
       e = max(helpers.max_rel(y, yo), helpers.max_rel(h, ho))
       assert e < BF16_TOL, (key, e)
@@ -222,7 +235,10 @@ def test_rglru_golden(golden):
       h = h_new
     y_nc, none = lru(_dev(x), _dev(seg), _dev(h0), return_cache=False)
     assert none is None and torch.equal(y_nc, y)
-  print("worst max-rel error", worst)
+  print("worst max-rel error vs fp32 golden / widened oracle", worst)
+  print("bf16 vs the reference's all-bf16 golden: max-rel", worst_ref_rel[0],
+        "excess over rtol=1e-2,atol=3e-2:", worst_ref_form[0])
+  assert worst_ref_form[0] <= 0.0, worst_ref_form[0]
 
 
 # ------------------------------------------------- fused conv -> rg_lru ----
