@@ -41,6 +41,9 @@ struct Act;
 template <>
 struct Act<float, 1> {
   static constexpr bool kIsBf16 = false;
+  typedef float Raw;
+  __device__ static Raw load_raw(const float* p) { return *p; }
+  __device__ static void unpack(Raw r, float (&v)[1]) { v[0] = r; }
   __device__ static void load(const float* p, float (&v)[1]) { v[0] = *p; }
   __device__ static void store(float* p, const float (&v)[1]) { *p = v[0]; }
   __device__ static float round(float v) { return v; }
@@ -48,6 +51,14 @@ struct Act<float, 1> {
 template <>
 struct Act<float, 2> {
   static constexpr bool kIsBf16 = false;
+  typedef f32x2 Raw;
+  __device__ static Raw load_raw(const float* p) {
+    return *reinterpret_cast<const f32x2*>(p);
+  }
+  __device__ static void unpack(Raw r, float (&v)[2]) {
+    v[0] = r.x;
+    v[1] = r.y;
+  }
   __device__ static void load(const float* p, float (&v)[2]) {
     f32x2 t = *reinterpret_cast<const f32x2*>(p);
     v[0] = t.x;
@@ -62,6 +73,11 @@ struct Act<float, 2> {
 template <>
 struct Act<uint16_t, 1> {
   static constexpr bool kIsBf16 = true;
+  typedef uint16_t Raw;
+  __device__ static Raw load_raw(const uint16_t* p) { return *p; }
+  __device__ static void unpack(Raw r, float (&v)[1]) {
+    v[0] = bf16_bits_to_f32(r);
+  }
   __device__ static void load(const uint16_t* p, float (&v)[1]) {
     v[0] = bf16_bits_to_f32(*p);
   }
@@ -73,6 +89,14 @@ struct Act<uint16_t, 1> {
 template <>
 struct Act<uint16_t, 2> {
   static constexpr bool kIsBf16 = true;
+  typedef uint32_t Raw;  // two bf16 stay packed in one register until used
+  __device__ static Raw load_raw(const uint16_t* p) {
+    return *reinterpret_cast<const uint32_t*>(p);
+  }
+  __device__ static void unpack(Raw r, float (&v)[2]) {
+    v[0] = __uint_as_float(r << 16);
+    v[1] = __uint_as_float(r & 0xffff0000u);
+  }
   __device__ static void load(const uint16_t* p, float (&v)[2]) {
     uint32_t u = *reinterpret_cast<const uint32_t*>(p);
     v[0] = __uint_as_float(u << 16);

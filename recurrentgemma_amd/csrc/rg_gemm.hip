@@ -164,25 +164,19 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
   for (int nt = 0; nt < 2; ++nt)
     biasv[nt] = bf16_bits_to_f32(
         ((const uint16_t*)p.b[gate])[h * kBW + n0 + nt * 32 + (lane & 31)]);
-  uint16_t* outp = (uint16_t*)p.out[gate] + h * kBW + n0 + (lane & 31);
+  // Output addressing: a wave-uniform row pointer plus this 32-bit lane offset
+  // (lanes 32-63 sit four rows below lanes 0-31 in the 32x32 result layout).
+  const uint32_t out_lane_bytes =
+      2u * ((uint32_t)(4 * (lane >> 5)) * (uint32_t)p.W + h * kBW + n0 +
+            (lane & 31));
+  char* const outbase = (char*)p.out[gate];
 
   // ---- x staging: thread -> (channel pair, group of 16 rows) -----------
   const int cp = tid & 127;
   const int rg = __builtin_amdgcn_readfirstlane(tid >> 7);
-  const int c = h * kBW + cp * 2;
-  const uint16_t* xcol = (const uint16_t*)p.x + c;
-  float cw0[2], cw1[2], cw2[2], cw3[2], cb[2];
-  if (CONV) {
-    const uint16_t* cw = (const uint16_t*)p.conv_w;
-#pragma unroll
-    for (int ch = 0; ch < 2; ++ch) {
-      cw0[ch] = bf16_bits_to_f32(cw[c + ch]);
-      cw1[ch] = bf16_bits_to_f32(cw[W + c + ch]);
-      cw2[ch] = bf16_bits_to_f32(cw[2 * W + c + ch]);
-      cw3[ch] = bf16_bits_to_f32(cw[3 * W + c + ch]);
-      cb[ch] = bf16_bits_to_f32(((const uint16_t*)p.conv_b)[c + ch]);
-    }
-  }
+  const uint32_t c = h * kBW + cp * 2;  // lane offset inside a row of x
+  const uint32_t c_bytes = 2u * c;
+  const uint16_t* const xbase = (const uint16_t*)p.x;
   constexpr int kHalo = CONV ? 3 : 0;
   constexpr int kRaw = kRowsPerGroup + kHalo;
   uint32_t raw[kRaw];
@@ -191,9 +185,10 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
     const int64_t mbase = tile * kTM + rg * kRowsPerGroup - kHalo;
 #pragma unroll
     for (int j = 0; j < kRaw; ++j) {
-      int64_t m = mbase + j;
+      int64_t m = mbase + j;  // wave-uniform
       m = m < 0 ? 0 : (m >= M ? M - 1 : m);
-      raw[j] = *reinterpret_cast<const uint32_t*>(xcol + m * W);
+      raw[j] = *reinterpret_cast<const uint32_t*>(
+          reinterpret_cast<const char*>(xbase + m * W) + c_bytes);
     }
   };
 
@@ -206,20 +201,36 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
         *reinterpret_cast<uint32_t*>(dst + (size_t)i * kLdsStride) = raw[i];
       return;
     }
+    // conv taps and bias of this thread's two channels (L1/L2 hits; not kept
+    // in registers across the MFMA phase)
+    float cw0[2], cw1[2], cw2[2], cw3[2], cb[2];
+    {
+      const uint16_t* cw = (const uint16_t*)p.conv_w + c;
+      const uint32_t u0 = *reinterpret_cast<const uint32_t*>(cw);
+      const uint32_t u1 = *reinterpret_cast<const uint32_t*>(cw + W);
+      const uint32_t u2 = *reinterpret_cast<const uint32_t*>(cw + 2 * W);
+      const uint32_t u3 = *reinterpret_cast<const uint32_t*>(cw + 3 * W);
+      const uint32_t ub =
+          *reinterpret_cast<const uint32_t*>((const uint16_t*)p.conv_b + c);
+      cw0[0] = __uint_as_float(u0 << 16); cw0[1] = __uint_as_float(u0 & 0xffff0000u);
+      cw1[0] = __uint_as_float(u1 << 16); cw1[1] = __uint_as_float(u1 & 0xffff0000u);
+      cw2[0] = __uint_as_float(u2 << 16); cw2[1] = __uint_as_float(u2 & 0xffff0000u);
+      cw3[0] = __uint_as_float(u3 << 16); cw3[1] = __uint_as_float(u3 & 0xffff0000u);
+      cb[0] = __uint_as_float(ub << 16);  cb[1] = __uint_as_float(ub & 0xffff0000u);
+    }
     const int64_t mbase = tile * kTM + rg * kRowsPerGroup - kHalo;
     // bit j: row mbase+j begins a sequence row (t == 0) or a document; the
-    // conv must not look past it.
-    uint32_t cut = 0;
-    int t = (int)(((mbase % T_len) + T_len) % T_len);  // token index of row 0
-#pragma unroll
-    for (int j = 0; j < kRaw; ++j) {
-      const int64_t m = mbase + j;
-      if (m >= 0 && m < M) {
-        const bool st = (t == 0) || is_doc_start(p.segpos, p.seg_kind, m);
-        if (st) cut |= 1u << j;
-      }
-      t = (t + 1 == T_len) ? 0 : t + 1;
+    // conv must not look past it.  Lane j of the wave looks at row mbase+j
+    // (all lanes of a wave stage the same rows): one load and one ballot.
+    bool st = false;
+    {
+      const int64_t m = mbase + lane;
+      const uint32_t t_base = (uint32_t)(((mbase % T_len) + T_len) % T_len);
+      if (lane < kRaw && m >= 0 && m < M)
+        st = ((t_base + (uint32_t)lane) % (uint32_t)T_len == 0u) ||
+             is_doc_start(p.segpos, p.seg_kind, m);
     }
+    const uint32_t cut = (uint32_t)__ballot(st);
     float h0[2] = {0.f, 0.f}, h1[2] = {0.f, 0.f}, h2[2] = {0.f, 0.f};
 #pragma unroll
     for (int j = 0; j < kRaw; ++j) {
@@ -282,13 +293,18 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
                                                        acc1, 0, 0, 0);
       }
       // epilogue: D[i][j], i = 8*(r/4) + 4*(lane/32) + r%4, j = lane%32
-      const int64_t mrow0 = tile * kTM + mt * 32 + 4 * (lane >> 5);
+      const int64_t row_first = tile * kTM + mt * 32;          // uniform
+      const int64_t rows_left = M - row_first;                 // uniform, > 0
+      const int lane_row = 4 * (lane >> 5);
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int64_t m = mrow0 + 8 * (r >> 2) + (r & 3);
-        if (m < M) {
-          outp[m * W] = f32_to_bf16_bits(acc0[r] + biasv[0]);
-          outp[m * W + 32] = f32_to_bf16_bits(acc1[r] + biasv[1]);
+        const int i = 8 * (r >> 2) + (r & 3);                  // uniform part
+        char* rowp = outbase + (row_first + i) * W * 2;        // uniform
+        if (i + lane_row < rows_left) {
+          *reinterpret_cast<uint16_t*>(rowp + out_lane_bytes) =
+              f32_to_bf16_bits(acc0[r] + biasv[0]);
+          *reinterpret_cast<uint16_t*>(rowp + out_lane_bytes + 64) =
+              f32_to_bf16_bits(acc1[r] + biasv[1]);
         }
       }
     }

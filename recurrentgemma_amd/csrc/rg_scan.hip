@@ -39,21 +39,35 @@ struct ChanConst {
 // inside the sequence and no document start among them.
 template <typename T, int CH, bool CONV, bool FAST, bool PLAIN, bool CHECK>
 __device__ __forceinline__ void phase1(
-    const T* __restrict__ xrow, const T* __restrict__ gxrow,
-    const T* __restrict__ garow, int64_t W, int t0, int T_len, uint32_t starts,
+    const char* __restrict__ xrow, const char* __restrict__ gxrow,
+    const char* __restrict__ garow, uint32_t lane_bytes, int64_t row_bytes,
+    int t0, int T_len, uint32_t starts,
     const ChanConst<CH>& k, float (&hist)[3][CH], float (&a_)[kL][CH],
     float (&xn_)[kL][CH], float (&P)[CH], float (&H)[CH]) {
   using A = Act<T, CH>;
+  // All loads of the wave's kL tokens are issued before any arithmetic so that
+  // 3*kL row segments per wave are in flight; the (a, xn) results then take
+  // over the registers of the raw inputs.
+  typename A::Raw xr[kL], gxr[kL], gar[kL];
+#pragma unroll
+  for (int i = 0; i < kL; ++i) {
+    const int t = t0 + i;
+    // wave-uniform row address + 32-bit lane offset
+    const int64_t off =
+        (int64_t)(CHECK ? (t < T_len ? t : T_len - 1) : t) * row_bytes;
+    xr[i] = A::load_raw((const T*)(xrow + off + lane_bytes));
+    if (!PLAIN) gxr[i] = A::load_raw((const T*)(gxrow + off + lane_bytes));
+    gar[i] = A::load_raw((const T*)(garow + off + lane_bytes));
+  }
 #pragma unroll
   for (int i = 0; i < kL; ++i) {
     const int t = t0 + i;
     const bool valid = !CHECK || (t < T_len);
     const bool start = CHECK && ((starts >> (i + 3)) & 1u);
-    const int64_t off = (int64_t)(CHECK ? (t < T_len ? t : T_len - 1) : t) * W;
     float xv[CH], gxv[CH], gav[CH];
-    A::load(xrow + off, xv);
-    if (!PLAIN) A::load(gxrow + off, gxv);
-    A::load(garow + off, gav);
+    A::unpack(xr[i], xv);
+    if (!PLAIN) A::unpack(gxr[i], gxv);
+    A::unpack(gar[i], gav);
 #pragma unroll
     for (int ch = 0; ch < CH; ++ch) {
       float xc;
@@ -103,7 +117,7 @@ __device__ __forceinline__ void phase1(
 }
 
 template <typename T, int CH, bool CONV, bool FAST, bool PLAIN>
-__global__ void __launch_bounds__(kMaxNW* kWave)
+__global__ void __launch_bounds__(kMaxNW* kWave, (sizeof(T) == 2 ? 4 : 2))
 lru_scan_kernel(ScanArgs p) {
   using A = Act<T, CH>;
   __shared__ float agg[2][kMaxNW][kWave][2 * CH];  // (P.., Hloc..) per lane
@@ -144,10 +158,13 @@ lru_scan_kernel(ScanArgs p) {
   }
 
   const int64_t row0 = (int64_t)b * T_len;
-  const T* xrow = (const T*)p.x + row0 * W + c;
-  const T* gxrow = (const T*)p.gx + row0 * W + c;
-  const T* garow = (const T*)p.ga + row0 * W + c;
-  T* yrow = (T*)p.y + row0 * W + c;
+  const int64_t row_bytes = W * (int64_t)sizeof(T);
+  const uint32_t lane_bytes = (uint32_t)c * (uint32_t)sizeof(T);
+  // wave-uniform pointers to token 0 of this batch row
+  const char* xrow = (const char*)p.x + row0 * row_bytes;
+  const char* gxrow = (const char*)p.gx + row0 * row_bytes;
+  const char* garow = (const char*)p.ga + row0 * row_bytes;
+  char* yrow = (char*)p.y + row0 * row_bytes;
 
   float h_first[CH];
 #pragma unroll
@@ -172,21 +189,23 @@ lru_scan_kernel(ScanArgs p) {
     if (any) {
       // bit j <-> token t0-3+j starts a document (only tokens inside the row;
       // the three look-back tokens matter only for the conv history).
-      uint32_t starts = 0;
-#pragma unroll
-      for (int j = CONV ? 0 : 3; j < kL + 3; ++j) {
-        const int t = t0 - 3 + j;
-        const int tc = t < 0 ? 0 : (t >= T_len ? T_len - 1 : t);
-        const bool st = is_doc_start(p.segpos, p.seg_kind, row0 + tc);
-        if (st && t >= 0 && t < T_len) starts |= 1u << j;
+      // Lane j looks at token t0-3+j: one coalesced load and one ballot for
+      // the whole wave instead of kL+3 dependent loads.
+      bool st = false;
+      {
+        const int t = t0 - 3 + lane;
+        if (lane < kL + 3 && (CONV || lane >= 3) && t >= 0 && t < T_len)
+          st = is_doc_start(p.segpos, p.seg_kind, row0 + t);
       }
+      const uint32_t starts = (uint32_t)__ballot(st);
       float hist[3][CH];
       if (CONV) {
 #pragma unroll
         for (int s = 1; s <= 3; ++s) {
           const int t = t0 - s;
           float v[CH];
-          A::load(xrow + (int64_t)(t < 0 ? 0 : t) * W, v);
+          A::load((const T*)(xrow + (int64_t)(t < 0 ? 0 : t) * row_bytes +
+                             lane_bytes), v);
 #pragma unroll
           for (int ch = 0; ch < CH; ++ch) hist[s - 1][ch] = t < 0 ? 0.0f : v[ch];
         }
@@ -207,11 +226,13 @@ lru_scan_kernel(ScanArgs p) {
       }
       const bool plain = (t0 + kL <= T_len) && ((starts >> 3) == 0u);
       if (plain)
-        phase1<T, CH, CONV, FAST, PLAIN, false>(xrow, gxrow, garow, W, t0, T_len,
-                                         starts, k, hist, a_, xn_, P, H);
+        phase1<T, CH, CONV, FAST, PLAIN, false>(xrow, gxrow, garow, lane_bytes,
+                                                row_bytes, t0, T_len, starts, k,
+                                                hist, a_, xn_, P, H);
       else
-        phase1<T, CH, CONV, FAST, PLAIN, true>(xrow, gxrow, garow, W, t0, T_len,
-                                        starts, k, hist, a_, xn_, P, H);
+        phase1<T, CH, CONV, FAST, PLAIN, true>(xrow, gxrow, garow, lane_bytes,
+                                               row_bytes, t0, T_len, starts, k,
+                                               hist, a_, xn_, P, H);
     }
 
     // exchange
@@ -242,7 +263,8 @@ lru_scan_kernel(ScanArgs p) {
           h[ch] = __builtin_fmaf(a_[i][ch], h[ch], xn_[i][ch]);
           out[ch] = h[ch];
         }
-        if (t0 + i < T_len && active) A::store(yrow + (int64_t)(t0 + i) * W, out);
+        if (t0 + i < T_len && active)
+          A::store((T*)(yrow + (int64_t)(t0 + i) * row_bytes + lane_bytes), out);
       }
     }
     if (wave == nw - 1) {
@@ -269,7 +291,8 @@ lru_scan_kernel(ScanArgs p) {
 #pragma unroll
       for (int ch = 0; ch < CH; ++ch) v[ch] = 0.0f;
       if (t >= 0) {
-        if (!later_start) A::load(xrow + (int64_t)t * W, v);
+        if (!later_start)
+          A::load((const T*)(xrow + (int64_t)t * row_bytes + lane_bytes), v);
         if (is_doc_start(p.segpos, p.seg_kind, row0 + t))
           later_start = true;
       }
