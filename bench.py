@@ -102,6 +102,11 @@ def main():
   ap.add_argument("--warmup", type=int, default=10)
   ap.add_argument("--workload", default="9b_prefill", choices=sorted(WORKLOADS))
   ap.add_argument("--no-cpu-baseline", action="store_true")
+  ap.add_argument("--calibration-copy", action="store_true",
+                  help="after the timed steps, run one plain device copy of x "
+                       "(known size) so that a counter run of this command "
+                       "holds a reference dispatch to scale FETCH_SIZE / "
+                       "WRITE_SIZE by")
   args = ap.parse_args()
   if args.gpus != 1:
     sys.exit("bench.py measures one GPU: this build has no multi-GPU path "
@@ -158,6 +163,10 @@ def main():
     out = step(evs[i])
   torch.cuda.synchronize()
   elapsed = time.perf_counter() - t0
+
+  if args.calibration_copy:
+    torch.empty_like(x).copy_(x)  # reads and writes x.numel()*2 bytes
+    torch.cuda.synchronize()
 
   gemm_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / args.steps
   scan_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / args.steps

@@ -184,6 +184,17 @@ __device__ __forceinline__ float conv_point(const T* x, const void* segpos,
   return round_act<T>(acc);
 }
 
+// ---------------------------------------------------------- barriers ----
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits
+// for every outstanding global load and store of the wave (its fence covers
+// global memory), which would drain loads that were issued early on purpose.
+// Use only where the waves exchange data through LDS and nothing else.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // ------------------------------------------------------------- math ----
 constexpr float kLog2e = 1.4426950408889634f;
 

@@ -20,14 +20,108 @@
 // end of the sequence are the operator's identity (1, 0).  A document start
 // (segment_pos == 0) sets a = 0 and the input scale to 1, and zeroes the conv
 // history, which is exactly the reference's masking rule.
+//
+// Addressing.  All row traffic goes through buffer instructions: a scalar
+// resource descriptor whose base is the wave's first token of the step and
+// whose size is the wave's kL rows, a per-lane byte offset that never changes,
+// and a scalar row offset.  No per-access vector address arithmetic is needed.
+// Lanes past the last channel carry an offset beyond any descriptor's size, so
+// the hardware range check returns 0 for their loads and drops their stores.
 #include "rg_common.h"
 #include "rg_internal.h"
 
 namespace rg {
 namespace {
 
-constexpr int kL = 16;     // tokens per wave per step
+constexpr int kL = 8;      // tokens per wave per step
 constexpr int kMaxNW = 8;  // waves per workgroup
+
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base,
+                                                            uint32_t bytes) {
+  // raw buffer (stride 0), 32-bit data format
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0,
+                                           (int)bytes, 0x00020000);
+}
+
+// Buffer access of CH adjacent channels.  Raw keeps bf16 pairs packed in one
+// register until they are used.
+template <typename T, int CH>
+struct Buf;
+template <>
+struct Buf<uint16_t, 2> {
+  typedef uint32_t Raw;
+  __device__ static Raw load(__amdgpu_buffer_rsrc_t r, uint32_t voff,
+                             uint32_t soff) {
+    return __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
+  }
+  __device__ static void unpack(Raw u, float (&v)[2]) {
+    v[0] = __uint_as_float(u << 16);
+    v[1] = __uint_as_float(u & 0xffff0000u);
+  }
+  __device__ static void store(__amdgpu_buffer_rsrc_t r, uint32_t voff,
+                               uint32_t soff, const float (&v)[2]) {
+    __builtin_amdgcn_raw_buffer_store_b32(pack_bf16x2(v[0], v[1]), r, voff,
+                                          soff, 0);
+  }
+  // round both channels to bf16 with one convert
+  __device__ static void round(float (&v)[2]) {
+    unpack(pack_bf16x2(v[0], v[1]), v);
+  }
+};
+template <>
+struct Buf<uint16_t, 1> {
+  typedef uint16_t Raw;
+  __device__ static Raw load(__amdgpu_buffer_rsrc_t r, uint32_t voff,
+                             uint32_t soff) {
+    return __builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, 0);
+  }
+  __device__ static void unpack(Raw u, float (&v)[1]) {
+    v[0] = bf16_bits_to_f32(u);
+  }
+  __device__ static void store(__amdgpu_buffer_rsrc_t r, uint32_t voff,
+                               uint32_t soff, const float (&v)[1]) {
+    __builtin_amdgcn_raw_buffer_store_b16(f32_to_bf16_bits(v[0]), r, voff, soff,
+                                          0);
+  }
+  __device__ static void round(float (&v)[1]) { v[0] = round_to_bf16(v[0]); }
+};
+template <>
+struct Buf<float, 2> {
+  typedef u32x2 Raw;
+  __device__ static Raw load(__amdgpu_buffer_rsrc_t r, uint32_t voff,
+                             uint32_t soff) {
+    return __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0);
+  }
+  __device__ static void unpack(Raw u, float (&v)[2]) {
+    v[0] = __uint_as_float(u.x);
+    v[1] = __uint_as_float(u.y);
+  }
+  __device__ static void store(__amdgpu_buffer_rsrc_t r, uint32_t voff,
+                               uint32_t soff, const float (&v)[2]) {
+    u32x2 u = {__float_as_uint(v[0]), __float_as_uint(v[1])};
+    __builtin_amdgcn_raw_buffer_store_b64(u, r, voff, soff, 0);
+  }
+  __device__ static void round(float (&)[2]) {}
+};
+template <>
+struct Buf<float, 1> {
+  typedef uint32_t Raw;
+  __device__ static Raw load(__amdgpu_buffer_rsrc_t r, uint32_t voff,
+                             uint32_t soff) {
+    return __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
+  }
+  __device__ static void unpack(Raw u, float (&v)[1]) {
+    v[0] = __uint_as_float(u);
+  }
+  __device__ static void store(__amdgpu_buffer_rsrc_t r, uint32_t voff,
+                               uint32_t soff, const float (&v)[1]) {
+    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v[0]), r, voff, soff,
+                                          0);
+  }
+  __device__ static void round(float (&)[1]) {}
+};
 
 template <int CH>
 struct ChanConst {
@@ -35,83 +129,288 @@ struct ChanConst {
   float decay[CH];  // FAST: -8 softplus(L) log2(e);  precise: softplus(L)
 };
 
-// Phase 1 for one wave.  CHECK=false is the straight-line case: all kL tokens
-// inside the sequence and no document start among them.
-template <typename T, int CH, bool CONV, bool FAST, bool PLAIN, bool CHECK>
-__device__ __forceinline__ void phase1(
-    const char* __restrict__ xrow, const char* __restrict__ gxrow,
-    const char* __restrict__ garow, uint32_t lane_bytes, int64_t row_bytes,
-    int t0, int T_len, uint32_t starts,
-    const ChanConst<CH>& k, float (&hist)[3][CH], float (&a_)[kL][CH],
-    float (&xn_)[kL][CH], float (&P)[CH], float (&H)[CH]) {
-  using A = Act<T, CH>;
-  // All loads of the wave's kL tokens are issued before any arithmetic so that
-  // 3*kL row segments per wave are in flight; the (a, xn) results then take
-  // over the registers of the raw inputs.
-  typename A::Raw xr[kL], gxr[kL], gar[kL];
-#pragma unroll
-  for (int i = 0; i < kL; ++i) {
-    const int t = t0 + i;
-    // wave-uniform row address + 32-bit lane offset
-    const int64_t off =
-        (int64_t)(CHECK ? (t < T_len ? t : T_len - 1) : t) * row_bytes;
-    xr[i] = A::load_raw((const T*)(xrow + off + lane_bytes));
-    if (!PLAIN) gxr[i] = A::load_raw((const T*)(gxrow + off + lane_bytes));
-    gar[i] = A::load_raw((const T*)(garow + off + lane_bytes));
+// Raw inputs of one wave for one step, as loaded (bf16 pairs still packed).
+template <typename T, int CH>
+struct Tile {
+  typename Buf<T, CH>::Raw x[kL], gx[kL], ga[kL], halo[3];
+};
+
+// Where a wave's rows for one step live: descriptors based at the wave's first
+// token (clamped into the sequence) and the scalar row offset of each token,
+// with tokens past the end of the sequence redirected to the last valid row.
+struct StepAddr {
+  __amdgpu_buffer_rsrc_t rx, rgx, rga, rhalo;
+  int first;  // clamped first token
+  int last;   // last token of the sequence (T-1)
+  uint32_t row_bytes;
+  bool has_halo;  // three look-back rows exist (first token >= 3)
+  __device__ __forceinline__ uint32_t soff(int i) const {
+    const int t = first + i < last ? first + i : last;
+    return (uint32_t)(t - first) * row_bytes;
   }
+};
+
+__device__ __forceinline__ StepAddr step_addr(const char* xrow,
+                                              const char* gxrow,
+                                              const char* garow, int t0,
+                                              int T_len, uint32_t row_bytes) {
+  StepAddr a;
+  a.last = T_len - 1;
+  a.first = t0 < a.last ? t0 : a.last;
+  a.row_bytes = row_bytes;
+  const int64_t tok_bytes = (int64_t)a.first * row_bytes;
+  const uint32_t span_bytes = (uint32_t)kL * row_bytes;
+  a.rx = make_rsrc(xrow + tok_bytes, span_bytes);
+  a.rgx = make_rsrc(gxrow + tok_bytes, span_bytes);
+  a.rga = make_rsrc(garow + tok_bytes, span_bytes);
+  a.has_halo = a.first >= 3;
+  a.rhalo = make_rsrc(xrow + tok_bytes - (a.has_halo ? 3 : 0) * (int64_t)row_bytes,
+                      3 * row_bytes);
+  return a;
+}
+
+template <typename T, int CH, bool PLAIN>
+__device__ __forceinline__ void load_token(Tile<T, CH>& tl, int i,
+                                           const StepAddr& a, uint32_t voff) {
+  using B = Buf<T, CH>;
+  const uint32_t so = a.soff(i);
+  tl.x[i] = B::load(a.rx, voff, so);
+  if (!PLAIN) tl.gx[i] = B::load(a.rgx, voff, so);
+  tl.ga[i] = B::load(a.rga, voff, so);
+}
+
+template <typename T, int CH, bool CONV>
+__device__ __forceinline__ void load_halo(Tile<T, CH>& tl, const StepAddr& a,
+                                          uint32_t voff) {
+  using B = Buf<T, CH>;
+  if (CONV && a.has_halo) {
+#pragma unroll
+    for (int s = 0; s < 3; ++s)  // halo[s] = x[first-1-s]
+      tl.halo[s] = B::load(a.rhalo, voff, (uint32_t)(2 - s) * a.row_bytes);
+  } else {
+#pragma unroll
+    for (int s = 0; s < 3; ++s) tl.halo[s] = typename B::Raw{};
+  }
+}
+
+// Raw segment value this lane looks at for the step starting at token t0
+// (token t0-3+lane).  One member per encoding, each written by its own guarded
+// load and defaulting to "no document start": the three are never merged into
+// one register, so issuing the load does not wait for anything.
+struct SegRaw {
+  int64_t v64;
+  int32_t v32;
+  uint32_t v8;
+};
+
+template <bool CONV>
+__device__ __forceinline__ SegRaw load_seg(const ScanArgs& p, int64_t row0,
+                                           int t0, int T_len, int lane) {
+  const int t = t0 - 3 + lane;
+  const bool look =
+      lane < kL + 3 && (CONV || lane >= 3) && t >= 0 && t < T_len;
+  SegRaw r;
+  r.v64 = 1;
+  r.v32 = 1;
+  r.v8 = 0;
+  if (look && p.seg_kind == kSegI64)
+    r.v64 = reinterpret_cast<const int64_t*>(p.segpos)[row0 + t];
+  if (look && p.seg_kind == kSegI32)
+    r.v32 = reinterpret_cast<const int32_t*>(p.segpos)[row0 + t];
+  if (look && p.seg_kind == kSegMaskU8)
+    r.v8 = reinterpret_cast<const uint8_t*>(p.segpos)[row0 + t];
+  return r;
+}
+
+// Keeps a rarely taken, wave-uniform block a real branch (the compiler would
+// otherwise turn it into per-lane selects that every token pays for).
+#define RG_RARE_BLOCK() asm volatile("" ::: "memory")
+
+// Gating arithmetic of one token: (xc, gate pre-activations) -> (a, xn).
+template <int CH, bool FAST, bool PLAIN>
+__device__ __forceinline__ void gate_math(const float (&xc)[CH],
+                                          const float (&gxv)[CH],
+                                          const float (&gav)[CH],
+                                          const float (&decay)[CH], bool start,
+                                          float (&a)[CH], float (&xn)[CH]) {
+#pragma unroll
+  for (int ch = 0; ch < CH; ++ch) {
+    float mult, gate_x;
+    if (PLAIN) {
+      a[ch] = gav[ch];
+      mult = 1.0f;
+      gate_x = 1.0f;
+    } else if (FAST) {
+      gate_x = sigmoid_fast(gxv[ch]);
+      const float gate_a = sigmoid_fast(gav[ch]);
+      a[ch] = __builtin_amdgcn_exp2f(gate_a * decay[ch]);
+      mult = __builtin_amdgcn_sqrtf(__builtin_fmaf(-a[ch], a[ch], 1.0f));
+    } else {
+      gate_x = sigmoid_precise(gxv[ch]);
+      const float gate_a = sigmoid_precise(gav[ch]);
+      const float log_a = (-8.0f * gate_a) * decay[ch];
+      a[ch] = expf(log_a);
+      mult = sqrtf(1.0f - expf(2.0f * log_a));
+    }
+    if (start) {  // only the slow path passes a non-constant `start`
+      a[ch] = 0.0f;
+      mult = 1.0f;
+    }
+    xn[ch] = PLAIN ? xc[ch] : (xc[ch] * gate_x) * mult;
+  }
+}
+
+// Phase 1, hot path: straight-line code for a step without a document start
+// among the wave's tokens or its three look-back tokens.  Tokens past the end
+// of the sequence are computed on a re-read of the last valid row; their
+// results are never stored and can only reach state that nothing reads any
+// more.  As soon as a token's raw inputs have been consumed, the same
+// registers are reloaded with that token's row of the NEXT step (`next`), so
+// the next step's data is in flight for a whole step without a second set of
+// registers.  After the last step the reload is redundant but harmless:
+// `next` is clamped into the sequence.
+template <typename T, int CH, bool CONV, bool FAST, bool PLAIN>
+__device__ __forceinline__ void phase1(
+    Tile<T, CH>& tl, const StepAddr& next, uint32_t voff,
+    const ChanConst<CH>& k, float (&a_)[kL][CH], float (&xn_)[kL][CH],
+    float (&P)[CH], float (&H)[CH]) {
+  using B = Buf<T, CH>;
+  float hist[3][CH];
+#pragma unroll
+  for (int s = 0; s < 3; ++s) B::unpack(tl.halo[s], hist[s]);
+  __builtin_amdgcn_sched_barrier(0);
+  load_halo<T, CH, CONV>(tl, next, voff);
 #pragma unroll
   for (int i = 0; i < kL; ++i) {
-    const int t = t0 + i;
-    const bool valid = !CHECK || (t < T_len);
-    const bool start = CHECK && ((starts >> (i + 3)) & 1u);
-    float xv[CH], gxv[CH], gav[CH];
-    A::unpack(xr[i], xv);
-    if (!PLAIN) A::unpack(gxr[i], gxv);
-    A::unpack(gar[i], gav);
+    float xv[CH], gxv[CH], gav[CH], xc[CH];
+    B::unpack(tl.x[i], xv);
+    if (!PLAIN) B::unpack(tl.gx[i], gxv);
+    B::unpack(tl.ga[i], gav);
+    // The reload must follow the last read of the registers it overwrites;
+    // without these fences the scheduler hoists it, the old and new values
+    // overlap, and the new tile needs copies (and full waits) every step.
+    __builtin_amdgcn_sched_barrier(0);
+    load_token<T, CH, PLAIN>(tl, i, next, voff);
+    __builtin_amdgcn_sched_barrier(0);
+    if (CONV) {
 #pragma unroll
-    for (int ch = 0; ch < CH; ++ch) {
-      float xc;
-      if (CONV) {
-        if (start) hist[0][ch] = hist[1][ch] = hist[2][ch] = 0.0f;
-        xc = A::round(conv4(xv[ch], hist[0][ch], hist[1][ch], hist[2][ch],
-                            k.w0[ch], k.w1[ch], k.w2[ch], k.w3[ch],
-                            k.bias[ch]));
+      for (int ch = 0; ch < CH; ++ch) {
+        xc[ch] = conv4(xv[ch], hist[0][ch], hist[1][ch], hist[2][ch], k.w0[ch],
+                       k.w1[ch], k.w2[ch], k.w3[ch], k.bias[ch]);
         hist[2][ch] = hist[1][ch];
         hist[1][ch] = hist[0][ch];
         hist[0][ch] = xv[ch];
-      } else {
-        xc = xv[ch];
       }
-      float a, mult, gate_x;
-      if (PLAIN) {
-        a = gav[ch];
-        mult = 1.0f;
-        gate_x = 1.0f;
-      } else if (FAST) {
-        gate_x = sigmoid_fast(gxv[ch]);
-        const float gate_a = sigmoid_fast(gav[ch]);
-        a = __builtin_amdgcn_exp2f(gate_a * k.decay[ch]);
-        mult = __builtin_amdgcn_sqrtf(__builtin_fmaf(-a, a, 1.0f));
-      } else {
-        gate_x = sigmoid_precise(gxv[ch]);
-        const float gate_a = sigmoid_precise(gav[ch]);
-        const float log_a = (-8.0f * gate_a) * k.decay[ch];
-        a = expf(log_a);
-        mult = sqrtf(1.0f - expf(2.0f * log_a));
+      B::round(xc);  // the conv output is a module output: activation dtype
+    } else {
+#pragma unroll
+      for (int ch = 0; ch < CH; ++ch) xc[ch] = xv[ch];
+    }
+    gate_math<CH, FAST, PLAIN>(xc, gxv, gav, k.decay, false, a_[i], xn_[i]);
+#pragma unroll
+    for (int ch = 0; ch < CH; ++ch) {
+      H[ch] = __builtin_fmaf(a_[i][ch], H[ch], xn_[i][ch]);
+      P[ch] = P[ch] * a_[i][ch];
+    }
+  }
+}
+
+// Phase 1, slow path: a step with a document start.  Recomputes the wave's
+// (a, xn) pairs from memory (the rows are still in cache), token by token,
+// with the conv history cut at every start, a = 0 and input scale 1 there.
+// It does not touch the prefetched tile.
+template <typename T, int CH, bool CONV, bool FAST, bool PLAIN>
+__device__ __forceinline__ void phase1_with_starts(
+    const StepAddr& cur, uint32_t voff, uint32_t starts,
+    const ChanConst<CH>& k, float (&a_)[kL][CH], float (&xn_)[kL][CH],
+    float (&P)[CH], float (&H)[CH]) {
+  using B = Buf<T, CH>;
+  float hist[3][CH];
+#pragma unroll
+  for (int s = 0; s < 3; ++s)
+#pragma unroll
+    for (int ch = 0; ch < CH; ++ch) hist[s][ch] = 0.0f;
+  if (CONV && cur.has_halo) {
+#pragma unroll
+    for (int s = 0; s < 3; ++s)  // hist[s] = x[first-1-s]
+      B::unpack(B::load(cur.rhalo, voff, (uint32_t)(2 - s) * cur.row_bytes),
+                hist[s]);
+    // a document start at first-1 hides x[first-2], x[first-3]; one at first-2
+    // hides x[first-3]
+    if (starts & 4u) {
+#pragma unroll
+      for (int ch = 0; ch < CH; ++ch) hist[1][ch] = hist[2][ch] = 0.0f;
+    }
+    if (starts & 2u) {
+#pragma unroll
+      for (int ch = 0; ch < CH; ++ch) hist[2][ch] = 0.0f;
+    }
+  }
+#pragma unroll
+  for (int ch = 0; ch < CH; ++ch) {
+    P[ch] = 1.0f;
+    H[ch] = 0.0f;
+  }
+#pragma unroll
+  for (int i = 0; i < kL; ++i) {
+    const bool start = (starts >> (i + 3)) & 1u;
+    const uint32_t so = cur.soff(i);
+    float xv[CH], gxv[CH], gav[CH], xc[CH], a[CH], xn[CH];
+    B::unpack(B::load(cur.rx, voff, so), xv);
+    if (!PLAIN) B::unpack(B::load(cur.rgx, voff, so), gxv);
+    B::unpack(B::load(cur.rga, voff, so), gav);
+    if (CONV) {
+#pragma unroll
+      for (int ch = 0; ch < CH; ++ch) {
+        if (start) hist[0][ch] = hist[1][ch] = hist[2][ch] = 0.0f;
+        xc[ch] = conv4(xv[ch], hist[0][ch], hist[1][ch], hist[2][ch], k.w0[ch],
+                       k.w1[ch], k.w2[ch], k.w3[ch], k.bias[ch]);
+        hist[2][ch] = hist[1][ch];
+        hist[1][ch] = hist[0][ch];
+        hist[0][ch] = xv[ch];
       }
-      if (start) {
-        a = 0.0f;
-        mult = 1.0f;
-      }
-      float xn = PLAIN ? xc : (xc * gate_x) * mult;
-      if (!valid) {
-        a = 1.0f;
-        xn = 0.0f;
-      }
-      a_[i][ch] = a;
-      xn_[i][ch] = xn;
-      H[ch] = __builtin_fmaf(a, H[ch], xn);
-      P[ch] = P[ch] * a;
+      B::round(xc);
+    } else {
+#pragma unroll
+      for (int ch = 0; ch < CH; ++ch) xc[ch] = xv[ch];
+    }
+    gate_math<CH, FAST, PLAIN>(xc, gxv, gav, k.decay, start, a, xn);
+#pragma unroll
+    for (int ch = 0; ch < CH; ++ch) {
+      a_[i][ch] = a[ch];
+      xn_[i][ch] = xn[ch];
+      H[ch] = __builtin_fmaf(a[ch], H[ch], xn[ch]);
+      P[ch] = P[ch] * a[ch];
+    }
+  }
+}
+
+// Phase 2: replay the recurrence from the incoming state and write y.  Stores
+// of tokens past the end of the sequence get a scalar offset outside the
+// descriptor and are dropped by the range check.  The state after token T-1
+// is written to h_last by the wave that holds that token.
+template <typename T, int CH>
+__device__ __forceinline__ void phase2(__amdgpu_buffer_rsrc_t ry, uint32_t voff,
+                                       uint32_t row_bytes, int n_valid,
+                                       float* h_last_lane,
+                                       const float (&a_)[kL][CH],
+                                       const float (&xn_)[kL][CH],
+                                       float (&h)[CH]) {
+  using B = Buf<T, CH>;
+#pragma unroll
+  for (int i = 0; i < kL; ++i) {
+    float out[CH];
+#pragma unroll
+    for (int ch = 0; ch < CH; ++ch) {
+      h[ch] = __builtin_fmaf(a_[i][ch], h[ch], xn_[i][ch]);
+      out[ch] = h[ch];
+    }
+    B::store(ry, voff, i < n_valid ? (uint32_t)i * row_bytes : 0x80000000u,
+             out);
+    if (h_last_lane && i == n_valid - 1) {
+      RG_RARE_BLOCK();
+#pragma unroll
+      for (int ch = 0; ch < CH; ++ch) h_last_lane[ch] = h[ch];
     }
   }
 }
@@ -120,6 +419,7 @@ template <typename T, int CH, bool CONV, bool FAST, bool PLAIN>
 __global__ void __launch_bounds__(kMaxNW* kWave, (sizeof(T) == 2 ? 4 : 2))
 lru_scan_kernel(ScanArgs p) {
   using A = Act<T, CH>;
+  using B = Buf<T, CH>;
   __shared__ float agg[2][kMaxNW][kWave][2 * CH];  // (P.., Hloc..) per lane
   __shared__ float carry_s[2][kWave][CH];
 
@@ -133,7 +433,7 @@ lru_scan_kernel(ScanArgs p) {
   const int slab = blockIdx.x - b * nslab;
   const int c_raw = (slab * kWave + lane) * CH;
   const bool active = c_raw < p.W;  // W % CH == 0, so the whole vector is in
-  const int c = active ? c_raw : 0;
+  const int c = active ? c_raw : 0;  // for the few plain-pointer accesses
 
   ChanConst<CH> k;
 #pragma unroll
@@ -158,90 +458,88 @@ lru_scan_kernel(ScanArgs p) {
   }
 
   const int64_t row0 = (int64_t)b * T_len;
-  const int64_t row_bytes = W * (int64_t)sizeof(T);
-  const uint32_t lane_bytes = (uint32_t)c * (uint32_t)sizeof(T);
+  const uint32_t row_bytes = (uint32_t)p.W * (uint32_t)sizeof(T);
+  // lanes past the last channel get an offset beyond every descriptor's range
+  // (whether or not the scalar row offset takes part in the range check):
+  // their loads return 0 and their stores are dropped
+  const uint32_t voff =
+      active ? (uint32_t)c_raw * (uint32_t)sizeof(T) : 0x80000000u;
+  const uint32_t span_bytes = (uint32_t)kL * row_bytes;
   // wave-uniform pointers to token 0 of this batch row
   const char* xrow = (const char*)p.x + row0 * row_bytes;
   const char* gxrow = (const char*)p.gx + row0 * row_bytes;
   const char* garow = (const char*)p.ga + row0 * row_bytes;
   char* yrow = (char*)p.y + row0 * row_bytes;
 
-  float h_first[CH];
-#pragma unroll
-  for (int ch = 0; ch < CH; ++ch)
-    h_first[ch] = p.h0 ? p.h0[(int64_t)b * W + c + ch] : 0.0f;
-
-  const int span = nw * kL;
   float h[CH];
 #pragma unroll
-  for (int ch = 0; ch < CH; ++ch) h[ch] = h_first[ch];
+  for (int ch = 0; ch < CH; ++ch)
+    h[ch] = p.h0 ? p.h0[(int64_t)b * W + c + ch] : 0.0f;
+
+  const int span = nw * kL;
+
+  // bit j of `starts` = token t0-3+j of the step at hand starts a document.
+  // It is a scalar: the next step's mask is formed (one ballot) at the end of
+  // the current step and costs no vector register in between.
+  auto doc_starts = [&](SegRaw seg) {
+    // The empty asm pins the comparison here: without it the compiler tests
+    // the value right behind its load, i.e. waits for the load (and for every
+    // older load and store) at the top of the step.
+    uint32_t lo = (uint32_t)seg.v64, hi = (uint32_t)((uint64_t)seg.v64 >> 32);
+    asm volatile("" : "+v"(lo), "+v"(hi), "+v"(seg.v32), "+v"(seg.v8));
+    const bool st = ((lo | hi) == 0u) | (seg.v32 == 0) | (seg.v8 != 0u);
+    return (uint32_t)__ballot(st);
+  };
+
+  // Every wave runs every step with the same code, so that the prefetched
+  // tile is never merged with a copy of itself at a branch join (that would
+  // cost register copies and a full wait per step).  A wave whose tokens lie
+  // past the end of the sequence works on a re-read of the last row, drops
+  // its stores and contributes the identity pair.
+
+  // prologue: the first step's rows
+  Tile<T, CH> tl;
+  uint32_t starts;
+  {
+    const SegRaw seg = load_seg<CONV>(p, row0, wave * kL, T_len, lane);
+    const StepAddr a0 =
+        step_addr(xrow, gxrow, garow, wave * kL, T_len, row_bytes);
+    load_halo<T, CH, CONV>(tl, a0, voff);
+#pragma unroll
+    for (int i = 0; i < kL; ++i) load_token<T, CH, PLAIN>(tl, i, a0, voff);
+    starts = doc_starts(seg);
+  }
 
   for (int step = 0, tb = 0; tb < T_len; ++step, tb += span) {
     const int buf = step & 1;
     const int t0 = tb + wave * kL;
     const bool any = t0 < T_len;
+    // tokens of this wave inside the sequence (<= 0: none)
+    const int n_valid = T_len - t0 < kL ? T_len - t0 : kL;
     float a_[kL][CH], xn_[kL][CH], P[CH], H[CH];
 #pragma unroll
     for (int ch = 0; ch < CH; ++ch) {
       P[ch] = 1.0f;
       H[ch] = 0.0f;
     }
-    if (any) {
-      // bit j <-> token t0-3+j starts a document (only tokens inside the row;
-      // the three look-back tokens matter only for the conv history).
-      // Lane j looks at token t0-3+j: one coalesced load and one ballot for
-      // the whole wave instead of kL+3 dependent loads.
-      bool st = false;
-      {
-        const int t = t0 - 3 + lane;
-        if (lane < kL + 3 && (CONV || lane >= 3) && t >= 0 && t < T_len)
-          st = is_doc_start(p.segpos, p.seg_kind, row0 + t);
-      }
-      const uint32_t starts = (uint32_t)__ballot(st);
-      float hist[3][CH];
-      if (CONV) {
-#pragma unroll
-        for (int s = 1; s <= 3; ++s) {
-          const int t = t0 - s;
-          float v[CH];
-          A::load((const T*)(xrow + (int64_t)(t < 0 ? 0 : t) * row_bytes +
-                             lane_bytes), v);
-#pragma unroll
-          for (int ch = 0; ch < CH; ++ch) hist[s - 1][ch] = t < 0 ? 0.0f : v[ch];
-        }
-        // a document start at t0-1 hides x[t0-2], x[t0-3]; one at t0-2 hides
-        // x[t0-3].
-        if (starts & 4u) {
-#pragma unroll
-          for (int ch = 0; ch < CH; ++ch) hist[1][ch] = hist[2][ch] = 0.0f;
-        }
-        if (starts & 2u) {
-#pragma unroll
-          for (int ch = 0; ch < CH; ++ch) hist[2][ch] = 0.0f;
-        }
-      } else {
-#pragma unroll
-        for (int ch = 0; ch < CH; ++ch)
-          hist[0][ch] = hist[1][ch] = hist[2][ch] = 0.0f;
-      }
-      const bool plain = (t0 + kL <= T_len) && ((starts >> 3) == 0u);
-      if (plain)
-        phase1<T, CH, CONV, FAST, PLAIN, false>(xrow, gxrow, garow, lane_bytes,
-                                                row_bytes, t0, T_len, starts, k,
-                                                hist, a_, xn_, P, H);
-      else
-        phase1<T, CH, CONV, FAST, PLAIN, true>(xrow, gxrow, garow, lane_bytes,
-                                               row_bytes, t0, T_len, starts, k,
-                                               hist, a_, xn_, P, H);
+    const StepAddr next =
+        step_addr(xrow, gxrow, garow, t0 + span, T_len, row_bytes);
+    const SegRaw seg_next = load_seg<CONV>(p, row0, t0 + span, T_len, lane);
+    phase1<T, CH, CONV, FAST, PLAIN>(tl, next, voff, k, a_, xn_, P, H);
+    if (starts != 0u) {
+      RG_RARE_BLOCK();
+      const StepAddr cur = step_addr(xrow, gxrow, garow, t0, T_len, row_bytes);
+      phase1_with_starts<T, CH, CONV, FAST, PLAIN>(cur, voff, starts, k, a_,
+                                                   xn_, P, H);
     }
 
     // exchange
 #pragma unroll
     for (int ch = 0; ch < CH; ++ch) {
-      agg[buf][wave][lane][ch] = P[ch];
-      agg[buf][wave][lane][CH + ch] = H[ch];
+      agg[buf][wave][lane][ch] = any ? P[ch] : 1.0f;
+      agg[buf][wave][lane][CH + ch] = any ? H[ch] : 0.0f;
     }
-    __syncthreads();
+    lds_barrier();  // LDS only: prefetched rows stay in flight
     if (step > 0) {
 #pragma unroll
       for (int ch = 0; ch < CH; ++ch) h[ch] = carry_s[buf ^ 1][lane][ch];
@@ -253,30 +551,26 @@ lru_scan_kernel(ScanArgs p) {
                                agg[buf][v][lane][CH + ch]);
     }
 
-    // phase 2
-    if (any) {
+    {
+      const __amdgpu_buffer_rsrc_t ry = make_rsrc(
+          yrow + (int64_t)(t0 < T_len ? t0 : T_len - 1) * row_bytes, span_bytes);
+      // this wave holds token T-1 iff its valid tokens end the sequence
+      float* const h_last_lane =
+          (p.h_last && active && any && t0 + n_valid == T_len)
+              ? p.h_last + (int64_t)b * W + c
+              : nullptr;
+      float hw[CH];  // the replay runs on a copy: an empty wave must not
+#pragma unroll       // disturb the carry it may have to hand on
+      for (int ch = 0; ch < CH; ++ch) hw[ch] = h[ch];
+      phase2<T, CH>(ry, voff, row_bytes, n_valid, h_last_lane, a_, xn_, hw);
 #pragma unroll
-      for (int i = 0; i < kL; ++i) {
-        float out[CH];
-#pragma unroll
-        for (int ch = 0; ch < CH; ++ch) {
-          h[ch] = __builtin_fmaf(a_[i][ch], h[ch], xn_[i][ch]);
-          out[ch] = h[ch];
-        }
-        if (t0 + i < T_len && active)
-          A::store((T*)(yrow + (int64_t)(t0 + i) * row_bytes + lane_bytes), out);
-      }
+      for (int ch = 0; ch < CH; ++ch) h[ch] = any ? hw[ch] : h[ch];
     }
     if (wave == nw - 1) {
 #pragma unroll
       for (int ch = 0; ch < CH; ++ch) carry_s[buf][lane][ch] = h[ch];
     }
-  }
-
-  // The last wave's h after the final step is h_{T-1}.
-  if (wave == nw - 1 && p.h_last && active) {
-#pragma unroll
-    for (int ch = 0; ch < CH; ++ch) p.h_last[(int64_t)b * W + c + ch] = h[ch];
+    starts = doc_starts(seg_next);
   }
 
   // Masked conv state: rows T-3..T-1 of x, each zeroed if a document starts in
@@ -292,7 +586,7 @@ lru_scan_kernel(ScanArgs p) {
       for (int ch = 0; ch < CH; ++ch) v[ch] = 0.0f;
       if (t >= 0) {
         if (!later_start)
-          A::load((const T*)(xrow + (int64_t)t * row_bytes + lane_bytes), v);
+          A::load((const T*)(xrow + (int64_t)t * row_bytes) + c, v);
         if (is_doc_start(p.segpos, p.seg_kind, row0 + t))
           later_start = true;
       }
@@ -307,7 +601,9 @@ hipError_t launch_t(const ScanArgs& a, hipStream_t s) {
   int nw = 1;
   while (nw < kMaxNW && nw * kL < a.T) nw *= 2;
   const int64_t blocks = (int64_t)a.B * nslab;
-  if (blocks > 0x7fffffff) return hipErrorInvalidValue;
+  // one row must fit a buffer descriptor's 32-bit scalar offsets
+  if (blocks > 0x7fffffff || (int64_t)a.W * sizeof(T) * (kL + 3) > 0x7fffffff)
+    return hipErrorInvalidValue;
   lru_scan_kernel<T, CH, CONV, FAST, PLAIN>
       <<<dim3((unsigned)blocks), dim3(nw * kWave), 0, s>>>(a);
   return hipGetLastError();
