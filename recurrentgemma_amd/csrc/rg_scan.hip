@@ -3,8 +3,8 @@
 // Work decomposition.  Lanes map to channels (CH adjacent channels per lane),
 // so every global access of a wave is one contiguous row segment.  A workgroup
 // owns one batch row and one slab of 64*CH channels and walks the sequence in
-// steps of nw*kL tokens (nw = waves in the group).  Inside a step, wave v
-// takes the kL consecutive tokens [v*kL, (v+1)*kL):
+// steps of nw*KL tokens (nw = waves in the group).  Inside a step, wave v
+// takes the KL consecutive tokens [v*KL, (v+1)*KL):
 //
 //   phase 1  each wave reads x / gate pre-activations for its tokens, applies
 //            the conv, the sigmoids, a = exp(-8 softplus(L) sigmoid(ga)) and
@@ -16,25 +16,36 @@
 //            incoming state;
 //   phase 2  each wave replays h = a_t h + xn_t from that state and writes y.
 //
-// The carry into the next step is the last wave's final h.  Tokens past the
-// end of the sequence are the operator's identity (1, 0).  A document start
-// (segment_pos == 0) sets a = 0 and the input scale to 1, and zeroes the conv
-// history, which is exactly the reference's masking rule.
+// The carry into the next step is the last wave's final h.  A document start
+// (segment_pos == 0) sets a = 0 and the input scale to 1 and cuts the conv
+// history, which is exactly the reference's masking rule; steps that contain
+// one are recomputed on a separate, rarely taken path so that the common path
+// is straight-line code.  Tokens past the end of the sequence are computed on
+// a re-read of the last valid row; their stores are dropped and their results
+// can only reach state that nothing reads any more.
+//
+// The kernel is bound by the memory system, not by arithmetic: on MI355X the
+// achieved rate depends on the bytes per lane and the step length (8 bytes per
+// lane and short steps stream best) and on marking the streamed rows
+// non-temporal.
 //
 // Addressing.  All row traffic goes through buffer instructions: a scalar
-// resource descriptor whose base is the wave's first token of the step and
-// whose size is the wave's kL rows, a per-lane byte offset that never changes,
-// and a scalar row offset.  No per-access vector address arithmetic is needed.
-// Lanes past the last channel carry an offset beyond any descriptor's size, so
-// the hardware range check returns 0 for their loads and drops their stores.
+// resource descriptor based at the wave's first token of the step, a per-lane
+// byte offset that never changes, and a scalar row offset.  No per-access
+// vector address arithmetic is needed.  The hardware range check covers the
+// scalar offset as well, which is used twice: lanes past the last channel
+// carry a huge lane offset and rows past the end of the sequence a huge scalar
+// offset, so their loads return 0 and their stores are dropped.
 #include "rg_common.h"
 #include "rg_internal.h"
 
 namespace rg {
 namespace {
 
-constexpr int kL = 8;      // tokens per wave per step
-constexpr int kMaxNW = 8;  // waves per workgroup
+constexpr int kMaxNW = 16;  // waves per workgroup
+constexpr uint32_t kOutOfRange = 0x80000000u;
+// cache policy of the streamed rows: non-temporal (read or written once)
+constexpr int kStream = 2;
 
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
@@ -45,27 +56,54 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base,
                                            (int)bytes, 0x00020000);
 }
 
-// Buffer access of CH adjacent channels.  Raw keeps bf16 pairs packed in one
-// register until they are used.
+// Buffer access of CH adjacent channels.  Raw keeps bf16 values packed until
+// they are used.
 template <typename T, int CH>
 struct Buf;
 template <>
-struct Buf<uint16_t, 2> {
-  typedef uint32_t Raw;
+struct Buf<uint16_t, 4> {
+  typedef u32x2 Raw;
+  template <int AUX>
   __device__ static Raw load(__amdgpu_buffer_rsrc_t r, uint32_t voff,
                              uint32_t soff) {
-    return __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
+    return __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, AUX);
+  }
+  __device__ static void unpack(Raw u, float (&v)[4]) {
+    v[0] = __uint_as_float(u.x << 16);
+    v[1] = __uint_as_float(u.x & 0xffff0000u);
+    v[2] = __uint_as_float(u.y << 16);
+    v[3] = __uint_as_float(u.y & 0xffff0000u);
+  }
+  template <int AUX>
+  __device__ static void store(__amdgpu_buffer_rsrc_t r, uint32_t voff,
+                               uint32_t soff, const float (&v)[4]) {
+    u32x2 u = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+    __builtin_amdgcn_raw_buffer_store_b64(u, r, voff, soff, AUX);
+  }
+  // round to bf16, two channels per convert
+  __device__ static void round(float (&v)[4]) {
+    u32x2 u = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+    unpack(u, v);
+  }
+};
+template <>
+struct Buf<uint16_t, 2> {
+  typedef uint32_t Raw;
+  template <int AUX>
+  __device__ static Raw load(__amdgpu_buffer_rsrc_t r, uint32_t voff,
+                             uint32_t soff) {
+    return __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, AUX);
   }
   __device__ static void unpack(Raw u, float (&v)[2]) {
     v[0] = __uint_as_float(u << 16);
     v[1] = __uint_as_float(u & 0xffff0000u);
   }
+  template <int AUX>
   __device__ static void store(__amdgpu_buffer_rsrc_t r, uint32_t voff,
                                uint32_t soff, const float (&v)[2]) {
     __builtin_amdgcn_raw_buffer_store_b32(pack_bf16x2(v[0], v[1]), r, voff,
-                                          soff, 0);
+                                          soff, AUX);
   }
-  // round both channels to bf16 with one convert
   __device__ static void round(float (&v)[2]) {
     unpack(pack_bf16x2(v[0], v[1]), v);
   }
@@ -73,52 +111,58 @@ struct Buf<uint16_t, 2> {
 template <>
 struct Buf<uint16_t, 1> {
   typedef uint16_t Raw;
+  template <int AUX>
   __device__ static Raw load(__amdgpu_buffer_rsrc_t r, uint32_t voff,
                              uint32_t soff) {
-    return __builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, 0);
+    return __builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, AUX);
   }
   __device__ static void unpack(Raw u, float (&v)[1]) {
     v[0] = bf16_bits_to_f32(u);
   }
+  template <int AUX>
   __device__ static void store(__amdgpu_buffer_rsrc_t r, uint32_t voff,
                                uint32_t soff, const float (&v)[1]) {
     __builtin_amdgcn_raw_buffer_store_b16(f32_to_bf16_bits(v[0]), r, voff, soff,
-                                          0);
+                                          AUX);
   }
   __device__ static void round(float (&v)[1]) { v[0] = round_to_bf16(v[0]); }
 };
 template <>
 struct Buf<float, 2> {
   typedef u32x2 Raw;
+  template <int AUX>
   __device__ static Raw load(__amdgpu_buffer_rsrc_t r, uint32_t voff,
                              uint32_t soff) {
-    return __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0);
+    return __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, AUX);
   }
   __device__ static void unpack(Raw u, float (&v)[2]) {
     v[0] = __uint_as_float(u.x);
     v[1] = __uint_as_float(u.y);
   }
+  template <int AUX>
   __device__ static void store(__amdgpu_buffer_rsrc_t r, uint32_t voff,
                                uint32_t soff, const float (&v)[2]) {
     u32x2 u = {__float_as_uint(v[0]), __float_as_uint(v[1])};
-    __builtin_amdgcn_raw_buffer_store_b64(u, r, voff, soff, 0);
+    __builtin_amdgcn_raw_buffer_store_b64(u, r, voff, soff, AUX);
   }
   __device__ static void round(float (&)[2]) {}
 };
 template <>
 struct Buf<float, 1> {
   typedef uint32_t Raw;
+  template <int AUX>
   __device__ static Raw load(__amdgpu_buffer_rsrc_t r, uint32_t voff,
                              uint32_t soff) {
-    return __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
+    return __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, AUX);
   }
   __device__ static void unpack(Raw u, float (&v)[1]) {
     v[0] = __uint_as_float(u);
   }
+  template <int AUX>
   __device__ static void store(__amdgpu_buffer_rsrc_t r, uint32_t voff,
                                uint32_t soff, const float (&v)[1]) {
     __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v[0]), r, voff, soff,
-                                          0);
+                                          AUX);
   }
   __device__ static void round(float (&)[1]) {}
 };
@@ -129,15 +173,10 @@ struct ChanConst {
   float decay[CH];  // FAST: -8 softplus(L) log2(e);  precise: softplus(L)
 };
 
-// Raw inputs of one wave for one step, as loaded (bf16 pairs still packed).
-template <typename T, int CH>
-struct Tile {
-  typename Buf<T, CH>::Raw x[kL], gx[kL], ga[kL], halo[3];
-};
-
 // Where a wave's rows for one step live: descriptors based at the wave's first
 // token (clamped into the sequence) and the scalar row offset of each token,
 // with tokens past the end of the sequence redirected to the last valid row.
+template <int KL>
 struct StepAddr {
   __amdgpu_buffer_rsrc_t rx, rgx, rga, rhalo;
   int first;  // clamped first token
@@ -150,43 +189,55 @@ struct StepAddr {
   }
 };
 
-__device__ __forceinline__ StepAddr step_addr(const char* xrow,
-                                              const char* gxrow,
-                                              const char* garow, int t0,
-                                              int T_len, uint32_t row_bytes) {
-  StepAddr a;
+template <int KL>
+__device__ __forceinline__ StepAddr<KL> step_addr(const char* xrow,
+                                                  const char* gxrow,
+                                                  const char* garow, int t0,
+                                                  int T_len,
+                                                  uint32_t row_bytes) {
+  StepAddr<KL> a;
   a.last = T_len - 1;
   a.first = t0 < a.last ? t0 : a.last;
   a.row_bytes = row_bytes;
   const int64_t tok_bytes = (int64_t)a.first * row_bytes;
-  const uint32_t span_bytes = (uint32_t)kL * row_bytes;
+  const uint32_t span_bytes = (uint32_t)KL * row_bytes;
   a.rx = make_rsrc(xrow + tok_bytes, span_bytes);
   a.rgx = make_rsrc(gxrow + tok_bytes, span_bytes);
   a.rga = make_rsrc(garow + tok_bytes, span_bytes);
   a.has_halo = a.first >= 3;
-  a.rhalo = make_rsrc(xrow + tok_bytes - (a.has_halo ? 3 : 0) * (int64_t)row_bytes,
-                      3 * row_bytes);
+  a.rhalo =
+      make_rsrc(xrow + tok_bytes - (a.has_halo ? 3 : 0) * (int64_t)row_bytes,
+                3 * row_bytes);
   return a;
 }
 
-template <typename T, int CH, bool PLAIN>
-__device__ __forceinline__ void load_token(Tile<T, CH>& tl, int i,
-                                           const StepAddr& a, uint32_t voff) {
+// Raw inputs of one wave for one step, as loaded (bf16 values still packed).
+template <typename T, int CH, int KL>
+struct Tile {
+  typename Buf<T, CH>::Raw x[KL], gx[KL], ga[KL], halo[3];
+};
+
+template <typename T, int CH, int KL, bool PLAIN>
+__device__ __forceinline__ void load_token(Tile<T, CH, KL>& tl, int i,
+                                           const StepAddr<KL>& a,
+                                           uint32_t voff) {
   using B = Buf<T, CH>;
   const uint32_t so = a.soff(i);
-  tl.x[i] = B::load(a.rx, voff, so);
-  if (!PLAIN) tl.gx[i] = B::load(a.rgx, voff, so);
-  tl.ga[i] = B::load(a.rga, voff, so);
+  tl.x[i] = B::template load<kStream>(a.rx, voff, so);
+  if (!PLAIN) tl.gx[i] = B::template load<kStream>(a.rgx, voff, so);
+  tl.ga[i] = B::template load<kStream>(a.rga, voff, so);
 }
 
-template <typename T, int CH, bool CONV>
-__device__ __forceinline__ void load_halo(Tile<T, CH>& tl, const StepAddr& a,
+template <typename T, int CH, int KL, bool CONV>
+__device__ __forceinline__ void load_halo(Tile<T, CH, KL>& tl,
+                                          const StepAddr<KL>& a,
                                           uint32_t voff) {
   using B = Buf<T, CH>;
   if (CONV && a.has_halo) {
 #pragma unroll
     for (int s = 0; s < 3; ++s)  // halo[s] = x[first-1-s]
-      tl.halo[s] = B::load(a.rhalo, voff, (uint32_t)(2 - s) * a.row_bytes);
+      tl.halo[s] =
+          B::template load<0>(a.rhalo, voff, (uint32_t)(2 - s) * a.row_bytes);
   } else {
 #pragma unroll
     for (int s = 0; s < 3; ++s) tl.halo[s] = typename B::Raw{};
@@ -203,12 +254,12 @@ struct SegRaw {
   uint32_t v8;
 };
 
-template <bool CONV>
+template <int KL, bool CONV>
 __device__ __forceinline__ SegRaw load_seg(const ScanArgs& p, int64_t row0,
                                            int t0, int T_len, int lane) {
   const int t = t0 - 3 + lane;
   const bool look =
-      lane < kL + 3 && (CONV || lane >= 3) && t >= 0 && t < T_len;
+      lane < KL + 3 && (CONV || lane >= 3) && t >= 0 && t < T_len;
   SegRaw r;
   r.v64 = 1;
   r.v32 = 1;
@@ -220,6 +271,17 @@ __device__ __forceinline__ SegRaw load_seg(const ScanArgs& p, int64_t row0,
   if (look && p.seg_kind == kSegMaskU8)
     r.v8 = reinterpret_cast<const uint8_t*>(p.segpos)[row0 + t];
   return r;
+}
+
+// bit j = token t0-3+j starts a document.  The empty asm pins the comparison
+// to the call site: without it the compiler tests the value right behind its
+// load, i.e. waits for that load before the rows of the step are even
+// requested.
+__device__ __forceinline__ uint32_t doc_starts(SegRaw seg) {
+  uint32_t lo = (uint32_t)seg.v64, hi = (uint32_t)((uint64_t)seg.v64 >> 32);
+  asm volatile("" : "+v"(lo), "+v"(hi), "+v"(seg.v32), "+v"(seg.v8));
+  const bool st = ((lo | hi) == 0u) | (seg.v32 == 0) | (seg.v8 != 0u);
+  return (uint32_t)__ballot(st);
 }
 
 // Keeps a rarely taken, wave-uniform block a real branch (the compiler would
@@ -261,36 +323,38 @@ __device__ __forceinline__ void gate_math(const float (&xc)[CH],
 }
 
 // Phase 1, hot path: straight-line code for a step without a document start
-// among the wave's tokens or its three look-back tokens.  Tokens past the end
-// of the sequence are computed on a re-read of the last valid row; their
-// results are never stored and can only reach state that nothing reads any
-// more.  As soon as a token's raw inputs have been consumed, the same
-// registers are reloaded with that token's row of the NEXT step (`next`), so
-// the next step's data is in flight for a whole step without a second set of
-// registers.  After the last step the reload is redundant but harmless:
-// `next` is clamped into the sequence.
-template <typename T, int CH, bool CONV, bool FAST, bool PLAIN>
+// among the wave's tokens or its three look-back tokens.  As soon as a token's
+// raw inputs have been unpacked, the same registers are reloaded with that
+// token's row of the NEXT step (`next`), so the next step's rows are in flight
+// for a whole step without a second set of registers.  After the last step
+// the reload is redundant but harmless: `next` is clamped into the sequence.
+template <typename T, int CH, int KL, bool CONV, bool FAST, bool PLAIN>
 __device__ __forceinline__ void phase1(
-    Tile<T, CH>& tl, const StepAddr& next, uint32_t voff,
-    const ChanConst<CH>& k, float (&a_)[kL][CH], float (&xn_)[kL][CH],
+    Tile<T, CH, KL>& tl, const StepAddr<KL>& next, uint32_t voff,
+    const ChanConst<CH>& k, float (&a_)[KL][CH], float (&xn_)[KL][CH],
     float (&P)[CH], float (&H)[CH]) {
   using B = Buf<T, CH>;
   float hist[3][CH];
 #pragma unroll
   for (int s = 0; s < 3; ++s) B::unpack(tl.halo[s], hist[s]);
+  // The reload must follow the last read of the registers it overwrites;
+  // without these fences the scheduler hoists it, old and new values overlap,
+  // and the new tile needs register copies (and full waits) every step.
   __builtin_amdgcn_sched_barrier(0);
-  load_halo<T, CH, CONV>(tl, next, voff);
+  load_halo<T, CH, KL, CONV>(tl, next, voff);
 #pragma unroll
-  for (int i = 0; i < kL; ++i) {
+  for (int ch = 0; ch < CH; ++ch) {
+    P[ch] = 1.0f;
+    H[ch] = 0.0f;
+  }
+#pragma unroll
+  for (int i = 0; i < KL; ++i) {
     float xv[CH], gxv[CH], gav[CH], xc[CH];
     B::unpack(tl.x[i], xv);
     if (!PLAIN) B::unpack(tl.gx[i], gxv);
     B::unpack(tl.ga[i], gav);
-    // The reload must follow the last read of the registers it overwrites;
-    // without these fences the scheduler hoists it, the old and new values
-    // overlap, and the new tile needs copies (and full waits) every step.
     __builtin_amdgcn_sched_barrier(0);
-    load_token<T, CH, PLAIN>(tl, i, next, voff);
+    load_token<T, CH, KL, PLAIN>(tl, i, next, voff);
     __builtin_amdgcn_sched_barrier(0);
     if (CONV) {
 #pragma unroll
@@ -316,13 +380,13 @@ __device__ __forceinline__ void phase1(
 }
 
 // Phase 1, slow path: a step with a document start.  Recomputes the wave's
-// (a, xn) pairs from memory (the rows are still in cache), token by token,
-// with the conv history cut at every start, a = 0 and input scale 1 there.
-// It does not touch the prefetched tile.
-template <typename T, int CH, bool CONV, bool FAST, bool PLAIN>
+// (a, xn) pairs from memory (the rows are still in cache), with the conv
+// history cut at every start and a = 0, input scale 1 there.  It does not
+// touch the prefetched tile.
+template <typename T, int CH, int KL, bool CONV, bool FAST, bool PLAIN>
 __device__ __forceinline__ void phase1_with_starts(
-    const StepAddr& cur, uint32_t voff, uint32_t starts,
-    const ChanConst<CH>& k, float (&a_)[kL][CH], float (&xn_)[kL][CH],
+    const StepAddr<KL>& at, uint32_t voff, uint32_t starts,
+    const ChanConst<CH>& k, float (&a_)[KL][CH], float (&xn_)[KL][CH],
     float (&P)[CH], float (&H)[CH]) {
   using B = Buf<T, CH>;
   float hist[3][CH];
@@ -330,13 +394,14 @@ __device__ __forceinline__ void phase1_with_starts(
   for (int s = 0; s < 3; ++s)
 #pragma unroll
     for (int ch = 0; ch < CH; ++ch) hist[s][ch] = 0.0f;
-  if (CONV && cur.has_halo) {
+  if (CONV && at.has_halo) {
 #pragma unroll
     for (int s = 0; s < 3; ++s)  // hist[s] = x[first-1-s]
-      B::unpack(B::load(cur.rhalo, voff, (uint32_t)(2 - s) * cur.row_bytes),
+      B::unpack(B::template load<0>(at.rhalo, voff,
+                                    (uint32_t)(2 - s) * at.row_bytes),
                 hist[s]);
-    // a document start at first-1 hides x[first-2], x[first-3]; one at first-2
-    // hides x[first-3]
+    // a document start at first-1 hides x[first-2], x[first-3]; one at
+    // first-2 hides x[first-3]
     if (starts & 4u) {
 #pragma unroll
       for (int ch = 0; ch < CH; ++ch) hist[1][ch] = hist[2][ch] = 0.0f;
@@ -352,13 +417,13 @@ __device__ __forceinline__ void phase1_with_starts(
     H[ch] = 0.0f;
   }
 #pragma unroll
-  for (int i = 0; i < kL; ++i) {
+  for (int i = 0; i < KL; ++i) {
     const bool start = (starts >> (i + 3)) & 1u;
-    const uint32_t so = cur.soff(i);
-    float xv[CH], gxv[CH], gav[CH], xc[CH], a[CH], xn[CH];
-    B::unpack(B::load(cur.rx, voff, so), xv);
-    if (!PLAIN) B::unpack(B::load(cur.rgx, voff, so), gxv);
-    B::unpack(B::load(cur.rga, voff, so), gav);
+    const uint32_t so = at.soff(i);
+    float xv[CH], gxv[CH], gav[CH], xc[CH];
+    B::unpack(B::template load<0>(at.rx, voff, so), xv);
+    if (!PLAIN) B::unpack(B::template load<0>(at.rgx, voff, so), gxv);
+    B::unpack(B::template load<0>(at.rga, voff, so), gav);
     if (CONV) {
 #pragma unroll
       for (int ch = 0; ch < CH; ++ch) {
@@ -374,13 +439,11 @@ __device__ __forceinline__ void phase1_with_starts(
 #pragma unroll
       for (int ch = 0; ch < CH; ++ch) xc[ch] = xv[ch];
     }
-    gate_math<CH, FAST, PLAIN>(xc, gxv, gav, k.decay, start, a, xn);
+    gate_math<CH, FAST, PLAIN>(xc, gxv, gav, k.decay, start, a_[i], xn_[i]);
 #pragma unroll
     for (int ch = 0; ch < CH; ++ch) {
-      a_[i][ch] = a[ch];
-      xn_[i][ch] = xn[ch];
-      H[ch] = __builtin_fmaf(a[ch], H[ch], xn[ch]);
-      P[ch] = P[ch] * a[ch];
+      H[ch] = __builtin_fmaf(a_[i][ch], H[ch], xn_[i][ch]);
+      P[ch] = P[ch] * a_[i][ch];
     }
   }
 }
@@ -389,24 +452,24 @@ __device__ __forceinline__ void phase1_with_starts(
 // of tokens past the end of the sequence get a scalar offset outside the
 // descriptor and are dropped by the range check.  The state after token T-1
 // is written to h_last by the wave that holds that token.
-template <typename T, int CH>
+template <typename T, int CH, int KL>
 __device__ __forceinline__ void phase2(__amdgpu_buffer_rsrc_t ry, uint32_t voff,
                                        uint32_t row_bytes, int n_valid,
                                        float* h_last_lane,
-                                       const float (&a_)[kL][CH],
-                                       const float (&xn_)[kL][CH],
+                                       const float (&a_)[KL][CH],
+                                       const float (&xn_)[KL][CH],
                                        float (&h)[CH]) {
   using B = Buf<T, CH>;
 #pragma unroll
-  for (int i = 0; i < kL; ++i) {
+  for (int i = 0; i < KL; ++i) {
     float out[CH];
 #pragma unroll
     for (int ch = 0; ch < CH; ++ch) {
       h[ch] = __builtin_fmaf(a_[i][ch], h[ch], xn_[i][ch]);
       out[ch] = h[ch];
     }
-    B::store(ry, voff, i < n_valid ? (uint32_t)i * row_bytes : 0x80000000u,
-             out);
+    B::template store<kStream>(
+        ry, voff, i < n_valid ? (uint32_t)i * row_bytes : kOutOfRange, out);
     if (h_last_lane && i == n_valid - 1) {
       RG_RARE_BLOCK();
 #pragma unroll
@@ -415,17 +478,21 @@ __device__ __forceinline__ void phase2(__amdgpu_buffer_rsrc_t ry, uint32_t voff,
   }
 }
 
-template <typename T, int CH, bool CONV, bool FAST, bool PLAIN>
+template <typename T, int CH, int KL, bool CONV, bool FAST, bool PLAIN>
 __global__ void __launch_bounds__(kMaxNW* kWave, (sizeof(T) == 2 ? 4 : 2))
 lru_scan_kernel(ScanArgs p) {
-  using A = Act<T, CH>;
-  using B = Buf<T, CH>;
-  __shared__ float agg[2][kMaxNW][kWave][2 * CH];  // (P.., Hloc..) per lane
-  __shared__ float carry_s[2][kWave][CH];
+  // LDS (sized at launch): per buffer and wave the lanes' (P.., Hloc..)
+  // pairs, then the two carry rows
+  extern __shared__ __align__(16) float lds_f[];
+  typedef float AggRow[kWave][2 * CH];
+  typedef float CarryRow[kWave][CH];
 
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int nw = blockDim.x >> 6;
+  AggRow* const agg0 = reinterpret_cast<AggRow*>(lds_f);   // [2][nw]
+  CarryRow* const carry_s =
+      reinterpret_cast<CarryRow*>(lds_f + 2 * nw * kWave * 2 * CH);  // [2]
   const int T_len = p.T;
   const int64_t W = p.W;
   const int nslab = (p.W + kWave * CH - 1) / (kWave * CH);
@@ -459,12 +526,9 @@ lru_scan_kernel(ScanArgs p) {
 
   const int64_t row0 = (int64_t)b * T_len;
   const uint32_t row_bytes = (uint32_t)p.W * (uint32_t)sizeof(T);
-  // lanes past the last channel get an offset beyond every descriptor's range
-  // (whether or not the scalar row offset takes part in the range check):
-  // their loads return 0 and their stores are dropped
   const uint32_t voff =
-      active ? (uint32_t)c_raw * (uint32_t)sizeof(T) : 0x80000000u;
-  const uint32_t span_bytes = (uint32_t)kL * row_bytes;
+      active ? (uint32_t)c_raw * (uint32_t)sizeof(T) : kOutOfRange;
+  const uint32_t span_bytes = (uint32_t)KL * row_bytes;
   // wave-uniform pointers to token 0 of this batch row
   const char* xrow = (const char*)p.x + row0 * row_bytes;
   const char* gxrow = (const char*)p.gx + row0 * row_bytes;
@@ -476,20 +540,7 @@ lru_scan_kernel(ScanArgs p) {
   for (int ch = 0; ch < CH; ++ch)
     h[ch] = p.h0 ? p.h0[(int64_t)b * W + c + ch] : 0.0f;
 
-  const int span = nw * kL;
-
-  // bit j of `starts` = token t0-3+j of the step at hand starts a document.
-  // It is a scalar: the next step's mask is formed (one ballot) at the end of
-  // the current step and costs no vector register in between.
-  auto doc_starts = [&](SegRaw seg) {
-    // The empty asm pins the comparison here: without it the compiler tests
-    // the value right behind its load, i.e. waits for the load (and for every
-    // older load and store) at the top of the step.
-    uint32_t lo = (uint32_t)seg.v64, hi = (uint32_t)((uint64_t)seg.v64 >> 32);
-    asm volatile("" : "+v"(lo), "+v"(hi), "+v"(seg.v32), "+v"(seg.v8));
-    const bool st = ((lo | hi) == 0u) | (seg.v32 == 0) | (seg.v8 != 0u);
-    return (uint32_t)__ballot(st);
-  };
+  const int span = nw * KL;
 
   // Every wave runs every step with the same code, so that the prefetched
   // tile is never merged with a copy of itself at a branch join (that would
@@ -498,48 +549,46 @@ lru_scan_kernel(ScanArgs p) {
   // its stores and contributes the identity pair.
 
   // prologue: the first step's rows
-  Tile<T, CH> tl;
+  Tile<T, CH, KL> tl;
   uint32_t starts;
   {
-    const SegRaw seg = load_seg<CONV>(p, row0, wave * kL, T_len, lane);
-    const StepAddr a0 =
-        step_addr(xrow, gxrow, garow, wave * kL, T_len, row_bytes);
-    load_halo<T, CH, CONV>(tl, a0, voff);
+    const SegRaw seg = load_seg<KL, CONV>(p, row0, wave * KL, T_len, lane);
+    const StepAddr<KL> a0 =
+        step_addr<KL>(xrow, gxrow, garow, wave * KL, T_len, row_bytes);
+    load_halo<T, CH, KL, CONV>(tl, a0, voff);
 #pragma unroll
-    for (int i = 0; i < kL; ++i) load_token<T, CH, PLAIN>(tl, i, a0, voff);
+    for (int i = 0; i < KL; ++i) load_token<T, CH, KL, PLAIN>(tl, i, a0, voff);
     starts = doc_starts(seg);
   }
 
   for (int step = 0, tb = 0; tb < T_len; ++step, tb += span) {
     const int buf = step & 1;
-    const int t0 = tb + wave * kL;
+    const int t0 = tb + wave * KL;
     const bool any = t0 < T_len;
     // tokens of this wave inside the sequence (<= 0: none)
-    const int n_valid = T_len - t0 < kL ? T_len - t0 : kL;
-    float a_[kL][CH], xn_[kL][CH], P[CH], H[CH];
-#pragma unroll
-    for (int ch = 0; ch < CH; ++ch) {
-      P[ch] = 1.0f;
-      H[ch] = 0.0f;
-    }
-    const StepAddr next =
-        step_addr(xrow, gxrow, garow, t0 + span, T_len, row_bytes);
-    const SegRaw seg_next = load_seg<CONV>(p, row0, t0 + span, T_len, lane);
-    phase1<T, CH, CONV, FAST, PLAIN>(tl, next, voff, k, a_, xn_, P, H);
+    const int n_valid = T_len - t0 < KL ? T_len - t0 : KL;
+    float a_[KL][CH], xn_[KL][CH], P[CH], H[CH];
+    const StepAddr<KL> next =
+        step_addr<KL>(xrow, gxrow, garow, t0 + span, T_len, row_bytes);
+    // next step's document starts: loaded now, looked at after this step
+    const SegRaw seg_next = load_seg<KL, CONV>(p, row0, t0 + span, T_len, lane);
+    phase1<T, CH, KL, CONV, FAST, PLAIN>(tl, next, voff, k, a_, xn_, P, H);
     if (starts != 0u) {
       RG_RARE_BLOCK();
-      const StepAddr cur = step_addr(xrow, gxrow, garow, t0, T_len, row_bytes);
-      phase1_with_starts<T, CH, CONV, FAST, PLAIN>(cur, voff, starts, k, a_,
-                                                   xn_, P, H);
+      const StepAddr<KL> cur =
+          step_addr<KL>(xrow, gxrow, garow, t0, T_len, row_bytes);
+      phase1_with_starts<T, CH, KL, CONV, FAST, PLAIN>(cur, voff, starts, k, a_,
+                                                       xn_, P, H);
     }
 
     // exchange
+    AggRow* const agg = agg0 + buf * nw;
 #pragma unroll
     for (int ch = 0; ch < CH; ++ch) {
-      agg[buf][wave][lane][ch] = any ? P[ch] : 1.0f;
-      agg[buf][wave][lane][CH + ch] = any ? H[ch] : 0.0f;
+      agg[wave][lane][ch] = any ? P[ch] : 1.0f;
+      agg[wave][lane][CH + ch] = any ? H[ch] : 0.0f;
     }
-    lds_barrier();  // LDS only: prefetched rows stay in flight
+    lds_barrier();  // LDS only: prefetched rows and earlier stores stay in flight
     if (step > 0) {
 #pragma unroll
       for (int ch = 0; ch < CH; ++ch) h[ch] = carry_s[buf ^ 1][lane][ch];
@@ -547,22 +596,21 @@ lru_scan_kernel(ScanArgs p) {
     for (int v = 0; v < wave; ++v) {
 #pragma unroll
       for (int ch = 0; ch < CH; ++ch)
-        h[ch] = __builtin_fmaf(agg[buf][v][lane][ch], h[ch],
-                               agg[buf][v][lane][CH + ch]);
+        h[ch] = __builtin_fmaf(agg[v][lane][ch], h[ch], agg[v][lane][CH + ch]);
     }
 
     {
       const __amdgpu_buffer_rsrc_t ry = make_rsrc(
-          yrow + (int64_t)(t0 < T_len ? t0 : T_len - 1) * row_bytes, span_bytes);
+          yrow + (int64_t)(any ? t0 : T_len - 1) * row_bytes, span_bytes);
       // this wave holds token T-1 iff its valid tokens end the sequence
       float* const h_last_lane =
           (p.h_last && active && any && t0 + n_valid == T_len)
               ? p.h_last + (int64_t)b * W + c
               : nullptr;
-      float hw[CH];  // the replay runs on a copy: an empty wave must not
-#pragma unroll       // disturb the carry it may have to hand on
+      float hw[CH];  // replay on a copy: a wave without tokens must hand the
+#pragma unroll       // carry on unchanged
       for (int ch = 0; ch < CH; ++ch) hw[ch] = h[ch];
-      phase2<T, CH>(ry, voff, row_bytes, n_valid, h_last_lane, a_, xn_, hw);
+      phase2<T, CH, KL>(ry, voff, row_bytes, n_valid, h_last_lane, a_, xn_, hw);
 #pragma unroll
       for (int ch = 0; ch < CH; ++ch) h[ch] = any ? hw[ch] : h[ch];
     }
@@ -581,54 +629,62 @@ lru_scan_kernel(ScanArgs p) {
 #pragma unroll
     for (int kk = 2; kk >= 0; --kk) {
       const int t = T_len - 3 + kk;
-      float v[CH];
+      const bool copy = t >= 0 && !later_start;
+      const T* src = (const T*)(xrow + (int64_t)(t >= 0 ? t : 0) * row_bytes) + c;
 #pragma unroll
-      for (int ch = 0; ch < CH; ++ch) v[ch] = 0.0f;
-      if (t >= 0) {
-        if (!later_start)
-          A::load((const T*)(xrow + (int64_t)t * row_bytes) + c, v);
-        if (is_doc_start(p.segpos, p.seg_kind, row0 + t))
-          later_start = true;
-      }
-      A::store(cache + (int64_t)kk * W, v);
+      for (int ch = 0; ch < CH; ++ch)
+        store_scalar(cache + (int64_t)kk * W + ch,
+                     copy ? load_scalar(src + ch) : 0.0f);
+      if (t >= 0 && is_doc_start(p.segpos, p.seg_kind, row0 + t))
+        later_start = true;
     }
   }
 }
 
-template <typename T, int CH, bool CONV, bool FAST, bool PLAIN>
+template <typename T, int CH, int KL, bool CONV, bool FAST, bool PLAIN>
 hipError_t launch_t(const ScanArgs& a, hipStream_t s) {
   const int nslab = (a.W + kWave * CH - 1) / (kWave * CH);
-  int nw = 1;
-  while (nw < kMaxNW && nw * kL < a.T) nw *= 2;
   const int64_t blocks = (int64_t)a.B * nslab;
-  // one row must fit a buffer descriptor's 32-bit scalar offsets
-  if (blocks > 0x7fffffff || (int64_t)a.W * sizeof(T) * (kL + 3) > 0x7fffffff)
+  // Waves per workgroup: enough to cover the sequence, and 16 rather than 8
+  // when the grid alone would leave most of the 256 CUs' wave slots empty.
+  int max_nw = blocks * 8 >= 4096 ? 8 : kMaxNW;
+  int nw = 1;
+  while (nw < max_nw && nw * KL < a.T) nw *= 2;
+  // a wave's rows of one step must fit a descriptor's 32-bit offsets
+  if (blocks > 0x7fffffff ||
+      (int64_t)a.W * sizeof(T) * (KL + 3) >= (int64_t)kOutOfRange)
     return hipErrorInvalidValue;
-  lru_scan_kernel<T, CH, CONV, FAST, PLAIN>
-      <<<dim3((unsigned)blocks), dim3(nw * kWave), 0, s>>>(a);
+  const size_t lds = sizeof(float) * (2 * nw * kWave * 2 * CH + 2 * kWave * CH);
+  auto kern = lru_scan_kernel<T, CH, KL, CONV, FAST, PLAIN>;
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(
+        (const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+  }
+  kern<<<dim3((unsigned)blocks), dim3(nw * kWave), lds, s>>>(a);
   return hipGetLastError();
 }
 
-template <typename T, bool FAST>
-hipError_t launch_dt(const ScanArgs& a, hipStream_t s) {
-  // Two channels per lane need the channel count even (every row then starts
-  // on a vector boundary; base pointers are checked by the caller).
-  const bool vec2 = (a.W % 2) == 0;
-  if (a.plain)
-    return vec2 ? launch_t<T, 2, false, FAST, true>(a, s)
-                : launch_t<T, 1, false, FAST, true>(a, s);
-  if (a.apply_conv)
-    return vec2 ? launch_t<T, 2, true, FAST, false>(a, s)
-                : launch_t<T, 1, true, FAST, false>(a, s);
-  return vec2 ? launch_t<T, 2, false, FAST, false>(a, s)
-              : launch_t<T, 1, false, FAST, false>(a, s);
+template <typename T, int CH, int KL, bool FAST>
+hipError_t launch_mode(const ScanArgs& a, hipStream_t s) {
+  if (a.plain) return launch_t<T, CH, KL, false, FAST, true>(a, s);
+  if (a.apply_conv) return launch_t<T, CH, KL, true, FAST, false>(a, s);
+  return launch_t<T, CH, KL, false, FAST, false>(a, s);
 }
 
 }  // namespace
 
 hipError_t launch_lru_scan(const ScanArgs& a, int dtype, hipStream_t s) {
-  return dtype == 0 ? launch_dt<float, false>(a, s)
-                    : launch_dt<uint16_t, true>(a, s);
+  // Channels per lane: 8 bytes per lane where the width allows it (every row
+  // then starts on a vector boundary; base pointers are checked by the
+  // caller), with short steps; narrower vectors take longer steps.
+  if (dtype == 0) {
+    if (a.W % 2 == 0) return launch_mode<float, 2, 4, false>(a, s);
+    return launch_mode<float, 1, 8, false>(a, s);
+  }
+  if (a.W % 4 == 0) return launch_mode<uint16_t, 4, 4, true>(a, s);
+  if (a.W % 2 == 0) return launch_mode<uint16_t, 2, 8, true>(a, s);
+  return launch_mode<uint16_t, 1, 8, true>(a, s);
 }
 
 }  // namespace rg
