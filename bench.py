@@ -40,7 +40,10 @@ WORKLOADS = {
 
 # HBM bytes per scan launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # (scaled by a copy kernel of known size); None until measured for a workload.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    # profiles/hbm_traffic_9b_prefill.txt: 3.334 GB read + 1.074 GB written
+    "9b_prefill": 4.408e9,
+}
 
 
 def scan_algorithmic_bytes(B, T, W, esize, seg_bytes, has_h0):

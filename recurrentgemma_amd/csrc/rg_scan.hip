@@ -682,7 +682,11 @@ hipError_t launch_lru_scan(const ScanArgs& a, int dtype, hipStream_t s) {
     if (a.W % 2 == 0) return launch_mode<float, 2, 4, false>(a, s);
     return launch_mode<float, 1, 8, false>(a, s);
   }
-  if (a.W % 4 == 0) return launch_mode<uint16_t, 4, 4, true>(a, s);
+  // 8-byte lanes halve the number of workgroups (B * ceil(W/256)); below
+  // about 200 of them too many of the 256 CUs idle and 4-byte lanes win.
+  const int64_t wide_blocks = (int64_t)a.B * ((a.W + 255) / 256);
+  if (a.W % 4 == 0 && wide_blocks >= 200)
+    return launch_mode<uint16_t, 4, 4, true>(a, s);
   if (a.W % 2 == 0) return launch_mode<uint16_t, 2, 8, true>(a, s);
   return launch_mode<uint16_t, 1, 8, true>(a, s);
 }
