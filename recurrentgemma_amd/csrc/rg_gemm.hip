@@ -179,10 +179,35 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
   const uint16_t* const xbase = (const uint16_t*)p.x;
   constexpr int kHalo = CONV ? 3 : 0;
   constexpr int kRaw = kRowsPerGroup + kHalo;
+  uint32_t cwp[5] = {0, 0, 0, 0, 0};  // conv w[0..3] and bias, two bf16 each
+  if (CONV) {
+    const uint16_t* cw = (const uint16_t*)p.conv_w + c;
+    cwp[0] = *reinterpret_cast<const uint32_t*>(cw);
+    cwp[1] = *reinterpret_cast<const uint32_t*>(cw + W);
+    cwp[2] = *reinterpret_cast<const uint32_t*>(cw + 2 * W);
+    cwp[3] = *reinterpret_cast<const uint32_t*>(cw + 3 * W);
+    cwp[4] = *reinterpret_cast<const uint32_t*>((const uint16_t*)p.conv_b + c);
+  }
   uint32_t raw[kRaw];
+  // Document-start lookup of the tile being fetched: lane j of the wave looks
+  // at row mbase+j (all lanes of a wave stage the same rows).  The raw values
+  // are loaded together with the rows and only tested in stage(); one member
+  // per encoding so that the loads are never merged into one register.
+  int64_t seg64 = 1;
+  int32_t seg32 = 1;
 
   auto fetch = [&](int64_t tile) {
     const int64_t mbase = tile * kTM + rg * kRowsPerGroup - kHalo;
+    if (CONV) {
+      const int64_t m = mbase + lane;
+      const bool look = lane < kRaw && m >= 0 && m < M;
+      seg64 = 1;
+      seg32 = 1;
+      if (look && p.seg_kind == kSegI64)
+        seg64 = reinterpret_cast<const int64_t*>(p.segpos)[m];
+      if (look && p.seg_kind == kSegI32)
+        seg32 = reinterpret_cast<const int32_t*>(p.segpos)[m];
+    }
 #pragma unroll
     for (int j = 0; j < kRaw; ++j) {
       int64_t m = mbase + j;  // wave-uniform
@@ -201,17 +226,12 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
         *reinterpret_cast<uint32_t*>(dst + (size_t)i * kLdsStride) = raw[i];
       return;
     }
-    // conv taps and bias of this thread's two channels (L1/L2 hits; not kept
-    // in registers across the MFMA phase)
+    // conv taps and bias of this thread's two channels: kept packed (five
+    // registers) across the MFMA phase, unpacked here
     float cw0[2], cw1[2], cw2[2], cw3[2], cb[2];
     {
-      const uint16_t* cw = (const uint16_t*)p.conv_w + c;
-      const uint32_t u0 = *reinterpret_cast<const uint32_t*>(cw);
-      const uint32_t u1 = *reinterpret_cast<const uint32_t*>(cw + W);
-      const uint32_t u2 = *reinterpret_cast<const uint32_t*>(cw + 2 * W);
-      const uint32_t u3 = *reinterpret_cast<const uint32_t*>(cw + 3 * W);
-      const uint32_t ub =
-          *reinterpret_cast<const uint32_t*>((const uint16_t*)p.conv_b + c);
+      const uint32_t u0 = cwp[0], u1 = cwp[1], u2 = cwp[2], u3 = cwp[3],
+                     ub = cwp[4];
       cw0[0] = __uint_as_float(u0 << 16); cw0[1] = __uint_as_float(u0 & 0xffff0000u);
       cw1[0] = __uint_as_float(u1 << 16); cw1[1] = __uint_as_float(u1 & 0xffff0000u);
       cw2[0] = __uint_as_float(u2 << 16); cw2[1] = __uint_as_float(u2 & 0xffff0000u);
@@ -226,9 +246,13 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
     {
       const int64_t m = mbase + lane;
       const uint32_t t_base = (uint32_t)(((mbase % T_len) + T_len) % T_len);
+      // pin the test here (see fetch): the values were loaded a tile ago
+      uint32_t lo = (uint32_t)seg64, hi = (uint32_t)((uint64_t)seg64 >> 32);
+      int32_t v32 = seg32;
+      asm volatile("" : "+v"(lo), "+v"(hi), "+v"(v32));
       if (lane < kRaw && m >= 0 && m < M)
         st = ((t_base + (uint32_t)lane) % (uint32_t)T_len == 0u) ||
-             is_doc_start(p.segpos, p.seg_kind, m);
+             ((lo | hi) == 0u) || (v32 == 0);
     }
     const uint32_t cut = (uint32_t)__ballot(st);
     float h0[2] = {0.f, 0.f}, h1[2] = {0.f, 0.f}, h2[2] = {0.f, 0.f};
@@ -262,7 +286,7 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
     fetch(tile);
     stage(tile, 0);
   }
-  __syncthreads();
+  lds_barrier();
 
   int buf = 0;
   for (; tile < ntiles; tile += gridDim.x, buf ^= 1) {
@@ -310,7 +334,9 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
     }
 
     if (has_next) stage(next, buf ^ 1);
-    __syncthreads();
+    // LDS-only barrier: the x rows fetched ahead and the stores of this tile
+    // stay in flight across it
+    lds_barrier();
   }
 }
 

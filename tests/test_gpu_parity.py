@@ -437,8 +437,12 @@ def _full_size_properties(B, T, W, H, seg, seed):
   # (5) a row's result does not depend on its neighbours (first row alone)
   y_row, c_row = rg.recurrent_core(blk.conv_1d, blk.rg_lru, x[:1].contiguous(),
                                    segd[:1].contiguous())
-  assert torch.equal(y_row, y[:1])
-  assert torch.equal(c_row.rg_lru_state, cache.rg_lru_state[:1])
+  # (a one-row launch may use another lane width / step length, i.e. another
+  # fp32 association of the carry: equal up to rare 1-ulp bf16 flips)
+  assert (y_row != y[:1]).float().mean().item() < 1e-3
+  assert (y_row.float() - y[:1].float()).abs().max().item() <= 0.0625
+  assert helpers.max_rel(c_row.rg_lru_state, cache.rg_lru_state[:1]) < 1e-5
+  assert torch.equal(c_row.conv1d_state, cache.conv1d_state[:1])
   # (6) spot parity against the oracle on one row's first tokens
   n = 300
   yo, _ = R.widened_recurrent_core(x[:1, :n].cpu(), seg[:1, :n], p)
