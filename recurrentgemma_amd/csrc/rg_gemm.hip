@@ -103,7 +103,12 @@ constexpr int kBW = 256;          // block width (K and per-gate N)
 constexpr int kTM = 64;           // rows of x per tile
 constexpr int kLdsStride = 264;   // bf16 elements per LDS row (256 + 8 pad)
 constexpr int kRowsPerGroup = 16; // rows each thread converts per tile
-constexpr size_t kMfmaLdsBytes = 2ull * kTM * kLdsStride * sizeof(uint16_t);
+constexpr size_t kStageLdsBytes = 2ull * kTM * kLdsStride * sizeof(uint16_t);
+// Per-wave output staging: one 32 x 64 result block in bf16, rows padded to
+// 144 bytes so that the 16-byte row reads stay aligned.
+constexpr int kEpiStride = 144;
+constexpr size_t kEpiBytesPerWave = 32ull * kEpiStride;
+constexpr size_t kMfmaLdsBytes = kStageLdsBytes + 8 * kEpiBytesPerWave;
 
 union Frag {
   bf16x8 v;
@@ -164,11 +169,19 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
   for (int nt = 0; nt < 2; ++nt)
     biasv[nt] = bf16_bits_to_f32(
         ((const uint16_t*)p.b[gate])[h * kBW + n0 + nt * 32 + (lane & 31)]);
-  // Output addressing: a wave-uniform row pointer plus this 32-bit lane offset
-  // (lanes 32-63 sit four rows below lanes 0-31 in the 32x32 result layout).
+  // Output addressing: a wave-uniform tile pointer plus this 32-bit lane
+  // offset.  Lane l stores the 16-byte chunk l%8 of rows l/8, l/8+8, ... of
+  // the wave's 32 x 64 block.
+  const uint32_t out_row_bytes = 2u * (uint32_t)p.W;
   const uint32_t out_lane_bytes =
-      2u * ((uint32_t)(4 * (lane >> 5)) * (uint32_t)p.W + h * kBW + n0 +
-            (lane & 31));
+      (uint32_t)(lane >> 3) * out_row_bytes + 2u * (h * kBW + n0) +
+      16u * (lane & 7);
+  unsigned char* const epi =
+      lds_raw + kStageLdsBytes + (size_t)wave * kEpiBytesPerWave;
+  // write side: result row 4*(lane/32) (+ i), column lane%32 (+ 32)
+  unsigned char* const epi_w =
+      epi + 4 * (lane >> 5) * kEpiStride + 2 * (lane & 31);
+  unsigned char* const epi_r = epi + (lane >> 3) * kEpiStride + 16 * (lane & 7);
   char* const outbase = (char*)p.out[gate];
 
   // ---- x staging: thread -> (channel pair, group of 16 rows) -----------
@@ -316,21 +329,32 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
         acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, bfrag[ks][1].v,
                                                        acc1, 0, 0, 0);
       }
-      // epilogue: D[i][j], i = 8*(r/4) + 4*(lane/32) + r%4, j = lane%32
-      const int64_t row_first = tile * kTM + mt * 32;          // uniform
-      const int64_t rows_left = M - row_first;                 // uniform, > 0
-      const int lane_row = 4 * (lane >> 5);
+      // epilogue: D[i][j], i = 8*(r/4) + 4*(lane/32) + r%4, j = lane%32.
+      // The block goes through this wave's LDS patch so that each lane
+      // stores 16 contiguous bytes (8 rows x 128 bytes per instruction).
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int i = 8 * (r >> 2) + (r & 3);                  // uniform part
-        char* rowp = outbase + (row_first + i) * W * 2;        // uniform
-        if (i + lane_row < rows_left) {
-          *reinterpret_cast<uint16_t*>(rowp + out_lane_bytes) =
-              f32_to_bf16_bits(acc0[r] + biasv[0]);
-          *reinterpret_cast<uint16_t*>(rowp + out_lane_bytes + 64) =
-              f32_to_bf16_bits(acc1[r] + biasv[1]);
-        }
+        const int i = 8 * (r >> 2) + (r & 3);
+        unsigned char* q = epi_w + i * kEpiStride;
+        *reinterpret_cast<uint16_t*>(q) = f32_to_bf16_bits(acc0[r] + biasv[0]);
+        *reinterpret_cast<uint16_t*>(q + 64) =
+            f32_to_bf16_bits(acc1[r] + biasv[1]);
       }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      const int64_t row_first = tile * kTM + mt * 32;          // uniform
+      const int rows_left =
+          (int)((M - row_first) < 32 ? (M - row_first) : 32);  // uniform, > 0
+      char* const tilep = outbase + row_first * W * 2;          // uniform
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(epi_r + q * 8 * kEpiStride);
+        if (q * 8 + (lane >> 3) < rows_left)
+          *reinterpret_cast<f32x4*>(tilep + out_lane_bytes +
+                                    (uint32_t)(q * 8) * out_row_bytes) = v;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
     }
 
     if (has_next) stage(next, buf ^ 1);
