@@ -9,6 +9,7 @@ namespace rg {
 
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -183,6 +184,16 @@ __device__ __forceinline__ float conv_point(const T* x, const void* segpos,
   }
   return round_act<T>(acc);
 }
+
+// Raw buffer descriptor (stride 0, 32-bit data format) over `bytes` bytes at
+// `base`.  Accesses whose offset (vector + scalar part) falls outside are
+// dropped (stores) or return zero (loads).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base,
+                                                            uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0,
+                                           (int)bytes, 0x00020000);
+}
+constexpr uint32_t kBufferOutOfRange = 0x80000000u;
 
 // ---------------------------------------------------------- barriers ----
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits

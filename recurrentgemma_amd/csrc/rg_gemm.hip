@@ -116,6 +116,32 @@ union Frag {
   f32x4 q;
 };
 
+// Instruction-order hints for one 32-row half (16 k-steps of one LDS read and
+// two MFMAs each).  Group masks: 0x008 MFMA, 0x020 global load, 0x040 global
+// store, 0x100 LDS read.
+template <int KS, int NLOADS>
+__device__ __forceinline__ void interleave_loads() {
+  if constexpr (KS == 0) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+  if constexpr (KS < 16) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+    __builtin_amdgcn_sched_group_barrier(0x020, (KS < NLOADS - 16) ? 2 : 1, 0);
+    if constexpr (KS < 14) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    interleave_loads<KS + 1, NLOADS>();
+  }
+}
+template <int KS>
+__device__ __forceinline__ void interleave_stores() {
+  // four patch reads and two operand reads up front, then one store after
+  // each of the first four MFMA pairs
+  if constexpr (KS == 0) __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+  if constexpr (KS < 16) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+    if constexpr (KS < 4) __builtin_amdgcn_sched_group_barrier(0x040, 1, 0);
+    if constexpr (KS < 14) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    interleave_stores<KS + 1>();
+  }
+}
+
 template <bool CONV>
 __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
@@ -190,6 +216,7 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
   const uint32_t c = h * kBW + cp * 2;  // lane offset inside a row of x
   const uint32_t c_bytes = 2u * c;
   const uint16_t* const xbase = (const uint16_t*)p.x;
+  const uint32_t x_row_bytes = 2u * (uint32_t)p.W;
   constexpr int kHalo = CONV ? 3 : 0;
   constexpr int kRaw = kRowsPerGroup + kHalo;
   uint32_t cwp[5] = {0, 0, 0, 0, 0};  // conv w[0..3] and bias, two bf16 each
@@ -209,9 +236,11 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
   int64_t seg64 = 1;
   int32_t seg32 = 1;
 
-  auto fetch = [&](int64_t tile) {
-    const int64_t mbase = tile * kTM + rg * kRowsPerGroup - kHalo;
+  // Rows past the end clamp to the last row, so both fetch parts are safe for
+  // a tile index beyond the last tile (the values are then never used).
+  auto fetch_seg = [&](int64_t tile) {
     if (CONV) {
+      const int64_t mbase = tile * kTM + rg * kRowsPerGroup - kHalo;
       const int64_t m = mbase + lane;
       const bool look = lane < kRaw && m >= 0 && m < M;
       seg64 = 1;
@@ -221,12 +250,24 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
       if (look && p.seg_kind == kSegI32)
         seg32 = reinterpret_cast<const int32_t*>(p.segpos)[m];
     }
+  };
+  auto fetch_rows = [&](int64_t tile) {
+    const int64_t mbase = tile * kTM + rg * kRowsPerGroup - kHalo;
+    // Descriptor over this thread group's rows that exist: rows past the end
+    // of x fall outside it, rows before the start (first tile only) get an
+    // out-of-range scalar offset.  Both read as zero and are never used: a
+    // row before the start is always cut off by the sequence boundary.
+    const int before = mbase < 0 ? (int)-mbase : 0;             // 0..kHalo
+    const int64_t first = mbase < 0 ? 0 : mbase;
+    int64_t nrows = M - first;
+    nrows = nrows < 0 ? 0 : (nrows > kRaw ? kRaw : nrows);
+    const __amdgpu_buffer_rsrc_t rx = make_rsrc(
+        xbase + (first < M ? first : 0) * W, (uint32_t)nrows * x_row_bytes);
 #pragma unroll
     for (int j = 0; j < kRaw; ++j) {
-      int64_t m = mbase + j;  // wave-uniform
-      m = m < 0 ? 0 : (m >= M ? M - 1 : m);
-      raw[j] = *reinterpret_cast<const uint32_t*>(
-          reinterpret_cast<const char*>(xbase + m * W) + c_bytes);
+      const uint32_t soff = j < before ? kBufferOutOfRange
+                                       : (uint32_t)(j - before) * x_row_bytes;
+      raw[j] = __builtin_amdgcn_raw_buffer_load_b32(rx, c_bytes, soff, 0);
     }
   };
 
@@ -296,24 +337,30 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
 
   int64_t tile = blockIdx.x;
   if (tile < ntiles) {
-    fetch(tile);
+    fetch_seg(tile);
+    fetch_rows(tile);
     stage(tile, 0);
   }
   lds_barrier();
 
+  // Per tile, three scheduling regions in which memory traffic is spread
+  // between the matrix instructions instead of being issued in bursts:
+  //   A  row loads of the next tile   | MFMA of rows 0-31  | result -> LDS
+  //   B  stores of rows 0-31          | MFMA of rows 32-63 | result -> LDS
+  //   C  stores of rows 32-63         | conv of the next tile -> LDS
   int buf = 0;
   for (; tile < ntiles; tile += gridDim.x, buf ^= 1) {
     const int64_t next = tile + gridDim.x;
-    const bool has_next = next < ntiles;
-    if (has_next) fetch(next);
+    fetch_seg(next);
 
-    // One 32-row half of the tile at a time keeps only 32 accumulator
-    // registers live next to the 128 registers of resident weights.
     const uint16_t* abase = lds + (size_t)buf * kTM * kLdsStride +
                             (size_t)(lane & 31) * kLdsStride + 8 * (lane >> 5);
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
-      f32x16 acc0, acc1;
+    const int64_t row_first = tile * kTM;                       // uniform
+    char* const tilep = outbase + row_first * W * 2;            // uniform
+    const int rows_left =
+        (int)((M - row_first) < kTM ? (M - row_first) : kTM);   // uniform, > 0
+
+    auto mfma_half = [&](int mt, f32x16& acc0, f32x16& acc1) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         acc0[r] = 0.0f;
@@ -329,9 +376,11 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
         acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, bfrag[ks][1].v,
                                                        acc1, 0, 0, 0);
       }
-      // epilogue: D[i][j], i = 8*(r/4) + 4*(lane/32) + r%4, j = lane%32.
-      // The block goes through this wave's LDS patch so that each lane
-      // stores 16 contiguous bytes (8 rows x 128 bytes per instruction).
+    };
+    // D[i][j], i = 8*(r/4) + 4*(lane/32) + r%4, j = lane%32, goes through
+    // this wave's LDS patch so that each lane stores 16 contiguous bytes
+    // (8 rows x 128 bytes per instruction).
+    auto result_to_lds = [&](const f32x16& acc0, const f32x16& acc1) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int i = 8 * (r >> 2) + (r & 3);
@@ -342,22 +391,38 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
-      const int64_t row_first = tile * kTM + mt * 32;          // uniform
-      const int rows_left =
-          (int)((M - row_first) < 32 ? (M - row_first) : 32);  // uniform, > 0
-      char* const tilep = outbase + row_first * W * 2;          // uniform
+    };
+    const __amdgpu_buffer_rsrc_t ro =
+        make_rsrc(tilep, (uint32_t)rows_left * out_row_bytes);
+    auto lds_to_global = [&](int mt) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const f32x4 v = *reinterpret_cast<const f32x4*>(epi_r + q * 8 * kEpiStride);
-        if (q * 8 + (lane >> 3) < rows_left)
-          *reinterpret_cast<f32x4*>(tilep + out_lane_bytes +
-                                    (uint32_t)(q * 8) * out_row_bytes) = v;
+        const u32x4 v =
+            *reinterpret_cast<const u32x4*>(epi_r + q * 8 * kEpiStride);
+        // rows past the end of the output fall outside the descriptor
+        __builtin_amdgcn_raw_buffer_store_b128(
+            v, ro, out_lane_bytes, (uint32_t)(mt * 32 + q * 8) * out_row_bytes,
+            0);
       }
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-    }
+    };
 
-    if (has_next) stage(next, buf ^ 1);
+    {  // ---- region A
+      fetch_rows(next);
+      f32x16 acc0, acc1;
+      mfma_half(0, acc0, acc1);
+      interleave_loads<0, kRaw>();
+      result_to_lds(acc0, acc1);
+    }
+    {  // ---- region B
+      lds_to_global(0);
+      f32x16 acc0, acc1;
+      mfma_half(1, acc0, acc1);
+      interleave_stores<0>();
+      result_to_lds(acc0, acc1);
+    }
+    // ---- region C
+    lds_to_global(1);
+    stage(next, buf ^ 1);
     // LDS-only barrier: the x rows fetched ahead and the stores of this tile
     // stay in flight across it
     lds_barrier();

@@ -49,13 +49,6 @@ constexpr int kStream = 2;
 
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base,
-                                                            uint32_t bytes) {
-  // raw buffer (stride 0), 32-bit data format
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0,
-                                           (int)bytes, 0x00020000);
-}
-
 // Buffer access of CH adjacent channels.  Raw keeps bf16 values packed until
 // they are used.
 template <typename T, int CH>
