@@ -12,6 +12,8 @@
 #include "rg_common.h"
 #include "rg_internal.h"
 
+#include <type_traits>
+
 namespace rg {
 namespace {
 
@@ -115,32 +117,6 @@ union Frag {
   uint16_t u[8];
   f32x4 q;
 };
-
-// Instruction-order hints for one 32-row half (16 k-steps of one LDS read and
-// two MFMAs each).  Group masks: 0x008 MFMA, 0x020 global load, 0x040 global
-// store, 0x100 LDS read.
-template <int KS, int NLOADS>
-__device__ __forceinline__ void interleave_loads() {
-  if constexpr (KS == 0) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-  if constexpr (KS < 16) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-    __builtin_amdgcn_sched_group_barrier(0x020, (KS < NLOADS - 16) ? 2 : 1, 0);
-    if constexpr (KS < 14) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    interleave_loads<KS + 1, NLOADS>();
-  }
-}
-template <int KS>
-__device__ __forceinline__ void interleave_stores() {
-  // four patch reads and two operand reads up front, then one store after
-  // each of the first four MFMA pairs
-  if constexpr (KS == 0) __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
-  if constexpr (KS < 16) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-    if constexpr (KS < 4) __builtin_amdgcn_sched_group_barrier(0x040, 1, 0);
-    if constexpr (KS < 14) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    interleave_stores<KS + 1>();
-  }
-}
 
 template <bool CONV>
 __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
@@ -251,47 +227,58 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
         seg32 = reinterpret_cast<const int32_t*>(p.segpos)[m];
     }
   };
-  auto fetch_rows = [&](int64_t tile) {
+  struct RowFetch {
+    __amdgpu_buffer_rsrc_t rx;
+    int before;
+  };
+  // Descriptor over this thread group's rows that exist: rows past the end
+  // of x fall outside it, rows before the start (first tile only) get an
+  // out-of-range scalar offset.  Both read as zero and are never used: a
+  // row before the start is always cut off by the sequence boundary.
+  auto fetch_rows_begin = [&](int64_t tile) {
     const int64_t mbase = tile * kTM + rg * kRowsPerGroup - kHalo;
-    // Descriptor over this thread group's rows that exist: rows past the end
-    // of x fall outside it, rows before the start (first tile only) get an
-    // out-of-range scalar offset.  Both read as zero and are never used: a
-    // row before the start is always cut off by the sequence boundary.
-    const int before = mbase < 0 ? (int)-mbase : 0;             // 0..kHalo
+    RowFetch f;
+    f.before = mbase < 0 ? (int)-mbase : 0;                     // 0..kHalo
     const int64_t first = mbase < 0 ? 0 : mbase;
     int64_t nrows = M - first;
     nrows = nrows < 0 ? 0 : (nrows > kRaw ? kRaw : nrows);
-    const __amdgpu_buffer_rsrc_t rx = make_rsrc(
-        xbase + (first < M ? first : 0) * W, (uint32_t)nrows * x_row_bytes);
+    f.rx = make_rsrc(xbase + (first < M ? first : 0) * W,
+                     (uint32_t)nrows * x_row_bytes);
+    return f;
+  };
+  auto fetch_row = [&](const RowFetch& f, int j) {
+    const uint32_t soff = j < f.before
+                              ? kBufferOutOfRange
+                              : (uint32_t)(j - f.before) * x_row_bytes;
+    raw[j] = __builtin_amdgcn_raw_buffer_load_b32(f.rx, c_bytes, soff, 0);
+  };
+  auto fetch_rows = [&](int64_t tile) {
+    const RowFetch f = fetch_rows_begin(tile);
 #pragma unroll
-    for (int j = 0; j < kRaw; ++j) {
-      const uint32_t soff = j < before ? kBufferOutOfRange
-                                       : (uint32_t)(j - before) * x_row_bytes;
-      raw[j] = __builtin_amdgcn_raw_buffer_load_b32(rx, c_bytes, soff, 0);
-    }
+    for (int j = 0; j < kRaw; ++j) fetch_row(f, j);
   };
 
-  auto stage = [&](int64_t tile, int buf) {
-    uint16_t* dst = lds + (size_t)buf * kTM * kLdsStride +
-                    (size_t)(rg * kRowsPerGroup) * kLdsStride + cp * 2;
-    if (!CONV) {
-#pragma unroll
-      for (int i = 0; i < kRowsPerGroup; ++i)
-        *reinterpret_cast<uint32_t*>(dst + (size_t)i * kLdsStride) = raw[i];
-      return;
-    }
-    // conv taps and bias of this thread's two channels: kept packed (five
-    // registers) across the MFMA phase, unpacked here
-    float cw0[2], cw1[2], cw2[2], cw3[2], cb[2];
-    {
-      const uint32_t u0 = cwp[0], u1 = cwp[1], u2 = cwp[2], u3 = cwp[3],
-                     ub = cwp[4];
-      cw0[0] = __uint_as_float(u0 << 16); cw0[1] = __uint_as_float(u0 & 0xffff0000u);
-      cw1[0] = __uint_as_float(u1 << 16); cw1[1] = __uint_as_float(u1 & 0xffff0000u);
-      cw2[0] = __uint_as_float(u2 << 16); cw2[1] = __uint_as_float(u2 & 0xffff0000u);
-      cw3[0] = __uint_as_float(u3 << 16); cw3[1] = __uint_as_float(u3 & 0xffff0000u);
-      cb[0] = __uint_as_float(ub << 16);  cb[1] = __uint_as_float(ub & 0xffff0000u);
-    }
+  // Conv of one tile, one row at a time so that the rows can be placed
+  // between the matrix instructions of the previous tile.
+  //   stage_begin: document-start mask of the tile's rows, history cleared
+  //   stage_row(j): j < kHalo feeds the history; j >= kHalo writes LDS row
+  //                 j - kHalo of this thread's group
+  float cw0[2], cw1[2], cw2[2], cw3[2], cb[2];
+  if (CONV) {
+    // unpacked once: ten registers, but no unpacking between the MFMAs
+    cw0[0] = __uint_as_float(cwp[0] << 16); cw0[1] = __uint_as_float(cwp[0] & 0xffff0000u);
+    cw1[0] = __uint_as_float(cwp[1] << 16); cw1[1] = __uint_as_float(cwp[1] & 0xffff0000u);
+    cw2[0] = __uint_as_float(cwp[2] << 16); cw2[1] = __uint_as_float(cwp[2] & 0xffff0000u);
+    cw3[0] = __uint_as_float(cwp[3] << 16); cw3[1] = __uint_as_float(cwp[3] & 0xffff0000u);
+    cb[0] = __uint_as_float(cwp[4] << 16);  cb[1] = __uint_as_float(cwp[4] & 0xffff0000u);
+  }
+  uint32_t cut = 0;
+  float h0[2], h1[2], h2[2];
+  uint16_t* const stage_dst0 =
+      lds + (size_t)(rg * kRowsPerGroup) * kLdsStride + cp * 2;
+
+  auto stage_begin = [&](int64_t tile) {
+    if (!CONV) return;
     const int64_t mbase = tile * kTM + rg * kRowsPerGroup - kHalo;
     // bit j: row mbase+j begins a sequence row (t == 0) or a document; the
     // conv must not look past it.  Lane j of the wave looks at row mbase+j
@@ -300,7 +287,7 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
     {
       const int64_t m = mbase + lane;
       const uint32_t t_base = (uint32_t)(((mbase % T_len) + T_len) % T_len);
-      // pin the test here (see fetch): the values were loaded a tile ago
+      // pin the test here: the values were loaded a tile ago
       uint32_t lo = (uint32_t)seg64, hi = (uint32_t)((uint64_t)seg64 >> 32);
       int32_t v32 = seg32;
       asm volatile("" : "+v"(lo), "+v"(hi), "+v"(v32));
@@ -308,50 +295,67 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
         st = ((t_base + (uint32_t)lane) % (uint32_t)T_len == 0u) ||
              ((lo | hi) == 0u) || (v32 == 0);
     }
-    const uint32_t cut = (uint32_t)__ballot(st);
-    float h0[2] = {0.f, 0.f}, h1[2] = {0.f, 0.f}, h2[2] = {0.f, 0.f};
+    cut = (uint32_t)__ballot(st);
+    h0[0] = h0[1] = h1[0] = h1[1] = h2[0] = h2[1] = 0.0f;
+  };
+  // CUTS = false is the straight-line form for a tile without any sequence or
+  // document start among its rows (cut == 0).
+  auto stage_row = [&](int j, int buf, auto cuts) {
+    constexpr bool CUTS = decltype(cuts)::value;
+    uint16_t* dst = stage_dst0 + (size_t)buf * kTM * kLdsStride;
+    if (!CONV) {
+      *reinterpret_cast<uint32_t*>(dst + (size_t)j * kLdsStride) = raw[j];
+      return;
+    }
+    float xv[2];
+    xv[0] = __uint_as_float(raw[j] << 16);
+    xv[1] = __uint_as_float(raw[j] & 0xffff0000u);
+    if (CUTS && ((cut >> j) & 1u)) {
+      h0[0] = h0[1] = h1[0] = h1[1] = h2[0] = h2[1] = 0.0f;
+    }
+    if (j >= kHalo) {
+      const float o0 = conv4(xv[0], h0[0], h1[0], h2[0], cw0[0], cw1[0],
+                             cw2[0], cw3[0], cb[0]);
+      const float o1 = conv4(xv[1], h0[1], h1[1], h2[1], cw0[1], cw1[1],
+                             cw2[1], cw3[1], cb[1]);
+      *reinterpret_cast<uint32_t*>(dst + (size_t)(j - kHalo) * kLdsStride) =
+          pack_bf16x2(o0, o1);
+    }
 #pragma unroll
-    for (int j = 0; j < kRaw; ++j) {
-      float xv[2];
-      xv[0] = __uint_as_float(raw[j] << 16);
-      xv[1] = __uint_as_float(raw[j] & 0xffff0000u);
-      if ((cut >> j) & 1u) {
-        h0[0] = h0[1] = h1[0] = h1[1] = h2[0] = h2[1] = 0.0f;
-      }
-      if (j >= kHalo) {
-        const float o0 = conv4(xv[0], h0[0], h1[0], h2[0], cw0[0], cw1[0],
-                               cw2[0], cw3[0], cb[0]);
-        const float o1 = conv4(xv[1], h0[1], h1[1], h2[1], cw0[1], cw1[1],
-                               cw2[1], cw3[1], cb[1]);
-        *reinterpret_cast<uint32_t*>(dst + (size_t)(j - kHalo) * kLdsStride) =
-            pack_bf16x2(o0, o1);
-      }
-#pragma unroll
-      for (int ch = 0; ch < 2; ++ch) {
-        h2[ch] = h1[ch];
-        h1[ch] = h0[ch];
-        h0[ch] = xv[ch];
-      }
+    for (int ch = 0; ch < 2; ++ch) {
+      h2[ch] = h1[ch];
+      h1[ch] = h0[ch];
+      h0[ch] = xv[ch];
     }
   };
+  using WithCuts = std::integral_constant<bool, true>;
+  using NoCuts = std::integral_constant<bool, false>;
 
+  // Software pipeline over this workgroup's tiles i0, i0+G, ...: while the
+  // MFMAs of tile i run, the conv of tile i+G is written to the other LDS
+  // buffer and the rows of tile i+2G are loaded.  Per tile, three regions;
+  // inside A and B the work is cut into 16 chunks (one k-step each) whose
+  // order is pinned with scheduling barriers:
+  //   A  chunk: LDS read k+1 | 2 MFMA (rows 0-31)  | conv row k of next tile
+  //   B  chunk: LDS read k+1 | 2 MFMA (rows 32-63) | a store of rows 0-31 (first
+  //      four chunks) | load of row k (+16) of the tile after next
+  //   C  stores of rows 32-63
   int64_t tile = blockIdx.x;
   if (tile < ntiles) {
     fetch_seg(tile);
     fetch_rows(tile);
-    stage(tile, 0);
+    stage_begin(tile);
+#pragma unroll
+    for (int j = 0; j < kRaw; ++j) stage_row(j, 0, WithCuts{});
+    fetch_seg(tile + gridDim.x);
+    fetch_rows(tile + gridDim.x);
   }
   lds_barrier();
 
-  // Per tile, three scheduling regions in which memory traffic is spread
-  // between the matrix instructions instead of being issued in bursts:
-  //   A  row loads of the next tile   | MFMA of rows 0-31  | result -> LDS
-  //   B  stores of rows 0-31          | MFMA of rows 32-63 | result -> LDS
-  //   C  stores of rows 32-63         | conv of the next tile -> LDS
   int buf = 0;
   for (; tile < ntiles; tile += gridDim.x, buf ^= 1) {
     const int64_t next = tile + gridDim.x;
-    fetch_seg(next);
+    const int64_t next2 = next + gridDim.x;
 
     const uint16_t* abase = lds + (size_t)buf * kTM * kLdsStride +
                             (size_t)(lane & 31) * kLdsStride + 8 * (lane >> 5);
@@ -359,24 +363,9 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
     char* const tilep = outbase + row_first * W * 2;            // uniform
     const int rows_left =
         (int)((M - row_first) < kTM ? (M - row_first) : kTM);   // uniform, > 0
+    const __amdgpu_buffer_rsrc_t ro =
+        make_rsrc(tilep, (uint32_t)rows_left * out_row_bytes);
 
-    auto mfma_half = [&](int mt, f32x16& acc0, f32x16& acc1) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        acc0[r] = 0.0f;
-        acc1[r] = 0.0f;
-      }
-      const uint16_t* arow = abase + (size_t)mt * 32 * kLdsStride;
-#pragma unroll
-      for (int ks = 0; ks < 16; ++ks) {
-        Frag a;
-        a.q = *reinterpret_cast<const f32x4*>(arow + ks * 16);
-        acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, bfrag[ks][0].v,
-                                                       acc0, 0, 0, 0);
-        acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, bfrag[ks][1].v,
-                                                       acc1, 0, 0, 0);
-      }
-    };
     // D[i][j], i = 8*(r/4) + 4*(lane/32) + r%4, j = lane%32, goes through
     // this wave's LDS patch so that each lane stores 16 contiguous bytes
     // (8 rows x 128 bytes per instruction).
@@ -392,37 +381,96 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
     };
-    const __amdgpu_buffer_rsrc_t ro =
-        make_rsrc(tilep, (uint32_t)rows_left * out_row_bytes);
-    auto lds_to_global = [&](int mt) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const u32x4 v =
-            *reinterpret_cast<const u32x4*>(epi_r + q * 8 * kEpiStride);
-        // rows past the end of the output fall outside the descriptor
-        __builtin_amdgcn_raw_buffer_store_b128(
-            v, ro, out_lane_bytes, (uint32_t)(mt * 32 + q * 8) * out_row_bytes,
-            0);
-      }
+    auto patch_read = [&](int q) {
+      return *reinterpret_cast<const u32x4*>(epi_r + q * 8 * kEpiStride);
+    };
+    // rows past the end of the output fall outside the descriptor
+    auto patch_store = [&](int mt, int q, u32x4 v) {
+      __builtin_amdgcn_raw_buffer_store_b128(
+          v, ro, out_lane_bytes, (uint32_t)(mt * 32 + q * 8) * out_row_bytes, 0);
+    };
+    auto a_read = [&](int mt, int ks) {
+      Frag a;
+      a.q = *reinterpret_cast<const f32x4*>(
+          abase + (size_t)mt * 32 * kLdsStride + ks * 16);
+      return a;
     };
 
     {  // ---- region A
-      fetch_rows(next);
+      stage_begin(next);
       f32x16 acc0, acc1;
-      mfma_half(0, acc0, acc1);
-      interleave_loads<0, kRaw>();
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        acc0[r] = 0.0f;
+        acc1[r] = 0.0f;
+      }
+      Frag a[2];
+      if (cut == 0) {
+#pragma unroll
+        for (int j = 0; j < kHalo; ++j) stage_row(j, buf ^ 1, NoCuts{});
+        a[0] = a_read(0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < 16; ++ks) {
+          if (ks < 15) a[(ks + 1) & 1] = a_read(0, ks + 1);
+          acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              a[ks & 1].v, bfrag[ks][0].v, acc0, 0, 0, 0);
+          acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              a[ks & 1].v, bfrag[ks][1].v, acc1, 0, 0, 0);
+          stage_row(kHalo + ks, buf ^ 1, NoCuts{});
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+        // a sequence or document starts among the rows of the next tile
+        // (one tile in T/64, plus one per document): conv first, with the
+        // history cuts, then the matrix instructions
+#pragma unroll
+        for (int j = 0; j < kRaw; ++j) stage_row(j, buf ^ 1, WithCuts{});
+        a[0] = a_read(0, 0);
+#pragma unroll
+        for (int ks = 0; ks < 16; ++ks) {
+          if (ks < 15) a[(ks + 1) & 1] = a_read(0, ks + 1);
+          acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              a[ks & 1].v, bfrag[ks][0].v, acc0, 0, 0, 0);
+          acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              a[ks & 1].v, bfrag[ks][1].v, acc1, 0, 0, 0);
+        }
+      }
       result_to_lds(acc0, acc1);
     }
+    fetch_seg(next2);
     {  // ---- region B
-      lds_to_global(0);
+      const RowFetch rf = fetch_rows_begin(next2);
       f32x16 acc0, acc1;
-      mfma_half(1, acc0, acc1);
-      interleave_stores<0>();
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        acc0[r] = 0.0f;
+        acc1[r] = 0.0f;
+      }
+      Frag a[2];
+      a[0] = a_read(1, 0);
+      u32x4 pv = patch_read(0);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ks = 0; ks < 16; ++ks) {
+        if (ks < 15) a[(ks + 1) & 1] = a_read(1, ks + 1);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+            a[ks & 1].v, bfrag[ks][0].v, acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+            a[ks & 1].v, bfrag[ks][1].v, acc1, 0, 0, 0);
+        if (ks < 4) {
+          patch_store(0, ks, pv);
+          if (ks < 3) pv = patch_read(ks + 1);
+        }
+        fetch_row(rf, ks);
+        if (ks + 16 < kRaw) fetch_row(rf, ks + 16);
+        __builtin_amdgcn_sched_barrier(0);
+      }
       result_to_lds(acc0, acc1);
     }
     // ---- region C
-    lds_to_global(1);
-    stage(next, buf ^ 1);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) patch_store(1, q, patch_read(q));
     // LDS-only barrier: the x rows fetched ahead and the stores of this tile
     // stay in flight across it
     lds_barrier();
