@@ -110,7 +110,8 @@ constexpr size_t kStageLdsBytes = 2ull * kTM * kLdsStride * sizeof(uint16_t);
 // 144 bytes so that the 16-byte row reads stay aligned.
 constexpr int kEpiStride = 144;
 constexpr size_t kEpiBytesPerWave = 32ull * kEpiStride;
-constexpr size_t kMfmaLdsBytes = kStageLdsBytes + 8 * kEpiBytesPerWave;
+constexpr size_t kBiasLdsOffset = kStageLdsBytes + 8 * kEpiBytesPerWave;
+constexpr size_t kMfmaLdsBytes = kBiasLdsOffset + 8 * 64 * sizeof(float);
 
 union Frag {
   bf16x8 v;
@@ -166,11 +167,16 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
       __syncthreads();
     }
   }
-  float biasv[2];
-#pragma unroll
-  for (int nt = 0; nt < 2; ++nt)
-    biasv[nt] = bf16_bits_to_f32(
-        ((const uint16_t*)p.b[gate])[h * kBW + n0 + nt * 32 + (lane & 31)]);
+  // The MFMAs compute the transposed block (weights as the A operand): lane l
+  // then holds, for x row l%32, the channels 8*g + 4*(l/32) + 0..3 of each
+  // 32-channel block, g = 0..3, i.e. four adjacent channels per register
+  // quad.  The accumulators start from the bias, which each wave keeps in LDS
+  // as 64 floats (one 16-byte read per quad).
+  float* const bias_lds =
+      reinterpret_cast<float*>(lds_raw + kBiasLdsOffset) + wave * 64;
+  bias_lds[lane] = bf16_bits_to_f32(
+      ((const uint16_t*)p.b[gate])[h * kBW + n0 + lane]);
+  const float* const bias_r = bias_lds + 4 * (lane >> 5);
   // Output addressing: a wave-uniform tile pointer plus this 32-bit lane
   // offset.  Lane l stores the 16-byte chunk l%8 of rows l/8, l/8+8, ... of
   // the wave's 32 x 64 block.
@@ -180,9 +186,9 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
       16u * (lane & 7);
   unsigned char* const epi =
       lds_raw + kStageLdsBytes + (size_t)wave * kEpiBytesPerWave;
-  // write side: result row 4*(lane/32) (+ i), column lane%32 (+ 32)
+  // write side: x row lane%32, channels 4*(lane/32) + 8*g (+ 32)
   unsigned char* const epi_w =
-      epi + 4 * (lane >> 5) * kEpiStride + 2 * (lane & 31);
+      epi + (lane & 31) * kEpiStride + 8 * (lane >> 5);
   unsigned char* const epi_r = epi + (lane >> 3) * kEpiStride + 16 * (lane & 7);
   char* const outbase = (char*)p.out[gate];
 
@@ -366,17 +372,31 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
     const __amdgpu_buffer_rsrc_t ro =
         make_rsrc(tilep, (uint32_t)rows_left * out_row_bytes);
 
-    // D[i][j], i = 8*(r/4) + 4*(lane/32) + r%4, j = lane%32, goes through
-    // this wave's LDS patch so that each lane stores 16 contiguous bytes
-    // (8 rows x 128 bytes per instruction).
+    // The block goes through this wave's LDS patch (row-major, bf16) so that
+    // each lane stores 16 contiguous bytes (8 rows x 128 bytes per
+    // instruction).
+    auto acc_init = [&](f32x16& acc0, f32x16& acc1) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 b0 = *reinterpret_cast<const f32x4*>(bias_r + 8 * g);
+        const f32x4 b1 = *reinterpret_cast<const f32x4*>(bias_r + 32 + 8 * g);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          acc0[4 * g + q] = b0[q];
+          acc1[4 * g + q] = b1[q];
+        }
+      }
+    };
     auto result_to_lds = [&](const f32x16& acc0, const f32x16& acc1) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int i = 8 * (r >> 2) + (r & 3);
-        unsigned char* q = epi_w + i * kEpiStride;
-        *reinterpret_cast<uint16_t*>(q) = f32_to_bf16_bits(acc0[r] + biasv[0]);
-        *reinterpret_cast<uint16_t*>(q + 64) =
-            f32_to_bf16_bits(acc1[r] + biasv[1]);
+      for (int g = 0; g < 4; ++g) {
+        u32x2 v0, v1;
+        v0[0] = pack_bf16x2(acc0[4 * g], acc0[4 * g + 1]);
+        v0[1] = pack_bf16x2(acc0[4 * g + 2], acc0[4 * g + 3]);
+        v1[0] = pack_bf16x2(acc1[4 * g], acc1[4 * g + 1]);
+        v1[1] = pack_bf16x2(acc1[4 * g + 2], acc1[4 * g + 3]);
+        *reinterpret_cast<u32x2*>(epi_w + 16 * g) = v0;
+        *reinterpret_cast<u32x2*>(epi_w + 64 + 16 * g) = v1;
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
@@ -399,11 +419,7 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
     {  // ---- region A
       stage_begin(next);
       f32x16 acc0, acc1;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        acc0[r] = 0.0f;
-        acc1[r] = 0.0f;
-      }
+      acc_init(acc0, acc1);
       Frag a[2];
       if (cut == 0) {
 #pragma unroll
@@ -414,9 +430,9 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
         for (int ks = 0; ks < 16; ++ks) {
           if (ks < 15) a[(ks + 1) & 1] = a_read(0, ks + 1);
           acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              a[ks & 1].v, bfrag[ks][0].v, acc0, 0, 0, 0);
+              bfrag[ks][0].v, a[ks & 1].v, acc0, 0, 0, 0);
           acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              a[ks & 1].v, bfrag[ks][1].v, acc1, 0, 0, 0);
+              bfrag[ks][1].v, a[ks & 1].v, acc1, 0, 0, 0);
           stage_row(kHalo + ks, buf ^ 1, NoCuts{});
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -431,9 +447,9 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
         for (int ks = 0; ks < 16; ++ks) {
           if (ks < 15) a[(ks + 1) & 1] = a_read(0, ks + 1);
           acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              a[ks & 1].v, bfrag[ks][0].v, acc0, 0, 0, 0);
+              bfrag[ks][0].v, a[ks & 1].v, acc0, 0, 0, 0);
           acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              a[ks & 1].v, bfrag[ks][1].v, acc1, 0, 0, 0);
+              bfrag[ks][1].v, a[ks & 1].v, acc1, 0, 0, 0);
         }
       }
       result_to_lds(acc0, acc1);
@@ -442,11 +458,7 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
     {  // ---- region B
       const RowFetch rf = fetch_rows_begin(next2);
       f32x16 acc0, acc1;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        acc0[r] = 0.0f;
-        acc1[r] = 0.0f;
-      }
+      acc_init(acc0, acc1);
       Frag a[2];
       a[0] = a_read(1, 0);
       u32x4 pv = patch_read(0);
@@ -455,9 +467,9 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
       for (int ks = 0; ks < 16; ++ks) {
         if (ks < 15) a[(ks + 1) & 1] = a_read(1, ks + 1);
         acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            a[ks & 1].v, bfrag[ks][0].v, acc0, 0, 0, 0);
+            bfrag[ks][0].v, a[ks & 1].v, acc0, 0, 0, 0);
         acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            a[ks & 1].v, bfrag[ks][1].v, acc1, 0, 0, 0);
+            bfrag[ks][1].v, a[ks & 1].v, acc1, 0, 0, 0);
         if (ks < 4) {
           patch_store(0, ks, pv);
           if (ks < 3) pv = patch_read(ks + 1);

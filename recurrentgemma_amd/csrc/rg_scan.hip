@@ -47,7 +47,6 @@ constexpr uint32_t kOutOfRange = 0x80000000u;
 // cache policy of the streamed rows: non-temporal (read or written once)
 constexpr int kStream = 2;
 
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 // Buffer access of CH adjacent channels.  Raw keeps bf16 values packed until
 // they are used.
