@@ -212,25 +212,29 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
   }
   uint32_t raw[kRaw];
   // Document-start lookup of the tile being fetched: lane j of the wave looks
-  // at row mbase+j (all lanes of a wave stage the same rows).  The raw values
-  // are loaded together with the rows and only tested in stage(); one member
-  // per encoding so that the loads are never merged into one register.
-  int64_t seg64 = 1;
-  int32_t seg32 = 1;
+  // at row mbase+j (all lanes of a wave stage the same rows).  Two
+  // unconditional 32-bit buffer loads (low and high half of an int64
+  // position; for int32 positions the high half is sent out of range and
+  // reads as zero), tested a tile later in stage_begin(): a position is a
+  // start iff both halves are zero.  Lanes without a row read out of range
+  // and are masked in the test.
+  uint32_t seg_lo = 1, seg_hi = 0;
+  const bool seg_is64 = p.seg_kind == kSegI64;
+  const uint32_t seg_esize = seg_is64 ? 8u : 4u;
+  const __amdgpu_buffer_rsrc_t rseg =
+      make_rsrc(CONV ? p.segpos : nullptr, CONV ? (uint32_t)M * seg_esize : 0u);
 
-  // Rows past the end clamp to the last row, so both fetch parts are safe for
-  // a tile index beyond the last tile (the values are then never used).
+  // Both fetch parts are safe for a tile index beyond the last tile (the
+  // values are then never used).
   auto fetch_seg = [&](int64_t tile) {
     if (CONV) {
       const int64_t mbase = tile * kTM + rg * kRowsPerGroup - kHalo;
       const int64_t m = mbase + lane;
       const bool look = lane < kRaw && m >= 0 && m < M;
-      seg64 = 1;
-      seg32 = 1;
-      if (look && p.seg_kind == kSegI64)
-        seg64 = reinterpret_cast<const int64_t*>(p.segpos)[m];
-      if (look && p.seg_kind == kSegI32)
-        seg32 = reinterpret_cast<const int32_t*>(p.segpos)[m];
+      const uint32_t off = look ? (uint32_t)m * seg_esize : kBufferOutOfRange;
+      seg_lo = __builtin_amdgcn_raw_buffer_load_b32(rseg, off, 0, 0);
+      seg_hi = __builtin_amdgcn_raw_buffer_load_b32(
+          rseg, seg_is64 ? off + 4u : kBufferOutOfRange, 0, 0);
     }
   };
   struct RowFetch {
@@ -294,12 +298,18 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
       const int64_t m = mbase + lane;
       const uint32_t t_base = (uint32_t)(((mbase % T_len) + T_len) % T_len);
       // pin the test here: the values were loaded a tile ago
-      uint32_t lo = (uint32_t)seg64, hi = (uint32_t)((uint64_t)seg64 >> 32);
-      int32_t v32 = seg32;
-      asm volatile("" : "+v"(lo), "+v"(hi), "+v"(v32));
-      if (lane < kRaw && m >= 0 && m < M)
-        st = ((t_base + (uint32_t)lane) % (uint32_t)T_len == 0u) ||
-             ((lo | hi) == 0u) || (v32 == 0);
+      uint32_t lo = seg_lo, hi = seg_hi;
+      asm volatile("" : "+v"(lo), "+v"(hi));
+      // lanes whose row starts a sequence row (t == 0): one lane at most when
+      // the sequence is longer than the rows looked at
+      bool seq_start;
+      if (T_len >= 64) {
+        const uint32_t j0 = t_base == 0 ? 0u : (uint32_t)T_len - t_base;
+        seq_start = (uint32_t)lane == j0;
+      } else {
+        seq_start = (t_base + (uint32_t)lane) % (uint32_t)T_len == 0u;
+      }
+      if (lane < kRaw && m >= 0 && m < M) st = seq_start || ((lo | hi) == 0u);
     }
     cut = (uint32_t)__ballot(st);
     h0[0] = h0[1] = h1[0] = h1[1] = h2[0] = h2[1] = 0.0f;
@@ -420,19 +430,20 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
       stage_begin(next);
       f32x16 acc0, acc1;
       acc_init(acc0, acc1);
-      Frag a[2];
+      Frag a[3];  // operand reads run two k-steps ahead
       if (cut == 0) {
 #pragma unroll
         for (int j = 0; j < kHalo; ++j) stage_row(j, buf ^ 1, NoCuts{});
         a[0] = a_read(0, 0);
+        a[1] = a_read(0, 1);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int ks = 0; ks < 16; ++ks) {
-          if (ks < 15) a[(ks + 1) & 1] = a_read(0, ks + 1);
+          if (ks < 14) a[(ks + 2) % 3] = a_read(0, ks + 2);
           acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              bfrag[ks][0].v, a[ks & 1].v, acc0, 0, 0, 0);
+              bfrag[ks][0].v, a[ks % 3].v, acc0, 0, 0, 0);
           acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              bfrag[ks][1].v, a[ks & 1].v, acc1, 0, 0, 0);
+              bfrag[ks][1].v, a[ks % 3].v, acc1, 0, 0, 0);
           stage_row(kHalo + ks, buf ^ 1, NoCuts{});
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -445,11 +456,11 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
         a[0] = a_read(0, 0);
 #pragma unroll
         for (int ks = 0; ks < 16; ++ks) {
-          if (ks < 15) a[(ks + 1) & 1] = a_read(0, ks + 1);
+          if (ks < 15) a[(ks + 1) % 3] = a_read(0, ks + 1);
           acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              bfrag[ks][0].v, a[ks & 1].v, acc0, 0, 0, 0);
+              bfrag[ks][0].v, a[ks % 3].v, acc0, 0, 0, 0);
           acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              bfrag[ks][1].v, a[ks & 1].v, acc1, 0, 0, 0);
+              bfrag[ks][1].v, a[ks % 3].v, acc1, 0, 0, 0);
         }
       }
       result_to_lds(acc0, acc1);
@@ -459,17 +470,18 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
       const RowFetch rf = fetch_rows_begin(next2);
       f32x16 acc0, acc1;
       acc_init(acc0, acc1);
-      Frag a[2];
+      Frag a[3];
       a[0] = a_read(1, 0);
+      a[1] = a_read(1, 1);
       u32x4 pv = patch_read(0);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 0; ks < 16; ++ks) {
-        if (ks < 15) a[(ks + 1) & 1] = a_read(1, ks + 1);
+        if (ks < 14) a[(ks + 2) % 3] = a_read(1, ks + 2);
         acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            bfrag[ks][0].v, a[ks & 1].v, acc0, 0, 0, 0);
+            bfrag[ks][0].v, a[ks % 3].v, acc0, 0, 0, 0);
         acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            bfrag[ks][1].v, a[ks & 1].v, acc1, 0, 0, 0);
+            bfrag[ks][1].v, a[ks % 3].v, acc1, 0, 0, 0);
         if (ks < 4) {
           patch_store(0, ks, pv);
           if (ks < 3) pv = patch_read(ks + 1);
