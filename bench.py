@@ -12,6 +12,9 @@ Workloads (BASELINE.json configs):
               (the configuration the >= 70 % HBM-roofline target is stated on;
               default)
   2b_prefill  B8 T4096 W2560 H10 bf16, documents ~ Geometric(mean 1024)
+  9b_decode   B256 W4096 H16 bf16, one token per row and step with the caches
+              carried in place (rg_recurrent_step); `roofline` then describes
+              the whole step (all its launches) against its algorithmic bytes
 
 `roofline` describes the scan kernel: algorithmic bytes per launch (read x,
 read both gate pre-activations, write y, plus the small terms) over the mean
@@ -36,6 +39,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 WORKLOADS = {
     "9b_prefill": dict(B=16, T=8192, W=4096, H=16, mean_doc=None, seed=1003),
     "2b_prefill": dict(B=8, T=4096, W=2560, H=10, mean_doc=1024, seed=1002),
+    "9b_decode": dict(B=256, T=1, W=4096, H=16, mean_doc=None, seed=1004,
+                      decode=True),
 }
 
 # HBM bytes per scan launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
@@ -98,6 +103,83 @@ def cpu_baseline(torch, R, wl, params, seconds_target=20.0):
   }
 
 
+def decode_algorithmic_bytes(B, W, H, esize):
+  """One decode step: x in, y out, fp32 state and conv state read and written,
+  both gate weight matrices, the per-channel parameters."""
+  return (2 * B * W * esize + 2 * B * W * 4 + 2 * B * 3 * W * esize
+          + 2 * H * (W // H) ** 2 * esize + W * esize * 8 + B * 8)
+
+
+def run_decode(args, torch, rg, R, ops, wl):
+  """Times rg_recurrent_step (conv step, both gate projections, gate
+  activations, state update) on B rows with the caches updated in place."""
+  B, W, H = wl["B"], wl["W"], wl["H"]
+  dev = torch.device("cuda:0")
+  dtype = torch.bfloat16
+  params = R.make_params(W, H, dtype, seed=wl["seed"] + 100)
+  P = {k: v.to(dev) for k, v in params.items()}
+  g = torch.Generator().manual_seed(wl["seed"])
+  x = torch.randn(B, 1, W, generator=g).to(dtype).to(dev)
+  conv_cache = torch.randn(B, 3, W, generator=g).to(dtype).to(dev)
+  h = torch.randn(B, W, generator=g).to(dev)
+  seg = torch.full((B, 1), 2048, dtype=torch.int64, device=dev)
+
+  def step():
+    return ops.recurrent_step(x, seg, conv_cache, h, P["conv_w"], P["conv_b"],
+                              P["w_x"], P["b_x"], P["w_a"], P["b_a"],
+                              P["a_param"], in_place=True)
+
+  for _ in range(args.warmup):
+    step()
+  torch.cuda.synchronize()
+  e0 = torch.cuda.Event(enable_timing=True)
+  e1 = torch.cuda.Event(enable_timing=True)
+  t0 = time.perf_counter()
+  e0.record()
+  for _ in range(args.steps):
+    step()
+  e1.record()
+  torch.cuda.synchronize()
+  elapsed = time.perf_counter() - t0
+  dev_ms = e0.elapsed_time(e1) / args.steps
+  algo = decode_algorithmic_bytes(B, W, H, 2)
+  achieved = algo / (dev_ms * 1e-3) / 1e9
+  result = {
+      "metric": "RG-LRU block tokens/s + scan HBM GB/s (% of roofline)",
+      "value": B / (elapsed / args.steps), "unit": "tokens/s", "n_gpus": 1,
+      "steps": args.steps, "warmup": args.warmup,
+      "ms_per_step": elapsed * 1e3 / args.steps, "higher_is_better": True,
+      "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+      "data": "synthetic",
+      "config": {"workload": args.workload, "batch": B, "seq_len": 1,
+                 "lru_width": W, "heads": H, "activations": "bf16",
+                 "state": "f32", "path": "rg_recurrent_step, caches in place"},
+      "roofline": {"kernel": "rg_recurrent_step (all launches of one step)",
+                   "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
+                   "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                   "traffic": None, "algorithmic_bytes": algo,
+                   "avg_launch_ms": dev_ms},
+  }
+  if not args.no_cpu_baseline:
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    xc, cc, hc = x.cpu(), conv_cache.cpu(), h.cpu()
+    segc = seg.cpu()
+    cache = R.CoreCache(rg_lru_state=hc, conv1d_state=cc)
+    R.recurrent_core(xc, segc, params, cache)
+    n = 20
+    t0 = time.perf_counter()
+    for _ in range(n):
+      _, cache = R.recurrent_core(xc, segc, params, cache)
+    dt = (time.perf_counter() - t0) / n
+    result["cpu_baseline"] = {
+        "value": B / dt, "unit": "tokens/s", "cores": cores, "kind": "port",
+        "sample": (f"oracle/torch_ref.recurrent_core with caches, bf16, {n} "
+                   f"decode steps of {B} rows (W={W}, H={H}), mean, torch "
+                   f"threads={torch.get_num_threads()}")}
+  print(json.dumps(result))
+
+
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--gpus", type=int, default=1)
@@ -122,6 +204,9 @@ def main():
   from recurrentgemma_amd import ops
 
   wl = WORKLOADS[args.workload]
+  if wl.get("decode"):
+    run_decode(args, torch, rg, R, ops, wl)
+    return
   B, T, W, H = wl["B"], wl["T"], wl["W"], wl["H"]
   dev = torch.device("cuda:0")
   dtype = torch.bfloat16
