@@ -125,6 +125,26 @@ int rg_linear_scan(const void* x, const void* a, const void* reset,
                    const void* h0, void* y, void* h_last, int B, int T, int W,
                    int dtype, void* stream);
 
+/* Prefill of the conv -> RG-LRU core in ONE launch, as RecurrentBlock.forward
+ * chains the two modules without a cache (recurrentgemma/torch/modules.py:
+ * 632-643: Conv1D.forward layers.py:447-529, then RGLRU.forward :313-365 with
+ * rnn_scan :140-191).  x, y [B,T,W]; segpos [B,T]; conv_w [4,W], conv_b [W];
+ * w_x, w_a [H,W/H,W/H], b_x, b_a [H,W/H]; a_param [W]; h0 (nullable) and
+ * h_last (nullable) float32 [B,W]; conv_cache_out (nullable) [B,3,W], the
+ * masked tail described at rg_conv1d_prefill.  Same arithmetic as
+ * rg_gates_gemm(apply_conv) followed by rg_lru_scan_fused(apply_conv), but the
+ * conv output and the gate pre-activations stay on chip: one persistent
+ * workgroup per (b, head) walks the sequence in 64-token tiles (conv -> LDS ->
+ * bf16 MFMA -> gates -> in-register recurrence).  Returns RG_ERR_UNSUPPORTED
+ * unless dtype is bf16, W/H == 256 and T*W*2 < 2^31; callers then use the
+ * two-call form. */
+int rg_recurrent_prefill(const void* x, const void* segpos, int segpos_is_i64,
+                         const void* conv_w, const void* conv_b,
+                         const void* w_x, const void* b_x, const void* w_a,
+                         const void* b_a, const void* a_param, const void* h0,
+                         void* y, void* h_last, void* conv_cache_out, int B,
+                         int T, int W, int H, int dtype, void* stream);
+
 /* One decode step of the conv -> RG-LRU core, as RecurrentBlock.forward chains
  * them with a cache (recurrentgemma/torch/modules.py:632-643 with
  * layers.py:469-474 and :170-177): x [B,1,W], segpos [B,1],

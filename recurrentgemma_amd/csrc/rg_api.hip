@@ -222,6 +222,63 @@ int rg_lru_scan_fused(const void* x, int apply_conv, const void* conv_w,
                        rg::launch_lru_scan(a, dtype, (hipStream_t)stream));
 }
 
+int rg_recurrent_prefill(const void* x, const void* segpos, int segpos_is_i64,
+                         const void* conv_w, const void* conv_b,
+                         const void* w_x, const void* b_x, const void* w_a,
+                         const void* b_a, const void* a_param, const void* h0,
+                         void* y, void* h_last, void* conv_cache_out, int B,
+                         int T, int W, int H, int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(B > 0 && T > 0 && W > 0 && H > 0,
+             "%s: B=%d T=%d W=%d H=%d must be positive", __func__, B, T, W, H);
+  RG_REQUIRE(W % H == 0, "%s: W=%d is not a multiple of H=%d", __func__, W, H);
+  RG_CHECK_PTR(x);
+  RG_CHECK_PTR(segpos);
+  RG_CHECK_PTR(conv_w);
+  RG_CHECK_PTR(conv_b);
+  RG_CHECK_PTR(w_x);
+  RG_CHECK_PTR(b_x);
+  RG_CHECK_PTR(w_a);
+  RG_CHECK_PTR(b_a);
+  RG_CHECK_PTR(a_param);
+  RG_CHECK_PTR(y);
+  RG_CHECK_OPT_PTR(h0);
+  RG_CHECK_OPT_PTR(h_last);
+  RG_CHECK_OPT_PTR(conv_cache_out);
+  RG_REQUIRE(y != x, "%s: y must not alias x", __func__);
+  // The single-launch kernel exists for bf16 with 256-wide heads and
+  // sequences whose byte offsets fit 31 bits; everything else is served by
+  // rg_gates_gemm + rg_lru_scan_fused.
+  if (dtype != RG_DTYPE_BF16 || W / H != 256 ||
+      (int64_t)T * W * 2 >= (int64_t)0x7fffffff) {
+    return fail(RG_ERR_UNSUPPORTED,
+                "%s: unsupported shape or dtype (needs bf16, W/H == 256, "
+                "T*W*2 < 2^31): dtype=%d W=%d H=%d T=%d",
+                __func__, dtype, W, H, T);
+  }
+  rg::FusedArgs a{};
+  a.x = x;
+  a.segpos = segpos;
+  a.seg_kind = segpos_is_i64 ? 1 : 0;
+  a.conv_w = conv_w;
+  a.conv_b = conv_b;
+  a.w[0] = w_x;
+  a.b[0] = b_x;
+  a.w[1] = w_a;
+  a.b[1] = b_a;
+  a.a_param = a_param;
+  a.h0 = (const float*)h0;
+  a.y = y;
+  a.h_last = (float*)h_last;
+  a.cache_out = conv_cache_out;
+  a.B = B;
+  a.T = T;
+  a.W = W;
+  a.H = H;
+  return launch_status(__func__,
+                       rg::launch_block_fused_bf16(a, (hipStream_t)stream));
+}
+
 int rg_linear_scan(const void* x, const void* a, const void* reset,
                    const void* h0, void* y, void* h_last, int B, int T, int W,
                    int dtype, void* stream) {

@@ -1,0 +1,498 @@
+// Whole recurrent core in one launch (bf16, 256-wide heads): width-4 conv ->
+// both gate projections on MFMA -> gate activations -> linear recurrence.
+//
+// One persistent workgroup per (sequence row b, head h) walks the sequence in
+// tiles of 64 tokens.  Neither the conv output nor the gate pre-activations
+// ever go to memory: per element the kernel reads x once and writes y once.
+//
+// Replaces the chain Conv1D.forward -> RGLRU.forward of
+// recurrentgemma/torch/modules.py:632-643 (layers.py:447-529, 313-365,
+// 140-191) for prefill.
+#include <type_traits>
+
+#include "rg_common.h"
+#include "rg_internal.h"
+
+namespace rg {
+namespace {
+
+constexpr int kBW = 256;           // head width (K and per-gate N)
+constexpr int kTM = 64;            // tokens per tile
+constexpr int kLdsStride = 264;    // bf16 elements per staged row (256 + 8 pad)
+constexpr int kRowsPerGroup = 16;  // rows each thread converts per tile
+constexpr int kHalo = 3;
+constexpr int kRaw = kRowsPerGroup + kHalo;
+constexpr size_t kStageLdsBytes = 2ull * kTM * kLdsStride * sizeof(uint16_t);
+// Per-wave output patch: 32 tokens x 32 channels in bf16, rows padded to 80
+// bytes (16-byte aligned row reads, spread over the banks).
+constexpr int kPatchStride = 80;
+constexpr size_t kPatchBytesPerWave = 32ull * kPatchStride;
+// Conv taps and bias of the 128 channel pairs as floats, 12 per pair (w0..w3
+// and bias for both channels, padded): read back at the start of every conv
+// so that they do not occupy registers in between.
+constexpr size_t kConvTabOffset = kStageLdsBytes + 8 * kPatchBytesPerWave;
+constexpr size_t kFusedLdsBytes = kConvTabOffset + 128 * 12 * sizeof(float);
+
+union Frag {
+  bf16x8 v;
+  uint16_t u[8];
+  f32x4 q;
+};
+
+using WithCuts = std::integral_constant<bool, true>;
+using NoCuts = std::integral_constant<bool, false>;
+
+// Broadcast of the two 32-lane halves of a register: lo = the value lanes
+// 0-31 hold (in all 64 lanes), hi = the value lanes 32-63 hold.
+__device__ __forceinline__ void halves(float v, float& lo, float& hi) {
+  const uint32_t u = __float_as_uint(v);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  lo = __uint_as_float(r[0]);
+  hi = __uint_as_float(r[1]);
+}
+
+__global__ void __launch_bounds__(512) block_fused_bf16_kernel(FusedArgs p) {
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  uint16_t* lds = reinterpret_cast<uint16_t*>(lds_raw);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int b = blockIdx.x / p.H;
+  const int h = blockIdx.x % p.H;
+  const int T_len = p.T;
+  const int64_t W = p.W;
+  const int ntiles = (T_len + kTM - 1) / kTM;
+  const bool upper = lane >= 32;
+
+  // ---- this wave's weights: 32 channels of the head, both gates ----------
+  // The weights are [k][n] with n contiguous, the MFMA B operand wants 8
+  // consecutive k per lane: transpose through LDS, 128 k-rows of one gate at
+  // a time (coalesced 16-byte global reads, 2-byte LDS reads).
+  const int n0 = wave * 32;
+  Frag bfrag[16][2];
+#pragma unroll
+  for (int g = 0; g < 2; ++g) {
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh) {
+      const uint16_t* src =
+          (const uint16_t*)p.w[g] + ((int64_t)h * kBW + kh * 128) * kBW;
+      for (int e = tid; e < 128 * 32; e += 512) {
+        const int r = e >> 5, q = e & 31;
+        *reinterpret_cast<f32x4*>(lds + (size_t)r * kLdsStride + q * 8) =
+            *reinterpret_cast<const f32x4*>(src + (size_t)r * kBW + q * 8);
+      }
+      __syncthreads();
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        const int n = n0 + (lane & 31);
+        const int kb = ks * 16 + 8 * (lane >> 5);
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          bfrag[kh * 8 + ks][g].u[e] = lds[(size_t)(kb + e) * kLdsStride + n];
+      }
+      __syncthreads();
+    }
+  }
+  // Per-lane channel (the MFMA result has channel = lane % 32): gate biases,
+  // decay constant -8 softplus(a_param) log2(e), running state.
+  const int ch = h * kBW + n0 + (lane & 31);
+  const float bias_x = bf16_bits_to_f32(((const uint16_t*)p.b[0])[ch]);
+  const float bias_a = bf16_bits_to_f32(((const uint16_t*)p.b[1])[ch]);
+  const float decay =
+      (-8.0f * kLog2e) *
+      softplus_precise(bf16_bits_to_f32(((const uint16_t*)p.a_param)[ch]));
+  float hc = p.h0 ? p.h0[(int64_t)b * W + ch] : 0.0f;
+
+  // ---- addressing ---------------------------------------------------------
+  const uint32_t row_bytes = 2u * (uint32_t)p.W;
+  const uint32_t seq_bytes = (uint32_t)T_len * row_bytes;  // < 2^31 (launcher)
+  const __amdgpu_buffer_rsrc_t rx =
+      make_rsrc((const char*)p.x + (int64_t)b * seq_bytes, seq_bytes);
+  const __amdgpu_buffer_rsrc_t ry =
+      make_rsrc((char*)p.y + (int64_t)b * seq_bytes, seq_bytes);
+  const bool seg_is64 = p.seg_kind == kSegI64;
+  const uint32_t seg_esize = seg_is64 ? 8u : 4u;
+  const __amdgpu_buffer_rsrc_t rseg =
+      make_rsrc((const char*)p.segpos + (int64_t)b * T_len * seg_esize,
+                (uint32_t)T_len * seg_esize);
+
+  // x staging: thread -> (channel pair, group of 16 tokens)
+  const int cp = tid & 127;
+  const int rg = __builtin_amdgcn_readfirstlane(tid >> 7);
+  const uint32_t c = h * kBW + cp * 2;
+  const uint32_t c_bytes = 2u * c;
+  float cw0[2], cw1[2], cw2[2], cw3[2], cb[2];
+  float* const conv_tab =
+      reinterpret_cast<float*>(lds_raw + kConvTabOffset) + cp * 12;
+  if (tid < 128) {
+    const uint16_t* cw = (const uint16_t*)p.conv_w + c;
+    const uint32_t u0 = *reinterpret_cast<const uint32_t*>(cw);
+    const uint32_t u1 = *reinterpret_cast<const uint32_t*>(cw + W);
+    const uint32_t u2 = *reinterpret_cast<const uint32_t*>(cw + 2 * W);
+    const uint32_t u3 = *reinterpret_cast<const uint32_t*>(cw + 3 * W);
+    const uint32_t ub =
+        *reinterpret_cast<const uint32_t*>((const uint16_t*)p.conv_b + c);
+    f32x4 t0 = {__uint_as_float(u0 << 16), __uint_as_float(u0 & 0xffff0000u),
+                __uint_as_float(u1 << 16), __uint_as_float(u1 & 0xffff0000u)};
+    f32x4 t1 = {__uint_as_float(u2 << 16), __uint_as_float(u2 & 0xffff0000u),
+                __uint_as_float(u3 << 16), __uint_as_float(u3 & 0xffff0000u)};
+    f32x4 t2 = {__uint_as_float(ub << 16), __uint_as_float(ub & 0xffff0000u),
+                0.0f, 0.0f};
+    reinterpret_cast<f32x4*>(conv_tab)[0] = t0;
+    reinterpret_cast<f32x4*>(conv_tab)[1] = t1;
+    reinterpret_cast<f32x4*>(conv_tab)[2] = t2;
+  }
+  __syncthreads();
+  auto load_conv_consts = [&]() {
+    const f32x4 t0 = reinterpret_cast<const f32x4*>(conv_tab)[0];
+    const f32x4 t1 = reinterpret_cast<const f32x4*>(conv_tab)[1];
+    const f32x4 t2 = reinterpret_cast<const f32x4*>(conv_tab)[2];
+    cw0[0] = t0[0]; cw0[1] = t0[1]; cw1[0] = t0[2]; cw1[1] = t0[3];
+    cw2[0] = t1[0]; cw2[1] = t1[1]; cw3[0] = t1[2]; cw3[1] = t1[3];
+    cb[0] = t2[0];  cb[1] = t2[1];
+  };
+  uint32_t raw[kRaw];
+  uint32_t seg_lo = 1, seg_hi = 0;
+
+  // Document starts of a tile: lane j looks at token 64*tile + j.  Two
+  // unconditional 32-bit loads (for int32 positions the high half is sent out
+  // of range and reads as zero); tokens past the end read as zero too and are
+  // masked in start_mask().
+  auto fetch_seg = [&](int tile) {
+    const int t = tile * kTM + lane;
+    const uint32_t off =
+        (tile < ntiles && t < T_len) ? (uint32_t)t * seg_esize : kBufferOutOfRange;
+    seg_lo = __builtin_amdgcn_raw_buffer_load_b32(rseg, off, 0, 0);
+    seg_hi = __builtin_amdgcn_raw_buffer_load_b32(
+        rseg, seg_is64 ? off + 4u : kBufferOutOfRange, 0, 0);
+  };
+  auto start_mask = [&](int tile) -> uint64_t {
+    uint32_t lo = seg_lo, hi = seg_hi;
+    asm volatile("" : "+v"(lo), "+v"(hi));  // test here, a tile after the load
+    const int t = tile * kTM + lane;
+    return __ballot(tile < ntiles && t < T_len && (lo | hi) == 0u);
+  };
+  // Rows before the sequence get an out-of-range scalar offset, rows past its
+  // end fall outside the descriptor: both read as zero, which is what the
+  // conv sees there.
+  auto fetch_row = [&](int tile, int j) {
+    const int t = tile * kTM + rg * kRowsPerGroup - kHalo + j;  // uniform
+    const uint32_t soff =
+        (t < 0 || tile >= ntiles) ? kBufferOutOfRange : (uint32_t)t * row_bytes;
+    raw[j] = __builtin_amdgcn_raw_buffer_load_b32(rx, c_bytes, soff, 0);
+  };
+
+  // Conv of one tile, one row at a time.  cut bit j: token j of this thread
+  // group's 19 rows starts a document; the conv must not look past it.
+  uint32_t cut = 0;
+  float h0v[2], h1v[2], h2v[2];
+  uint16_t* const stage_dst0 =
+      lds + (size_t)(rg * kRowsPerGroup) * kLdsStride + cp * 2;
+  auto stage_begin = [&](uint64_t m_tile, uint64_t m_before) {
+    // rows 16*rg-3 .. 16*rg+15 of the tile; the three rows before the tile
+    // are the last three of the previous one
+    if (rg == 0)
+      cut = ((uint32_t)(m_tile << 3) | (uint32_t)(m_before >> 61)) & 0x7ffffu;
+    else
+      cut = (uint32_t)(m_tile >> (16 * rg - 3)) & 0x7ffffu;
+    h0v[0] = h0v[1] = h1v[0] = h1v[1] = h2v[0] = h2v[1] = 0.0f;
+    load_conv_consts();
+  };
+  auto stage_row = [&](int j, int buf, auto cuts) {
+    constexpr bool CUTS = decltype(cuts)::value;
+    uint16_t* dst = stage_dst0 + (size_t)buf * kTM * kLdsStride;
+    float xv[2];
+    xv[0] = __uint_as_float(raw[j] << 16);
+    xv[1] = __uint_as_float(raw[j] & 0xffff0000u);
+    if (CUTS && ((cut >> j) & 1u)) {
+      h0v[0] = h0v[1] = h1v[0] = h1v[1] = h2v[0] = h2v[1] = 0.0f;
+    }
+    if (j >= kHalo) {
+      const float o0 = conv4(xv[0], h0v[0], h1v[0], h2v[0], cw0[0], cw1[0],
+                             cw2[0], cw3[0], cb[0]);
+      const float o1 = conv4(xv[1], h0v[1], h1v[1], h2v[1], cw0[1], cw1[1],
+                             cw2[1], cw3[1], cb[1]);
+      *reinterpret_cast<uint32_t*>(dst + (size_t)(j - kHalo) * kLdsStride) =
+          pack_bf16x2(o0, o1);
+    }
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      h2v[k] = h1v[k];
+      h1v[k] = h0v[k];
+      h0v[k] = xv[k];
+    }
+  };
+
+  // ---- per-wave output patch ----------------------------------------------
+  unsigned char* const patch =
+      lds_raw + kStageLdsBytes + (size_t)wave * kPatchBytesPerWave;
+  // (written as token 4*(lane/32) + i, channel lane%32; read back as 16-byte
+  // row chunks)
+
+  // ---- prologue -------------------------------------------------------------
+  uint64_t m_cur = 0;
+  {
+    fetch_seg(0);
+#pragma unroll
+    for (int j = 0; j < kRaw; ++j) fetch_row(0, j);
+    m_cur = start_mask(0);
+    stage_begin(m_cur, 0);
+#pragma unroll
+    for (int j = 0; j < kRaw; ++j) stage_row(j, 0, WithCuts{});
+    fetch_seg(1);
+#pragma unroll
+    for (int j = 0; j < kRaw; ++j) fetch_row(1, j);
+  }
+  lds_barrier();
+
+  // Gate arithmetic + recurrence of one 32-token half of a tile.  On entry
+  // acc_x / acc_a hold the gate pre-activations (bias included) of tokens
+  // i = 8*(r/4) + 4*(lane/32) + r%4 for channel lane%32.  `general` also
+  // handles document starts (a = 0, unit input scale) and tokens past the end
+  // of the sequence (identity: a = 1, no input).
+  auto half_epilogue = [&](int it, int mt, int buf, f32x16& acc_x, f32x16& acc_a,
+                           bool general) {
+    int l1 = lane;
+    asm volatile("" : "+v"(l1));  // address recomputed per call, not kept
+    const uint16_t* xcp = lds + (size_t)buf * kTM * kLdsStride +
+                          (size_t)(mt * 32 + 4 * (l1 >> 5)) * kLdsStride + n0 +
+                          (l1 & 31);
+    const int t_half = it * kTM + mt * 32;  // first token of this half
+    // `general` (wave-uniform, rare): bit r of these per-lane words says that
+    // token r of this lane starts a document / lies inside the sequence.
+    uint32_t start_bits = 0, valid_bits = 0xffffu;
+    if (general) {
+      uint32_t s_lo = 0, s_hi = 0, v_lo = 0, v_hi = 0;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int row = mt * 32 + 8 * g;  // lanes 0-31: row..row+3, 32-63: +4
+        s_lo |= ((uint32_t)(m_cur >> row) & 0xfu) << (4 * g);
+        s_hi |= ((uint32_t)(m_cur >> (row + 4)) & 0xfu) << (4 * g);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          v_lo |= (uint32_t)(t_half + 8 * g + q < T_len) << (4 * g + q);
+          v_hi |= (uint32_t)(t_half + 8 * g + 4 + q < T_len) << (4 * g + q);
+        }
+      }
+      start_bits = upper ? s_hi : s_lo;
+      valid_bits = upper ? v_hi : v_lo;
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r += 2) {
+      // pre-activations are a bf16 module output in the reference
+      const uint32_t px2 = pack_bf16x2(acc_x[r], acc_x[r + 1]);
+      const uint32_t pa2 = pack_bf16x2(acc_a[r], acc_a[r + 1]);
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const int rr = r + e;
+        const int i = 8 * (rr >> 2) + (rr & 3);
+        const float xc = bf16_bits_to_f32(xcp[(size_t)i * kLdsStride]);
+        const float px = e == 0 ? __uint_as_float(px2 << 16)
+                                : __uint_as_float(px2 & 0xffff0000u);
+        const float pa = e == 0 ? __uint_as_float(pa2 << 16)
+                                : __uint_as_float(pa2 & 0xffff0000u);
+        const float gate_x = sigmoid_fast(px);
+        const float gate_a = sigmoid_fast(pa);
+        float a = __builtin_amdgcn_exp2f(gate_a * decay);
+        float mult = __builtin_amdgcn_sqrtf(__builtin_fmaf(-a, a, 1.0f));
+        if (general) {
+          if ((start_bits >> rr) & 1u) {  // document start: forget, unit scale
+            a = 0.0f;
+            mult = 1.0f;
+          }
+          if (!((valid_bits >> rr) & 1u)) {  // past the end: identity
+            a = 1.0f;
+            mult = 0.0f;
+          }
+        }
+        acc_a[rr] = a;
+        acc_x[rr] = (xc * gate_x) * mult;
+      }
+      // one pair at a time: keeps the temporaries of the gate arithmetic few
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // Recurrence.  In time order the runs of four tokens alternate between
+    // the lane halves: L0 U0 L1 U1 L2 U2 L3 U3 (run g of lanes 0-31 holds
+    // tokens 8g..8g+3, of lanes 32-63 tokens 8g+4..8g+7).  Per run the pair
+    // (P, Hh): h_out = P h_in + Hh; both halves' pairs are made visible to all
+    // lanes, every lane follows the chain and keeps the h_in of its own runs.
+    // The run is replayed from its h_in and written to the patch as soon as
+    // its h_in is known.
+    {
+      // lane-derived address, recomputed here rather than kept in a register
+      int l2 = lane;
+      asm volatile("" : "+v"(l2));
+      unsigned char* const patch_w =
+          patch + 4 * (l2 >> 5) * kPatchStride + 2 * (l2 & 31);
+      float c_run = hc;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        float P = acc_a[4 * g], Hh = acc_x[4 * g];
+#pragma unroll
+        for (int q = 1; q < 4; ++q) {
+          Hh = __builtin_fmaf(acc_a[4 * g + q], Hh, acc_x[4 * g + q]);
+          P = P * acc_a[4 * g + q];
+        }
+        float PL, PU, HL, HU;
+        halves(P, PL, PU);
+        halves(Hh, HL, HU);
+        const float after_lower = __builtin_fmaf(PL, c_run, HL);
+        float hh = upper ? after_lower : c_run;
+        c_run = __builtin_fmaf(PU, after_lower, HU);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          hh = __builtin_fmaf(acc_a[4 * g + q], hh, acc_x[4 * g + q]);
+          *reinterpret_cast<uint16_t*>(patch_w + (8 * g + q) * kPatchStride) =
+              f32_to_bf16_bits(hh);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      hc = c_run;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    // tokens past the end of the sequence fall outside the descriptor
+    {
+      int l2 = lane;
+      asm volatile("" : "+v"(l2));
+      // read side: lane l takes the 16-byte chunk l%4 of tokens l/4, l/4+16
+      const unsigned char* patch_r =
+          patch + (l2 >> 2) * kPatchStride + 16 * (l2 & 3);
+      const uint32_t y_lane_bytes = (uint32_t)(l2 >> 2) * row_bytes +
+                                    2u * (h * kBW + n0) + 16u * (l2 & 3);
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        const u32x4 v =
+            *reinterpret_cast<const u32x4*>(patch_r + q * 16 * kPatchStride);
+        __builtin_amdgcn_raw_buffer_store_b128(
+            v, ry, y_lane_bytes, (uint32_t)(t_half + 16 * q) * row_bytes, 0);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  };
+
+  // ---- tile loop ------------------------------------------------------------
+  // Per tile: A  MFMA of tokens 0-31 with the conv of the next tile between
+  //              the matrix instructions; gates + recurrence of tokens 0-31
+  //           B  MFMA of tokens 32-63 with the row loads of the tile after
+  //              next; gates + recurrence of tokens 32-63
+  int buf = 0;
+  for (int it = 0; it < ntiles; ++it, buf ^= 1) {
+    const uint64_t m_next = start_mask(it + 1);
+    fetch_seg(it + 2);
+    const bool general = m_cur != 0 || (it + 1) * kTM > T_len;
+
+    const uint16_t* abase = lds + (size_t)buf * kTM * kLdsStride +
+                            (size_t)(lane & 31) * kLdsStride + 8 * (lane >> 5);
+    auto a_read = [&](int mt, int ks) {
+      Frag a;
+      a.q = *reinterpret_cast<const f32x4*>(
+          abase + (size_t)mt * 32 * kLdsStride + ks * 16);
+      return a;
+    };
+    auto acc_init = [&](f32x16& acc_x, f32x16& acc_a) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        acc_x[r] = bias_x;
+        acc_a[r] = bias_a;
+      }
+    };
+
+    {  // ---- A
+      stage_begin(m_next, m_cur);
+      f32x16 acc_x, acc_a;
+      acc_init(acc_x, acc_a);
+      Frag a[3];
+      if (cut == 0) {
+#pragma unroll
+        for (int j = 0; j < kHalo; ++j) stage_row(j, buf ^ 1, NoCuts{});
+        a[0] = a_read(0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < 16; ++ks) {
+          if (ks < 15) a[(ks + 1) % 3] = a_read(0, ks + 1);
+          acc_x = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              a[ks % 3].v, bfrag[ks][0].v, acc_x, 0, 0, 0);
+          acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              a[ks % 3].v, bfrag[ks][1].v, acc_a, 0, 0, 0);
+          stage_row(kHalo + ks, buf ^ 1, NoCuts{});
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < kRaw; ++j) stage_row(j, buf ^ 1, WithCuts{});
+        a[0] = a_read(0, 0);
+#pragma unroll
+        for (int ks = 0; ks < 16; ++ks) {
+          if (ks < 15) a[(ks + 1) % 3] = a_read(0, ks + 1);
+          acc_x = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              a[ks % 3].v, bfrag[ks][0].v, acc_x, 0, 0, 0);
+          acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              a[ks % 3].v, bfrag[ks][1].v, acc_a, 0, 0, 0);
+        }
+      }
+      half_epilogue(it, 0, buf, acc_x, acc_a, general);
+    }
+    {  // ---- B
+      f32x16 acc_x, acc_a;
+      acc_init(acc_x, acc_a);
+      Frag a[3];
+      a[0] = a_read(1, 0);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ks = 0; ks < 16; ++ks) {
+        if (ks < 15) a[(ks + 1) % 3] = a_read(1, ks + 1);
+        acc_x = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+            a[ks % 3].v, bfrag[ks][0].v, acc_x, 0, 0, 0);
+        acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+            a[ks % 3].v, bfrag[ks][1].v, acc_a, 0, 0, 0);
+        fetch_row(it + 2, ks);
+        if (ks + 16 < kRaw) fetch_row(it + 2, ks + 16);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      half_epilogue(it, 1, buf, acc_x, acc_a, general);
+    }
+    // LDS-only barrier: row loads and y stores stay in flight across it
+    lds_barrier();
+    m_cur = m_next;
+  }
+
+  if (p.h_last && !upper) p.h_last[(int64_t)b * W + ch] = hc;
+
+  // Masked conv state: rows T-3..T-1 of x, each zeroed if a document starts in
+  // a later position of the row; rows before the sequence start are zero.
+  if (p.cache_out && tid < 128) {
+    uint16_t* cache = (uint16_t*)p.cache_out + (int64_t)b * 3 * W + c;
+    bool later_start = false;
+#pragma unroll
+    for (int kk = 2; kk >= 0; --kk) {
+      const int t = T_len - 3 + kk;
+      uint32_t v = 0;
+      if (t >= 0 && !later_start)
+        v = __builtin_amdgcn_raw_buffer_load_b32(rx, c_bytes,
+                                                 (uint32_t)t * row_bytes, 0);
+      *reinterpret_cast<uint32_t*>(cache + (int64_t)kk * W) = v;
+      if (t >= 0 && is_doc_start(p.segpos, p.seg_kind, (int64_t)b * T_len + t))
+        later_start = true;
+    }
+  }
+}
+
+}  // namespace
+
+hipError_t launch_block_fused_bf16(const FusedArgs& a, hipStream_t s) {
+  // needs head width 256 and a sequence whose rows fit 31-bit byte offsets
+  // (checked by the caller)
+  const int64_t blocks = (int64_t)a.B * a.H;
+  if (blocks <= 0 || blocks > 0x7fffffff) return hipErrorInvalidValue;
+  hipError_t e = hipFuncSetAttribute(
+      (const void*)block_fused_bf16_kernel,
+      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFusedLdsBytes);
+  if (e != hipSuccess) return e;
+  block_fused_bf16_kernel<<<dim3((unsigned)blocks), 512, kFusedLdsBytes, s>>>(a);
+  return hipGetLastError();
+}
+
+}  // namespace rg

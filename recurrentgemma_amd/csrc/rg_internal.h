@@ -63,12 +63,29 @@ struct ScanArgs {
   int B, T, W;
 };
 
+struct FusedArgs {
+  const void* x;       // [B, T, W] bf16, the conv input
+  const void* segpos;  // [B, T]
+  int seg_kind;
+  const void* conv_w;  // [4, W]
+  const void* conv_b;  // [W]
+  const void* w[2];    // [H, 256, 256]: input gate, a gate
+  const void* b[2];    // [H, 256]
+  const void* a_param; // [W]
+  const float* h0;     // [B, W] or null
+  void* y;             // [B, T, W]
+  float* h_last;       // [B, W] or null
+  void* cache_out;     // [B, 3, W] or null
+  int B, T, W, H;
+};
+
 // Each returns hipSuccess or the launch error.  dtype: 0 = f32, 1 = bf16.
 hipError_t launch_conv1d_prefill(const ConvArgs& a, int dtype, hipStream_t s);
 hipError_t launch_conv1d_step(const ConvStepArgs& a, int dtype, hipStream_t s);
 hipError_t launch_gemm_generic(const GemmArgs& a, int dtype, hipStream_t s);
 hipError_t launch_gemm_mfma_bf16(const GemmArgs& a, hipStream_t s);
 hipError_t launch_lru_scan(const ScanArgs& a, int dtype, hipStream_t s);
+hipError_t launch_block_fused_bf16(const FusedArgs& a, hipStream_t s);
 
 }  // namespace rg
 #endif  // RG_INTERNAL_H_

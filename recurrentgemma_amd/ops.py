@@ -183,6 +183,49 @@ def lru_scan_fused(x, gx_pre, ga_pre, a_param, segment_pos, h0=None, conv=None,
   return y, h_last, cache
 
 
+def recurrent_prefill_supported(x, num_heads):
+  """Shapes the single-launch prefill kernel serves (rg_recurrent_prefill)."""
+  B, T, W = x.shape
+  return (x.dtype == torch.bfloat16 and W % num_heads == 0 and
+          W // num_heads == 256 and T * W * 2 < 2**31 - 1)
+
+
+def recurrent_prefill(x, segment_pos, conv_w, conv_b, w_x, b_x, w_a, b_a,
+                      a_param, h0=None, return_h=True, return_conv_cache=True):
+  """conv -> gates -> recurrence of a whole prefill in one launch.
+
+  Returns (y, h_last | None, conv_cache | None).  Only for the shapes
+  recurrent_prefill_supported() accepts; other shapes go through gates_gemm +
+  lru_scan_fused.
+  """
+  B, T, W = x.shape
+  H = w_x.shape[0]
+  assert conv_w.shape == (4, W) and conv_b.shape == (W,)
+  assert w_x.shape == w_a.shape == (H, W // H, W // H)
+  assert b_x.shape == b_a.shape == (H, W // H)
+  assert a_param.shape == (W,)
+  x = _dev(x, "x")
+  _same(x.dtype, x.device, conv_w=conv_w, conv_b=conv_b, w_x=w_x, b_x=b_x,
+        w_a=w_a, b_a=b_a, a_param=a_param)
+  args = [_dev(t, n) for t, n in ((conv_w, "conv_w"), (conv_b, "conv_b"),
+                                  (w_x, "w_x"), (b_x, "b_x"), (w_a, "w_a"),
+                                  (b_a, "b_a"), (a_param, "a_param"))]
+  seg, is64 = _segpos(segment_pos, B, T)
+  if h0 is not None:
+    assert h0.dtype == torch.float32, "the RG-LRU state is always float32"
+    assert h0.shape == (B, W)
+    h0 = _dev(h0, "h0")
+  y = torch.empty_like(x)
+  h_last = (torch.empty((B, W), dtype=torch.float32, device=x.device)
+            if return_h else None)
+  cache = x.new_empty((B, 3, W)) if return_conv_cache else None
+  with torch.cuda.device(x.device):
+    _lib.check(_lib.lib().rg_recurrent_prefill(
+        _p(x), _p(seg), is64, *[_p(t) for t in args], _p(h0), _p(y),
+        _p(h_last), _p(cache), B, T, W, H, _dtype_code(x), _stream(x)))
+  return y, h_last, cache
+
+
 def linear_scan(x, a, reset, h0=None):
   B, T, W = x.shape
   x = _dev(x, "x")
