@@ -2,10 +2,17 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
-A "step" is one pass of the hot path over one synthetic batch that is already
-resident in HBM: rg_gates_gemm (width-4 conv on load, both gate projections on
-bf16 MFMA) followed by rg_lru_scan_fused (conv + gates + chunked scan), called
-through the C ABI on torch's current stream.  Prints ONE JSON line.
+A "step" is one pass of the hot path (Conv1D -> RG-LRU of the recurrent block)
+over one synthetic batch that is already resident in HBM, called through the C
+ABI on torch's current stream.  Two forms of the path exist (--path):
+  single  rg_recurrent_prefill: conv, gate projections (bf16 MFMA), gate
+          arithmetic and recurrence in ONE launch, nothing but x and y moves
+          through HBM (default where one workgroup per row and head fills the
+          GPU)
+  split   rg_gates_gemm (conv on load, both gate projections on bf16 MFMA)
+          followed by rg_lru_scan_fused (conv + gates + chunked scan); the gate
+          pre-activations go through HBM
+Prints ONE JSON line.
 
 Workloads (BASELINE.json configs):
   9b_prefill  B16 T8192 W4096 H16 bf16 / fp32 state, one document per row
@@ -16,9 +23,12 @@ Workloads (BASELINE.json configs):
               carried in place (rg_recurrent_step); `roofline` then describes
               the whole step (all its launches) against its algorithmic bytes
 
-`roofline` describes the scan kernel: algorithmic bytes per launch (read x,
-read both gate pre-activations, write y, plus the small terms) over the mean
-launch duration measured with HIP events inside the timed region.
+`roofline` describes the dominant kernel of the timed path: its algorithmic
+bytes per launch (single: read x, write y; split: the scan kernel's read x,
+read both gate pre-activations, write y; plus the small terms) over the mean
+launch duration measured with HIP events inside the timed region.  With the
+default path the JSON also carries `two_kernel_path`, the split form measured
+after the timed region (scan-kernel roofline and gate GEMM figures).
 `cpu_baseline` times the CPU oracle (an op-for-op torch restatement of the
 reference's path, bf16 like the reference would run it) on a bounded sample of
 the same workload on this machine's host cores.
@@ -47,8 +57,18 @@ WORKLOADS = {
 # (scaled by a copy kernel of known size); None until measured for a workload.
 MEASURED_TRAFFIC_BYTES = {
     # profiles/hbm_traffic_9b_prefill.txt: 3.334 GB read + 1.074 GB written
-    "9b_prefill": 4.408e9,
+    ("9b_prefill", "scan"): 4.408e9,
 }
+
+
+def single_algorithmic_bytes(B, T, W, H, esize, seg_bytes, has_h0):
+  n = B * T * W
+  return (2 * esize * n            # x in, y out
+          + B * T * seg_bytes      # segment positions
+          + B * W * 4 * (int(has_h0) + 1)   # h0 in, h_last out (fp32)
+          + B * 3 * W * esize      # conv state out
+          + 2 * H * (W // H) ** 2 * esize   # both gate weight matrices
+          + W * esize * 8)         # conv w (4), conv b, a_param, gate biases
 
 
 def scan_algorithmic_bytes(B, T, W, esize, seg_bytes, has_h0):
@@ -186,6 +206,7 @@ def main():
   ap.add_argument("--steps", type=int, default=50)
   ap.add_argument("--warmup", type=int, default=10)
   ap.add_argument("--workload", default="9b_prefill", choices=sorted(WORKLOADS))
+  ap.add_argument("--path", default="auto", choices=["auto", "single", "split"])
   ap.add_argument("--no-cpu-baseline", action="store_true")
   ap.add_argument("--calibration-copy", action="store_true",
                   help="after the timed steps, run one plain device copy of x "
@@ -224,7 +245,7 @@ def main():
   blk = blk.to(dev)
   conv, lru = blk.conv_1d, blk.rg_lru
 
-  def step(events=None):
+  def step_split(events=None):
     if events:
       events[0].record()
     gx, ga = ops.gates_gemm(x, lru.input_gate.w, lru.input_gate.b,
@@ -239,33 +260,82 @@ def main():
       events[2].record()
     return y, h, cache
 
-  for _ in range(args.warmup):
-    out = step()
-  torch.cuda.synchronize()
+  def step_single(events=None):
+    if events:
+      events[0].record()
+    out = ops.recurrent_prefill(x, seg, conv.w, conv.b, lru.input_gate.w,
+                                lru.input_gate.b, lru.a_gate.w, lru.a_gate.b,
+                                lru.a_param)
+    if events:
+      events[1].record()
+      events[2].record()
+    return out
 
-  evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)]
-         for _ in range(args.steps)]
-  torch.cuda.synchronize()
-  t0 = time.perf_counter()
-  for i in range(args.steps):
-    out = step(evs[i])
-  torch.cuda.synchronize()
-  elapsed = time.perf_counter() - t0
+  path = args.path
+  if path == "auto":
+    path = ("single" if ops.recurrent_prefill_supported(x, H) and B * H >= 128
+            else "split")
+  step = step_single if path == "single" else step_split
+
+  def timed(fn, steps, warmup):
+    for _ in range(warmup):
+      fn()
+    torch.cuda.synchronize()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)]
+           for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+      fn(evs[i])
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    first = sum(e[0].elapsed_time(e[1]) for e in evs) / steps
+    second = sum(e[1].elapsed_time(e[2]) for e in evs) / steps
+    return elapsed, first, second
+
+  elapsed, first_ms, second_ms = timed(step, args.steps, args.warmup)
+
+  tokens = B * T
+  seg_bytes = seg.element_size()
+  scan_algo = scan_algorithmic_bytes(B, T, W, 2, seg_bytes, has_h0=False)
+  gemm_flops = 1024.0 * W * tokens
+  gemm_bytes = 3 * 2 * B * T * W
+
+  def split_figures(gemm_ms, scan_ms):
+    achieved = scan_algo / (scan_ms * 1e-3) / 1e9
+    return {
+        "scan": {
+            "kernel": "lru_scan_kernel (conv + gates + scan)",
+            "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
+            "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+            "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, "scan")),
+            "algorithmic_bytes": scan_algo, "avg_launch_ms": scan_ms},
+        "gate_gemm": {
+            "kernel": "gates_mfma_bf16_kernel", "avg_launch_ms": gemm_ms,
+            "tflops": gemm_flops / (gemm_ms * 1e-3) / 1e12,
+            "frac_of_bf16_mfma_peak": gemm_flops / (gemm_ms * 1e-3) / 2.5e15,
+            "gbs": gemm_bytes / (gemm_ms * 1e-3) / 1e9,
+            "frac_of_hbm_peak": gemm_bytes / (gemm_ms * 1e-3) / 1e9
+                                / HBM_PEAK_GBS}}
+
+  if path == "single":
+    algo = single_algorithmic_bytes(B, T, W, H, 2, seg_bytes, has_h0=False)
+    achieved = algo / (first_ms * 1e-3) / 1e9
+    roofline = {
+        "kernel": "block_fused_bf16_kernel (conv + gate GEMMs + gates + scan)",
+        "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
+        "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+        "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, "single")),
+        "algorithmic_bytes": algo, "avg_launch_ms": first_ms,
+        "mfma_tflops": gemm_flops / (first_ms * 1e-3) / 1e12,
+        "frac_of_bf16_mfma_peak": gemm_flops / (first_ms * 1e-3) / 2.5e15}
+  else:
+    figs = split_figures(first_ms, second_ms)
+    roofline = figs["scan"]
 
   if args.calibration_copy:
     torch.empty_like(x).copy_(x)  # reads and writes x.numel()*2 bytes
     torch.cuda.synchronize()
-
-  gemm_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / args.steps
-  scan_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / args.steps
-  ms_per_step = elapsed * 1e3 / args.steps
-  tokens = B * T
-
-  seg_bytes = seg.element_size()
-  algo = scan_algorithmic_bytes(B, T, W, 2, seg_bytes, has_h0=False)
-  achieved = algo / (scan_ms * 1e-3) / 1e9
-  gemm_flops = 1024.0 * W * tokens
-  gemm_bytes = 3 * 2 * B * T * W
 
   result = {
       "metric": "RG-LRU block tokens/s + scan HBM GB/s (% of roofline)",
@@ -274,7 +344,7 @@ def main():
       "n_gpus": 1,
       "steps": args.steps,
       "warmup": args.warmup,
-      "ms_per_step": ms_per_step,
+      "ms_per_step": elapsed * 1e3 / args.steps,
       "higher_is_better": True,
       "scaling": "weak",
       "vs_baseline": None,
@@ -285,21 +355,21 @@ def main():
           "heads": H, "activations": "bf16", "state": "f32",
           "documents": ("one per row" if wl["mean_doc"] is None
                         else f"geometric mean {wl['mean_doc']}"),
-          "path": "rg_gates_gemm(conv on load) + rg_lru_scan_fused(conv)"},
-      "roofline": {
-          "kernel": "lru_scan_kernel (conv + gates + scan)",
-          "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
-          "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-          "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-          "algorithmic_bytes": algo, "avg_launch_ms": scan_ms},
-      "gate_gemm": {
-          "kernel": "gates_mfma_bf16_kernel", "avg_launch_ms": gemm_ms,
-          "tflops": gemm_flops / (gemm_ms * 1e-3) / 1e12,
-          "frac_of_bf16_mfma_peak": gemm_flops / (gemm_ms * 1e-3) / 2.5e15,
-          "gbs": gemm_bytes / (gemm_ms * 1e-3) / 1e9,
-          "frac_of_hbm_peak": gemm_bytes / (gemm_ms * 1e-3) / 1e9
-                              / HBM_PEAK_GBS},
+          "path": ("rg_recurrent_prefill (single launch)" if path == "single"
+                   else "rg_gates_gemm(conv on load) + "
+                        "rg_lru_scan_fused(conv)")},
+      "roofline": roofline,
   }
+  if path == "split":
+    result["gate_gemm"] = figs["gate_gemm"]
+  elif args.path == "auto":
+    # the two-kernel form of the same step, measured after the timed region
+    n2 = max(5, args.steps // 2)
+    e2, g_ms, s_ms = timed(step_split, n2, 3)
+    figs = split_figures(g_ms, s_ms)
+    result["two_kernel_path"] = {
+        "value": tokens / (e2 / n2), "unit": "tokens/s", "steps": n2,
+        "scan": figs["scan"], "gate_gemm": figs["gate_gemm"]}
   if not args.no_cpu_baseline:
     result["cpu_baseline"] = cpu_baseline(torch, R, wl, params)
   print(json.dumps(result))

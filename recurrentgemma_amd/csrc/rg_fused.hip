@@ -22,7 +22,12 @@ constexpr int kLdsStride = 264;    // bf16 elements per staged row (256 + 8 pad)
 constexpr int kRowsPerGroup = 16;  // rows each thread converts per tile
 constexpr int kHalo = 3;
 constexpr int kRaw = kRowsPerGroup + kHalo;
-constexpr size_t kStageLdsBytes = 2ull * kTM * kLdsStride * sizeof(uint16_t);
+// Three staged tiles: the one the MFMAs read, the one being written for the
+// next tile, and the previous one, which half of the waves still read while
+// they finish its gate arithmetic (see the tile loop).
+constexpr int kStageBufs = 3;
+constexpr size_t kStageLdsBytes =
+    (size_t)kStageBufs * kTM * kLdsStride * sizeof(uint16_t);
 // Per-wave output patch: 32 tokens x 32 channels in bf16, rows padded to 80
 // bytes (16-byte aligned row reads, spread over the banks).
 constexpr int kPatchStride = 80;
@@ -31,13 +36,25 @@ constexpr size_t kPatchBytesPerWave = 32ull * kPatchStride;
 // and bias for both channels, padded): read back at the start of every conv
 // so that they do not occupy registers in between.
 constexpr size_t kConvTabOffset = kStageLdsBytes + 8 * kPatchBytesPerWave;
-constexpr size_t kFusedLdsBytes = kConvTabOffset + 128 * 12 * sizeof(float);
+// Gate biases and decay constant of the 256 channels (4 floats each, one
+// padding), read at the start of the phases that need them.
+constexpr size_t kChanTabOffset = kConvTabOffset + 128 * 12 * sizeof(float);
+constexpr size_t kFusedLdsBytes = kChanTabOffset + 256 * 4 * sizeof(float);
 
 union Frag {
   bf16x8 v;
   uint16_t u[8];
   f32x4 q;
 };
+
+// Build switch for the tile loop: 1 runs waves 4-7 one phase behind waves 0-3
+// (matrix phases of one group over vector phases of the other).  Measured at
+// B16 T8192 W4096 it is about 3 % slower than keeping all waves in the same
+// phase (the vector ALU, not the matrix pipe, bounds the tile), so it is off.
+#ifndef RG_FUSED_SKEW
+#define RG_FUSED_SKEW 0
+#endif
+constexpr bool kSkewGroups = RG_FUSED_SKEW != 0;
 
 using WithCuts = std::integral_constant<bool, true>;
 using NoCuts = std::integral_constant<bool, false>;
@@ -64,6 +81,14 @@ __global__ void __launch_bounds__(512) block_fused_bf16_kernel(FusedArgs p) {
   const int64_t W = p.W;
   const int ntiles = (T_len + kTM - 1) / kTM;
   const bool upper = lane >= 32;
+  // Lane-derived addresses are recomputed from the thread id where they are
+  // used (a few integer instructions) instead of being kept in registers for
+  // the whole tile: the optimiser cannot see through fresh_tid().
+  auto fresh_tid = [&]() {
+    int t = tid;
+    asm volatile("" : "+v"(t));
+    return t;
+  };
 
   // ---- this wave's weights: 32 channels of the head, both gates ----------
   // The weights are [k][n] with n contiguous, the MFMA B operand wants 8
@@ -97,11 +122,19 @@ __global__ void __launch_bounds__(512) block_fused_bf16_kernel(FusedArgs p) {
   // Per-lane channel (the MFMA result has channel = lane % 32): gate biases,
   // decay constant -8 softplus(a_param) log2(e), running state.
   const int ch = h * kBW + n0 + (lane & 31);
-  const float bias_x = bf16_bits_to_f32(((const uint16_t*)p.b[0])[ch]);
-  const float bias_a = bf16_bits_to_f32(((const uint16_t*)p.b[1])[ch]);
-  const float decay =
-      (-8.0f * kLog2e) *
-      softplus_precise(bf16_bits_to_f32(((const uint16_t*)p.a_param)[ch]));
+  auto chan_ptr = [&](int t) {
+    return reinterpret_cast<float*>(lds_raw + kChanTabOffset) +
+           4 * (n0 + (t & 31));
+  };
+  if (!upper) {
+    float* const chan_tab = chan_ptr(tid);
+    f32x4 t = {bf16_bits_to_f32(((const uint16_t*)p.b[0])[ch]),
+               bf16_bits_to_f32(((const uint16_t*)p.b[1])[ch]),
+               (-8.0f * kLog2e) * softplus_precise(bf16_bits_to_f32(
+                                      ((const uint16_t*)p.a_param)[ch])),
+               0.0f};
+    *reinterpret_cast<f32x4*>(chan_tab) = t;
+  }
   float hc = p.h0 ? p.h0[(int64_t)b * W + ch] : 0.0f;
 
   // ---- addressing ---------------------------------------------------------
@@ -123,9 +156,11 @@ __global__ void __launch_bounds__(512) block_fused_bf16_kernel(FusedArgs p) {
   const uint32_t c = h * kBW + cp * 2;
   const uint32_t c_bytes = 2u * c;
   float cw0[2], cw1[2], cw2[2], cw3[2], cb[2];
-  float* const conv_tab =
-      reinterpret_cast<float*>(lds_raw + kConvTabOffset) + cp * 12;
+  auto conv_ptr = [&](int t) {
+    return reinterpret_cast<float*>(lds_raw + kConvTabOffset) + (t & 127) * 12;
+  };
   if (tid < 128) {
+    float* const conv_tab = conv_ptr(tid);
     const uint16_t* cw = (const uint16_t*)p.conv_w + c;
     const uint32_t u0 = *reinterpret_cast<const uint32_t*>(cw);
     const uint32_t u1 = *reinterpret_cast<const uint32_t*>(cw + W);
@@ -144,7 +179,8 @@ __global__ void __launch_bounds__(512) block_fused_bf16_kernel(FusedArgs p) {
     reinterpret_cast<f32x4*>(conv_tab)[2] = t2;
   }
   __syncthreads();
-  auto load_conv_consts = [&]() {
+  auto load_conv_consts = [&](int t) {
+    const float* const conv_tab = conv_ptr(t);
     const f32x4 t0 = reinterpret_cast<const f32x4*>(conv_tab)[0];
     const f32x4 t1 = reinterpret_cast<const f32x4*>(conv_tab)[1];
     const f32x4 t2 = reinterpret_cast<const f32x4*>(conv_tab)[2];
@@ -176,20 +212,26 @@ __global__ void __launch_bounds__(512) block_fused_bf16_kernel(FusedArgs p) {
   // Rows before the sequence get an out-of-range scalar offset, rows past its
   // end fall outside the descriptor: both read as zero, which is what the
   // conv sees there.
-  auto fetch_row = [&](int tile, int j) {
+  auto fetch_row = [&](int tile, int j, uint32_t cb_off) {
     const int t = tile * kTM + rg * kRowsPerGroup - kHalo + j;  // uniform
     const uint32_t soff =
         (t < 0 || tile >= ntiles) ? kBufferOutOfRange : (uint32_t)t * row_bytes;
-    raw[j] = __builtin_amdgcn_raw_buffer_load_b32(rx, c_bytes, soff, 0);
+    raw[j] = __builtin_amdgcn_raw_buffer_load_b32(rx, cb_off, soff, 0);
   };
+  auto chan_bytes = [&](int t) {  // byte offset of thread t's channel pair
+    return 2u * (uint32_t)(h * kBW + (t & 127) * 2);
+  };
+
 
   // Conv of one tile, one row at a time.  cut bit j: token j of this thread
   // group's 19 rows starts a document; the conv must not look past it.
   uint32_t cut = 0;
   float h0v[2], h1v[2], h2v[2];
-  uint16_t* const stage_dst0 =
-      lds + (size_t)(rg * kRowsPerGroup) * kLdsStride + cp * 2;
-  auto stage_begin = [&](uint64_t m_tile, uint64_t m_before) {
+  auto stage_dst = [&](int t, int buf) {
+    return lds + (size_t)buf * kTM * kLdsStride +
+           (size_t)(rg * kRowsPerGroup) * kLdsStride + (t & 127) * 2;
+  };
+  auto stage_begin = [&](int t, uint64_t m_tile, uint64_t m_before) {
     // rows 16*rg-3 .. 16*rg+15 of the tile; the three rows before the tile
     // are the last three of the previous one
     if (rg == 0)
@@ -197,11 +239,10 @@ __global__ void __launch_bounds__(512) block_fused_bf16_kernel(FusedArgs p) {
     else
       cut = (uint32_t)(m_tile >> (16 * rg - 3)) & 0x7ffffu;
     h0v[0] = h0v[1] = h1v[0] = h1v[1] = h2v[0] = h2v[1] = 0.0f;
-    load_conv_consts();
+    load_conv_consts(t);
   };
-  auto stage_row = [&](int j, int buf, auto cuts) {
+  auto stage_row = [&](int j, uint16_t* dst, auto cuts) {
     constexpr bool CUTS = decltype(cuts)::value;
-    uint16_t* dst = stage_dst0 + (size_t)buf * kTM * kLdsStride;
     float xv[2];
     xv[0] = __uint_as_float(raw[j] << 16);
     xv[1] = __uint_as_float(raw[j] & 0xffff0000u);
@@ -235,14 +276,14 @@ __global__ void __launch_bounds__(512) block_fused_bf16_kernel(FusedArgs p) {
   {
     fetch_seg(0);
 #pragma unroll
-    for (int j = 0; j < kRaw; ++j) fetch_row(0, j);
+    for (int j = 0; j < kRaw; ++j) fetch_row(0, j, c_bytes);
     m_cur = start_mask(0);
-    stage_begin(m_cur, 0);
+    stage_begin(tid, m_cur, 0);
 #pragma unroll
-    for (int j = 0; j < kRaw; ++j) stage_row(j, 0, WithCuts{});
+    for (int j = 0; j < kRaw; ++j) stage_row(j, stage_dst(tid, 0), WithCuts{});
     fetch_seg(1);
 #pragma unroll
-    for (int j = 0; j < kRaw; ++j) fetch_row(1, j);
+    for (int j = 0; j < kRaw; ++j) fetch_row(1, j, c_bytes);
   }
   lds_barrier();
 
@@ -252,31 +293,32 @@ __global__ void __launch_bounds__(512) block_fused_bf16_kernel(FusedArgs p) {
   // handles document starts (a = 0, unit input scale) and tokens past the end
   // of the sequence (identity: a = 1, no input).
   auto half_epilogue = [&](int it, int mt, int buf, f32x16& acc_x, f32x16& acc_a,
-                           bool general) {
+                           uint64_t m_tile) {
+    const bool general = m_tile != 0 || (it + 1) * kTM > T_len;
     int l1 = lane;
     asm volatile("" : "+v"(l1));  // address recomputed per call, not kept
     const uint16_t* xcp = lds + (size_t)buf * kTM * kLdsStride +
                           (size_t)(mt * 32 + 4 * (l1 >> 5)) * kLdsStride + n0 +
                           (l1 & 31);
     const int t_half = it * kTM + mt * 32;  // first token of this half
-    // `general` (wave-uniform, rare): bit r of these per-lane words says that
-    // token r of this lane starts a document / lies inside the sequence.
-    uint32_t start_bits = 0, valid_bits = 0xffffu;
+    const float decay = chan_ptr(l1)[2];
+    // `general` (wave-uniform, rare): bit r of these words says that token r
+    // of a lane starts a document / lies inside the sequence.
+    // kept as wave-uniform words, one pair per lane half
+    uint32_t s_lo = 0, s_hi = 0, v_lo = 0xffffu, v_hi = 0xffffu;
     if (general) {
-      uint32_t s_lo = 0, s_hi = 0, v_lo = 0, v_hi = 0;
+      v_lo = v_hi = 0;
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int row = mt * 32 + 8 * g;  // lanes 0-31: row..row+3, 32-63: +4
-        s_lo |= ((uint32_t)(m_cur >> row) & 0xfu) << (4 * g);
-        s_hi |= ((uint32_t)(m_cur >> (row + 4)) & 0xfu) << (4 * g);
+        s_lo |= ((uint32_t)(m_tile >> row) & 0xfu) << (4 * g);
+        s_hi |= ((uint32_t)(m_tile >> (row + 4)) & 0xfu) << (4 * g);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           v_lo |= (uint32_t)(t_half + 8 * g + q < T_len) << (4 * g + q);
           v_hi |= (uint32_t)(t_half + 8 * g + 4 + q < T_len) << (4 * g + q);
         }
       }
-      start_bits = upper ? s_hi : s_lo;
-      valid_bits = upper ? v_hi : v_lo;
     }
 #pragma unroll
     for (int r = 0; r < 16; r += 2) {
@@ -297,11 +339,13 @@ __global__ void __launch_bounds__(512) block_fused_bf16_kernel(FusedArgs p) {
         float a = __builtin_amdgcn_exp2f(gate_a * decay);
         float mult = __builtin_amdgcn_sqrtf(__builtin_fmaf(-a, a, 1.0f));
         if (general) {
-          if ((start_bits >> rr) & 1u) {  // document start: forget, unit scale
+          const bool start = upper ? (s_hi >> rr) & 1u : (s_lo >> rr) & 1u;
+          const bool valid = upper ? (v_hi >> rr) & 1u : (v_lo >> rr) & 1u;
+          if (start) {  // document start: forget, unit scale
             a = 0.0f;
             mult = 1.0f;
           }
-          if (!((valid_bits >> rr) & 1u)) {  // past the end: identity
+          if (!valid) {  // past the end: identity
             a = 1.0f;
             mult = 0.0f;
           }
@@ -309,8 +353,10 @@ __global__ void __launch_bounds__(512) block_fused_bf16_kernel(FusedArgs p) {
         acc_a[rr] = a;
         acc_x[rr] = (xc * gate_x) * mult;
       }
-      // one pair at a time: keeps the temporaries of the gate arithmetic few
-      __builtin_amdgcn_sched_barrier(0);
+      // four tokens at a time: enough independent work to cover the latency
+      // of the transcendental chain, few enough temporaries to stay in
+      // registers
+      if ((r & 2) != 0) __builtin_amdgcn_sched_barrier(0);
     }
     // Recurrence.  In time order the runs of four tokens alternate between
     // the lane halves: L0 U0 L1 U1 L2 U2 L3 U3 (run g of lanes 0-31 holds
@@ -374,89 +420,135 @@ __global__ void __launch_bounds__(512) block_fused_bf16_kernel(FusedArgs p) {
   };
 
   // ---- tile loop ------------------------------------------------------------
-  // Per tile: A  MFMA of tokens 0-31 with the conv of the next tile between
-  //              the matrix instructions; gates + recurrence of tokens 0-31
-  //           B  MFMA of tokens 32-63 with the row loads of the tile after
-  //              next; gates + recurrence of tokens 32-63
-  int buf = 0;
-  for (int it = 0; it < ntiles; ++it, buf ^= 1) {
-    const uint64_t m_next = start_mask(it + 1);
-    fetch_seg(it + 2);
-    const bool general = m_cur != 0 || (it + 1) * kTM > T_len;
-
-    const uint16_t* abase = lds + (size_t)buf * kTM * kLdsStride +
-                            (size_t)(lane & 31) * kLdsStride + 8 * (lane >> 5);
-    auto a_read = [&](int mt, int ks) {
-      Frag a;
-      a.q = *reinterpret_cast<const f32x4*>(
-          abase + (size_t)mt * 32 * kLdsStride + ks * 16);
-      return a;
-    };
-    auto acc_init = [&](f32x16& acc_x, f32x16& acc_a) {
+  // Phases of one tile `it` (staged in buffer it % 3):
+  //   A   MFMA of tokens 0-31, with the conv of tile it+1 (into buffer
+  //       (it+1) % 3) between the matrix instructions
+  //   E0  gates + recurrence of tokens 0-31
+  //   B   MFMA of tokens 32-63, with the row loads of tile it+2
+  //   E1  gates + recurrence of tokens 32-63
+  // A and B keep the matrix pipe busy, E0 and E1 the vector ALU.  Each SIMD
+  // holds one wave of waves 0-3 and one of waves 4-7; the second group runs one
+  // phase behind the first (it finishes E1 of a tile after the barrier that
+  // ends the tile), so that on every SIMD a matrix phase of one wave overlaps a
+  // vector phase of the other:
+  //   waves 0-3:  A(it)    E0(it)  B(it)   E1(it)  | barrier
+  //   waves 4-7:  E1(it-1) A(it)   E0(it)  B(it)   | barrier
+  auto a_base = [&](int t, int bi, int mt) {
+    const int l = t & 63;
+    return lds + (size_t)bi * kTM * kLdsStride +
+           (size_t)(mt * 32 + (l & 31)) * kLdsStride + 8 * (l >> 5);
+  };
+  auto a_read = [&](const uint16_t* abase, int ks) {
+    Frag a;
+    a.q = *reinterpret_cast<const f32x4*>(abase + ks * 16);
+    return a;
+  };
+  auto acc_init = [&](int t, f32x16& acc_x, f32x16& acc_a) {
+    const f32x2 bias = *reinterpret_cast<const f32x2*>(chan_ptr(t));
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        acc_x[r] = bias_x;
-        acc_a[r] = bias_a;
-      }
-    };
-
-    {  // ---- A
-      stage_begin(m_next, m_cur);
-      f32x16 acc_x, acc_a;
-      acc_init(acc_x, acc_a);
-      Frag a[3];
-      if (cut == 0) {
-#pragma unroll
-        for (int j = 0; j < kHalo; ++j) stage_row(j, buf ^ 1, NoCuts{});
-        a[0] = a_read(0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int ks = 0; ks < 16; ++ks) {
-          if (ks < 15) a[(ks + 1) % 3] = a_read(0, ks + 1);
-          acc_x = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              a[ks % 3].v, bfrag[ks][0].v, acc_x, 0, 0, 0);
-          acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              a[ks % 3].v, bfrag[ks][1].v, acc_a, 0, 0, 0);
-          stage_row(kHalo + ks, buf ^ 1, NoCuts{});
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      } else {
-#pragma unroll
-        for (int j = 0; j < kRaw; ++j) stage_row(j, buf ^ 1, WithCuts{});
-        a[0] = a_read(0, 0);
-#pragma unroll
-        for (int ks = 0; ks < 16; ++ks) {
-          if (ks < 15) a[(ks + 1) % 3] = a_read(0, ks + 1);
-          acc_x = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              a[ks % 3].v, bfrag[ks][0].v, acc_x, 0, 0, 0);
-          acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              a[ks % 3].v, bfrag[ks][1].v, acc_a, 0, 0, 0);
-        }
-      }
-      half_epilogue(it, 0, buf, acc_x, acc_a, general);
+    for (int r = 0; r < 16; ++r) {
+      acc_x[r] = bias[0];
+      acc_a[r] = bias[1];
     }
-    {  // ---- B
-      f32x16 acc_x, acc_a;
-      acc_init(acc_x, acc_a);
-      Frag a[3];
-      a[0] = a_read(1, 0);
+  };
+  auto phase_a = [&](int bi, int bn, uint64_t m_next, uint64_t m_tile,
+                     f32x16& acc_x, f32x16& acc_a) {
+    const int t1 = fresh_tid();
+    const uint16_t* abase = a_base(t1, bi, 0);
+    uint16_t* const dst = stage_dst(t1, bn);
+    stage_begin(t1, m_next, m_tile);
+    acc_init(t1, acc_x, acc_a);
+    Frag a[2];
+    if (cut == 0) {
+#pragma unroll
+      for (int j = 0; j < kHalo; ++j) stage_row(j, dst, NoCuts{});
+      a[0] = a_read(abase, 0);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 0; ks < 16; ++ks) {
-        if (ks < 15) a[(ks + 1) % 3] = a_read(1, ks + 1);
+        if (ks < 15) a[(ks + 1) & 1] = a_read(abase, ks + 1);
         acc_x = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            a[ks % 3].v, bfrag[ks][0].v, acc_x, 0, 0, 0);
+            a[ks & 1].v, bfrag[ks][0].v, acc_x, 0, 0, 0);
         acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            a[ks % 3].v, bfrag[ks][1].v, acc_a, 0, 0, 0);
-        fetch_row(it + 2, ks);
-        if (ks + 16 < kRaw) fetch_row(it + 2, ks + 16);
+            a[ks & 1].v, bfrag[ks][1].v, acc_a, 0, 0, 0);
+        stage_row(kHalo + ks, dst, NoCuts{});
         __builtin_amdgcn_sched_barrier(0);
       }
-      half_epilogue(it, 1, buf, acc_x, acc_a, general);
+    } else {
+      // a document starts among the rows of the next tile: conv first, with
+      // the history cuts, then the matrix instructions
+#pragma unroll
+      for (int j = 0; j < kRaw; ++j) stage_row(j, dst, WithCuts{});
+      a[0] = a_read(abase, 0);
+#pragma unroll
+      for (int ks = 0; ks < 16; ++ks) {
+        if (ks < 15) a[(ks + 1) & 1] = a_read(abase, ks + 1);
+        acc_x = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+            a[ks & 1].v, bfrag[ks][0].v, acc_x, 0, 0, 0);
+        acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+            a[ks & 1].v, bfrag[ks][1].v, acc_a, 0, 0, 0);
+      }
     }
-    // LDS-only barrier: row loads and y stores stay in flight across it
-    lds_barrier();
-    m_cur = m_next;
+  };
+  auto phase_b = [&](int it, int bi, f32x16& acc_x, f32x16& acc_a) {
+    const int t1 = fresh_tid();
+    const uint32_t cb_off = chan_bytes(t1);
+    const uint16_t* abase = a_base(t1, bi, 1);
+    acc_init(t1, acc_x, acc_a);
+    Frag a[2];
+    a[0] = a_read(abase, 0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < 16; ++ks) {
+      if (ks < 15) a[(ks + 1) & 1] = a_read(abase, ks + 1);
+      acc_x = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+          a[ks & 1].v, bfrag[ks][0].v, acc_x, 0, 0, 0);
+      acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+          a[ks & 1].v, bfrag[ks][1].v, acc_a, 0, 0, 0);
+      fetch_row(it + 2, ks, cb_off);
+      if (ks + 16 < kRaw) fetch_row(it + 2, ks + 16, cb_off);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  if (!kSkewGroups || wave < 4) {
+    int bi = 0;
+    for (int it = 0; it < ntiles; ++it) {
+      const int bn = bi == kStageBufs - 1 ? 0 : bi + 1;
+      const uint64_t m_next = start_mask(it + 1);
+      fetch_seg(it + 2);
+      f32x16 acc_x, acc_a;
+      phase_a(bi, bn, m_next, m_cur, acc_x, acc_a);
+      half_epilogue(it, 0, bi, acc_x, acc_a, m_cur);
+      phase_b(it, bi, acc_x, acc_a);
+      half_epilogue(it, 1, bi, acc_x, acc_a, m_cur);
+      // LDS-only barrier: row loads and y stores stay in flight across it
+      lds_barrier();
+      m_cur = m_next;
+      bi = bn;
+    }
+  } else {
+    int bi = 0, bp = 0;
+    uint64_t m_prev = 0;
+    f32x16 late_x, late_a;  // tokens 32-63 of the previous tile, E1 pending
+#pragma unroll
+    for (int r = 0; r < 16; ++r) late_x[r] = late_a[r] = 0.0f;
+    for (int it = 0; it < ntiles; ++it) {
+      const int bn = bi == kStageBufs - 1 ? 0 : bi + 1;
+      const uint64_t m_next = start_mask(it + 1);
+      fetch_seg(it + 2);
+      if (it > 0) half_epilogue(it - 1, 1, bp, late_x, late_a, m_prev);
+      f32x16 acc_x, acc_a;
+      phase_a(bi, bn, m_next, m_cur, acc_x, acc_a);
+      half_epilogue(it, 0, bi, acc_x, acc_a, m_cur);
+      phase_b(it, bi, late_x, late_a);
+      lds_barrier();
+      m_prev = m_cur;
+      m_cur = m_next;
+      bp = bi;
+      bi = bn;
+    }
+    half_epilogue(ntiles - 1, 1, bp, late_x, late_a, m_prev);
   }
 
   if (p.h_last && !upper) p.h_last[(int64_t)b * W + ch] = hc;

@@ -30,6 +30,11 @@ def gelu(x: torch.Tensor) -> torch.Tensor:
   return nn.functional.gelu(x, approximate="tanh")
 
 
+# rg_recurrent_prefill runs one workgroup per (sequence row, head); with fewer
+# groups than this most of the 256 CUs would idle.
+_MIN_GROUPS_FOR_SINGLE_LAUNCH = 128
+
+
 @torch.no_grad()
 def recurrent_core(conv_1d: layers.Conv1D, rg_lru: layers.RGLRU, x,
                    segment_pos, cache: RecurrentBlockCache | None = None,
@@ -57,6 +62,14 @@ def recurrent_core(conv_1d: layers.Conv1D, rg_lru: layers.RGLRU, x,
                              return_cache)
     y, h = rg_lru(xc, segment_pos,
                   None if cache is None else cache.rg_lru_state, return_cache)
+  elif (ops.recurrent_prefill_supported(x, rg_lru.num_heads) and
+        bs * rg_lru.num_heads >= _MIN_GROUPS_FOR_SINGLE_LAUNCH):
+    # one workgroup per (row, head): pays once there are enough of them to
+    # fill the GPU; below that the two-kernel form spreads over more CUs
+    y, h, conv_state = ops.recurrent_prefill(
+        x, segment_pos, conv_1d.w, conv_1d.b, rg_lru.input_gate.w,
+        rg_lru.input_gate.b, rg_lru.a_gate.w, rg_lru.a_gate.b, rg_lru.a_param,
+        h0=None, return_h=return_cache, return_conv_cache=return_cache)
   else:
     gx_pre, ga_pre = ops.gates_gemm(
         x, rg_lru.input_gate.w, rg_lru.input_gate.b, rg_lru.a_gate.w,

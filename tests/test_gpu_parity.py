@@ -389,6 +389,70 @@ def test_recurrent_block_module():
   assert helpers.max_rel(got1, want[:, :1]) < 1e-4
 
 
+# ------------------------------------------- single-launch prefill kernel --
+
+
+@pytest.mark.parametrize("B,T,W,H,mean_doc,seg_dtype,with_h0", [
+    (1, 64, 256, 1, None, torch.int64, False),
+    (1, 128, 256, 1, None, torch.int64, False),
+    (2, 200, 512, 2, 50, torch.int64, True),
+    (3, 1, 256, 1, None, torch.int32, True),
+    (2, 3, 512, 2, 2, torch.int32, False),
+    (2, 65, 256, 1, 16, torch.int64, True),
+    (2, 1000, 768, 3, 250, torch.int32, False),
+    (1, 130, 256, 1, 3, torch.int64, False),   # documents of a few tokens
+])
+def test_recurrent_prefill_single_launch(B, T, W, H, mean_doc, seg_dtype,
+                                         with_h0):
+  """rg_recurrent_prefill against the oracle (bf16 tolerance) and against the
+  two-kernel form (same arithmetic up to the association of the recurrence)."""
+  _announce("recurrent_prefill", B, T, W, H, mean_doc, seg_dtype, with_h0)
+  seed = 7000 + T
+  p = R.make_params(W, H, torch.bfloat16, seed=seed, gate_bias_std=0.5)
+  g = torch.Generator().manual_seed(seed + 1)
+  x = torch.randn(B, T, W, generator=g).to(torch.bfloat16)
+  seg = (torch.arange(T).expand(B, T).contiguous() if mean_doc is None
+         else helpers.document_positions(B, T, mean_doc, seed=seed))
+  h0 = torch.randn(B, W, generator=g) if with_h0 else None
+  P = {k: _dev(v) for k, v in p.items()}
+  xd, segd = _dev(x), _dev(seg.to(seg_dtype))
+  h0d = None if h0 is None else _dev(h0)
+  assert ops.recurrent_prefill_supported(xd, H)
+  y, h, cache = ops.recurrent_prefill(
+      xd, segd, P["conv_w"], P["conv_b"], P["w_x"], P["b_x"], P["w_a"],
+      P["b_a"], P["a_param"], h0=h0d)
+  gx, ga = ops.gates_gemm(xd, P["w_x"], P["b_x"], P["w_a"], P["b_a"],
+                          conv=(segd, P["conv_w"], P["conv_b"]))
+  y2, h2, cache2 = ops.lru_scan_fused(
+      xd, gx, ga, P["a_param"], segd, h0=h0d,
+      conv=(P["conv_w"], P["conv_b"]), return_conv_cache=True)
+  assert (y != y2).float().mean().item() < 1e-3
+  assert (y.float() - y2.float()).abs().max().item() <= 0.0625
+  assert helpers.max_rel(h, h2) < 1e-5
+  assert torch.equal(cache, cache2)
+  xc, cc = R.widened_conv1d_forward(x, seg, p["conv_w"], p["conv_b"])
+  yo, ho = R.widened_rglru_forward(xc, seg, p["a_param"], p["w_x"], p["b_x"],
+                                   p["w_a"], p["b_a"], cache=h0)
+  assert helpers.max_rel(y, yo) < BF16_TOL
+  assert helpers.max_rel(h, ho) < BF16_TOL
+  assert torch.equal(cache.cpu(), cc)
+
+
+def test_recurrent_prefill_unsupported_shapes():
+  """fp32 and heads that are not 256 wide are refused with RG_ERR_UNSUPPORTED
+  (callers use the two-kernel form), nothing is launched."""
+  from recurrentgemma_amd import _lib
+  for dtype, W, H in ((torch.float32, 256, 1), (torch.bfloat16, 256, 2)):
+    p = {k: _dev(v) for k, v in R.make_params(W, H, dtype, seed=3).items()}
+    x = _dev(torch.zeros(1, 8, W, dtype=dtype))
+    seg = _dev(torch.arange(8).expand(1, 8).contiguous())
+    assert not ops.recurrent_prefill_supported(x, H)
+    with pytest.raises(_lib.KernelError) as e:
+      ops.recurrent_prefill(x, seg, p["conv_w"], p["conv_b"], p["w_x"],
+                            p["b_x"], p["w_a"], p["b_a"], p["a_param"])
+    assert "unsupported" in str(e.value)
+
+
 # --------------------------------- full-size, size-independent properties --
 
 
@@ -403,7 +467,32 @@ def _full_size_properties(B, T, W, H, seg, seed):
   y, cache = rg.recurrent_core(blk.conv_1d, blk.rg_lru, x, segd)
   torch.cuda.synchronize()
   assert torch.isfinite(y.float()).all()
-  # (1) module-by-module equals fused, bit for bit
+  # (0) recurrent_core may take the single-launch kernel (one workgroup per
+  #     row and head) or the two-kernel form; the two differ only in the fp32
+  #     association of the recurrence: rare 1-ulp bf16 flips in y
+  gx, ga = ops.gates_gemm(x, blk.rg_lru.input_gate.w, blk.rg_lru.input_gate.b,
+                          blk.rg_lru.a_gate.w, blk.rg_lru.a_gate.b,
+                          conv=(segd, blk.conv_1d.w, blk.conv_1d.b))
+  y1, h1, c1 = ops.lru_scan_fused(x, gx, ga, blk.rg_lru.a_param, segd,
+                                  conv=(blk.conv_1d.w, blk.conv_1d.b),
+                                  return_conv_cache=True)
+  assert (y1 != y).float().mean().item() < 1e-3
+  assert (y1.float() - y.float()).abs().max().item() <= 0.0625
+  assert helpers.max_rel(cache.rg_lru_state, h1) < 1e-5
+  assert torch.equal(c1, cache.conv1d_state)
+  if ops.recurrent_prefill_supported(x, H):
+    yf, hf, cf = ops.recurrent_prefill(
+        x, segd, blk.conv_1d.w, blk.conv_1d.b, blk.rg_lru.input_gate.w,
+        blk.rg_lru.input_gate.b, blk.rg_lru.a_gate.w, blk.rg_lru.a_gate.b,
+        blk.rg_lru.a_param)
+    assert (y1 != yf).float().mean().item() < 1e-3
+    assert (y1.float() - yf.float()).abs().max().item() <= 0.0625
+    assert helpers.max_rel(hf, h1) < 1e-5
+    assert torch.equal(cf, c1)
+  y_core, y = y, y1  # the exact statements below are about the two-kernel form
+  cache_core, cache = cache, rg.RecurrentBlockCache(rg_lru_state=h1,
+                                                    conv1d_state=c1)
+  # (1) module-by-module equals the two-kernel form, bit for bit
   xc, cstate = blk.conv_1d(x, segd)
   y2, h2 = blk.rg_lru(xc, segd)
   assert torch.equal(y2, y) and torch.equal(h2, cache.rg_lru_state)
@@ -420,14 +509,8 @@ def _full_size_properties(B, T, W, H, seg, seed):
   assert mism < 1e-3, mism
   # (3) with the gate pre-activations held fixed the path is linear in x:
   #     doubling x doubles y and h exactly (powers of two are exact)
-  gx, ga = ops.gates_gemm(x, blk.rg_lru.input_gate.w, blk.rg_lru.input_gate.b,
-                          blk.rg_lru.a_gate.w, blk.rg_lru.a_gate.b,
-                          conv=(segd, blk.conv_1d.w, blk.conv_1d.b))
-  y1, h1, _ = ops.lru_scan_fused(x, gx, ga, blk.rg_lru.a_param, segd,
-                                 conv=(blk.conv_1d.w, blk.conv_1d.b))
   yd, hd, _ = ops.lru_scan_fused(x * 2, gx, ga, blk.rg_lru.a_param, segd,
                                  conv=(blk.conv_1d.w, blk.conv_1d.b))
-  assert torch.equal(y1, y)
   assert torch.equal(yd.float(), y1.float() * 2) and torch.equal(hd, h1 * 2)
   # (4) at every document start y == conv(x) * sigmoid(gx_pre)
   starts = segd == 0
@@ -447,6 +530,7 @@ def _full_size_properties(B, T, W, H, seg, seed):
   n = 300
   yo, _ = R.widened_recurrent_core(x[:1, :n].cpu(), seg[:1, :n], p)
   assert helpers.max_rel(y[:1, :n], yo) < BF16_TOL
+  assert helpers.max_rel(y_core[:1, :n], yo) < BF16_TOL
 
 
 def test_config2_full_size_properties():
