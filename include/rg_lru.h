@@ -160,6 +160,31 @@ int rg_recurrent_step(const void* x, const void* segpos, int segpos_is_i64,
                       void* y, void* workspace, size_t workspace_bytes, int B,
                       int W, int H, int dtype, void* stream);
 
+/* The same decode step in ONE launch, for bf16 with 256-wide heads (no
+ * counterpart call in the reference: it is RecurrentBlock.forward with a
+ * cache, modules.py:632-643, after a one-time re-layout of the two gate
+ * matrices).  rg_pack_gate_weights writes w_x and w_a ([H,256,256] each, the
+ * reference's BlockDiagonalLinear layout, layers.py:105-112) into `packed`
+ * (rg_packed_gate_weights_bytes(W, H, dtype) bytes, 16-byte aligned) in the
+ * order the MFMA operand registers are filled: head, group of 32 output
+ * channels, 16-row k-step, gate, lane, 8 values.  Pack again whenever the
+ * weights change.  rg_recurrent_step_packed then takes `packed` in place of
+ * w_x / w_a and needs no workspace; all other arguments are as for
+ * rg_recurrent_step (outputs may alias inputs).  Both return
+ * RG_ERR_UNSUPPORTED for other dtypes or head widths (the byte count is 0
+ * then): use rg_recurrent_step. */
+size_t rg_packed_gate_weights_bytes(int W, int H, int dtype);
+int rg_pack_gate_weights(const void* w_x, const void* w_a, void* packed, int W,
+                         int H, int dtype, void* stream);
+int rg_recurrent_step_packed(const void* x, const void* segpos,
+                             int segpos_is_i64, const void* conv_cache_in,
+                             void* conv_cache_out, const void* h_in,
+                             void* h_out, const void* conv_w,
+                             const void* conv_b, const void* w_packed,
+                             const void* b_x, const void* b_a,
+                             const void* a_param, void* y, int B, int W, int H,
+                             int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -352,4 +352,79 @@ int rg_recurrent_step(const void* x, const void* segpos, int segpos_is_i64,
                            dtype, stream);
 }
 
+size_t rg_packed_gate_weights_bytes(int W, int H, int dtype) {
+  if (W <= 0 || H <= 0 || W % H != 0 || dtype != RG_DTYPE_BF16 || W / H != 256)
+    return 0;
+  return (size_t)2 * H * 256 * 256 * 2;
+}
+
+int rg_pack_gate_weights(const void* w_x, const void* w_a, void* packed, int W,
+                         int H, int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(W > 0 && H > 0 && W % H == 0, "%s: W=%d H=%d", __func__, W, H);
+  if (dtype != RG_DTYPE_BF16 || W / H != 256)
+    return fail(RG_ERR_UNSUPPORTED,
+                "%s: needs bf16 and W/H == 256 (dtype=%d W=%d H=%d)", __func__,
+                dtype, W, H);
+  RG_CHECK_PTR(w_x);
+  RG_CHECK_PTR(w_a);
+  RG_CHECK_PTR(packed);
+  RG_REQUIRE(packed != w_x && packed != w_a, "%s: packed must not alias",
+             __func__);
+  return launch_status(__func__, rg::launch_pack_gate_weights(
+                                     w_x, w_a, packed, H, (hipStream_t)stream));
+}
+
+int rg_recurrent_step_packed(const void* x, const void* segpos,
+                             int segpos_is_i64, const void* conv_cache_in,
+                             void* conv_cache_out, const void* h_in,
+                             void* h_out, const void* conv_w,
+                             const void* conv_b, const void* w_packed,
+                             const void* b_x, const void* b_a,
+                             const void* a_param, void* y, int B, int W, int H,
+                             int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(B > 0 && W > 0 && H > 0, "%s: B=%d W=%d H=%d must be positive",
+             __func__, B, W, H);
+  RG_REQUIRE(W % H == 0, "%s: W=%d is not a multiple of H=%d", __func__, W, H);
+  if (dtype != RG_DTYPE_BF16 || W / H != 256)
+    return fail(RG_ERR_UNSUPPORTED,
+                "%s: needs bf16 and W/H == 256 (dtype=%d W=%d H=%d)", __func__,
+                dtype, W, H);
+  RG_CHECK_PTR(x);
+  RG_CHECK_PTR(segpos);
+  RG_CHECK_PTR(conv_cache_in);
+  RG_CHECK_PTR(conv_cache_out);
+  RG_CHECK_PTR(h_in);
+  RG_CHECK_PTR(h_out);
+  RG_CHECK_PTR(conv_w);
+  RG_CHECK_PTR(conv_b);
+  RG_CHECK_PTR(w_packed);
+  RG_CHECK_PTR(b_x);
+  RG_CHECK_PTR(b_a);
+  RG_CHECK_PTR(a_param);
+  RG_CHECK_PTR(y);
+  RG_REQUIRE(y != x, "%s: y must not alias x", __func__);
+  rg::StepArgs a{};
+  a.x = x;
+  a.segpos = segpos;
+  a.seg_kind = segpos_is_i64 ? 1 : 0;
+  a.cache_in = conv_cache_in;
+  a.cache_out = conv_cache_out;
+  a.h_in = (const float*)h_in;
+  a.h_out = (float*)h_out;
+  a.conv_w = conv_w;
+  a.conv_b = conv_b;
+  a.w_packed = w_packed;
+  a.b[0] = b_x;
+  a.b[1] = b_a;
+  a.a_param = a_param;
+  a.y = y;
+  a.B = B;
+  a.W = W;
+  a.H = H;
+  return launch_status(__func__,
+                       rg::launch_block_step_bf16(a, (hipStream_t)stream));
+}
+
 }  // extern "C"

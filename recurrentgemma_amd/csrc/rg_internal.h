@@ -79,6 +79,23 @@ struct FusedArgs {
   int B, T, W, H;
 };
 
+struct StepArgs {
+  const void* x;         // [B, 1, W] bf16
+  const void* segpos;    // [B, 1]
+  int seg_kind;
+  const void* cache_in;  // [B, 3, W] bf16
+  void* cache_out;       // [B, 3, W] bf16 (may alias cache_in)
+  const float* h_in;     // [B, W]
+  float* h_out;          // [B, W] (may alias h_in)
+  const void* conv_w;
+  const void* conv_b;
+  const void* w_packed;  // both gate matrices, see launch_pack_gate_weights
+  const void* b[2];
+  const void* a_param;
+  void* y;               // [B, 1, W]
+  int B, W, H;
+};
+
 // Each returns hipSuccess or the launch error.  dtype: 0 = f32, 1 = bf16.
 hipError_t launch_conv1d_prefill(const ConvArgs& a, int dtype, hipStream_t s);
 hipError_t launch_conv1d_step(const ConvStepArgs& a, int dtype, hipStream_t s);
@@ -86,6 +103,11 @@ hipError_t launch_gemm_generic(const GemmArgs& a, int dtype, hipStream_t s);
 hipError_t launch_gemm_mfma_bf16(const GemmArgs& a, hipStream_t s);
 hipError_t launch_lru_scan(const ScanArgs& a, int dtype, hipStream_t s);
 hipError_t launch_block_fused_bf16(const FusedArgs& a, hipStream_t s);
+hipError_t launch_block_step_bf16(const StepArgs& a, hipStream_t s);
+// bf16 [H,256,256] x 2 -> one buffer of the same total size in MFMA operand
+// order (head, wave, k-step, gate, lane, 8 values).
+hipError_t launch_pack_gate_weights(const void* w_x, const void* w_a,
+                                    void* packed, int H, hipStream_t s);
 
 }  // namespace rg
 #endif  // RG_INTERNAL_H_

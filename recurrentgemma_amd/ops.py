@@ -258,9 +258,39 @@ def _workspace(B, W, dtype, device):
   return ws
 
 
+_packed_weights = {}  # (ptr_x, ver_x, ptr_a, ver_a) -> packed tensor
+
+
+def packed_gate_weights(w_x, w_a):
+  """Both gate matrices in MFMA operand order (rg_pack_gate_weights), cached
+  until either tensor is written to or re-allocated."""
+  key = (w_x.data_ptr(), w_x._version, w_a.data_ptr(), w_a._version)
+  hit = _packed_weights.get(key)
+  if hit is not None:
+    return hit
+  H, bw, _ = w_x.shape
+  W = H * bw
+  nbytes = _lib.lib().rg_packed_gate_weights_bytes(W, H, _dtype_code(w_x))
+  if nbytes == 0:
+    return None
+  packed = torch.empty(nbytes // 2, dtype=w_x.dtype, device=w_x.device)
+  with torch.cuda.device(w_x.device):
+    _lib.check(_lib.lib().rg_pack_gate_weights(
+        _p(_dev(w_x, "w_x")), _p(_dev(w_a, "w_a")), _p(packed), W, H,
+        _dtype_code(w_x), _stream(w_x)))
+  if len(_packed_weights) > 64:
+    _packed_weights.clear()
+  _packed_weights[key] = packed
+  return packed
+
+
 def recurrent_step(x, segment_pos, conv_cache, h, conv_w, conv_b, w_x, b_x, w_a,
                    b_a, a_param, in_place=False):
-  """One decode step of conv -> RG-LRU.  Returns (y, h_new, conv_cache_new)."""
+  """One decode step of conv -> RG-LRU.  Returns (y, h_new, conv_cache_new).
+
+  bf16 with 256-wide heads runs as one launch on re-laid-out gate weights
+  (packed once per weight version); other shapes as conv step + gate GEMM +
+  scan step."""
   B, n_tok, W = x.shape
   assert n_tok == 1
   assert conv_cache.shape == (B, 3, W)
@@ -280,6 +310,19 @@ def recurrent_step(x, segment_pos, conv_cache, h, conv_w, conv_b, w_x, b_x, w_a,
   else:
     cache_out, h_out = torch.empty_like(cache_in), torch.empty_like(h_in)
   y = torch.empty_like(x)
+  packed = None
+  if x.dtype == torch.bfloat16 and W // H == 256 and W % H == 0:
+    packed = packed_gate_weights(w_x, w_a)
+  if packed is not None:
+    cw, cb, wx_, bx_, wa_, ba_, ap_ = args
+    with torch.cuda.device(x.device):
+      _lib.check(_lib.lib().rg_recurrent_step_packed(
+          _p(x), _p(seg), is64, _p(cache_in), _p(cache_out), _p(h_in),
+          _p(h_out), _p(cw), _p(cb), _p(packed), _p(bx_), _p(ba_), _p(ap_),
+          _p(y), B, W, H, _dtype_code(x), _stream(x)))
+    if cache_out.dtype != conv_cache.dtype:
+      cache_out = cache_out.to(conv_cache.dtype)
+    return y, h_out, cache_out
   ws = _workspace(B, W, x.dtype, x.device)
   with torch.cuda.device(x.device):
     _lib.check(_lib.lib().rg_recurrent_step(

@@ -438,6 +438,57 @@ def test_recurrent_prefill_single_launch(B, T, W, H, mean_doc, seg_dtype,
   assert torch.equal(cache.cpu(), cc)
 
 
+@pytest.mark.parametrize("B,W,H,in_place", [(1, 256, 1, False),
+                                              (5, 512, 2, True),
+                                              (33, 256, 1, False),
+                                              (70, 768, 3, True)])
+def test_recurrent_step_single_launch(B, W, H, in_place):
+  """rg_recurrent_step_packed (decode, one launch on re-laid-out gate weights)
+  against rg_recurrent_step (conv step + gate GEMM + scan step, same
+  arithmetic: bit for bit) and the oracle, over three chained steps with a
+  position 0 (state reset) in some rows."""
+  from recurrentgemma_amd import _lib
+  _announce("recurrent_step packed", B, W, H, in_place)
+  seed = 8100 + B
+  p = R.make_params(W, H, torch.bfloat16, seed=seed, gate_bias_std=0.5)
+  P = {k: _dev(v) for k, v in p.items()}
+  g = torch.Generator().manual_seed(seed + 1)
+  h = torch.randn(B, W, generator=g)
+  cc = torch.randn(B, 3, W, generator=g).to(torch.bfloat16)
+  hd, ccd = _dev(h), _dev(cc)          # single-launch chain
+  h3, cc3 = _dev(h), _dev(cc)          # three-launch chain
+  ho, cco = h.clone(), cc.clone()      # oracle chain
+  lib = _lib.lib()
+  for step in range(3):
+    x = torch.randn(B, 1, W, generator=g).to(torch.bfloat16)
+    seg = torch.full((B, 1), 40 + step, dtype=torch.int64)
+    seg[step % B, 0] = 0  # one row starts a document
+    xd, segd = _dev(x), _dev(seg)
+    y, hd, ccd = ops.recurrent_step(xd, segd, ccd, hd, P["conv_w"],
+                                    P["conv_b"], P["w_x"], P["b_x"], P["w_a"],
+                                    P["b_a"], P["a_param"], in_place=in_place)
+    # three-launch form through the C ABI
+    y3 = torch.empty_like(xd)
+    h3n, cc3n = torch.empty_like(h3), torch.empty_like(cc3)
+    ws = torch.empty(lib.rg_recurrent_step_workspace_bytes(B, W, 1),
+                     dtype=torch.uint8, device=DEV)
+    ptr = lambda t: t.data_ptr()
+    _lib.check(lib.rg_recurrent_step(
+        ptr(xd), ptr(segd), 1, ptr(cc3), ptr(cc3n), ptr(h3), ptr(h3n),
+        ptr(P["conv_w"]), ptr(P["conv_b"]), ptr(P["w_x"]), ptr(P["b_x"]),
+        ptr(P["w_a"]), ptr(P["b_a"]), ptr(P["a_param"]), ptr(y3), ptr(ws),
+        ws.numel(), B, W, H, 1, torch.cuda.current_stream().cuda_stream))
+    h3, cc3 = h3n, cc3n
+    assert torch.equal(y, y3) and torch.equal(hd, h3) and torch.equal(ccd, cc3)
+    xc, cco = R.widened_conv1d_forward(x, seg, p["conv_w"], p["conv_b"],
+                                       cache=cco)
+    yo, ho = R.widened_rglru_forward(xc, seg, p["a_param"], p["w_x"], p["b_x"],
+                                     p["w_a"], p["b_a"], cache=ho)
+    assert helpers.max_rel(y, yo) < BF16_TOL
+    assert helpers.max_rel(hd, ho) < BF16_TOL
+    assert torch.equal(ccd.cpu(), cco)
+
+
 def test_recurrent_prefill_unsupported_shapes():
   """fp32 and heads that are not 256 wide are refused with RG_ERR_UNSUPPORTED
   (callers use the two-kernel form), nothing is launched."""
