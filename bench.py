@@ -19,6 +19,8 @@ Workloads (BASELINE.json configs):
               (the configuration the >= 70 % HBM-roofline target is stated on;
               default)
   2b_prefill  B8 T4096 W2560 H10 bf16, documents ~ Geometric(mean 1024)
+  2b_f32      B1 T512 W2560 H10 fp32 (the reference's own CPU-runnable case;
+              21 MB, i.e. cache resident: warm-cache figures)
   9b_decode   B256 W4096 H16 bf16, one token per row and step with the caches
               carried in place (rg_recurrent_step); `roofline` then describes
               the whole step (all its launches) against its algorithmic bytes
@@ -49,6 +51,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 WORKLOADS = {
     "9b_prefill": dict(B=16, T=8192, W=4096, H=16, mean_doc=None, seed=1003),
     "2b_prefill": dict(B=8, T=4096, W=2560, H=10, mean_doc=1024, seed=1002),
+    "2b_f32": dict(B=1, T=512, W=2560, H=10, mean_doc=None, seed=1001,
+                   dtype="f32"),
     "9b_decode": dict(B=256, T=1, W=4096, H=16, mean_doc=None, seed=1004,
                       decode=True),
 }
@@ -104,7 +108,8 @@ def cpu_baseline(torch, R, wl, params, seconds_target=20.0):
   torch.set_num_threads(cores)
   Bs, Ts = min(wl["B"], 4), wl["T"]
   g = torch.Generator().manual_seed(wl["seed"])
-  x = torch.randn(Bs, Ts, wl["W"], generator=g).to(torch.bfloat16)
+  dt = torch.float32 if wl.get("dtype") == "f32" else torch.bfloat16
+  x = torch.randn(Bs, Ts, wl["W"], generator=g).to(dt)
   seg = make_segment_pos(torch, Bs, Ts, wl["mean_doc"], wl["seed"])
   R.recurrent_core(x[:, :64], seg[:, :64], params)  # warm-up
   times = []
@@ -118,7 +123,8 @@ def cpu_baseline(torch, R, wl, params, seconds_target=20.0):
   return {
       "value": Bs * Ts / best, "unit": "tokens/s", "cores": cores,
       "kind": "port",
-      "sample": (f"oracle/torch_ref.recurrent_core, bf16, {Bs}x{Ts} tokens of "
+      "sample": (f"oracle/torch_ref.recurrent_core, "
+                 f"{'f32' if dt == torch.float32 else 'bf16'}, {Bs}x{Ts} tokens of "
                  f"the workload (W={wl['W']}, H={wl['H']}), median of "
                  f"{len(times)} runs, torch threads={torch.get_num_threads()}"),
   }
@@ -231,7 +237,8 @@ def main():
     return
   B, T, W, H = wl["B"], wl["T"], wl["W"], wl["H"]
   dev = torch.device("cuda:0")
-  dtype = torch.bfloat16
+  dtype = torch.float32 if wl.get("dtype") == "f32" else torch.bfloat16
+  esize = 4 if dtype == torch.float32 else 2
 
   params = R.make_params(W, H, dtype, seed=wl["seed"] + 100)
   g = torch.Generator().manual_seed(wl["seed"])
@@ -298,9 +305,9 @@ def main():
 
   tokens = B * T
   seg_bytes = seg.element_size()
-  scan_algo = scan_algorithmic_bytes(B, T, W, 2, seg_bytes, has_h0=False)
+  scan_algo = scan_algorithmic_bytes(B, T, W, esize, seg_bytes, has_h0=False)
   gemm_flops = 1024.0 * W * tokens
-  gemm_bytes = 3 * 2 * B * T * W
+  gemm_bytes = 3 * esize * B * T * W
 
   def split_figures(gemm_ms, scan_ms):
     achieved = scan_algo / (scan_ms * 1e-3) / 1e9
@@ -312,7 +319,9 @@ def main():
             "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, "scan")),
             "algorithmic_bytes": scan_algo, "avg_launch_ms": scan_ms},
         "gate_gemm": {
-            "kernel": "gates_mfma_bf16_kernel", "avg_launch_ms": gemm_ms,
+            "kernel": ("gates_mfma_bf16_kernel" if esize == 2
+                       else "bdl_generic_kernel (fp32 FMA)"),
+            "avg_launch_ms": gemm_ms,
             "tflops": gemm_flops / (gemm_ms * 1e-3) / 1e12,
             "frac_of_bf16_mfma_peak": gemm_flops / (gemm_ms * 1e-3) / 2.5e15,
             "gbs": gemm_bytes / (gemm_ms * 1e-3) / 1e9,
@@ -349,11 +358,12 @@ def main():
       "higher_is_better": True,
       "scaling": "weak",
       "vs_baseline": None,
-      "dtype": "bf16",
+      "dtype": "bf16" if esize == 2 else "f32",
       "data": "synthetic",
       "config": {
           "workload": args.workload, "batch": B, "seq_len": T, "lru_width": W,
-          "heads": H, "activations": "bf16", "state": "f32",
+          "heads": H, "activations": "bf16" if esize == 2 else "f32",
+          "state": "f32",
           "documents": ("one per row" if wl["mean_doc"] is None
                         else f"geometric mean {wl['mean_doc']}"),
           "path": ("rg_recurrent_prefill (single launch)" if path == "single"
