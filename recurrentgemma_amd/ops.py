@@ -258,16 +258,20 @@ def _workspace(B, W, dtype, device):
   return ws
 
 
-_packed_weights = {}  # (ptr_x, ver_x, ptr_a, ver_a) -> packed tensor
+_packed_weights = {}  # (id(w_x), id(w_a)) -> (ref_x, ref_a, stamp, packed)
 
 
 def packed_gate_weights(w_x, w_a):
-  """Both gate matrices in MFMA operand order (rg_pack_gate_weights), cached
-  until either tensor is written to or re-allocated."""
-  key = (w_x.data_ptr(), w_x._version, w_a.data_ptr(), w_a._version)
+  """Both gate matrices in MFMA operand order (rg_pack_gate_weights), cached per
+  pair of tensor objects until either is written to, re-pointed or dies."""
+  import weakref
+  key = (id(w_x), id(w_a))
+  stamp = (w_x.data_ptr(), w_x._version, w_a.data_ptr(), w_a._version)
   hit = _packed_weights.get(key)
   if hit is not None:
-    return hit
+    ref_x, ref_a, old_stamp, packed = hit
+    if ref_x() is w_x and ref_a() is w_a and old_stamp == stamp:
+      return packed
   H, bw, _ = w_x.shape
   W = H * bw
   nbytes = _lib.lib().rg_packed_gate_weights_bytes(W, H, _dtype_code(w_x))
@@ -278,9 +282,10 @@ def packed_gate_weights(w_x, w_a):
     _lib.check(_lib.lib().rg_pack_gate_weights(
         _p(_dev(w_x, "w_x")), _p(_dev(w_a, "w_a")), _p(packed), W, H,
         _dtype_code(w_x), _stream(w_x)))
-  if len(_packed_weights) > 64:
-    _packed_weights.clear()
-  _packed_weights[key] = packed
+  for k in [k for k, v in _packed_weights.items()
+            if v[0]() is None or v[1]() is None]:
+    del _packed_weights[k]  # entries whose tensors are gone
+  _packed_weights[key] = (weakref.ref(w_x), weakref.ref(w_a), stamp, packed)
   return packed
 
 

@@ -401,6 +401,8 @@ def test_recurrent_block_module():
     (2, 65, 256, 1, 16, torch.int64, True),
     (2, 1000, 768, 3, 250, torch.int32, False),
     (1, 130, 256, 1, 3, torch.int64, False),   # documents of a few tokens
+    (130, 70, 256, 1, 20, torch.int64, False),  # more workgroups than CUs/2
+    (2, 100, 256, 1, -7, torch.int32, False),   # left padding: positions < 0
 ])
 def test_recurrent_prefill_single_launch(B, T, W, H, mean_doc, seg_dtype,
                                          with_h0):
@@ -411,8 +413,12 @@ def test_recurrent_prefill_single_launch(B, T, W, H, mean_doc, seg_dtype,
   p = R.make_params(W, H, torch.bfloat16, seed=seed, gate_bias_std=0.5)
   g = torch.Generator().manual_seed(seed + 1)
   x = torch.randn(B, T, W, generator=g).to(torch.bfloat16)
-  seg = (torch.arange(T).expand(B, T).contiguous() if mean_doc is None
-         else helpers.document_positions(B, T, mean_doc, seed=seed))
+  if mean_doc is None:
+    seg = torch.arange(T).expand(B, T).contiguous()
+  elif mean_doc < 0:  # the sampler's left padding: -1 ... then 0, 1, 2, ...
+    seg = (torch.arange(T) + mean_doc).clamp(min=-1).expand(B, T).contiguous()
+  else:
+    seg = helpers.document_positions(B, T, mean_doc, seed=seed)
   h0 = torch.randn(B, W, generator=g) if with_h0 else None
   P = {k: _dev(v) for k, v in p.items()}
   xd, segd = _dev(x), _dev(seg.to(seg_dtype))
