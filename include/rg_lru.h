@@ -135,15 +135,18 @@ int rg_linear_scan(const void* x, const void* a, const void* reset,
  * rg_gates_gemm(apply_conv) followed by rg_lru_scan_fused(apply_conv), but the
  * conv output and the gate pre-activations stay on chip: one persistent
  * workgroup per (b, head) walks the sequence in 64-token tiles (conv -> LDS ->
- * bf16 MFMA -> gates -> in-register recurrence).  Returns RG_ERR_UNSUPPORTED
+ * bf16 MFMA -> gates -> in-register recurrence).  w_packed (nullable) is the
+ * output of rg_pack_gate_weights for the same w_x / w_a (see below): with it
+ * the kernel skips its own re-layout of the weights.  Returns RG_ERR_UNSUPPORTED
  * unless dtype is bf16, W/H == 256 and T*W*2 < 2^31; callers then use the
  * two-call form. */
 int rg_recurrent_prefill(const void* x, const void* segpos, int segpos_is_i64,
                          const void* conv_w, const void* conv_b,
                          const void* w_x, const void* b_x, const void* w_a,
-                         const void* b_a, const void* a_param, const void* h0,
-                         void* y, void* h_last, void* conv_cache_out, int B,
-                         int T, int W, int H, int dtype, void* stream);
+                         const void* b_a, const void* w_packed,
+                         const void* a_param, const void* h0, void* y,
+                         void* h_last, void* conv_cache_out, int B, int T,
+                         int W, int H, int dtype, void* stream);
 
 /* One decode step of the conv -> RG-LRU core, as RecurrentBlock.forward chains
  * them with a cache (recurrentgemma/torch/modules.py:632-643 with

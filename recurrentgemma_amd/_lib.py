@@ -37,8 +37,8 @@ SIGNATURES = {
     "rg_lru_scan_fused": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp,
                                _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "rg_recurrent_prefill": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp,
-                                  _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i,
-                                  _vp]),
+                                  _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i,
+                                  _i, _vp]),
     "rg_linear_scan": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "rg_recurrent_step_workspace_bytes": (_sz, [_i, _i, _i]),
     "rg_packed_gate_weights_bytes": (_sz, [_i, _i, _i]),

@@ -225,9 +225,10 @@ int rg_lru_scan_fused(const void* x, int apply_conv, const void* conv_w,
 int rg_recurrent_prefill(const void* x, const void* segpos, int segpos_is_i64,
                          const void* conv_w, const void* conv_b,
                          const void* w_x, const void* b_x, const void* w_a,
-                         const void* b_a, const void* a_param, const void* h0,
-                         void* y, void* h_last, void* conv_cache_out, int B,
-                         int T, int W, int H, int dtype, void* stream) {
+                         const void* b_a, const void* w_packed,
+                         const void* a_param, const void* h0, void* y,
+                         void* h_last, void* conv_cache_out, int B, int T,
+                         int W, int H, int dtype, void* stream) {
   RG_CHECK_DTYPE(dtype);
   RG_REQUIRE(B > 0 && T > 0 && W > 0 && H > 0,
              "%s: B=%d T=%d W=%d H=%d must be positive", __func__, B, T, W, H);
@@ -242,6 +243,7 @@ int rg_recurrent_prefill(const void* x, const void* segpos, int segpos_is_i64,
   RG_CHECK_PTR(b_a);
   RG_CHECK_PTR(a_param);
   RG_CHECK_PTR(y);
+  RG_CHECK_OPT_PTR(w_packed);
   RG_CHECK_OPT_PTR(h0);
   RG_CHECK_OPT_PTR(h_last);
   RG_CHECK_OPT_PTR(conv_cache_out);
@@ -266,6 +268,7 @@ int rg_recurrent_prefill(const void* x, const void* segpos, int segpos_is_i64,
   a.b[0] = b_x;
   a.w[1] = w_a;
   a.b[1] = b_a;
+  a.w_packed = w_packed;
   a.a_param = a_param;
   a.h0 = (const float*)h0;
   a.y = y;

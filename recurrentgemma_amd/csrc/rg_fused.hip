@@ -92,31 +92,42 @@ __global__ void __launch_bounds__(512) block_fused_bf16_kernel(FusedArgs p) {
 
   // ---- this wave's weights: 32 channels of the head, both gates ----------
   // The weights are [k][n] with n contiguous, the MFMA B operand wants 8
-  // consecutive k per lane: transpose through LDS, 128 k-rows of one gate at
-  // a time (coalesced 16-byte global reads, 2-byte LDS reads).
+  // consecutive k per lane: either the caller supplies them re-laid-out, or
+  // they are transposed through LDS here, 128 k-rows of one gate at a time
+  // (coalesced 16-byte global reads, 2-byte LDS reads).
   const int n0 = wave * 32;
   Frag bfrag[16][2];
+  if (p.w_packed) {
+    // already in operand order (pack_gate_weights_kernel): 32 x 16 bytes
+    const f32x4* src = reinterpret_cast<const f32x4*>(p.w_packed) +
+                       ((int64_t)(h * 8 + wave) * 16 * 2) * 64 + lane;
 #pragma unroll
-  for (int g = 0; g < 2; ++g) {
+    for (int ks = 0; ks < 16; ++ks)
 #pragma unroll
-    for (int kh = 0; kh < 2; ++kh) {
-      const uint16_t* src =
-          (const uint16_t*)p.w[g] + ((int64_t)h * kBW + kh * 128) * kBW;
-      for (int e = tid; e < 128 * 32; e += 512) {
-        const int r = e >> 5, q = e & 31;
-        *reinterpret_cast<f32x4*>(lds + (size_t)r * kLdsStride + q * 8) =
-            *reinterpret_cast<const f32x4*>(src + (size_t)r * kBW + q * 8);
+      for (int g = 0; g < 2; ++g) bfrag[ks][g].q = src[(ks * 2 + g) * 64];
+  } else {
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+#pragma unroll
+      for (int kh = 0; kh < 2; ++kh) {
+        const uint16_t* src =
+            (const uint16_t*)p.w[g] + ((int64_t)h * kBW + kh * 128) * kBW;
+        for (int e = tid; e < 128 * 32; e += 512) {
+          const int r = e >> 5, q = e & 31;
+          *reinterpret_cast<f32x4*>(lds + (size_t)r * kLdsStride + q * 8) =
+              *reinterpret_cast<const f32x4*>(src + (size_t)r * kBW + q * 8);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+          const int n = n0 + (lane & 31);
+          const int kb = ks * 16 + 8 * (lane >> 5);
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            bfrag[kh * 8 + ks][g].u[e] = lds[(size_t)(kb + e) * kLdsStride + n];
+        }
+        __syncthreads();
       }
-      __syncthreads();
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        const int n = n0 + (lane & 31);
-        const int kb = ks * 16 + 8 * (lane >> 5);
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          bfrag[kh * 8 + ks][g].u[e] = lds[(size_t)(kb + e) * kLdsStride + n];
-      }
-      __syncthreads();
     }
   }
   // Per-lane channel (the MFMA result has channel = lane % 32): gate biases,

@@ -70,6 +70,7 @@ struct FusedArgs {
   const void* conv_w;  // [4, W]
   const void* conv_b;  // [W]
   const void* w[2];    // [H, 256, 256]: input gate, a gate
+  const void* w_packed;  // or null: both, see launch_pack_gate_weights
   const void* b[2];    // [H, 256]
   const void* a_param; // [W]
   const float* h0;     // [B, W] or null

@@ -219,10 +219,13 @@ def recurrent_prefill(x, segment_pos, conv_w, conv_b, w_x, b_x, w_a, b_a,
   h_last = (torch.empty((B, W), dtype=torch.float32, device=x.device)
             if return_h else None)
   cache = x.new_empty((B, 3, W)) if return_conv_cache else None
+  cw, cb, wx_, bx_, wa_, ba_, ap_ = args
+  packed = packed_gate_weights(w_x, w_a)  # cached per weight version
   with torch.cuda.device(x.device):
     _lib.check(_lib.lib().rg_recurrent_prefill(
-        _p(x), _p(seg), is64, *[_p(t) for t in args], _p(h0), _p(y),
-        _p(h_last), _p(cache), B, T, W, H, _dtype_code(x), _stream(x)))
+        _p(x), _p(seg), is64, _p(cw), _p(cb), _p(wx_), _p(bx_), _p(wa_),
+        _p(ba_), _p(packed), _p(ap_), _p(h0), _p(y), _p(h_last), _p(cache), B,
+        T, W, H, _dtype_code(x), _stream(x)))
   return y, h_last, cache
 
 
