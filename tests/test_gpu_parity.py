@@ -495,6 +495,46 @@ def test_recurrent_step_single_launch(B, W, H, in_place):
     assert torch.equal(ccd.cpu(), cco)
 
 
+def test_decode_step_under_graph_capture():
+  """The decode step allocates nothing, never synchronises and only uses the
+  stream it is given, so a HIP graph can hold it: capture one in-place step,
+  replay it several times with eager work and synchronisation in between, and
+  compare every replay with the same step run eagerly."""
+  B, W, H = 48, 512, 2
+  p = R.make_params(W, H, torch.bfloat16, seed=91, gate_bias_std=0.5)
+  P = {k: _dev(v) for k, v in p.items()}
+  g = torch.Generator().manual_seed(92)
+  x = _dev(torch.randn(B, 1, W, generator=g).to(torch.bfloat16))
+  seg = _dev(torch.full((B, 1), 17, dtype=torch.int64))
+  h_g = _dev(torch.randn(B, W, generator=g))
+  cc_g = _dev(torch.randn(B, 3, W, generator=g).to(torch.bfloat16))
+  h_e, cc_e = h_g.clone(), cc_g.clone()
+  ops.packed_gate_weights(P["w_x"], P["w_a"])  # packed outside the capture
+
+  def step(h, cc):
+    return ops.recurrent_step(x, seg, cc, h, P["conv_w"], P["conv_b"],
+                              P["w_x"], P["b_x"], P["w_a"], P["b_a"],
+                              P["a_param"], in_place=True)
+
+  side = torch.cuda.Stream()
+  side.wait_stream(torch.cuda.current_stream())
+  with torch.cuda.stream(side):
+    step(h_g.clone(), cc_g.clone())  # warm-up off the capture
+  torch.cuda.current_stream().wait_stream(side)
+  torch.cuda.synchronize()
+  graph = torch.cuda.CUDAGraph()
+  with torch.cuda.graph(graph):
+    y_g, _, _ = step(h_g, cc_g)
+  for i in range(4):
+    x.copy_(torch.randn(B, 1, W, generator=g).to(torch.bfloat16))  # eager work
+    torch.cuda.synchronize()
+    graph.replay()
+    y_e, h_e, cc_e = step(h_e, cc_e)
+    torch.cuda.synchronize()
+    assert torch.equal(y_g, y_e), i
+    assert torch.equal(h_g, h_e) and torch.equal(cc_g, cc_e), i
+
+
 def test_recurrent_prefill_unsupported_shapes():
   """fp32 and heads that are not 256 wide are refused with RG_ERR_UNSUPPORTED
   (callers use the two-kernel form), nothing is launched."""
