@@ -495,6 +495,29 @@ def test_recurrent_step_single_launch(B, W, H, in_place):
     assert torch.equal(ccd.cpu(), cco)
 
 
+def test_recurrent_core_picks_single_launch():
+  """With enough (row, head) pairs recurrent_core runs prefill as one launch
+  and decode as one launch; both against the oracle, chained."""
+  from recurrentgemma_amd import modules
+  B, T, W, H = 70, 90, 512, 2
+  assert B * H >= modules._MIN_GROUPS_FOR_SINGLE_LAUNCH
+  p, x, blk, (y, cache), (yo, co) = _core_case(
+      torch.bfloat16, B, T, W, H, helpers.document_positions(B, T, 30, seed=5),
+      seed=77)
+  assert helpers.max_rel(y, yo) < BF16_TOL
+  assert helpers.max_rel(cache.rg_lru_state, co.rg_lru_state) < BF16_TOL
+  assert torch.equal(cache.conv1d_state.cpu(), co.conv1d_state)
+  g = torch.Generator().manual_seed(78)
+  x1 = torch.randn(B, 1, W, generator=g).to(torch.bfloat16)
+  pos = torch.full((B, 1), T, dtype=torch.int64)
+  y1, cache1 = rg.recurrent_core(blk.conv_1d, blk.rg_lru, _dev(x1), _dev(pos),
+                                 cache)
+  yo1, co1 = R.widened_recurrent_core(x1, pos, p, co)
+  assert helpers.max_rel(y1, yo1) < BF16_TOL
+  assert helpers.max_rel(cache1.rg_lru_state, co1.rg_lru_state) < BF16_TOL
+  assert torch.equal(cache1.conv1d_state.cpu(), co1.conv1d_state)
+
+
 def test_decode_step_under_graph_capture():
   """The decode step allocates nothing, never synchronises and only uses the
   stream it is given, so a HIP graph can hold it: capture one in-place step,
