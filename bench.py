@@ -281,7 +281,7 @@ def main():
 
   path = args.path
   if path == "auto":
-    path = ("single" if ops.recurrent_prefill_supported(x, H) and B * H >= 128
+    path = ("single" if ops.recurrent_prefill_supported(x, H) and B * H >= 144
             else "split")
   step = step_single if path == "single" else step_split
 

@@ -30,9 +30,12 @@ def gelu(x: torch.Tensor) -> torch.Tensor:
   return nn.functional.gelu(x, approximate="tanh")
 
 
-# rg_recurrent_prefill runs one workgroup per (sequence row, head); with fewer
-# groups than this most of the 256 CUs would idle.
-_MIN_GROUPS_FOR_SINGLE_LAUNCH = 128
+# rg_recurrent_prefill runs one workgroup per (sequence row, head), so its time
+# does not shrink below 256 groups, while the two-kernel form scales with the
+# number of tokens.  Measured on MI355X (T = 1024 and 4096, 256-wide heads) the
+# two cross between 128 groups (two kernels 5 % ahead) and 160 (single launch
+# 25 % ahead).
+_MIN_GROUPS_FOR_SINGLE_LAUNCH = 144
 
 
 @torch.no_grad()

@@ -499,7 +499,7 @@ def test_recurrent_core_picks_single_launch():
   """With enough (row, head) pairs recurrent_core runs prefill as one launch
   and decode as one launch; both against the oracle, chained."""
   from recurrentgemma_amd import modules
-  B, T, W, H = 70, 90, 512, 2
+  B, T, W, H = 75, 90, 512, 2
   assert B * H >= modules._MIN_GROUPS_FOR_SINGLE_LAUNCH
   p, x, blk, (y, cache), (yo, co) = _core_case(
       torch.bfloat16, B, T, W, H, helpers.document_positions(B, T, 30, seed=5),
