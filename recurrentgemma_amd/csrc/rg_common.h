@@ -196,6 +196,20 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base,
 }
 constexpr uint32_t kBufferOutOfRange = 0x80000000u;
 
+// 16-byte buffer store at byte offset lane_off + uniform_off.  The whole offset
+// goes into the vector offset and the scalar offset stays the constant 0: for
+// a store of more than 8 bytes whose scalar offset is a register the compiler
+// does not keep the next vector instruction from overwriting the data
+// registers, and on gfx950 such an overwrite right after the store was seen to
+// reach memory (third dword of the 16 bytes, last lanes of each 16).  With a
+// constant scalar offset the compiler spaces the two instructions itself.
+__device__ __forceinline__ void buffer_store_16(u32x4 v,
+                                                __amdgpu_buffer_rsrc_t r,
+                                                uint32_t lane_off,
+                                                uint32_t uniform_off) {
+  __builtin_amdgcn_raw_buffer_store_b128(v, r, lane_off + uniform_off, 0, 0);
+}
+
 // ---------------------------------------------------------- barriers ----
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits
 // for every outstanding global load and store of the wave (its fence covers

@@ -427,8 +427,8 @@ __global__ void __launch_bounds__(512) block_fused_bf16_kernel(FusedArgs p) {
       for (int q = 0; q < 2; ++q) {
         const u32x4 v =
             *reinterpret_cast<const u32x4*>(patch_r + q * 16 * kPatchStride);
-        __builtin_amdgcn_raw_buffer_store_b128(
-            v, ry, y_lane_bytes, (uint32_t)(t_half + 16 * q) * row_bytes, 0);
+        buffer_store_16(v, ry, y_lane_bytes,
+                        (uint32_t)(t_half + 16 * q) * row_bytes);
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");

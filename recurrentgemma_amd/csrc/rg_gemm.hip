@@ -416,8 +416,8 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
     };
     // rows past the end of the output fall outside the descriptor
     auto patch_store = [&](int mt, int q, u32x4 v) {
-      __builtin_amdgcn_raw_buffer_store_b128(
-          v, ro, out_lane_bytes, (uint32_t)(mt * 32 + q * 8) * out_row_bytes, 0);
+      buffer_store_16(v, ro, out_lane_bytes,
+                      (uint32_t)(mt * 32 + q * 8) * out_row_bytes);
     };
     auto a_read = [&](int mt, int ks) {
       Frag a;
