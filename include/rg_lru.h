@@ -163,6 +163,16 @@ int rg_recurrent_step(const void* x, const void* segpos, int segpos_is_i64,
                       void* y, void* workspace, size_t workspace_bytes, int B,
                       int W, int H, int dtype, void* stream);
 
+/* The join of RecurrentBlock.forward's two branches in one pass:
+ * out = a * gelu(g) with the tanh approximation, for recurrentgemma/torch/
+ * modules.py:627-628 (`y = gelu(linear_y(x))`, gelu at :289-291) and :644
+ * (`x = x * y`): `a` is the RG-LRU output, `g` the linear_y output, n elements
+ * each in `dtype`.  bf16: gelu evaluated in float32 and rounded to bf16 (it is
+ * a tensor of its own in the reference), then the product rounded once.  out
+ * may alias a or g. */
+int rg_gelu_mul(const void* a, const void* g, void* out, int64_t n, int dtype,
+                void* stream);
+
 /* The same decode step in ONE launch, for bf16 with 256-wide heads (no
  * counterpart call in the reference: it is RecurrentBlock.forward with a
  * cache, modules.py:632-643, after a one-time re-layout of the two gate

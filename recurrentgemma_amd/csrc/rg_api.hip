@@ -355,6 +355,19 @@ int rg_recurrent_step(const void* x, const void* segpos, int segpos_is_i64,
                            dtype, stream);
 }
 
+int rg_gelu_mul(const void* a, const void* g, void* out, int64_t n, int dtype,
+                void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(n > 0, "%s: n=%lld must be positive", __func__, (long long)n);
+  RG_CHECK_PTR(a);
+  RG_CHECK_PTR(g);
+  RG_CHECK_PTR(out);
+  RG_REQUIRE((((uintptr_t)a | (uintptr_t)g | (uintptr_t)out) & 15) == 0,
+             "%s: a, g and out must be 16-byte aligned", __func__);
+  return launch_status(
+      __func__, rg::launch_gelu_mul(a, g, out, n, dtype, (hipStream_t)stream));
+}
+
 size_t rg_packed_gate_weights_bytes(int W, int H, int dtype) {
   if (W <= 0 || H <= 0 || W % H != 0 || dtype != RG_DTYPE_BF16 || W / H != 256)
     return 0;

@@ -107,6 +107,9 @@ hipError_t launch_block_fused_bf16(const FusedArgs& a, hipStream_t s);
 hipError_t launch_block_step_bf16(const StepArgs& a, hipStream_t s);
 // bf16 [H,256,256] x 2 -> one buffer of the same total size in MFMA operand
 // order (head, wave, k-step, gate, lane, 8 values).
+// out[i] = a[i] * gelu_tanh(g[i]) over n elements (out may alias a or g).
+hipError_t launch_gelu_mul(const void* a, const void* g, void* out, int64_t n,
+                           int dtype, hipStream_t s);
 hipError_t launch_pack_gate_weights(const void* w_x, const void* w_a,
                                     void* packed, int H, hipStream_t s);
 

@@ -129,11 +129,11 @@ class RecurrentBlock(nn.Module):
 
   @torch.no_grad()
   def forward(self, x, segment_pos, cache=None, return_cache=True):
-    y = gelu(self.linear_y(x))
+    y = self.linear_y(x)
     x = self.linear_x(x)
     x, new_cache = recurrent_core(self.conv_1d, self.rg_lru, x, segment_pos,
                                   cache, return_cache)
-    x = x * y
+    x = ops.gelu_mul(x, y)  # x * gelu(y), one pass (modules.py:627-628, 644)
     x = self.linear_out(x)
     if not return_cache:
       return x, None

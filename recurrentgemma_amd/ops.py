@@ -261,6 +261,19 @@ def _workspace(B, W, dtype, device):
   return ws
 
 
+def gelu_mul(a, g):
+  """a * gelu_tanh(g) in one pass (the x * y join of RecurrentBlock.forward)."""
+  assert a.shape == g.shape
+  a = _dev(a, "a")
+  _same(a.dtype, a.device, g=g)
+  g = _dev(g, "g")
+  out = torch.empty_like(a)
+  with torch.cuda.device(a.device):
+    _lib.check(_lib.lib().rg_gelu_mul(_p(a), _p(g), _p(out), a.numel(),
+                                      _dtype_code(a), _stream(a)))
+  return out
+
+
 _packed_weights = {}  # (id(w_x), id(w_a)) -> (ref_x, ref_a, stamp, packed)
 
 

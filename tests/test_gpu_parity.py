@@ -598,6 +598,50 @@ def test_recurrent_prefill_unsupported_shapes():
     assert "unsupported" in str(e.value)
 
 
+# ------------------------------------------- the x * gelu(y) join, 1 pass --
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n", [1, 7, 8, 2055, 3 * 100 * 256, 8 * 1024 * 1024 + 3])
+def test_gelu_mul(dtype, n):
+  """rg_gelu_mul against torch's own two passes (gelu(approximate="tanh")
+  evaluated in float32 on the CPU, rounded to the activation dtype as the
+  reference's tensor `y` is, then the product): fp32 within 1e-5 of the
+  largest magnitude; bf16 within one bf16 ulp of each element (the fast
+  sigmoid may land a gelu value on the neighbouring bf16) plus 1e-6 |a|: in
+  the negative tail 1 + tanh(u) is a multiple of 2^-24, and two float32 tanh
+  that differ in the last place differ there by 0.5 |g| 2^-24 in gelu."""
+  _announce("gelu_mul", dtype, n)
+  gen = torch.Generator().manual_seed(n)
+  a = torch.randn(n, generator=gen).to(dtype)
+  g = (3.0 * torch.randn(n, generator=gen)).to(dtype)
+  if n >= 7:
+    g[:7] = torch.tensor([0.0, -0.0, 20.0, -20.0, 1e-3, -9.0, 9.0]).to(dtype)
+  y = torch.nn.functional.gelu(g.float(), approximate="tanh").to(dtype)
+  want = (a.float() * y.float()).to(dtype)
+  got = ops.gelu_mul(_dev(a), _dev(g)).cpu()
+  assert got.dtype == dtype and got.shape == a.shape
+  assert torch.isfinite(got.float()).all()
+  if dtype == torch.float32:
+    assert helpers.max_rel(got, want) < 1e-5
+  else:
+    err = (got.float() - want.float()).abs()
+    ulp = want.float().abs() * 2.0 ** -7 + 1e-6 * a.float().abs()
+    assert (err <= ulp).all(), float((err / ulp).max())
+    assert (err > 0).float().mean() < 0.02  # neighbouring-bf16 cases are rare
+  # in place on either operand
+  a_d, g_d = _dev(a), _dev(g)
+  from recurrentgemma_amd import _lib
+  code = 0 if dtype == torch.float32 else 1
+  a_io, g_io = a_d.clone(), g_d.clone()
+  for src_a, src_g, dst in ((a_io, g_d, a_io), (a_d, g_io, g_io)):
+    _lib.check(_lib.lib().rg_gelu_mul(src_a.data_ptr(), src_g.data_ptr(),
+                                      dst.data_ptr(), n, code,
+                                      torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert torch.equal(dst.cpu(), got)
+
+
 # --------------------------------- full-size, size-independent properties --
 
 
