@@ -19,13 +19,12 @@ namespace {
 constexpr int kBW = 256;           // head width (K and per-gate N)
 constexpr int kTM = 64;            // tokens per tile
 constexpr int kLdsStride = 264;    // bf16 elements per staged row (256 + 8 pad)
-constexpr int kRowsPerGroup = 16;  // rows each thread converts per tile
+constexpr int kRowsPerGroup = 32;  // rows each staging thread converts per tile
 constexpr int kHalo = 3;
 constexpr int kRaw = kRowsPerGroup + kHalo;
-// Three staged tiles: the one the MFMAs read, the one being written for the
-// next tile, and the previous one, which half of the waves still read while
-// they finish its gate arithmetic (see the tile loop).
-constexpr int kStageBufs = 3;
+// Two staged tiles: the one the matrix instructions and the gate arithmetic
+// read, and the one being written for the next tile (one barrier per tile).
+constexpr int kStageBufs = 2;
 constexpr size_t kStageLdsBytes =
     (size_t)kStageBufs * kTM * kLdsStride * sizeof(uint16_t);
 // Per-wave output patch: 32 tokens x 32 channels in bf16, rows padded to 80
@@ -46,15 +45,6 @@ union Frag {
   uint16_t u[8];
   f32x4 q;
 };
-
-// Build switch for the tile loop: 1 runs waves 4-7 one phase behind waves 0-3
-// (matrix phases of one group over vector phases of the other).  Measured at
-// B16 T8192 W4096 it is about 3 % slower than keeping all waves in the same
-// phase (the vector ALU, not the matrix pipe, bounds the tile), so it is off.
-#ifndef RG_FUSED_SKEW
-#define RG_FUSED_SKEW 0
-#endif
-constexpr bool kSkewGroups = RG_FUSED_SKEW != 0;
 
 using WithCuts = std::integral_constant<bool, true>;
 using NoCuts = std::integral_constant<bool, false>;
@@ -161,9 +151,14 @@ __global__ void __launch_bounds__(512) block_fused_bf16_kernel(FusedArgs p) {
       make_rsrc((const char*)p.segpos + (int64_t)b * T_len * seg_esize,
                 (uint32_t)T_len * seg_esize);
 
-  // x staging: thread -> (channel pair, group of 16 tokens)
+  // x staging: waves 0-3 only, thread -> (channel pair, 32 tokens of the
+  // tile).  The issue arbiter of a SIMD serves its older wave first, so waves
+  // 4-7 (the younger wave of each SIMD) progress at about two thirds of the
+  // rate of waves 0-3 while both run; leaving the conv to waves 0-3 evens out
+  // the time the two groups need per tile.
+  const bool stager = wave < 4;
   const int cp = tid & 127;
-  const int rg = __builtin_amdgcn_readfirstlane(tid >> 7);
+  const int rg = __builtin_amdgcn_readfirstlane((tid >> 7) & 1);
   const uint32_t c = h * kBW + cp * 2;
   const uint32_t c_bytes = 2u * c;
   float cw0[2], cw1[2], cw2[2], cw3[2], cb[2];
@@ -229,26 +224,38 @@ __global__ void __launch_bounds__(512) block_fused_bf16_kernel(FusedArgs p) {
         (t < 0 || tile >= ntiles) ? kBufferOutOfRange : (uint32_t)t * row_bytes;
     raw[j] = __builtin_amdgcn_raw_buffer_load_b32(rx, cb_off, soff, 0);
   };
+  // The same for a tile >= 1 (no row before the sequence): one scalar add per
+  // row.  A tile past the end keeps every row out of range (the marker plus a
+  // few rows stays above any sequence size).
+  auto row_base = [&](int tile) -> uint32_t {
+    return tile < ntiles ? (uint32_t)(tile * kTM + rg * kRowsPerGroup - kHalo) *
+                               row_bytes
+                         : kBufferOutOfRange;
+  };
+  auto fetch_row_at = [&](uint32_t base, int j, uint32_t cb_off) {
+    raw[j] = __builtin_amdgcn_raw_buffer_load_b32(
+        rx, cb_off, base + (uint32_t)j * row_bytes, 0);
+  };
   auto chan_bytes = [&](int t) {  // byte offset of thread t's channel pair
     return 2u * (uint32_t)(h * kBW + (t & 127) * 2);
   };
 
 
   // Conv of one tile, one row at a time.  cut bit j: token j of this thread
-  // group's 19 rows starts a document; the conv must not look past it.
-  uint32_t cut = 0;
+  // group's 35 rows starts a document; the conv must not look past it.
+  uint64_t cut = 0;
   float h0v[2], h1v[2], h2v[2];
   auto stage_dst = [&](int t, int buf) {
     return lds + (size_t)buf * kTM * kLdsStride +
            (size_t)(rg * kRowsPerGroup) * kLdsStride + (t & 127) * 2;
   };
   auto stage_begin = [&](int t, uint64_t m_tile, uint64_t m_before) {
-    // rows 16*rg-3 .. 16*rg+15 of the tile; the three rows before the tile
+    // rows 32*rg-3 .. 32*rg+31 of the tile; the three rows before the tile
     // are the last three of the previous one
     if (rg == 0)
-      cut = ((uint32_t)(m_tile << 3) | (uint32_t)(m_before >> 61)) & 0x7ffffu;
+      cut = ((m_tile << 3) | (m_before >> 61)) & ((1ull << kRaw) - 1);
     else
-      cut = (uint32_t)(m_tile >> (16 * rg - 3)) & 0x7ffffu;
+      cut = m_tile >> (kRowsPerGroup - kHalo);
     h0v[0] = h0v[1] = h1v[0] = h1v[1] = h2v[0] = h2v[1] = 0.0f;
     load_conv_consts(t);
   };
@@ -257,7 +264,7 @@ __global__ void __launch_bounds__(512) block_fused_bf16_kernel(FusedArgs p) {
     float xv[2];
     xv[0] = __uint_as_float(raw[j] << 16);
     xv[1] = __uint_as_float(raw[j] & 0xffff0000u);
-    if (CUTS && ((cut >> j) & 1u)) {
+    if (CUTS && ((cut >> j) & 1ull)) {
       h0v[0] = h0v[1] = h1v[0] = h1v[1] = h2v[0] = h2v[1] = 0.0f;
     }
     if (j >= kHalo) {
@@ -286,169 +293,210 @@ __global__ void __launch_bounds__(512) block_fused_bf16_kernel(FusedArgs p) {
   uint64_t m_cur = 0;
   {
     fetch_seg(0);
+    if (stager) {
 #pragma unroll
-    for (int j = 0; j < kRaw; ++j) fetch_row(0, j, c_bytes);
+      for (int j = 0; j < kRaw; ++j) fetch_row(0, j, c_bytes);
+    }
     m_cur = start_mask(0);
-    stage_begin(tid, m_cur, 0);
+    if (stager) {
+      stage_begin(tid, m_cur, 0);
 #pragma unroll
-    for (int j = 0; j < kRaw; ++j) stage_row(j, stage_dst(tid, 0), WithCuts{});
+      for (int j = 0; j < kRaw; ++j) stage_row(j, stage_dst(tid, 0), WithCuts{});
+    }
     fetch_seg(1);
+    if (stager) {
 #pragma unroll
-    for (int j = 0; j < kRaw; ++j) fetch_row(1, j, c_bytes);
+      for (int j = 0; j < kRaw; ++j) fetch_row(1, j, c_bytes);
+    }
   }
   lds_barrier();
 
-  // Gate arithmetic + recurrence of one 32-token half of a tile.  On entry
-  // acc_x / acc_a hold the gate pre-activations (bias included) of tokens
-  // i = 8*(r/4) + 4*(lane/32) + r%4 for channel lane%32.  `general` also
-  // handles document starts (a = 0, unit input scale) and tokens past the end
-  // of the sequence (identity: a = 1, no input).
-  auto half_epilogue = [&](int it, int mt, int buf, f32x16& acc_x, f32x16& acc_a,
-                           uint64_t m_tile) {
+  // Gate pre-activations of one 32-token half of a tile (bias included),
+  // rounded to bf16 -- they are a bf16 module output in the reference -- and
+  // kept packed: word i holds accumulator registers 2i and 2i+1, i.e. tokens
+  // 8*(i/2) + 4*(lane/32) + 2*(i%2) + {0,1} of channel lane%32.
+  struct Packed {
+    uint32_t x[8], a[8];
+  };
+  auto pack_acc = [&](const f32x16& acc_x, const f32x16& acc_a, Packed& pk) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      pk.x[i] = pack_bf16x2(acc_x[2 * i], acc_x[2 * i + 1]);
+      pk.a[i] = pack_bf16x2(acc_a[2 * i], acc_a[2 * i + 1]);
+    }
+  };
+
+  // Gate arithmetic + recurrence of one 32-token half of a tile, one run of
+  // four tokens at a time.  In time order the runs alternate between the lane
+  // halves: L0 U0 L1 U1 L2 U2 L3 U3 (run g of lanes 0-31 holds tokens
+  // 8g..8g+3, of lanes 32-63 tokens 8g+4..8g+7).  Per run the pair (P, Hh):
+  // h_out = P h_in + Hh; both halves' pairs are made visible to all lanes,
+  // every lane follows the chain, replays its own run from its h_in and writes
+  // it to the wave's patch.  `general` also handles document starts (a = 0,
+  // unit input scale) and tokens past the end of the sequence (identity:
+  // a = 1, no input).
+  // The work of a run is cut into eight chunks, and hook(8g + c) runs after
+  // chunk c of run g, pinned there: the caller passes the matrix instructions
+  // of the next half tile (32 of them) so that they issue from this wave's own
+  // instruction stream, evenly spread under the vector work.
+  auto half_epilogue = [&](int it, int mt, int buf, const Packed& pk,
+                           uint64_t m_tile, auto&& hook) {
     const bool general = m_tile != 0 || (it + 1) * kTM > T_len;
     int l1 = lane;
-    asm volatile("" : "+v"(l1));  // address recomputed per call, not kept
+    asm volatile("" : "+v"(l1));  // addresses recomputed per call, not kept
     const uint16_t* xcp = lds + (size_t)buf * kTM * kLdsStride +
                           (size_t)(mt * 32 + 4 * (l1 >> 5)) * kLdsStride + n0 +
                           (l1 & 31);
+    unsigned char* const patch_w =
+        patch + 4 * (l1 >> 5) * kPatchStride + 2 * (l1 & 31);
+    // read side of the patch: lane l takes the 16-byte chunk l%4 of tokens
+    // l/4 and l/4+16
+    const unsigned char* patch_r =
+        patch + (l1 >> 2) * kPatchStride + 16 * (l1 & 3);
+    const uint32_t y_lane_bytes = (uint32_t)(l1 >> 2) * row_bytes +
+                                  2u * (h * kBW + n0) + 16u * (l1 & 3);
     const int t_half = it * kTM + mt * 32;  // first token of this half
     const float decay = chan_ptr(l1)[2];
-    // `general` (wave-uniform, rare): bit r of these words says that token r
-    // of a lane starts a document / lies inside the sequence.
-    // kept as wave-uniform words, one pair per lane half
-    uint32_t s_lo = 0, s_hi = 0, v_lo = 0xffffu, v_hi = 0xffffu;
-    if (general) {
-      v_lo = v_hi = 0;
+    // End of a chunk: its memory operations stay on this side, then the hook,
+    // fenced for the instruction scheduler.  The values a chunk produces are
+    // pinned by keep4() before this is called (pure arithmetic would otherwise
+    // drift to its first use).
+    auto pinned = [&](int i) {
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+      hook(i);
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("" ::: "memory");
+    };
+    auto keep4 = [](float (&v)[4]) {
+      asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]));
+    };
+    float c_run = hc;
+    uint16_t xraw[4];
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int row = mt * 32 + 8 * g;  // lanes 0-31: row..row+3, 32-63: +4
-        s_lo |= ((uint32_t)(m_tile >> row) & 0xfu) << (4 * g);
-        s_hi |= ((uint32_t)(m_tile >> (row + 4)) & 0xfu) << (4 * g);
+    for (int q = 0; q < 4; ++q) xraw[q] = xcp[(size_t)q * kLdsStride];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          v_lo |= (uint32_t)(t_half + 8 * g + q < T_len) << (4 * g + q);
-          v_hi |= (uint32_t)(t_half + 8 * g + 4 + q < T_len) << (4 * g + q);
-        }
-      }
-    }
-    // Pass 1 (straight-line): a = exp2(sigmoid(pa) * decay) -> acc_a,
-    // xc * sigmoid(px) -> acc_x.
-#pragma unroll
-    for (int r = 0; r < 16; r += 2) {
-      // pre-activations are a bf16 module output in the reference
-      const uint32_t px2 = pack_bf16x2(acc_x[r], acc_x[r + 1]);
-      const uint32_t pa2 = pack_bf16x2(acc_a[r], acc_a[r + 1]);
+    for (int g = 0; g < 4; ++g) {
+      // chunk 0: unpack
+      float px[4], pa[4], xc[4];
 #pragma unroll
       for (int e = 0; e < 2; ++e) {
-        const int rr = r + e;
-        const int i = 8 * (rr >> 2) + (rr & 3);
-        const float xc = bf16_bits_to_f32(xcp[(size_t)i * kLdsStride]);
-        const float px = e == 0 ? __uint_as_float(px2 << 16)
-                                : __uint_as_float(px2 & 0xffff0000u);
-        const float pa = e == 0 ? __uint_as_float(pa2 << 16)
-                                : __uint_as_float(pa2 & 0xffff0000u);
-        const float gate_x = sigmoid_fast(px);
-        const float gate_a = sigmoid_fast(pa);
-        acc_a[rr] = __builtin_amdgcn_exp2f(gate_a * decay);
-        acc_x[rr] = xc * gate_x;
+        px[2 * e] = __uint_as_float(pk.x[2 * g + e] << 16);
+        px[2 * e + 1] = __uint_as_float(pk.x[2 * g + e] & 0xffff0000u);
+        pa[2 * e] = __uint_as_float(pk.a[2 * g + e] << 16);
+        pa[2 * e + 1] = __uint_as_float(pk.a[2 * g + e] & 0xffff0000u);
       }
-      // eight tokens at a time: enough independent work to cover the latency
-      // of the transcendental chains, few enough temporaries to stay in
-      // registers
-      if ((r & 6) == 6) __builtin_amdgcn_sched_barrier(0);
-    }
-    // Document start: a = 0; past the end of the sequence: a = 1.  The input
-    // scale sqrt(1 - a^2) of pass 2 then comes out as 1 and 0 by itself.
-    if (general) {
 #pragma unroll
-      for (int rr = 0; rr < 16; ++rr) {
-        const bool start = upper ? (s_hi >> rr) & 1u : (s_lo >> rr) & 1u;
-        const bool valid = upper ? (v_hi >> rr) & 1u : (v_lo >> rr) & 1u;
-        acc_a[rr] = start ? 0.0f : acc_a[rr];
-        acc_a[rr] = valid ? acc_a[rr] : 1.0f;
+      for (int q = 0; q < 4; ++q) xc[q] = bf16_bits_to_f32(xraw[q]);
+      keep4(px);
+      keep4(pa);
+      keep4(xc);
+      pinned(8 * g + 0);
+      // chunks 1, 2: the two sigmoids, eight independent chains
+      float ex[4], ea[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        ex[q] = __builtin_amdgcn_exp2f(-kLog2e * px[q]);
+        ea[q] = __builtin_amdgcn_exp2f(-kLog2e * pa[q]);
       }
-    }
-    // Pass 2: xn = (xc * gate_x) * sqrt(1 - a^2)
+      keep4(ex);
+      keep4(ea);
+      pinned(8 * g + 1);
+      float av[4], xn[4];
 #pragma unroll
-    for (int rr = 0; rr < 16; ++rr)
-      acc_x[rr] = acc_x[rr] * __builtin_amdgcn_sqrtf(__builtin_fmaf(
-                                  -acc_a[rr], acc_a[rr], 1.0f));
-    __builtin_amdgcn_sched_barrier(0);
-    // Recurrence.  In time order the runs of four tokens alternate between
-    // the lane halves: L0 U0 L1 U1 L2 U2 L3 U3 (run g of lanes 0-31 holds
-    // tokens 8g..8g+3, of lanes 32-63 tokens 8g+4..8g+7).  Per run the pair
-    // (P, Hh): h_out = P h_in + Hh; both halves' pairs are made visible to all
-    // lanes, every lane follows the chain and keeps the h_in of its own runs.
-    // The run is replayed from its h_in and written to the patch as soon as
-    // its h_in is known.
-    {
-      // lane-derived address, recomputed here rather than kept in a register
-      int l2 = lane;
-      asm volatile("" : "+v"(l2));
-      unsigned char* const patch_w =
-          patch + 4 * (l2 >> 5) * kPatchStride + 2 * (l2 & 31);
-      float c_run = hc;
+      for (int q = 0; q < 4; ++q) {
+        ex[q] = __builtin_amdgcn_rcpf(1.0f + ex[q]);
+        ea[q] = __builtin_amdgcn_rcpf(1.0f + ea[q]);
+      }
+      keep4(ex);
+      keep4(ea);
+      pinned(8 * g + 2);
+      // chunk 3: a = exp2(sigmoid(pa) * decay), xc * sigmoid(px); the conv
+      // outputs of the next run are requested here
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        float P = acc_a[4 * g], Hh = acc_x[4 * g];
+      for (int q = 0; q < 4; ++q) {
+        av[q] = __builtin_amdgcn_exp2f(ea[q] * decay);
+        xn[q] = xc[q] * ex[q];
+      }
+      keep4(av);
+      keep4(xn);
+      if (g < 3) {
 #pragma unroll
-        for (int q = 1; q < 4; ++q) {
-          Hh = __builtin_fmaf(acc_a[4 * g + q], Hh, acc_x[4 * g + q]);
-          P = P * acc_a[4 * g + q];
-        }
-        float PL, PU, HL, HU;
-        halves(P, PL, PU);
-        halves(Hh, HL, HU);
-        const float after_lower = __builtin_fmaf(PL, c_run, HL);
-        float hh = upper ? after_lower : c_run;
-        c_run = __builtin_fmaf(PU, after_lower, HU);
+        for (int q = 0; q < 4; ++q)
+          xraw[q] = xcp[(size_t)(8 * (g + 1) + q) * kLdsStride];
+      }
+      pinned(8 * g + 3);
+      // chunk 4: document start: a = 0; past the end of the sequence: a = 1.
+      // The input scale sqrt(1 - a^2) then comes out as 1 and 0 by itself.
+      if (general) {
+        const int row = mt * 32 + 8 * g + (upper ? 4 : 0);
+        const uint32_t starts = (uint32_t)(m_tile >> row) & 0xfu;
+        const int t_run = t_half + 8 * g + (upper ? 4 : 0);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          hh = __builtin_fmaf(acc_a[4 * g + q], hh, acc_x[4 * g + q]);
-          *reinterpret_cast<uint16_t*>(patch_w + (8 * g + q) * kPatchStride) =
-              f32_to_bf16_bits(hh);
+          av[q] = ((starts >> q) & 1u) ? 0.0f : av[q];
+          av[q] = (t_run + q < T_len) ? av[q] : 1.0f;
         }
-        __builtin_amdgcn_sched_barrier(0);
       }
-      hc = c_run;
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    // tokens past the end of the sequence fall outside the descriptor
-    {
-      int l2 = lane;
-      asm volatile("" : "+v"(l2));
-      // read side: lane l takes the 16-byte chunk l%4 of tokens l/4, l/4+16
-      const unsigned char* patch_r =
-          patch + (l2 >> 2) * kPatchStride + 16 * (l2 & 3);
-      const uint32_t y_lane_bytes = (uint32_t)(l2 >> 2) * row_bytes +
-                                    2u * (h * kBW + n0) + 16u * (l2 & 3);
 #pragma unroll
-      for (int q = 0; q < 2; ++q) {
-        const u32x4 v =
-            *reinterpret_cast<const u32x4*>(patch_r + q * 16 * kPatchStride);
-        buffer_store_16(v, ry, y_lane_bytes,
-                        (uint32_t)(t_half + 16 * q) * row_bytes);
+      for (int q = 0; q < 4; ++q)
+        xn[q] = xn[q] * __builtin_amdgcn_sqrtf(
+                            __builtin_fmaf(-av[q], av[q], 1.0f));
+      keep4(av);
+      keep4(xn);
+      pinned(8 * g + 4);
+      // chunk 5: the run as a pair, the chain over both lane halves
+      float P = av[0], Hh = xn[0];
+#pragma unroll
+      for (int q = 1; q < 4; ++q) {
+        Hh = __builtin_fmaf(av[q], Hh, xn[q]);
+        P = P * av[q];
       }
+      float PL, PU, HL, HU;
+      halves(P, PL, PU);
+      halves(Hh, HL, HU);
+      const float after_lower = __builtin_fmaf(PL, c_run, HL);
+      float hh = upper ? after_lower : c_run;
+      c_run = __builtin_fmaf(PU, after_lower, HU);
+      asm volatile("" : "+v"(hh), "+v"(c_run));
+      pinned(8 * g + 5);
+      // chunk 6: replay from this lane's h_in
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        hh = __builtin_fmaf(av[q], hh, xn[q]);
+        *reinterpret_cast<uint16_t*>(patch_w + (8 * g + q) * kPatchStride) =
+            f32_to_bf16_bits(hh);
+      }
+      pinned(8 * g + 6);
+      // chunk 7: sixteen finished tokens leave as 16-byte row chunks; tokens
+      // past the end of the sequence fall outside the descriptor
+      if (g & 1) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        const u32x4 v = *reinterpret_cast<const u32x4*>(
+            patch_r + (g >> 1) * 16 * kPatchStride);
+        buffer_store_16(v, ry, y_lane_bytes,
+                        (uint32_t)(t_half + 16 * (g >> 1)) * row_bytes);
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+      }
+      pinned(8 * g + 7);
     }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
+    hc = c_run;
   };
 
   // ---- tile loop ------------------------------------------------------------
   // Phases of one tile `it` (staged in buffer it % 3):
   //   A   MFMA of tokens 0-31, with the conv of tile it+1 (into buffer
   //       (it+1) % 3) between the matrix instructions
-  //   E0  gates + recurrence of tokens 0-31
-  //   B   MFMA of tokens 32-63, with the row loads of tile it+2
+  //   E0  gates + recurrence of tokens 0-31, with the MFMA of tokens 32-63
+  //       and the row loads of tile it+2 spread through it
   //   E1  gates + recurrence of tokens 32-63
-  // A and B keep the matrix pipe busy, E0 and E1 the vector ALU.  Each SIMD
-  // holds one wave of waves 0-3 and one of waves 4-7; the second group runs one
-  // phase behind the first (it finishes E1 of a tile after the barrier that
-  // ends the tile), so that on every SIMD a matrix phase of one wave overlaps a
-  // vector phase of the other:
-  //   waves 0-3:  A(it)    E0(it)  B(it)   E1(it)  | barrier
-  //   waves 4-7:  E1(it-1) A(it)   E0(it)  B(it)   | barrier
+  // Every matrix instruction issues from a stream that also carries vector
+  // work of the same wave, so the matrix pipe runs under the vector ALU
+  // whatever the other wave of the SIMD is doing (the issue arbiter serves the
+  // older wave first: a wave that only has matrix instructions to issue
+  // starves next to one that only has vector instructions).
   auto a_base = [&](int t, int bi, int mt) {
     const int l = t & 63;
     return lds + (size_t)bi * kTM * kLdsStride +
@@ -467,53 +515,43 @@ __global__ void __launch_bounds__(512) block_fused_bf16_kernel(FusedArgs p) {
       acc_a[r] = bias[1];
     }
   };
-  auto phase_a = [&](int bi, int bn, uint64_t m_next, uint64_t m_tile,
-                     f32x16& acc_x, f32x16& acc_a) {
+  // A: the matrix instructions of tokens 0-31; waves 0-3 convolve their 32
+  // rows of the next tile between them, one row after each instruction.
+  auto phase_a = [&](auto staging, int bi, int bn, uint64_t m_next,
+                     uint64_t m_tile, f32x16& acc_x, f32x16& acc_a) {
+    constexpr bool STAGE = decltype(staging)::value;
     const int t1 = fresh_tid();
     const uint16_t* abase = a_base(t1, bi, 0);
-    uint16_t* const dst = stage_dst(t1, bn);
-    stage_begin(t1, m_next, m_tile);
     acc_init(t1, acc_x, acc_a);
     Frag a[2];
-    if (cut == 0) {
+    if (STAGE) {
+      uint16_t* const dst = stage_dst(t1, bn);
+      stage_begin(t1, m_next, m_tile);
+      if (cut == 0) {
 #pragma unroll
-      for (int j = 0; j < kHalo; ++j) stage_row(j, dst, NoCuts{});
-      a[0] = a_read(abase, 0);
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int ks = 0; ks < 16; ++ks) {
-        if (ks < 15) a[(ks + 1) & 1] = a_read(abase, ks + 1);
-        acc_x = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            a[ks & 1].v, bfrag[ks][0].v, acc_x, 0, 0, 0);
-        acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            a[ks & 1].v, bfrag[ks][1].v, acc_a, 0, 0, 0);
-        stage_row(kHalo + ks, dst, NoCuts{});
+        for (int j = 0; j < kHalo; ++j) stage_row(j, dst, NoCuts{});
+        a[0] = a_read(abase, 0);
         __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < 16; ++ks) {
+          if (ks < 15) a[(ks + 1) & 1] = a_read(abase, ks + 1);
+          acc_x = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              a[ks & 1].v, bfrag[ks][0].v, acc_x, 0, 0, 0);
+          stage_row(kHalo + 2 * ks, dst, NoCuts{});
+          __builtin_amdgcn_sched_barrier(0);
+          acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              a[ks & 1].v, bfrag[ks][1].v, acc_a, 0, 0, 0);
+          stage_row(kHalo + 2 * ks + 1, dst, NoCuts{});
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        return;
       }
-    } else {
       // a document starts among the rows of the next tile: conv first, with
       // the history cuts, then the matrix instructions
 #pragma unroll
       for (int j = 0; j < kRaw; ++j) stage_row(j, dst, WithCuts{});
-      a[0] = a_read(abase, 0);
-#pragma unroll
-      for (int ks = 0; ks < 16; ++ks) {
-        if (ks < 15) a[(ks + 1) & 1] = a_read(abase, ks + 1);
-        acc_x = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            a[ks & 1].v, bfrag[ks][0].v, acc_x, 0, 0, 0);
-        acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            a[ks & 1].v, bfrag[ks][1].v, acc_a, 0, 0, 0);
-      }
     }
-  };
-  auto phase_b = [&](int it, int bi, f32x16& acc_x, f32x16& acc_a) {
-    const int t1 = fresh_tid();
-    const uint32_t cb_off = chan_bytes(t1);
-    const uint16_t* abase = a_base(t1, bi, 1);
-    acc_init(t1, acc_x, acc_a);
-    Frag a[2];
     a[0] = a_read(abase, 0);
-    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ks = 0; ks < 16; ++ks) {
       if (ks < 15) a[(ks + 1) & 1] = a_read(abase, ks + 1);
@@ -521,51 +559,84 @@ __global__ void __launch_bounds__(512) block_fused_bf16_kernel(FusedArgs p) {
           a[ks & 1].v, bfrag[ks][0].v, acc_x, 0, 0, 0);
       acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
           a[ks & 1].v, bfrag[ks][1].v, acc_a, 0, 0, 0);
-      fetch_row(it + 2, ks, cb_off);
-      if (ks + 16 < kRaw) fetch_row(it + 2, ks + 16, cb_off);
-      __builtin_amdgcn_sched_barrier(0);
     }
   };
+  // One of the 32 matrix instructions of a half tile (hook index i): k-step
+  // i/2, gate i%2; the operand of the next k-step is requested two hooks ahead.
+  auto mfma_step = [&](int i, const uint16_t* abase, Frag (&a)[2],
+                       f32x16& acc_x, f32x16& acc_a) {
+    const int ks = i >> 1;
+    if ((i & 1) == 0) {
+      if (ks < 15) a[(ks + 1) & 1] = a_read(abase, ks + 1);
+      acc_x = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+          a[ks & 1].v, bfrag[ks][0].v, acc_x, 0, 0, 0);
+    } else {
+      acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+          a[ks & 1].v, bfrag[ks][1].v, acc_a, 0, 0, 0);
+    }
+  };
+  // E0 with the matrix instructions of tokens 32-63 spread through it (and,
+  // in waves 0-3, the first 19 row loads of tile it+2); leaves the packed
+  // pre-activations of tokens 32-63 in `out`.
+  constexpr int kRowsInE0 = 19;
+  static_assert(kRowsInE0 + 16 == kRaw, "row loads are split over E0 and E1");
+  auto phase_e0 = [&](auto staging, int it, int bi, const Packed& pk,
+                      uint64_t m_tile, Packed& out) {
+    constexpr bool STAGE = decltype(staging)::value;
+    const int t1 = fresh_tid();
+    const uint32_t cb_off = chan_bytes(t1);
+    const uint32_t base = row_base(it + 2);
+    const uint16_t* abase = a_base(t1, bi, 1);
+    f32x16 acc_x, acc_a;
+    acc_init(t1, acc_x, acc_a);
+    Frag a[2];
+    a[0] = a_read(abase, 0);
+    half_epilogue(it, 0, bi, pk, m_tile, [&](int i) {
+      mfma_step(i, abase, a, acc_x, acc_a);
+      if (STAGE && (i & 1) == 0) fetch_row_at(base, i >> 1, cb_off);
+      if (STAGE && (i & 1) == 1 && (i >> 1) + 16 < kRowsInE0)
+        fetch_row_at(base, (i >> 1) + 16, cb_off);
+    });
+    pack_acc(acc_x, acc_a, out);
+  };
 
-  if (!kSkewGroups || wave < 4) {
+  // E1; waves 0-3 issue the other 16 row loads of tile it+2 in it.
+  auto phase_e1 = [&](auto staging, int it, int bi, const Packed& pk,
+                      uint64_t m_tile) {
+    constexpr bool STAGE = decltype(staging)::value;
+    const int t1 = fresh_tid();
+    const uint32_t cb_off = chan_bytes(t1);
+    const uint32_t base = row_base(it + 2);
+    half_epilogue(it, 1, bi, pk, m_tile, [&](int i) {
+      if (STAGE && (i & 1) == 0)
+        fetch_row_at(base, kRowsInE0 + (i >> 1), cb_off);
+    });
+  };
+
+  auto tile_loop = [&](auto staging) {
     int bi = 0;
     for (int it = 0; it < ntiles; ++it) {
       const int bn = bi == kStageBufs - 1 ? 0 : bi + 1;
       const uint64_t m_next = start_mask(it + 1);
       fetch_seg(it + 2);
-      f32x16 acc_x, acc_a;
-      phase_a(bi, bn, m_next, m_cur, acc_x, acc_a);
-      half_epilogue(it, 0, bi, acc_x, acc_a, m_cur);
-      phase_b(it, bi, acc_x, acc_a);
-      half_epilogue(it, 1, bi, acc_x, acc_a, m_cur);
+      Packed pk, pk1;
+      {
+        f32x16 acc_x, acc_a;
+        phase_a(staging, bi, bn, m_next, m_cur, acc_x, acc_a);
+        pack_acc(acc_x, acc_a, pk);
+      }
+      phase_e0(staging, it, bi, pk, m_cur, pk1);
+      phase_e1(staging, it, bi, pk1, m_cur);
       // LDS-only barrier: row loads and y stores stay in flight across it
       lds_barrier();
       m_cur = m_next;
       bi = bn;
     }
-  } else {
-    int bi = 0, bp = 0;
-    uint64_t m_prev = 0;
-    f32x16 late_x, late_a;  // tokens 32-63 of the previous tile, E1 pending
-#pragma unroll
-    for (int r = 0; r < 16; ++r) late_x[r] = late_a[r] = 0.0f;
-    for (int it = 0; it < ntiles; ++it) {
-      const int bn = bi == kStageBufs - 1 ? 0 : bi + 1;
-      const uint64_t m_next = start_mask(it + 1);
-      fetch_seg(it + 2);
-      if (it > 0) half_epilogue(it - 1, 1, bp, late_x, late_a, m_prev);
-      f32x16 acc_x, acc_a;
-      phase_a(bi, bn, m_next, m_cur, acc_x, acc_a);
-      half_epilogue(it, 0, bi, acc_x, acc_a, m_cur);
-      phase_b(it, bi, late_x, late_a);
-      lds_barrier();
-      m_prev = m_cur;
-      m_cur = m_next;
-      bp = bi;
-      bi = bn;
-    }
-    half_epilogue(ntiles - 1, 1, bp, late_x, late_a, m_prev);
-  }
+  };
+  if (stager)
+    tile_loop(std::true_type{});
+  else
+    tile_loop(std::false_type{});
 
   if (p.h_last && !upper) p.h_last[(int64_t)b * W + ch] = hc;
 
