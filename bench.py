@@ -61,7 +61,7 @@ WORKLOADS = {
 # (scaled by a copy kernel of known size); None until measured for a workload.
 MEASURED_TRAFFIC_BYTES = {
     # profiles/hbm_traffic_9b_prefill.txt
-    ("9b_prefill", "single"): 2.161e9,   # 1.087 GB read + 1.074 GB written
+    ("9b_prefill", "single"): 2.164e9,   # 1.088 GB read + 1.076 GB written
     ("9b_prefill", "scan"): 4.40e9,      # 3.33 GB read + 1.074 GB written
 }
 
