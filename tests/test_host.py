@@ -58,6 +58,27 @@ def test_c_side_validation_without_launch():
   rc = lib.rg_recurrent_step(ok, ok, 1, ok, ok, ok, ok, ok, ok, ok, ok, ok, ok,
                              ok, ok, None, 0, 2, 256, 1, 1, None)
   assert rc == -4 and b"workspace" in lib.rg_last_error()
+  # the entries added for the whole block
+  rc = lib.rg_gelu_mul(ok, ok, ok, 0, 1, None)
+  assert rc == -1 and b"positive" in lib.rg_last_error()
+  rc = lib.rg_gelu_mul(ok, odd, ok, 8, 1, None)
+  assert rc == -1 and b"aligned" in lib.rg_last_error()
+  rc = lib.rg_gelu_mul(ok, ok, None, 8, 1, None)
+  assert rc == -1 and b"null" in lib.rg_last_error()
+  rc = lib.rg_gelu_mul(ok, ok, ok, 8, 3, None)
+  assert rc == -2 and b"dtype" in lib.rg_last_error()
+  args = [ok, ok, 1, ok, ok, ok, ok, ok, ok, None, ok, None, y, None, None]
+  rc = lib.rg_recurrent_prefill(*args, 1, 8, 256, 1, 0, None)
+  assert rc == -2 and b"unsupported" in lib.rg_last_error().lower()  # fp32
+  rc = lib.rg_recurrent_prefill(*args, 1, 8, 512, 1, 1, None)
+  assert rc == -2  # head width 512
+  rc = lib.rg_recurrent_prefill(*args, 1, 0, 256, 1, 1, None)
+  assert rc == -1 and b"positive" in lib.rg_last_error()
+  args[12] = ok  # y aliases x
+  rc = lib.rg_recurrent_prefill(*args, 1, 8, 256, 1, 1, None)
+  assert rc == -1 and b"alias" in lib.rg_last_error()
+  assert lib.rg_packed_gate_weights_bytes(4096, 16, 1) == 2 * 4096 * 256 * 2
+  assert lib.rg_packed_gate_weights_bytes(4096, 8, 1) == 0  # 512-wide heads
 
 
 def test_no_cpu_fallback():
