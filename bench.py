@@ -100,11 +100,36 @@ def make_segment_pos(torch, B, T, mean_doc, seed):
   return torch.from_numpy(out)
 
 
+def host_cores():
+  """Threads for the CPU leg: the cores this process may use (an
+  OMP_NUM_THREADS set by the environment is the share it was given)."""
+  n = os.cpu_count() or 1
+  try:
+    n = min(n, len(os.sched_getaffinity(0)))
+  except (AttributeError, OSError):
+    pass
+  env = os.environ.get("OMP_NUM_THREADS", "")
+  if env.isdigit() and int(env) > 0:
+    n = min(n, int(env))
+  return n
+
+
+def cpu_model():
+  try:
+    with open("/proc/cpuinfo") as f:
+      for line in f:
+        if line.startswith("model name"):
+          return line.split(":", 1)[1].strip()
+  except OSError:
+    pass
+  return "unknown"
+
+
 def cpu_baseline(torch, R, wl, params, seconds_target=20.0):
   """Oracle (port of the reference torch path) on the host cores, on a slice
   of the workload: the first Bs batch rows at full sequence length (about
   10-30 s of CPU work in total)."""
-  cores = os.cpu_count() or 1
+  cores = host_cores()
   torch.set_num_threads(cores)
   Bs, Ts = min(wl["B"], 4), wl["T"]
   g = torch.Generator().manual_seed(wl["seed"])
@@ -122,7 +147,7 @@ def cpu_baseline(torch, R, wl, params, seconds_target=20.0):
   best = sorted(times)[len(times) // 2]
   return {
       "value": Bs * Ts / best, "unit": "tokens/s", "cores": cores,
-      "kind": "port",
+      "kind": "port", "cpu": cpu_model(),
       "sample": (f"oracle/torch_ref.recurrent_core, "
                  f"{'f32' if dt == torch.float32 else 'bf16'}, {Bs}x{Ts} tokens of "
                  f"the workload (W={wl['W']}, H={wl['H']}), median of "
@@ -188,7 +213,7 @@ def run_decode(args, torch, rg, R, ops, wl):
                    "avg_launch_ms": dev_ms},
   }
   if not args.no_cpu_baseline:
-    cores = os.cpu_count() or 1
+    cores = host_cores()
     torch.set_num_threads(cores)
     xc, cc, hc = x.cpu(), conv_cache.cpu(), h.cpu()
     segc = seg.cpu()
@@ -201,6 +226,7 @@ def run_decode(args, torch, rg, R, ops, wl):
     dt = (time.perf_counter() - t0) / n
     result["cpu_baseline"] = {
         "value": B / dt, "unit": "tokens/s", "cores": cores, "kind": "port",
+        "cpu": cpu_model(),
         "sample": (f"oracle/torch_ref.recurrent_core with caches, bf16, {n} "
                    f"decode steps of {B} rows (W={W}, H={H}), mean, torch "
                    f"threads={torch.get_num_threads()}")}
