@@ -1,0 +1,472 @@
+"""The callers around the recurrent block: Griffin's residual stack.
+
+Mirrors the module surface of recurrentgemma/torch/modules.py (attention
+block :294-493, MLP block :683-760, residual block :763-932, embedder
+:935-1003), recurrentgemma/torch/griffin.py:27-209 (model, cache dictionary
+keyed "blocks.{i}") and the config types of recurrentgemma/common.py:22-190:
+same constructor arguments, parameter names (reference state dicts load
+unchanged), forward signatures and cache tuples.  Only the recurrent block
+runs on this package's kernels; everything else here is plain torch on the GPU
+(hipBLASLt GEMMs, scaled_dot_product_attention) and exists so that the
+recurrent path can be exercised and measured inside the model it belongs to.
+Inference only (no autograd through the kernels).
+"""
+
+from __future__ import annotations
+
+import enum
+import itertools
+import math
+from typing import Any, NamedTuple
+
+import torch
+from torch import nn
+
+from recurrentgemma_amd import modules
+
+_MAX_WAVELENGTH = 10_000
+
+
+@enum.unique
+class TemporalBlockType(enum.Enum):
+  ATTENTION = enum.auto()
+  RECURRENT = enum.auto()
+
+
+@enum.unique
+class Preset(enum.Enum):
+  """The published shapes (common.py:47-112)."""
+  GRIFFIN_PAPER_7B = enum.auto()
+  HAWK_PAPER_7B = enum.auto()
+  RECURRENT_GEMMA_2B_V1 = enum.auto()
+  RECURRENT_GEMMA_9B_V1 = enum.auto()
+
+  @property
+  def config_dict(self) -> dict[str, Any]:
+    r, a = TemporalBlockType.RECURRENT, TemporalBlockType.ATTENTION
+
+    def pattern(n):  # recurrent, recurrent, attention, ...
+      return tuple(itertools.islice(itertools.cycle((r, r, a)), n))
+
+    paper = dict(width=4096, mlp_expanded_width=3 * 4096, num_heads=32,
+                 lru_width=5632, embeddings_scale_by_sqrt_dim=False,
+                 attention_window_size=1024, logits_soft_cap=0.0)
+    gemma = dict(embeddings_scale_by_sqrt_dim=True, attention_window_size=2048,
+                 logits_soft_cap=30.0)
+    if self is Preset.GRIFFIN_PAPER_7B:
+      return dict(paper, block_types=pattern(32))
+    if self is Preset.HAWK_PAPER_7B:
+      return dict(paper, block_types=(r,) * 32)
+    if self is Preset.RECURRENT_GEMMA_2B_V1:
+      return dict(gemma, width=2560, mlp_expanded_width=3 * 2560, num_heads=10,
+                  lru_width=2560, block_types=pattern(26))
+    return dict(gemma, width=4096, mlp_expanded_width=3 * 4096, num_heads=16,
+                lru_width=4096, block_types=pattern(38))
+
+
+class GriffinConfig(NamedTuple):
+  """common.py:115-190 without the Flax-only scan_type field."""
+  vocab_size: int
+  width: int
+  mlp_expanded_width: int
+  num_heads: int
+  block_types: tuple[TemporalBlockType, ...]
+  embeddings_scale_by_sqrt_dim: bool
+  attention_window_size: int
+  logits_soft_cap: float
+  lru_width: int | None = None
+
+  @property
+  def max_cache_length(self) -> int:
+    return self.attention_window_size
+
+  @property
+  def num_layers(self) -> int:
+    return len(self.block_types)
+
+  @classmethod
+  def from_preset(cls, preset: Preset, vocab_size: int = 256_000,
+                  max_sequence_length: int | None = None) -> "GriffinConfig":
+    kw = preset.config_dict
+    if max_sequence_length is not None:
+      kw["attention_window_size"] = min(kw["attention_window_size"],
+                                        max_sequence_length)
+    return cls(vocab_size=vocab_size, **kw)
+
+
+class AttentionBlockCache(NamedTuple):
+  keys: torch.Tensor        # [B, window, 1, head_dim], ring buffer
+  values: torch.Tensor      # [B, window, 1, head_dim]
+  num_tokens: torch.Tensor  # [B] int32, tokens seen so far
+
+
+ResidualBlockCache = modules.RecurrentBlockCache | AttentionBlockCache
+Cache = dict[str, ResidualBlockCache]
+
+
+class RMSNorm(nn.Module):
+  """x / rms(x) * (1 + scale)  (layers.py:30-73); scale starts at zero."""
+
+  def __init__(self, width, eps=1e-6, device=None, dtype=None):
+    super().__init__()
+    self.width = width
+    self.eps = eps
+    self.scale = nn.Parameter(torch.empty([width], device=device, dtype=dtype))
+    self.reset_parameters()
+
+  def reset_parameters(self) -> None:
+    torch.nn.init.zeros_(self.scale)
+
+  def forward(self, x):
+    # the reference computes every step in the activation dtype
+    var = torch.mean(torch.square(x), dim=-1, keepdim=True)
+    return x * torch.rsqrt(var + self.eps) * (self.scale + 1)
+
+
+class _StackedLinear(nn.Module):
+  """Two width -> expanded projections with stacked parameters `w`
+  [2, width, expanded] and `b` [2, 1, 1, expanded]: the parameters of the
+  reference's `Einsum("...td,cdD->c...tD")` (layers.py:653-703) under the same
+  names."""
+
+  def __init__(self, width, expanded, device=None, dtype=None):
+    super().__init__()
+    self.w_shape = (2, width, expanded)
+    self.w = nn.Parameter(torch.empty(self.w_shape, device=device, dtype=dtype))
+    self.b = nn.Parameter(
+        torch.empty((2, 1, 1, expanded), device=device, dtype=dtype))
+    self.reset_parameters()
+
+  def reset_parameters(self) -> None:
+    torch.nn.init.normal_(self.w, mean=0.0,
+                          std=math.sqrt(1.0 / self.w_shape[1]))
+    torch.nn.init.zeros_(self.b)
+
+  def forward(self, x):
+    lead = x.shape[:-1]
+    x2 = x.reshape(-1, x.shape[-1])
+    gate = torch.addmm(self.b[0].reshape(-1), x2, self.w[0])
+    up = torch.addmm(self.b[1].reshape(-1), x2, self.w[1])
+    return gate.reshape(*lead, -1), up.reshape(*lead, -1)
+
+
+class MLPBlock(nn.Module):
+  """gelu(x W0 + b0) * (x W1 + b1) -> ffw_down  (modules.py:683-760)."""
+
+  def __init__(self, width, expanded_width, final_w_init_variance_scale=1.0,
+               device=None, dtype=None):
+    super().__init__()
+    self.width = width
+    self.expanded_width = expanded_width
+    self.final_w_init_variance_scale = final_w_init_variance_scale
+    self.ffw_up = _StackedLinear(width, expanded_width, device=device,
+                                 dtype=dtype)
+    self.ffw_down = nn.Linear(expanded_width, width, device=device, dtype=dtype)
+    self.reset_parameters()
+
+  def reset_parameters(self) -> None:
+    self.ffw_up.reset_parameters()
+    std = math.sqrt(self.final_w_init_variance_scale / self.expanded_width)
+    torch.nn.init.normal_(self.ffw_down.weight, mean=0.0, std=std)
+    torch.nn.init.zeros_(self.ffw_down.bias)
+
+  def forward(self, x):
+    gate, up = self.ffw_up(x)
+    return self.ffw_down(modules.gelu(gate) * up)
+
+
+def _rope(x, positions, max_wavelength=_MAX_WAVELENGTH):
+  """Rotary embedding on the first half of the head dimension
+  (modules.py:52-83): within that half, element i pairs with element
+  i + quarter, angle = position / max_wavelength^(2i / half)."""
+  half = x.shape[-1] // 2
+  quarter = half // 2
+  rot, keep = x[..., :half], x[..., half:]
+  freq = torch.arange(quarter, device=x.device)
+  inv = 1.0 / (max_wavelength ** (2 * freq / half))
+  angle = positions[:, :, None, None] * inv
+  sin, cos = torch.sin(angle).type_as(x), torch.cos(angle).type_as(x)
+  lo, hi = rot[..., :quarter], rot[..., quarter:]
+  return torch.cat([lo * cos - hi * sin, hi * cos + lo * sin, keep], dim=-1)
+
+
+def _visible(q_pos, k_pos, window, q_doc=None, k_doc=None):
+  """[B, Tq, Tk] mask (modules.py:86-127): keys not after the query, at most
+  `window` positions back, in the same document (or, without document ids, at
+  a real position >= 0)."""
+  q, k = q_pos[..., :, None], k_pos[..., None, :]
+  mask = (q >= k) & (q <= k + window)
+  if q_doc is not None:
+    return mask & (q_doc[..., :, None] == k_doc[..., None, :])
+  return mask & (k >= 0)
+
+
+class LocalAttentionBlock(nn.Module):
+  """Sliding-window multi-query attention with a ring KV cache
+  (modules.py:294-493)."""
+
+  def __init__(self, width, num_heads, window_size,
+               final_w_init_variance_scale=1.0, device=None, dtype=None):
+    super().__init__()
+    self.width = width
+    self.num_heads = num_heads
+    self.window_size = window_size
+    self.final_w_init_variance_scale = final_w_init_variance_scale
+    kw = dict(device=device, dtype=dtype)
+    self.proj_q = nn.Linear(width, width, bias=False, **kw)
+    self.proj_k = nn.Linear(width, self.head_dim, bias=False, **kw)
+    self.proj_v = nn.Linear(width, self.head_dim, bias=False, **kw)
+    self.proj_final = nn.Linear(width, width, bias=True, **kw)
+    self.reset_parameters()
+
+  @property
+  def head_dim(self) -> int:
+    return self.width // self.num_heads
+
+  def reset_parameters(self) -> None:
+    for proj in (self.proj_q, self.proj_k, self.proj_v):
+      torch.nn.init.normal_(proj.weight, mean=0.0,
+                            std=math.sqrt(1.0 / self.width))
+    std = math.sqrt(self.final_w_init_variance_scale / self.width)
+    torch.nn.init.normal_(self.proj_final.weight, mean=0.0, std=std)
+    torch.nn.init.zeros_(self.proj_final.bias)
+
+  @staticmethod
+  def _cache_from_prompt(keys, values, segment_pos, window):
+    """Ring buffer filled from a prompt (modules.py:253-283): the last
+    min(window, T) tokens, token with position p in slot p % window when the
+    prompt fills the window."""
+    w = min(window, keys.shape[1])
+    num_tokens = segment_pos[:, -1] + 1
+    shift = (num_tokens % window)[:, None]
+    src = (torch.arange(w, device=keys.device)[None] - shift) % w  # [B, w]
+
+    def place(x):
+      tail = x[:, -w:]
+      idx = src[:, :, None, None].expand(-1, -1, *tail.shape[2:])
+      out = torch.gather(tail, 1, idx)
+      if w < window:
+        pad = out.new_zeros(out.shape[0], window - w, *out.shape[2:])
+        out = torch.cat([out, pad], dim=1)
+      return out
+
+    return AttentionBlockCache(keys=place(keys), values=place(values),
+                               num_tokens=num_tokens)
+
+  @torch.no_grad()
+  def forward(self, x, segment_pos, cache=None, return_cache=True):
+    b, t, _ = x.shape
+    assert segment_pos.shape == (b, t), segment_pos.shape
+    q = self.proj_q(x).reshape(b, t, self.num_heads, self.head_dim)
+    k = self.proj_k(x).reshape(b, t, 1, self.head_dim)
+    v = self.proj_v(x).reshape(b, t, 1, self.head_dim)
+    q, k = _rope(q, segment_pos), _rope(k, segment_pos)
+
+    new_cache = None
+    if cache is not None:
+      # positions held by the ring: slot j keeps the largest position
+      # congruent to j that is below num_tokens (modules.py:152-183)
+      w = self.window_size
+      n = cache.num_tokens[:, None]
+      slot = torch.arange(w, device=x.device)[None]
+      now = slot + (n // w) * w
+      k_pos = torch.where(now < n, now, now - w)
+      q_pos = torch.arange(t, device=x.device)[None] + n
+      mask = _visible(q_pos, torch.cat([k_pos, q_pos], dim=-1), w)
+      k_all = torch.cat([cache.keys, k], dim=1)
+      v_all = torch.cat([cache.values, v], dim=1)
+      if return_cache:
+        if t == 1:
+          rows = torch.arange(b, device=x.device)
+          at = (cache.num_tokens % w).long()
+          cache.keys[rows, at] = k[:, 0]
+          cache.values[rows, at] = v[:, 0]
+          cache.num_tokens[:] = cache.num_tokens + 1
+          new_cache = cache
+        elif t >= w:
+          new_cache = self._cache_from_prompt(k, v, segment_pos, w)
+        else:
+          raise NotImplementedError(
+              "a cached call takes one token or at least a window of them")
+    else:
+      doc = torch.cumsum(segment_pos == 0, dim=-1)
+      pos = torch.arange(t, device=x.device)[None].expand(b, t)
+      mask = _visible(pos, pos, self.window_size, doc, doc)
+      k_all, v_all = k, v
+      if return_cache:
+        new_cache = self._cache_from_prompt(k, v, segment_pos,
+                                            self.window_size)
+
+    # [B, heads, T, head_dim] against one shared key/value head
+    out = nn.functional.scaled_dot_product_attention(
+        q.transpose(1, 2),
+        k_all.transpose(1, 2).expand(-1, self.num_heads, -1, -1),
+        v_all.transpose(1, 2).expand(-1, self.num_heads, -1, -1),
+        attn_mask=mask[:, None])
+    out = out.transpose(1, 2).reshape(b, t, self.width)
+    return self.proj_final(out), new_cache
+
+  @classmethod
+  def init_cache(cls, batch_size, window_size, heads_dim, dtype, device=None):
+    shape = (batch_size, window_size, 1, heads_dim)
+    return AttentionBlockCache(
+        keys=torch.zeros(shape, device=device, dtype=dtype),
+        values=torch.zeros(shape, device=device, dtype=dtype),
+        num_tokens=torch.zeros([batch_size], dtype=torch.int32, device=device))
+
+
+class ResidualBlock(nn.Module):
+  """norm -> temporal block -> +x -> norm -> MLP -> +  (modules.py:763-932)."""
+
+  def __init__(self, width, mlp_expanded_width, num_heads,
+               attention_window_size, temporal_block_type, lru_width=None,
+               conv1d_temporal_width=4, final_w_init_variance_scale=1.0,
+               device=None, dtype=None):
+    super().__init__()
+    self.width = width
+    self.mlp_expanded_width = mlp_expanded_width
+    self.num_heads = num_heads
+    self.attention_window_size = attention_window_size
+    self.temporal_block_type = temporal_block_type
+    self.lru_width = lru_width
+    self.conv1d_temporal_width = conv1d_temporal_width
+    self.final_w_init_variance_scale = final_w_init_variance_scale
+    kw = dict(device=device, dtype=dtype)
+    self.temporal_pre_norm = RMSNorm(width, **kw)
+    if temporal_block_type is TemporalBlockType.RECURRENT:
+      self.recurrent_block = modules.RecurrentBlock(
+          width=width, num_heads=num_heads, lru_width=lru_width,
+          conv1d_temporal_width=conv1d_temporal_width,
+          final_w_init_variance_scale=final_w_init_variance_scale, **kw)
+    else:
+      self.attention_block = LocalAttentionBlock(
+          width=width, num_heads=num_heads, window_size=attention_window_size,
+          final_w_init_variance_scale=final_w_init_variance_scale, **kw)
+    self.channel_pre_norm = RMSNorm(width, **kw)
+    self.mlp_block = MLPBlock(
+        width=width, expanded_width=mlp_expanded_width,
+        final_w_init_variance_scale=final_w_init_variance_scale, **kw)
+
+  @property
+  def temporal_block(self) -> nn.Module:
+    if self.temporal_block_type is TemporalBlockType.RECURRENT:
+      return self.recurrent_block
+    return self.attention_block
+
+  def reset_parameters(self) -> None:
+    self.temporal_pre_norm.reset_parameters()
+    self.temporal_block.reset_parameters()
+    self.channel_pre_norm.reset_parameters()
+    self.mlp_block.reset_parameters()
+
+  @torch.no_grad()
+  def forward(self, x, segment_pos, cache=None, return_cache=True):
+    mixed, new_cache = self.temporal_block(self.temporal_pre_norm(x),
+                                           segment_pos, cache,
+                                           return_cache=return_cache)
+    residual = mixed + x
+    return self.mlp_block(self.channel_pre_norm(residual)) + residual, new_cache
+
+  @classmethod
+  def init_cache(cls, batch_size, width, num_heads, attention_window_size,
+                 temporal_block_type, dtype, lru_width=None,
+                 conv1d_temporal_width=4, device=None):
+    if temporal_block_type is TemporalBlockType.RECURRENT:
+      return modules.RecurrentBlock.init_cache(
+          batch_size=batch_size, lru_width=lru_width or width, dtype=dtype,
+          conv1d_temporal_width=conv1d_temporal_width, device=device)
+    return LocalAttentionBlock.init_cache(
+        batch_size=batch_size, window_size=attention_window_size,
+        heads_dim=width // num_heads, dtype=dtype, device=device)
+
+
+class Embedder(nn.Module):
+  """Token table used for both the input embedding and the output logits
+  (modules.py:935-1003)."""
+
+  def __init__(self, vocab_size, embed_dim, scale_by_sqrt_dim, device=None,
+               dtype=None):
+    super().__init__()
+    self.vocab_size = vocab_size
+    self.embed_dim = embed_dim
+    self.scale_by_sqrt_dim = scale_by_sqrt_dim
+    self.input_embedding = nn.Parameter(
+        torch.empty([vocab_size, embed_dim], device=device, dtype=dtype))
+    self.reset_parameters()
+
+  def reset_parameters(self) -> None:
+    torch.nn.init.normal_(self.input_embedding, mean=0.0,
+                          std=math.sqrt(1.0 / self.embed_dim))
+
+  def encode(self, tokens):
+    x = self.input_embedding[(tokens,)]
+    if self.scale_by_sqrt_dim:
+      # the factor is rounded to bfloat16 whatever the model dtype
+      x = x * torch.tensor(math.sqrt(self.embed_dim)).type(torch.bfloat16)
+    return x
+
+  def decode(self, x):
+    return x @ self.input_embedding.T
+
+
+class Griffin(nn.Module):
+  """Embedder -> residual blocks -> final norm -> logits (soft-capped)
+  (griffin.py:27-209)."""
+
+  def __init__(self, config: GriffinConfig, gradient_checkpointing=True,
+               device=None, dtype=None):
+    super().__init__()
+    self.config = config
+    # accepted for signature compatibility; this build is inference only and
+    # never checkpoints
+    self.gradient_checkpointing = gradient_checkpointing
+    self.embedder = Embedder(
+        vocab_size=config.vocab_size, embed_dim=config.width,
+        scale_by_sqrt_dim=config.embeddings_scale_by_sqrt_dim, device=device,
+        dtype=dtype)
+    self.blocks = nn.ModuleList([
+        ResidualBlock(
+            width=config.width, mlp_expanded_width=config.mlp_expanded_width,
+            num_heads=config.num_heads,
+            attention_window_size=config.attention_window_size,
+            temporal_block_type=kind, lru_width=config.lru_width,
+            final_w_init_variance_scale=2.0 / config.num_layers, device=device,
+            dtype=dtype) for kind in config.block_types])
+    self.final_norm = RMSNorm(config.width, device=device, dtype=dtype)
+
+  def reset_parameters(self) -> None:
+    self.embedder.reset_parameters()
+    for block in self.blocks:
+      block.reset_parameters()
+    self.final_norm.reset_parameters()
+
+  @torch.no_grad()
+  def forward(self, tokens, segment_pos, cache: Cache | None = None,
+              return_logits=True, return_cache=True):
+    if not return_logits and not return_cache:
+      return None, None
+    x = self.embedder.encode(tokens)
+    new_cache = {}
+    for i, block in enumerate(self.blocks):
+      name = f"blocks.{i}"
+      x, new_cache[name] = block(x, segment_pos,
+                                 None if cache is None else cache[name],
+                                 return_cache=return_cache)
+    if not return_logits:
+      return None, new_cache
+    logits = self.embedder.decode(self.final_norm(x))
+    cap = self.config.logits_soft_cap
+    if cap:
+      logits = torch.tanh(logits / cap) * cap
+    return logits, (new_cache if return_cache else None)
+
+  def init_cache(self, batch_size, dtype, device=None) -> Cache:
+    c = self.config
+    if device is None:
+      device = self.embedder.input_embedding.device
+    return {
+        f"blocks.{i}": ResidualBlock.init_cache(
+            batch_size=batch_size, width=c.width, num_heads=c.num_heads,
+            attention_window_size=c.attention_window_size,
+            temporal_block_type=kind, dtype=dtype, lru_width=c.lru_width,
+            device=device) for i, kind in enumerate(c.block_types)}

@@ -1,0 +1,143 @@
+"""The residual stack and the sampler around the recurrent block, on the GPU,
+against vectors written by the reference model itself
+(tests/golden/make_griffin_golden.py; float32, tiny shapes).  Tolerance: 2e-4
+of the largest reference magnitude per tensor (GPU vs CPU float32 matmuls and
+softmax); sampled tokens must be identical."""
+
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from recurrentgemma_amd import griffin as G
+from recurrentgemma_amd import sampler as S
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "griffin_golden.npz")
+TOL = 2e-4
+
+
+@pytest.fixture(scope="module")
+def golden():
+  return np.load(GOLDEN)
+
+
+@pytest.fixture(scope="module")
+def model(golden):
+  R, A = G.TemporalBlockType.RECURRENT, G.TemporalBlockType.ATTENTION
+  cfg = G.GriffinConfig(
+      vocab_size=48, width=32, mlp_expanded_width=40, num_heads=2,
+      block_types=(R, A, R), embeddings_scale_by_sqrt_dim=True,
+      attention_window_size=6, logits_soft_cap=30.0, lru_width=64)
+  m = G.Griffin(cfg, dtype=torch.float32)
+  sd = {k[len("param/"):]: torch.from_numpy(golden[k])
+        for k in golden.files if k.startswith("param/")}
+  assert set(sd) == set(m.state_dict()), set(sd) ^ set(m.state_dict())
+  m.load_state_dict(sd)  # the reference's own keys and shapes
+  return m.to(DEV).eval()
+
+
+def close(got, want, what):
+  want = torch.from_numpy(np.asarray(want))
+  got = got.detach().cpu()
+  assert got.shape == want.shape, (what, got.shape, want.shape)
+  if want.numel() == 0:  # the reference cuts pad_length leading entries
+    return
+  if want.dtype in (torch.int32, torch.int64):
+    assert torch.equal(got.to(want.dtype), want), what
+    return
+  err = (got.float() - want.float()).abs().max().item()
+  scale = max(want.float().abs().max().item(), 1e-6)
+  assert err <= TOL * scale, (what, err, scale)
+
+
+def check_cache(cache, golden, prefix):
+  names = [k for k in golden.files if k.startswith(prefix + "/")]
+  assert names
+  for k in names:
+    block, field = k[len(prefix) + 1:].split("/")
+    close(getattr(cache[block], field), golden[k], k)
+
+
+def dev(a, dtype=None):
+  t = torch.from_numpy(np.asarray(a)).to(DEV)
+  return t if dtype is None else t.to(dtype)
+
+
+def test_forward_left_padded_then_step(model, golden):
+  logits, cache = model(dev(golden["c1/tokens"]), dev(golden["c1/pos"]))
+  close(logits, golden["c1/logits"], "c1/logits")
+  check_cache(cache, golden, "c1/cache")
+  assert isinstance(cache["blocks.0"], G.modules.RecurrentBlockCache)
+  assert isinstance(cache["blocks.1"], G.AttentionBlockCache)
+  logits2, cache2 = model(dev(golden["c1/next_tokens"]),
+                          dev(golden["c1/next_pos"]), cache)
+  close(logits2, golden["c1/next_logits"], "c1/next_logits")
+  check_cache(cache2, golden, "c1/next_cache")
+
+
+def test_prompt_longer_than_window_then_steps(model, golden):
+  pos = dev(golden["c2/pos"])
+  logits, cache = model(dev(golden["c2/tokens"]), pos)
+  close(logits, golden["c2/logits"], "c2/logits")
+  check_cache(cache, golden, "c2/cache")
+  steps = dev(golden["c2/step_tokens"])
+  p = pos[:, -1:] + 1
+  for i in range(3):
+    lg, cache = model(steps[:, i:i + 1], p, cache)
+    close(lg, golden[f"c2/step{i}_logits"], f"c2/step{i}")
+    p = p + 1
+  check_cache(cache, golden, "c2/final_cache")
+
+
+def test_flags(model, golden):
+  tokens, pos = dev(golden["c1/tokens"]), dev(golden["c1/pos"])
+  assert model(tokens, pos, return_logits=False, return_cache=False) == (None,
+                                                                         None)
+  logits, cache = model(tokens, pos, return_cache=False)
+  assert cache is None
+  close(logits, golden["c1/logits"], "no-cache logits")
+  none, cache = model(tokens, pos, return_logits=False)
+  assert none is None
+  check_cache(cache, golden, "c1/cache")
+  empty = model.init_cache(2, torch.float32)
+  assert set(empty) == {"blocks.0", "blocks.1", "blocks.2"}
+  assert empty["blocks.1"].keys.shape == (2, 6, 1, 16)
+  assert empty["blocks.0"].rg_lru_state.shape == (2, 64)
+
+
+class ToyVocab:
+  def bos_id(self): return 2
+  def eos_id(self): return 1
+  def pad_id(self): return 0
+  def EncodeAsIds(self, s): return [int(t) for t in s.split()]
+  def DecodeIds(self, ids): return " ".join(str(i) for i in ids)
+
+
+@pytest.mark.parametrize("echo", [False, True])
+def test_sampler_matches_reference(model, golden, echo):
+  smp = S.Sampler(model, ToyVocab(), greedy_sampling=True)
+  prompts = [str(p) for p in golden["c3/prompts"]]
+  res = smp(prompts, total_generation_steps=6, echo=echo, return_logits=True,
+            end_sampling_at_eos_token=False)
+  tag = "c3/echo" if echo else "c3/plain"
+  assert res.text == [str(t) for t in golden[f"{tag}/text"]]
+  for i in range(len(prompts)):
+    close(res.tokens[i], golden[f"{tag}/tokens{i}"], f"{tag}/tokens{i}")
+    close(res.logits[i], golden[f"{tag}/logits{i}"], f"{tag}/logits{i}")
+
+
+def test_sample_tokens_without_vocab(model, golden):
+  smp = S.Sampler(model)
+  toks = torch.tensor([[0, 0, 2, 7, 40, 3], [2, 5, 9, 13, 21, 8]], device=DEV,
+                      dtype=torch.int32)
+  lens = torch.tensor([4, 6], device=DEV, dtype=torch.int32)
+  out, logits = smp.sample_tokens(toks, lens, 5)
+  assert out.shape == (2, 5) and logits is None
+  # the same prompts one at a time (no padding) give the same continuation
+  for r in range(2):
+    single, _ = smp.sample_tokens(toks[r:r + 1, 6 - int(lens[r]):],
+                                  lens[r:r + 1], 5)
+    assert torch.equal(single[0], out[r])
