@@ -55,6 +55,10 @@ WORKLOADS = {
                    dtype="f32"),
     "9b_decode": dict(B=256, T=1, W=4096, H=16, mean_doc=None, seed=1004,
                       decode=True),
+    # random-init 2B residual stack, greedy decoding: 64 prompts of 2048 random
+    # token ids, 256 new tokens each (--steps sets the number of new tokens)
+    "2b_griffin_decode": dict(B=64, T=2048, new_tokens=256, seed=1005,
+                              griffin=True),
 }
 
 # HBM bytes per scan launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
@@ -162,6 +166,74 @@ def decode_algorithmic_bytes(B, W, H, esize):
           + 2 * H * (W // H) ** 2 * esize + W * esize * 8 + B * 8)
 
 
+def run_griffin(args, torch, rg, wl):
+  """Greedy decoding with the whole 2B-shape model: the recurrent blocks on
+  this package's kernels, the rest plain torch.  One step = one new token for
+  every sequence of the batch (a cached single-token pass through the 26
+  blocks); the prompt pass is timed separately."""
+  from recurrentgemma_amd import griffin as G
+  from recurrentgemma_amd import sampler as S
+  dev = torch.device("cuda:0")
+  B, T = wl["B"], wl["T"]
+  new_tokens = args.steps + 1 if args.steps != 50 else wl["new_tokens"]
+  cfg = G.GriffinConfig.from_preset(G.Preset.RECURRENT_GEMMA_2B_V1)
+  torch.manual_seed(wl["seed"])
+  model = G.Griffin(cfg, device=dev, dtype=torch.bfloat16).eval()
+  n_params = sum(p.numel() for p in model.parameters())
+  g = torch.Generator().manual_seed(wl["seed"])
+  tokens = torch.randint(0, cfg.vocab_size, (B, T), generator=g).to(
+      dev, torch.int32)
+  lens = torch.full((B,), T, device=dev, dtype=torch.int32)
+  smp = S.Sampler(model, greedy_sampling=True, use_graph=not args.eager)
+
+  def generate(n):
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    out, _ = smp.sample_tokens(tokens, lens, n)
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0, out
+
+  generate(min(args.warmup, 8) + 1)          # warm-up: prompt + a few steps
+  t_prompt, _ = generate(1)                  # prompt pass + first token
+  t_full, out = generate(new_tokens)
+  steps = new_tokens - 1
+  t_decode = t_full - t_prompt
+  # every decode step reads every parameter once (bf16); the embedding table
+  # only as the logits projection
+  step_bytes = 2 * n_params
+  achieved = step_bytes * steps / t_decode / 1e9
+  result = {
+      "metric": "greedy decoding tokens/s, 2B residual stack",
+      "value": B * steps / t_decode, "unit": "tokens/s", "n_gpus": 1,
+      "steps": steps, "warmup": min(args.warmup, 8),
+      "ms_per_step": t_decode * 1e3 / steps, "higher_is_better": True,
+      "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+      "data": "synthetic",
+      "config": {"workload": args.workload, "batch": B, "prompt_len": T,
+                 "new_tokens": new_tokens, "blocks": cfg.num_layers,
+                 "width": cfg.width, "vocab": cfg.vocab_size,
+                 "parameters": n_params,
+                 "path": "Sampler.sample_tokens ("
+                         + ("eager" if args.eager else "decode step replayed "
+                            "as a captured HIP graph")
+                         + "), recurrent blocks: "
+                         "rg_recurrent_prefill / two-kernel form + "
+                         "rg_recurrent_step_packed + rg_gelu_mul"},
+      "prompt_pass": {"ms": t_prompt * 1e3,
+                      "tokens_per_s": B * T / t_prompt},
+      "whole_generation": {"ms": t_full * 1e3,
+                           "new_tokens_per_s": B * new_tokens / t_full},
+      "roofline": {"kernel": "one decode step (all kernels of the 26 blocks "
+                             "and the logits projection)",
+                   "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
+                   "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                   "traffic": None, "algorithmic_bytes": step_bytes,
+                   "avg_launch_ms": t_decode * 1e3 / steps},
+      "checksum": int(out.sum().item()),
+  }
+  print(json.dumps(result))
+
+
 def run_decode(args, torch, rg, R, ops, wl):
   """Times rg_recurrent_step (conv step, both gate projections, gate
   activations, state update) on B rows with the caches updated in place."""
@@ -243,6 +315,9 @@ def main():
   ap.add_argument("--no-cpu-baseline", action="store_true",
                   help="lean run for the profiler: no CPU leg and no "
                        "additional 2B-width measurement")
+  ap.add_argument("--eager", action="store_true",
+                  help="2b_griffin_decode: launch every kernel of a decode "
+                       "step from Python instead of replaying a captured graph")
   ap.add_argument("--calibration-copy", action="store_true",
                   help="after the timed steps, run one plain device copy of x "
                        "(known size) so that a counter run of this command "
@@ -260,6 +335,9 @@ def main():
   from recurrentgemma_amd import ops
 
   wl = WORKLOADS[args.workload]
+  if wl.get("griffin"):
+    run_griffin(args, torch, rg, wl)
+    return
   if wl.get("decode"):
     run_decode(args, torch, rg, R, ops, wl)
     return

@@ -262,28 +262,18 @@ class LocalAttentionBlock(nn.Module):
     v = self.proj_v(x).reshape(b, t, 1, self.head_dim)
     q, k = _rope(q, segment_pos), _rope(k, segment_pos)
 
+    if cache is not None and t == 1:
+      return self._decode_step(x, q, k, v, cache, return_cache)
+
     new_cache = None
     if cache is not None:
-      # positions held by the ring: slot j keeps the largest position
-      # congruent to j that is below num_tokens (modules.py:152-183)
       w = self.window_size
-      n = cache.num_tokens[:, None]
-      slot = torch.arange(w, device=x.device)[None]
-      now = slot + (n // w) * w
-      k_pos = torch.where(now < n, now, now - w)
-      q_pos = torch.arange(t, device=x.device)[None] + n
+      k_pos, q_pos = self._ring_positions(cache.num_tokens, t)
       mask = _visible(q_pos, torch.cat([k_pos, q_pos], dim=-1), w)
       k_all = torch.cat([cache.keys, k], dim=1)
       v_all = torch.cat([cache.values, v], dim=1)
       if return_cache:
-        if t == 1:
-          rows = torch.arange(b, device=x.device)
-          at = (cache.num_tokens % w).long()
-          cache.keys[rows, at] = k[:, 0]
-          cache.values[rows, at] = v[:, 0]
-          cache.num_tokens[:] = cache.num_tokens + 1
-          new_cache = cache
-        elif t >= w:
+        if t >= w:
           new_cache = self._cache_from_prompt(k, v, segment_pos, w)
         else:
           raise NotImplementedError(
@@ -305,6 +295,47 @@ class LocalAttentionBlock(nn.Module):
         attn_mask=mask[:, None])
     out = out.transpose(1, 2).reshape(b, t, self.width)
     return self.proj_final(out), new_cache
+
+  def _ring_positions(self, num_tokens, t):
+    """Positions held by the ring (slot j keeps the largest position congruent
+    to j that is below num_tokens; negative = never written) and positions of
+    the t new tokens (modules.py:152-183)."""
+    w = self.window_size
+    n = num_tokens[:, None]
+    now = torch.arange(w, device=n.device)[None] + (n // w) * w
+    k_pos = torch.where(now < n, now, now - w)
+    q_pos = torch.arange(t, device=n.device)[None] + n
+    return k_pos, q_pos
+
+  def _decode_step(self, x, q, k, v, cache, return_cache):
+    """One new token against the ring and itself, without concatenating or
+    expanding the cached keys and values: all heads share them, so the scores
+    are one batched [heads, head_dim] x [head_dim, window] product per row.
+    Same order of roundings as the reference: scores in the activation dtype,
+    scaled, masked, softmax in float32, probabilities back in the activation
+    dtype (modules.py:462-474)."""
+    b = x.shape[0]
+    w = self.window_size
+    k_pos, q_pos = self._ring_positions(cache.num_tokens, 1)
+    ring_ok = _visible(q_pos, k_pos, w)                    # [B, 1, window]
+    qh = q[:, 0]                                           # [B, heads, hd]
+    ring_k, ring_v = cache.keys[:, :, 0], cache.values[:, :, 0]  # [B, w, hd]
+    scale = self.head_dim ** -0.5
+    s_ring = torch.bmm(qh, ring_k.transpose(1, 2)) * scale  # [B, heads, w]
+    s_self = (qh * k[:, 0]).sum(-1, keepdim=True).to(qh.dtype) * scale
+    s_ring = s_ring.float().masked_fill(~ring_ok, float("-inf"))
+    probs = torch.softmax(torch.cat([s_ring, s_self.float()], dim=-1),
+                          dim=-1).type_as(x)
+    out = torch.bmm(probs[..., :w], ring_v) + probs[..., w:] * v[:, 0]
+    out = self.proj_final(out.reshape(b, 1, self.width))
+    if not return_cache:
+      return out, None
+    rows = torch.arange(b, device=x.device)
+    at = (cache.num_tokens % w).long()
+    cache.keys[rows, at] = k[:, 0]
+    cache.values[rows, at] = v[:, 0]
+    cache.num_tokens[:] = cache.num_tokens + 1
+    return out, cache
 
   @classmethod
   def init_cache(cls, batch_size, window_size, heads_dim, dtype, device=None):

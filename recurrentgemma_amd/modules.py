@@ -41,9 +41,12 @@ _MIN_GROUPS_FOR_SINGLE_LAUNCH = 144
 @torch.no_grad()
 def recurrent_core(conv_1d: layers.Conv1D, rg_lru: layers.RGLRU, x,
                    segment_pos, cache: RecurrentBlockCache | None = None,
-                   return_cache: bool = True):
+                   return_cache: bool = True, in_place: bool = False):
   """conv_1d -> rg_lru exactly as RecurrentBlock.forward chains them
-  (modules.py:632-643), fused.  Returns (y, RecurrentBlockCache | None)."""
+  (modules.py:632-643), fused.  Returns (y, RecurrentBlockCache | None).
+  in_place (decode only): the step overwrites the tensors of `cache` and
+  returns them, for callers that replay a captured step on fixed buffers; the
+  default returns new tensors like the reference."""
   bs, l, _ = x.shape
   assert segment_pos.shape == (bs, l)
   fused = conv_1d.temporal_width == 4
@@ -55,11 +58,13 @@ def recurrent_core(conv_1d: layers.Conv1D, rg_lru: layers.RGLRU, x,
       y, h, conv_state = ops.recurrent_step(
           x, segment_pos, cache.conv1d_state, cache.rg_lru_state, conv_1d.w,
           conv_1d.b, rg_lru.input_gate.w, rg_lru.input_gate.b, rg_lru.a_gate.w,
-          rg_lru.a_gate.b, rg_lru.a_param)
+          rg_lru.a_gate.b, rg_lru.a_param, in_place=in_place)
       if not return_cache:
         return y, None
       return y, RecurrentBlockCache(rg_lru_state=h, conv1d_state=conv_state)
   if not fused or cache is not None:
+    if in_place:
+      raise ValueError("in-place decode needs the fused step (conv width 4)")
     xc, conv_state = conv_1d(x, segment_pos,
                              None if cache is None else cache.conv1d_state,
                              return_cache)
@@ -108,6 +113,10 @@ class RecurrentBlock(nn.Module):
                                  device=device, dtype=dtype)
     self.rg_lru = layers.RGLRU(width=self.lru_width, num_heads=self.num_heads,
                                device=device, dtype=dtype)
+    # True: a cached single-token call updates the cache tensors it is given
+    # instead of returning new ones (set by callers that replay a captured
+    # decode step on fixed buffers)
+    self.decode_in_place = False
     self.reset_parameters()
 
   def reset_parameters(self) -> None:
@@ -131,8 +140,9 @@ class RecurrentBlock(nn.Module):
   def forward(self, x, segment_pos, cache=None, return_cache=True):
     y = self.linear_y(x)
     x = self.linear_x(x)
-    x, new_cache = recurrent_core(self.conv_1d, self.rg_lru, x, segment_pos,
-                                  cache, return_cache)
+    x, new_cache = recurrent_core(
+        self.conv_1d, self.rg_lru, x, segment_pos, cache, return_cache,
+        in_place=self.decode_in_place and cache is not None and return_cache)
     x = ops.gelu_mul(x, y)  # x * gelu(y), one pass (modules.py:627-628, 644)
     x = self.linear_out(x)
     if not return_cache:

@@ -27,15 +27,76 @@ class SamplerOutput(NamedTuple):
   tokens: list[torch.Tensor]
 
 
+class _CapturedStep:
+  """One cached single-token pass through the model, captured once as a HIP
+  graph on fixed buffers (token ids, positions, every block's cache, logits)
+  and replayed per generated token: the ~1300 kernel launches of a step cost
+  one graph launch.  The caches are updated in place inside the graph, the
+  positions advance inside it too.  Token selection stays outside (a reduction
+  over the whole vocabulary may clear its scratch with a memset node, which
+  must not be recorded into a graph on this platform)."""
+
+  def __init__(self, model, batch_size, dtype, device):
+    self.model = model
+    ints = dict(device=device, dtype=torch.int32)
+    self.tokens = torch.zeros((batch_size, 1), **ints)
+    self.pos = torch.ones((batch_size, 1), **ints)
+    self.cache = model.init_cache(batch_size, dtype, device=device)
+    self._recurrent = [b.recurrent_block for b in model.blocks
+                       if hasattr(b, "recurrent_block")]
+    with self._in_place():
+      side = torch.cuda.Stream(device=device)
+      side.wait_stream(torch.cuda.current_stream(device))
+      with torch.cuda.stream(side):
+        for _ in range(2):  # library handles, packed weights, allocator pools
+          model(self.tokens, self.pos, self.cache)
+      torch.cuda.current_stream(device).wait_stream(side)
+      self.graph = torch.cuda.CUDAGraph()
+      with torch.cuda.graph(self.graph):
+        self.logits, _ = model(self.tokens, self.pos, self.cache)
+        self.pos.add_(1)
+
+  def _in_place(self):
+    blocks = self._recurrent
+
+    class _Ctx:
+      def __enter__(self):
+        self.old = [b.decode_in_place for b in blocks]
+        for b in blocks:
+          b.decode_in_place = True
+
+      def __exit__(self, *exc):
+        for b, o in zip(blocks, self.old):
+          b.decode_in_place = o
+
+    return _Ctx()
+
+  def load(self, cache, pos):
+    """Takes over the state a prompt pass left behind."""
+    for name, c in cache.items():
+      for dst, src in zip(self.cache[name], c):
+        dst.copy_(src)
+    self.pos.copy_(pos)
+
+  def step(self, tokens):
+    self.tokens.copy_(tokens)
+    self.graph.replay()
+    return self.logits
+
+
 class Sampler:
   """Sampler for a Griffin model (greedy, or from the categorical
-  distribution of the logits)."""
+  distribution of the logits).  use_graph: decode steps replay a captured HIP
+  graph (same kernels, same results as the eager loop)."""
 
   def __init__(self, model: griffin_lib.Griffin, vocab=None,
-               greedy_sampling: bool = True, is_it_model: bool = False):
+               greedy_sampling: bool = True, is_it_model: bool = False,
+               use_graph: bool = False):
     self.model = model
     self.vocab = vocab
     self.greedy_sampling = greedy_sampling
+    self.use_graph = use_graph
+    self._captured = {}
     self._is_it_model = is_it_model
     self._eos_token = (None if vocab is None else torch.tensor(
         [vocab.eos_id()], device=self.device))
@@ -117,9 +178,19 @@ class Sampler:
 
     pos = positions[:, -1:] + 1
     done = False
+    captured = None
+    if self.use_graph and total_generation_steps > 2:
+      captured = self._captured.get(bsz)
+      if captured is None:
+        captured = self._captured[bsz] = _CapturedStep(model, bsz, self.dtype,
+                                                       dev)
+      captured.load(cache, pos)
     while total_generation_steps > 1 and step < total - 1 and not done:
-      logits, cache = model(tokens_buffer[:, step][:, None], pos, cache,
-                            return_logits=True, return_cache=True)
+      if captured is not None:
+        logits = captured.step(tokens_buffer[:, step][:, None])
+      else:
+        logits, cache = model(tokens_buffer[:, step][:, None], pos, cache,
+                              return_logits=True, return_cache=True)
       nxt = self._pick(logits[:, 0])
       tokens_buffer[:, step + 1] = nxt
       if logits_buffer is not None:
