@@ -173,6 +173,16 @@ int rg_recurrent_step(const void* x, const void* segpos, int segpos_is_i64,
 int rg_gelu_mul(const void* a, const void* g, void* out, int64_t n, int dtype,
                 void* stream);
 
+/* RMSNorm of the residual stack around the recurrent block, one pass:
+ * out[r, :] = x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * (scale + 1) for
+ * recurrentgemma/torch/layers.py:65-73 (RMSNorm.forward; eps 1e-6 there).
+ * x, out [rows, width], scale [width], all in `dtype`.  bf16 reproduces the
+ * reference's chain of bf16 tensors: x^2, their mean (float32 sum), var + eps,
+ * the rsqrt, x * rsqrt and scale + 1 are each rounded to bf16.  out may alias
+ * x. */
+int rg_rms_norm(const void* x, const void* scale, void* out, int64_t rows,
+                int width, float eps, int dtype, void* stream);
+
 /* The same decode step in ONE launch, for bf16 with 256-wide heads (no
  * counterpart call in the reference: it is RecurrentBlock.forward with a
  * cache, modules.py:632-643, after a one-time re-layout of the two gate

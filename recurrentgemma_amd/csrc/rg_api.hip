@@ -368,6 +368,19 @@ int rg_gelu_mul(const void* a, const void* g, void* out, int64_t n, int dtype,
       __func__, rg::launch_gelu_mul(a, g, out, n, dtype, (hipStream_t)stream));
 }
 
+int rg_rms_norm(const void* x, const void* scale, void* out, int64_t rows,
+                int width, float eps, int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(rows > 0 && width > 0, "%s: rows=%lld width=%d must be positive",
+             __func__, (long long)rows, width);
+  RG_CHECK_PTR(x);
+  RG_CHECK_PTR(scale);
+  RG_CHECK_PTR(out);
+  return launch_status(__func__,
+                       rg::launch_rms_norm(x, scale, out, rows, width, eps,
+                                           dtype, (hipStream_t)stream));
+}
+
 size_t rg_packed_gate_weights_bytes(int W, int H, int dtype) {
   if (W <= 0 || H <= 0 || W % H != 0 || dtype != RG_DTYPE_BF16 || W / H != 256)
     return 0;

@@ -73,6 +73,38 @@ gelu_mul_f32_kernel(const f32x4* __restrict__ a, const f32x4* __restrict__ g,
     out_tail[threadIdx.x] = one(a_tail[threadIdx.x], g_tail[threadIdx.x]);
 }
 
+// RMSNorm of the residual stack (recurrentgemma/torch/layers.py:65-73):
+//   var = mean(x^2);  out = x * rsqrt(var + eps) * (scale + 1)
+// with every step rounded to the activation dtype like the reference's chain
+// of tensor ops (for bf16: x^2, the mean, var + eps, the rsqrt, x * rsqrt and
+// scale + 1 are each a bf16 tensor there; sums accumulate in float32).  One
+// workgroup per row; the row is read twice, the second time from cache.
+template <typename T>
+__global__ void __launch_bounds__(256)
+rms_norm_kernel(const T* __restrict__ x, const T* __restrict__ scale,
+                T* __restrict__ out, int width, float eps) {
+  __shared__ float partial[4];
+  const T* xr = x + (int64_t)blockIdx.x * width;
+  T* outr = out + (int64_t)blockIdx.x * width;
+  float sum = 0.0f;
+  for (int i = threadIdx.x; i < width; i += 256) {
+    const float v = load_scalar<T>(xr + i);
+    sum += round_act<T>(v * v);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+  if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = sum;
+  __syncthreads();
+  sum = (partial[0] + partial[1]) + (partial[2] + partial[3]);
+  const float var = round_act<T>(sum * (1.0f / (float)width));
+  const float r = round_act<T>(1.0f / sqrtf(round_act<T>(var + eps)));
+  for (int i = threadIdx.x; i < width; i += 256) {
+    const float v = load_scalar<T>(xr + i);
+    const float g = round_act<T>(load_scalar<T>(scale + i) + 1.0f);
+    store_scalar<T>(outr + i, round_act<T>(v * r) * g);
+  }
+}
+
 }  // namespace
 
 hipError_t launch_gelu_mul(const void* a, const void* g, void* out, int64_t n,
@@ -93,6 +125,19 @@ hipError_t launch_gelu_mul(const void* a, const void* g, void* out, int64_t n,
         (const uint16_t*)a + items * per, (const uint16_t*)g + items * per,
         (uint16_t*)out + items * per, tail);
   }
+  return hipGetLastError();
+}
+
+hipError_t launch_rms_norm(const void* x, const void* scale, void* out,
+                           int64_t rows, int width, float eps, int dtype,
+                           hipStream_t s) {
+  if (rows > 0x7fffffff) return hipErrorInvalidValue;
+  if (dtype == 0)
+    rms_norm_kernel<float><<<dim3((unsigned)rows), 256, 0, s>>>(
+        (const float*)x, (const float*)scale, (float*)out, width, eps);
+  else
+    rms_norm_kernel<uint16_t><<<dim3((unsigned)rows), 256, 0, s>>>(
+        (const uint16_t*)x, (const uint16_t*)scale, (uint16_t*)out, width, eps);
   return hipGetLastError();
 }
 

@@ -110,6 +110,10 @@ hipError_t launch_block_step_bf16(const StepArgs& a, hipStream_t s);
 // out[i] = a[i] * gelu_tanh(g[i]) over n elements (out may alias a or g).
 hipError_t launch_gelu_mul(const void* a, const void* g, void* out, int64_t n,
                            int dtype, hipStream_t s);
+// out[r, :] = x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * (scale + 1)
+hipError_t launch_rms_norm(const void* x, const void* scale, void* out,
+                           int64_t rows, int width, float eps, int dtype,
+                           hipStream_t s);
 hipError_t launch_pack_gate_weights(const void* w_x, const void* w_a,
                                     void* packed, int H, hipStream_t s);
 

@@ -23,6 +23,7 @@ import torch
 from torch import nn
 
 from recurrentgemma_amd import modules
+from recurrentgemma_amd import ops
 
 _MAX_WAVELENGTH = 10_000
 
@@ -118,9 +119,9 @@ class RMSNorm(nn.Module):
     torch.nn.init.zeros_(self.scale)
 
   def forward(self, x):
-    # the reference computes every step in the activation dtype
-    var = torch.mean(torch.square(x), dim=-1, keepdim=True)
-    return x * torch.rsqrt(var + self.eps) * (self.scale + 1)
+    # one kernel; every step rounded to the activation dtype like the
+    # reference's chain of tensor ops
+    return ops.rms_norm(x, self.scale, self.eps)
 
 
 class _StackedLinear(nn.Module):
@@ -172,7 +173,7 @@ class MLPBlock(nn.Module):
 
   def forward(self, x):
     gate, up = self.ffw_up(x)
-    return self.ffw_down(modules.gelu(gate) * up)
+    return self.ffw_down(ops.gelu_mul(up, gate))  # gelu(gate) * up, one pass
 
 
 def _rope(x, positions, max_wavelength=_MAX_WAVELENGTH):

@@ -274,6 +274,21 @@ def gelu_mul(a, g):
   return out
 
 
+def rms_norm(x, scale, eps=1e-6):
+  """x * rsqrt(mean(x^2, -1) + eps) * (scale + 1), one pass."""
+  x = _dev(x, "x")
+  _same(x.dtype, x.device, scale=scale)
+  scale = _dev(scale, "scale")
+  width = x.shape[-1]
+  assert scale.shape == (width,)
+  out = torch.empty_like(x)
+  with torch.cuda.device(x.device):
+    _lib.check(_lib.lib().rg_rms_norm(_p(x), _p(scale), _p(out),
+                                      x.numel() // width, width, eps,
+                                      _dtype_code(x), _stream(x)))
+  return out
+
+
 _packed_weights = {}  # (id(w_x), id(w_a)) -> (ref_x, ref_a, stamp, packed)
 
 

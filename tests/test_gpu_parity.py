@@ -642,6 +642,40 @@ def test_gelu_mul(dtype, n):
     assert torch.equal(dst.cpu(), got)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,width", [(1, 1), (3, 7), (5, 256), (64, 2560),
+                                        (2 * 33, 4096), (2, 10007)])
+def test_rms_norm(dtype, rows, width):
+  """rg_rms_norm against the reference's chain of tensor ops (layers.py:65-73)
+  evaluated by torch in the same dtype: fp32 on the CPU, 1e-5 of the largest
+  magnitude; bf16 by torch's own GPU kernels (torch's CPU rsqrt rounds the
+  square root to bf16 before taking the reciprocal, its GPU kernel and this
+  one round once), one bf16 ulp per element: the sum of squares is taken in a
+  different order, which can move the rounded mean or rsqrt by one ulp, and
+  that moves every element of the row."""
+  _announce("rms_norm", dtype, rows, width)
+  gen = torch.Generator().manual_seed(rows * 131 + width)
+  x = (2.0 * torch.randn(rows, width, generator=gen)).to(dtype)
+  scale = (0.3 * torch.randn(width, generator=gen)).to(dtype)
+  eps = 1e-6
+
+  def chain(x, scale):
+    var = torch.mean(torch.square(x), dim=-1, keepdim=True)
+    return x * torch.rsqrt(var + eps) * (scale + 1)
+
+  got = ops.rms_norm(_dev(x), _dev(scale), eps).cpu()
+  assert got.dtype == dtype and got.shape == x.shape
+  if dtype == torch.float32:
+    assert helpers.max_rel(got, chain(x, scale)) < 1e-5
+  else:
+    want = chain(_dev(x), _dev(scale)).cpu()
+    err = (got.float() - want.float()).abs()
+    assert (err <= want.float().abs() * 2.0 ** -7 + 1e-30).all()
+    assert (err > 0).float().mean() < 0.35
+  x3 = x.reshape(1, rows, width)  # leading dimensions are rows
+  assert torch.equal(ops.rms_norm(_dev(x3), _dev(scale), eps).cpu()[0], got)
+
+
 # --------------------------------- full-size, size-independent properties --
 
 
