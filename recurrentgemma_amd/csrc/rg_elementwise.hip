@@ -105,6 +105,59 @@ rms_norm_kernel(const T* __restrict__ x, const T* __restrict__ scale,
   }
 }
 
+// bf16 rows of up to 4096 elements whose width is a multiple of 8: 16-byte
+// lanes, the row stays in registers between the two passes (one read, one
+// write; the scalar kernel above re-reads through the cache and moved
+// 1.7 TB/s on 131 072 rows of 2560).
+__global__ void __launch_bounds__(256)
+rms_norm_bf16_rows_kernel(const u32x4* __restrict__ x,
+                          const u32x4* __restrict__ scale,
+                          u32x4* __restrict__ out, int chunks, float inv_width,
+                          float eps) {
+  __shared__ float partial[4];
+  const u32x4* xr = x + (int64_t)blockIdx.x * chunks;
+  u32x4* outr = out + (int64_t)blockIdx.x * chunks;
+  u32x4 v[2];
+  float sum = 0.0f;
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    const int i = threadIdx.x + c * 256;
+    v[c] = u32x4{0u, 0u, 0u, 0u};
+    if (i < chunks) v[c] = __builtin_nontemporal_load(xr + i);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float lo = __uint_as_float(v[c][k] << 16);
+      const float hi = __uint_as_float(v[c][k] & 0xffff0000u);
+      sum += round_to_bf16(lo * lo);
+      sum += round_to_bf16(hi * hi);
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+  if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = sum;
+  __syncthreads();
+  sum = (partial[0] + partial[1]) + (partial[2] + partial[3]);
+  const float var = round_to_bf16(sum * inv_width);
+  const float r = round_to_bf16(1.0f / sqrtf(round_to_bf16(var + eps)));
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    const int i = threadIdx.x + c * 256;
+    if (i >= chunks) continue;
+    const u32x4 g = scale[i];
+    u32x4 o;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float lo = round_to_bf16(__uint_as_float(v[c][k] << 16) * r) *
+                       round_to_bf16(__uint_as_float(g[k] << 16) + 1.0f);
+      const float hi =
+          round_to_bf16(__uint_as_float(v[c][k] & 0xffff0000u) * r) *
+          round_to_bf16(__uint_as_float(g[k] & 0xffff0000u) + 1.0f);
+      o[k] = pack_bf16x2(lo, hi);
+    }
+    __builtin_nontemporal_store(o, outr + i);
+  }
+}
+
 }  // namespace
 
 hipError_t launch_gelu_mul(const void* a, const void* g, void* out, int64_t n,
@@ -132,9 +185,15 @@ hipError_t launch_rms_norm(const void* x, const void* scale, void* out,
                            int64_t rows, int width, float eps, int dtype,
                            hipStream_t s) {
   if (rows > 0x7fffffff) return hipErrorInvalidValue;
+  const bool aligned =
+      (((uintptr_t)x | (uintptr_t)scale | (uintptr_t)out) & 15) == 0;
   if (dtype == 0)
     rms_norm_kernel<float><<<dim3((unsigned)rows), 256, 0, s>>>(
         (const float*)x, (const float*)scale, (float*)out, width, eps);
+  else if (width % 8 == 0 && width <= 4096 && aligned)
+    rms_norm_bf16_rows_kernel<<<dim3((unsigned)rows), 256, 0, s>>>(
+        (const u32x4*)x, (const u32x4*)scale, (u32x4*)out, width / 8,
+        1.0f / (float)width, eps);
   else
     rms_norm_kernel<uint16_t><<<dim3((unsigned)rows), 256, 0, s>>>(
         (const uint16_t*)x, (const uint16_t*)scale, (uint16_t*)out, width, eps);
