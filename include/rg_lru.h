@@ -183,6 +183,48 @@ int rg_gelu_mul(const void* a, const void* g, void* out, int64_t n, int dtype,
 int rg_rms_norm(const void* x, const void* scale, void* out, int64_t rows,
                 int width, float eps, int dtype, void* stream);
 
+/* ---- the local-attention block around its matrix products ----------------
+ * Not part of the recurrent path: the steps of the attention block that the
+ * reference spells as dozens of elementwise tensor ops per block and decoded
+ * token, one kernel each.  Projections, scores and the weighted sum of the
+ * values remain batched GEMMs of the caller. */
+
+/* Rotary embedding on the first half of the head dimension
+ * (recurrentgemma/torch/modules.py:52-83 `_apply_rope`): x, out
+ * [rows, heads, head_dim] in `dtype`, positions [rows] int32/int64, inv_freq
+ * [head_dim / 4] float32 = 1 / max_wavelength^(2 i / (head_dim / 2)).  Element
+ * i < head_dim/4 pairs with element i + head_dim/4; sin, cos and every product
+ * are rounded to `dtype` like the reference's tensors. */
+int rg_rope(const void* x, const void* positions, int positions_is_i64,
+            const float* inv_freq, void* out, int64_t rows, int heads,
+            int head_dim, int dtype, void* stream);
+
+/* Masked softmax of one decoded token against the ring cache and itself
+ * (modules.py:152-183 `_compute_cache_mask`, :462-470): scores
+ * [B, heads, window] = q . k of the ring slots, unscaled, in `dtype`; q
+ * [B, heads, head_dim] and k_new [B, head_dim] after rg_rope; num_tokens [B]
+ * int32, tokens seen before this one; probs [B, heads, window + 1], last
+ * column = the new token.  Scores are scaled and rounded to `dtype`, the
+ * softmax is taken in float32 over the ring slots that were ever written and
+ * the new token, probabilities are rounded to `dtype`. */
+int rg_attention_decode_probs(const void* scores, const void* q,
+                              const void* k_new, const int32_t* num_tokens,
+                              void* probs, int B, int heads, int head_dim,
+                              int window, float scale, int dtype,
+                              void* stream);
+
+/* out = from_ring + probs[..., window] * v_new (modules.py:471-474), then, if
+ * update_cache, the ring update of modules.py:186-216 (`n_fill == 1`): k_new,
+ * v_new into slot num_tokens % window of ring_keys / ring_values
+ * [B, window, head_dim], num_tokens += 1.  from_ring, out [B, heads, head_dim]
+ * (out may alias from_ring). */
+int rg_attention_decode_finish(const void* from_ring, const void* probs,
+                               const void* k_new, const void* v_new, void* out,
+                               void* ring_keys, void* ring_values,
+                               int32_t* num_tokens, int B, int heads,
+                               int head_dim, int window, int update_cache,
+                               int dtype, void* stream);
+
 /* The same decode step in ONE launch, for bf16 with 256-wide heads (no
  * counterpart call in the reference: it is RecurrentBlock.forward with a
  * cache, modules.py:632-643, after a one-time re-layout of the two gate

@@ -44,6 +44,10 @@ SIGNATURES = {
     "rg_gelu_mul": (_i, [_vp, _vp, _vp, ctypes.c_int64, _i, _vp]),
     "rg_rms_norm": (_i, [_vp, _vp, _vp, ctypes.c_int64, _i, ctypes.c_float, _i,
                          _vp]),
+    "rg_rope": (_i, [_vp, _vp, _i, _vp, _vp, ctypes.c_int64, _i, _i, _i, _vp]),
+    "rg_attention_decode_probs": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i,
+                                       ctypes.c_float, _i, _vp]),
+    "rg_attention_decode_finish": (_i, [_vp] * 8 + [_i] * 6 + [_vp]),
     "rg_packed_gate_weights_bytes": (_sz, [_i, _i, _i]),
     "rg_pack_gate_weights": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "rg_recurrent_step_packed": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp,

@@ -381,6 +381,76 @@ int rg_rms_norm(const void* x, const void* scale, void* out, int64_t rows,
                                            dtype, (hipStream_t)stream));
 }
 
+int rg_rope(const void* x, const void* positions, int positions_is_i64,
+            const float* inv_freq, void* out, int64_t rows, int heads,
+            int head_dim, int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(rows > 0 && heads > 0 && head_dim > 0,
+             "%s: rows=%lld heads=%d head_dim=%d must be positive", __func__,
+             (long long)rows, heads, head_dim);
+  RG_REQUIRE(head_dim % 4 == 0, "%s: head_dim=%d is not a multiple of 4",
+             __func__, head_dim);
+  RG_CHECK_PTR(x);
+  RG_CHECK_PTR(positions);
+  RG_CHECK_PTR(inv_freq);
+  RG_CHECK_PTR(out);
+  RG_REQUIRE(out != x, "%s: out must not alias x", __func__);
+  return launch_status(
+      __func__, rg::launch_rope(x, positions, positions_is_i64 ? 1 : 0,
+                                inv_freq, out, rows, heads, head_dim, dtype,
+                                (hipStream_t)stream));
+}
+
+int rg_attention_decode_probs(const void* scores, const void* q,
+                              const void* k_new, const int32_t* num_tokens,
+                              void* probs, int B, int heads, int head_dim,
+                              int window, float scale, int dtype,
+                              void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(B > 0 && heads > 0 && head_dim > 0 && window > 0,
+             "%s: B=%d heads=%d head_dim=%d window=%d must be positive",
+             __func__, B, heads, head_dim, window);
+  RG_CHECK_PTR(scores);
+  RG_CHECK_PTR(q);
+  RG_CHECK_PTR(k_new);
+  RG_CHECK_PTR(num_tokens);
+  RG_CHECK_PTR(probs);
+  return launch_status(
+      __func__,
+      rg::launch_attn_decode_probs(scores, q, k_new, num_tokens, probs, B,
+                                   heads, head_dim, window, scale, dtype,
+                                   (hipStream_t)stream));
+}
+
+int rg_attention_decode_finish(const void* from_ring, const void* probs,
+                               const void* k_new, const void* v_new, void* out,
+                               void* ring_keys, void* ring_values,
+                               int32_t* num_tokens, int B, int heads,
+                               int head_dim, int window, int update_cache,
+                               int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(B > 0 && heads > 0 && head_dim > 0 && window > 0,
+             "%s: B=%d heads=%d head_dim=%d window=%d must be positive",
+             __func__, B, heads, head_dim, window);
+  RG_CHECK_PTR(from_ring);
+  RG_CHECK_PTR(probs);
+  RG_CHECK_PTR(k_new);
+  RG_CHECK_PTR(v_new);
+  RG_CHECK_PTR(out);
+  RG_CHECK_PTR(num_tokens);
+  if (update_cache) {
+    RG_CHECK_PTR(ring_keys);
+    RG_CHECK_PTR(ring_values);
+  }
+  return launch_status(
+      __func__,
+      rg::launch_attn_decode_finish(from_ring, probs, k_new, v_new, out,
+                                    ring_keys, ring_values, num_tokens, B,
+                                    heads, head_dim, window,
+                                    update_cache ? 1 : 0, dtype,
+                                    (hipStream_t)stream));
+}
+
 size_t rg_packed_gate_weights_bytes(int W, int H, int dtype) {
   if (W <= 0 || H <= 0 || W % H != 0 || dtype != RG_DTYPE_BF16 || W / H != 256)
     return 0;

@@ -1,0 +1,198 @@
+// The small steps of the local-attention block around its matrix products
+// (recurrentgemma/torch/modules.py:52-83 rotary embedding, :152-183 positions
+// held by the ring cache, :186-216 ring update, :462-474 masked softmax): one
+// kernel each instead of a few dozen elementwise launches per block and
+// decoded token.  The products themselves (projections, scores, weighted sum
+// of the values) stay batched GEMMs of the caller.  Every step rounds to the
+// activation dtype where the reference's chain of tensor ops does.
+#include "rg_common.h"
+#include "rg_internal.h"
+
+namespace rg {
+namespace {
+
+__device__ __forceinline__ float position_as_float(const void* pos, int kind,
+                                                   int64_t i) {
+  return kind == kSegI64 ? (float)reinterpret_cast<const int64_t*>(pos)[i]
+                         : (float)reinterpret_cast<const int32_t*>(pos)[i];
+}
+
+// x, out [rows, n, hd]; positions [rows]; inv_freq [hd / 4] float32.
+// First half of the head dimension: element i pairs with element i + hd/4,
+// rotated by position * inv_freq[i]; second half copied.
+template <typename T>
+__global__ void __launch_bounds__(256)
+rope_kernel(const T* __restrict__ x, const void* __restrict__ pos,
+            int pos_kind, const float* __restrict__ inv_freq,
+            T* __restrict__ out, int64_t total, int n, int hd) {
+  // products and their sum are separate tensors in the reference: no fused
+  // multiply-add (matters in float32, where nothing is rounded in between)
+#pragma clang fp contract(off)
+  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const int d = (int)(e % hd);
+  const int half = hd / 2, quarter = hd / 4;
+  if (d >= half) {
+    out[e] = x[e];
+    return;
+  }
+  const int64_t row = e / ((int64_t)n * hd);
+  const int i = d % quarter;
+  const float angle = position_as_float(pos, pos_kind, row) * inv_freq[i];
+  const float s = round_act<T>(sinf(angle)), c = round_act<T>(cosf(angle));
+  const int64_t base = e - d;
+  const float lo = load_scalar<T>(x + base + i);
+  const float hi = load_scalar<T>(x + base + i + quarter);
+  const float v = d < quarter
+                      ? round_act<T>(lo * c) - round_act<T>(hi * s)
+                      : round_act<T>(hi * c) + round_act<T>(lo * s);
+  store_scalar<T>(out + e, v);
+}
+
+__device__ __forceinline__ float block_reduce(float v, float* scratch,
+                                              bool take_max) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float o = __shfl_xor(v, off, 64);
+    v = take_max ? fmaxf(v, o) : v + o;
+  }
+  __syncthreads();  // scratch may still be read from the previous reduction
+  if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
+  __syncthreads();
+  const float a = scratch[0], b = scratch[1], c = scratch[2], d = scratch[3];
+  return take_max ? fmaxf(fmaxf(a, b), fmaxf(c, d)) : (a + b) + (c + d);
+}
+
+// One workgroup per (row, head).  scores [B, heads, window]: q . k of the ring
+// slots as the caller's batched product left them (activation dtype,
+// unscaled); q [B, heads, hd], k_new [B, hd] (both after the rotary
+// embedding); num_tokens [B] tokens seen before this one; probs
+// [B, heads, window + 1]: softmax over the visible ring slots and, last
+// column, the new token itself.  Slot j holds the largest position congruent
+// to j below num_tokens, so it is visible iff it was ever written: j <
+// num_tokens, or the ring has wrapped.
+template <typename T>
+__global__ void __launch_bounds__(256)
+attn_decode_probs_kernel(const T* __restrict__ scores, const T* __restrict__ q,
+                         const T* __restrict__ k_new,
+                         const int32_t* __restrict__ num_tokens,
+                         T* __restrict__ probs, int heads, int hd, int window,
+                         float scale) {
+  __shared__ float scratch[4];
+  const int b = blockIdx.x / heads;
+  const int nt = num_tokens[b];
+  const T* srow = scores + (int64_t)blockIdx.x * window;
+  const T* qrow = q + (int64_t)blockIdx.x * hd;
+  const T* krow = k_new + (int64_t)b * hd;
+  T* prow = probs + (int64_t)blockIdx.x * (window + 1);
+  float dot = 0.0f;
+  for (int d = threadIdx.x; d < hd; d += 256)
+    dot += load_scalar<T>(qrow + d) * load_scalar<T>(krow + d);
+  dot = block_reduce(dot, scratch, false);
+  const float self = round_act<T>(round_act<T>(dot) * scale);
+  const bool wrapped = nt >= window;
+  float mx = self;
+  for (int j = threadIdx.x; j < window; j += 256)
+    if (wrapped || j < nt)
+      mx = fmaxf(mx, round_act<T>(load_scalar<T>(srow + j) * scale));
+  mx = block_reduce(mx, scratch, true);
+  float sum = 0.0f;
+  for (int j = threadIdx.x; j < window; j += 256)
+    if (wrapped || j < nt)
+      sum += expf(round_act<T>(load_scalar<T>(srow + j) * scale) - mx);
+  if (threadIdx.x == 0) sum += expf(self - mx);
+  sum = block_reduce(sum, scratch, false);
+  const float inv = 1.0f / sum;
+  for (int j = threadIdx.x; j < window; j += 256) {
+    float p = 0.0f;
+    if (wrapped || j < nt)
+      p = expf(round_act<T>(load_scalar<T>(srow + j) * scale) - mx) * inv;
+    store_scalar<T>(prow + j, p);
+  }
+  if (threadIdx.x == 0) store_scalar<T>(prow + window, expf(self - mx) * inv);
+}
+
+// One workgroup per row.  from_ring [B, heads, hd]: probs[..., :window] times
+// the ring's values (the caller's batched product); adds the new token's share
+// probs[..., window] * v_new, then (update != 0) stores the new key and value
+// in slot num_tokens % window and counts the token.
+template <typename T>
+__global__ void __launch_bounds__(256)
+attn_decode_finish_kernel(const T* __restrict__ from_ring,
+                          const T* __restrict__ probs,
+                          const T* __restrict__ k_new,
+                          const T* __restrict__ v_new, T* __restrict__ out,
+                          T* __restrict__ ring_k, T* __restrict__ ring_v,
+                          int32_t* __restrict__ num_tokens, int heads, int hd,
+                          int window, int update) {
+  const int b = blockIdx.x;
+  const int nt = num_tokens[b];
+  const T* vrow = v_new + (int64_t)b * hd;
+  for (int e = threadIdx.x; e < heads * hd; e += 256) {
+    const int h = e / hd, d = e % hd;
+    const float p = load_scalar<T>(
+        probs + ((int64_t)b * heads + h) * (window + 1) + window);
+    const int64_t at = (int64_t)b * heads * hd + e;
+    store_scalar<T>(out + at, load_scalar<T>(from_ring + at) +
+                                  round_act<T>(p * load_scalar<T>(vrow + d)));
+  }
+  if (!update) return;
+  const int64_t slot = ((int64_t)b * window + nt % window) * hd;
+  for (int d = threadIdx.x; d < hd; d += 256) {
+    ring_k[slot + d] = k_new[(int64_t)b * hd + d];
+    ring_v[slot + d] = vrow[d];
+  }
+  __syncthreads();  // every thread has read num_tokens[b]
+  if (threadIdx.x == 0) num_tokens[b] = nt + 1;
+}
+
+template <typename F>
+hipError_t by_dtype(int dtype, F&& f) {
+  if (dtype == 0) f((float*)nullptr);
+  else f((uint16_t*)nullptr);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_rope(const void* x, const void* pos, int pos_kind,
+                       const float* inv_freq, void* out, int64_t rows, int n,
+                       int hd, int dtype, hipStream_t s) {
+  const int64_t total = rows * n * hd;
+  const int64_t blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffff) return hipErrorInvalidValue;
+  return by_dtype(dtype, [&](auto* tag) {
+    typedef std::remove_pointer_t<decltype(tag)> T;
+    rope_kernel<T><<<dim3((unsigned)blocks), 256, 0, s>>>(
+        (const T*)x, pos, pos_kind, inv_freq, (T*)out, total, n, hd);
+  });
+}
+
+hipError_t launch_attn_decode_probs(const void* scores, const void* q,
+                                    const void* k_new,
+                                    const int32_t* num_tokens, void* probs,
+                                    int B, int heads, int hd, int window,
+                                    float scale, int dtype, hipStream_t s) {
+  return by_dtype(dtype, [&](auto* tag) {
+    typedef std::remove_pointer_t<decltype(tag)> T;
+    attn_decode_probs_kernel<T><<<dim3((unsigned)(B * heads)), 256, 0, s>>>(
+        (const T*)scores, (const T*)q, (const T*)k_new, num_tokens, (T*)probs,
+        heads, hd, window, scale);
+  });
+}
+
+hipError_t launch_attn_decode_finish(const void* from_ring, const void* probs,
+                                     const void* k_new, const void* v_new,
+                                     void* out, void* ring_k, void* ring_v,
+                                     int32_t* num_tokens, int B, int heads,
+                                     int hd, int window, int update, int dtype,
+                                     hipStream_t s) {
+  return by_dtype(dtype, [&](auto* tag) {
+    typedef std::remove_pointer_t<decltype(tag)> T;
+    attn_decode_finish_kernel<T><<<dim3((unsigned)B), 256, 0, s>>>(
+        (const T*)from_ring, (const T*)probs, (const T*)k_new, (const T*)v_new,
+        (T*)out, (T*)ring_k, (T*)ring_v, num_tokens, heads, hd, window, update);
+  });
+}
+
+}  // namespace rg

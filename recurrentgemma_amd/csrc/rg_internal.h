@@ -114,6 +114,22 @@ hipError_t launch_gelu_mul(const void* a, const void* g, void* out, int64_t n,
 hipError_t launch_rms_norm(const void* x, const void* scale, void* out,
                            int64_t rows, int width, float eps, int dtype,
                            hipStream_t s);
+// Steps of the local-attention block around its matrix products
+// (rg_attention.hip).
+hipError_t launch_rope(const void* x, const void* pos, int pos_kind,
+                       const float* inv_freq, void* out, int64_t rows, int n,
+                       int hd, int dtype, hipStream_t s);
+hipError_t launch_attn_decode_probs(const void* scores, const void* q,
+                                    const void* k_new,
+                                    const int32_t* num_tokens, void* probs,
+                                    int B, int heads, int hd, int window,
+                                    float scale, int dtype, hipStream_t s);
+hipError_t launch_attn_decode_finish(const void* from_ring, const void* probs,
+                                     const void* k_new, const void* v_new,
+                                     void* out, void* ring_k, void* ring_v,
+                                     int32_t* num_tokens, int B, int heads,
+                                     int hd, int window, int update, int dtype,
+                                     hipStream_t s);
 hipError_t launch_pack_gate_weights(const void* w_x, const void* w_a,
                                     void* packed, int H, hipStream_t s);
 

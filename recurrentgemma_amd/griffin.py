@@ -176,19 +176,13 @@ class MLPBlock(nn.Module):
     return self.ffw_down(ops.gelu_mul(up, gate))  # gelu(gate) * up, one pass
 
 
-def _rope(x, positions, max_wavelength=_MAX_WAVELENGTH):
-  """Rotary embedding on the first half of the head dimension
-  (modules.py:52-83): within that half, element i pairs with element
-  i + quarter, angle = position / max_wavelength^(2i / half)."""
-  half = x.shape[-1] // 2
-  quarter = half // 2
-  rot, keep = x[..., :half], x[..., half:]
-  freq = torch.arange(quarter, device=x.device)
-  inv = 1.0 / (max_wavelength ** (2 * freq / half))
-  angle = positions[:, :, None, None] * inv
-  sin, cos = torch.sin(angle).type_as(x), torch.cos(angle).type_as(x)
-  lo, hi = rot[..., :quarter], rot[..., quarter:]
-  return torch.cat([lo * cos - hi * sin, hi * cos + lo * sin, keep], dim=-1)
+def _inv_frequencies(head_dim, device, max_wavelength=_MAX_WAVELENGTH):
+  """1 / max_wavelength^(2i / half) for the i-th rotated pair, with the
+  reference's own tensor expression (modules.py:70-73) so that the table has
+  its float32 values."""
+  half = head_dim // 2
+  freq = torch.arange(half // 2, device=device)
+  return 1.0 / (max_wavelength ** (2 * freq / half))
 
 
 def _visible(q_pos, k_pos, window, q_doc=None, k_doc=None):
@@ -218,7 +212,15 @@ class LocalAttentionBlock(nn.Module):
     self.proj_k = nn.Linear(width, self.head_dim, bias=False, **kw)
     self.proj_v = nn.Linear(width, self.head_dim, bias=False, **kw)
     self.proj_final = nn.Linear(width, width, bias=True, **kw)
+    self._inv_freq = None
     self.reset_parameters()
+
+  def _rope(self, x, positions):
+    """Rotary embedding on the first half of the head dimension
+    (modules.py:52-83), one kernel."""
+    if self._inv_freq is None or self._inv_freq.device != x.device:
+      self._inv_freq = _inv_frequencies(self.head_dim, x.device)
+    return ops.rope(x, positions, self._inv_freq)
 
   @property
   def head_dim(self) -> int:
@@ -238,7 +240,8 @@ class LocalAttentionBlock(nn.Module):
     min(window, T) tokens, token with position p in slot p % window when the
     prompt fills the window."""
     w = min(window, keys.shape[1])
-    num_tokens = segment_pos[:, -1] + 1
+    # int32 like init_cache (the reference keeps the dtype of segment_pos)
+    num_tokens = (segment_pos[:, -1] + 1).to(torch.int32)
     shift = (num_tokens % window)[:, None]
     src = (torch.arange(w, device=keys.device)[None] - shift) % w  # [B, w]
 
@@ -261,7 +264,7 @@ class LocalAttentionBlock(nn.Module):
     q = self.proj_q(x).reshape(b, t, self.num_heads, self.head_dim)
     k = self.proj_k(x).reshape(b, t, 1, self.head_dim)
     v = self.proj_v(x).reshape(b, t, 1, self.head_dim)
-    q, k = _rope(q, segment_pos), _rope(k, segment_pos)
+    q, k = self._rope(q, segment_pos), self._rope(k, segment_pos)
 
     if cache is not None and t == 1:
       return self._decode_step(x, q, k, v, cache, return_cache)
@@ -311,32 +314,27 @@ class LocalAttentionBlock(nn.Module):
   def _decode_step(self, x, q, k, v, cache, return_cache):
     """One new token against the ring and itself, without concatenating or
     expanding the cached keys and values: all heads share them, so the scores
-    are one batched [heads, head_dim] x [head_dim, window] product per row.
-    Same order of roundings as the reference: scores in the activation dtype,
-    scaled, masked, softmax in float32, probabilities back in the activation
-    dtype (modules.py:462-474)."""
+    are one batched [heads, head_dim] x [head_dim, window] product per row on
+    the cache as it lies.  Scaling, mask, softmax and the new token's own
+    score are one kernel; the new token's share of the output, the ring update
+    and the token count another.  Same order of roundings as the reference:
+    scores in the activation dtype, scaled, masked, softmax in float32,
+    probabilities back in the activation dtype (modules.py:462-474)."""
     b = x.shape[0]
     w = self.window_size
-    k_pos, q_pos = self._ring_positions(cache.num_tokens, 1)
-    ring_ok = _visible(q_pos, k_pos, w)                    # [B, 1, window]
+    if cache.num_tokens.dtype != torch.int32:
+      raise TypeError("AttentionBlockCache.num_tokens must be int32")
     qh = q[:, 0]                                           # [B, heads, hd]
     ring_k, ring_v = cache.keys[:, :, 0], cache.values[:, :, 0]  # [B, w, hd]
-    scale = self.head_dim ** -0.5
-    s_ring = torch.bmm(qh, ring_k.transpose(1, 2)) * scale  # [B, heads, w]
-    s_self = (qh * k[:, 0]).sum(-1, keepdim=True).to(qh.dtype) * scale
-    s_ring = s_ring.float().masked_fill(~ring_ok, float("-inf"))
-    probs = torch.softmax(torch.cat([s_ring, s_self.float()], dim=-1),
-                          dim=-1).type_as(x)
-    out = torch.bmm(probs[..., :w], ring_v) + probs[..., w:] * v[:, 0]
+    scores = torch.bmm(qh, ring_k.transpose(1, 2))         # [B, heads, w]
+    probs = ops.attention_decode_probs(scores, qh, k[:, 0, 0],
+                                       cache.num_tokens, self.head_dim ** -0.5)
+    from_ring = torch.bmm(probs[..., :w], ring_v)
+    out = ops.attention_decode_finish(
+        from_ring, probs, k[:, 0, 0], v[:, 0, 0], cache.keys, cache.values,
+        cache.num_tokens, update_cache=return_cache)
     out = self.proj_final(out.reshape(b, 1, self.width))
-    if not return_cache:
-      return out, None
-    rows = torch.arange(b, device=x.device)
-    at = (cache.num_tokens % w).long()
-    cache.keys[rows, at] = k[:, 0]
-    cache.values[rows, at] = v[:, 0]
-    cache.num_tokens[:] = cache.num_tokens + 1
-    return out, cache
+    return out, (cache if return_cache else None)
 
   @classmethod
   def init_cache(cls, batch_size, window_size, heads_dim, dtype, device=None):

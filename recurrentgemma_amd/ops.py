@@ -289,6 +289,69 @@ def rms_norm(x, scale, eps=1e-6):
   return out
 
 
+def rope(x, positions, inv_freq):
+  """Rotary embedding on the first half of the last dimension of
+  x [B, T, heads, head_dim]; positions [B, T]; inv_freq [head_dim / 4] f32."""
+  B, T, n, hd = x.shape
+  x = _dev(x, "x")
+  pos, is64 = _segpos(positions, B, T)
+  inv = _dev(inv_freq, "inv_freq")
+  assert inv.dtype == torch.float32 and inv.shape == (hd // 4,)
+  out = torch.empty_like(x)
+  with torch.cuda.device(x.device):
+    _lib.check(_lib.lib().rg_rope(_p(x), _p(pos), is64, _p(inv), _p(out),
+                                  B * T, n, hd, _dtype_code(x), _stream(x)))
+  return out
+
+
+def attention_decode_probs(scores, q, k_new, num_tokens, scale):
+  """softmax over the written ring slots and the new token: scores
+  [B, heads, window] (unscaled), q [B, heads, hd], k_new [B, hd], num_tokens
+  [B] int32 -> probs [B, heads, window + 1]."""
+  B, heads, window = scores.shape
+  hd = q.shape[-1]
+  scores, q, k_new = _dev(scores, "scores"), _dev(q, "q"), _dev(k_new, "k_new")
+  _same(scores.dtype, scores.device, q=q, k_new=k_new)
+  assert q.shape == (B, heads, hd) and k_new.shape == (B, hd)
+  assert num_tokens.dtype == torch.int32 and num_tokens.shape == (B,)
+  nt = _dev(num_tokens, "num_tokens")
+  probs = torch.empty((B, heads, window + 1), dtype=scores.dtype,
+                      device=scores.device)
+  with torch.cuda.device(scores.device):
+    _lib.check(_lib.lib().rg_attention_decode_probs(
+        _p(scores), _p(q), _p(k_new), _p(nt), _p(probs), B, heads, hd, window,
+        scale, _dtype_code(scores), _stream(scores)))
+  return probs
+
+
+def attention_decode_finish(from_ring, probs, k_new, v_new, ring_keys,
+                            ring_values, num_tokens, update_cache):
+  """from_ring + probs[..., -1] * v_new; with update_cache the new key and
+  value go into slot num_tokens % window of the ring (in place) and num_tokens
+  is incremented (in place)."""
+  B, heads, hd = from_ring.shape
+  window = probs.shape[-1] - 1
+  from_ring, probs = _dev(from_ring, "from_ring"), _dev(probs, "probs")
+  k_new, v_new = _dev(k_new, "k_new"), _dev(v_new, "v_new")
+  _same(from_ring.dtype, from_ring.device, probs=probs, k_new=k_new,
+        v_new=v_new, ring_keys=ring_keys, ring_values=ring_values)
+  for t, name in ((ring_keys, "ring_keys"), (ring_values, "ring_values"),
+                  (num_tokens, "num_tokens")):
+    # updated in place: no silent copies
+    if not (t.is_cuda and t.is_contiguous() and t.data_ptr() % 16 == 0):
+      raise ValueError(f"{name} must be a contiguous, 16-byte aligned GPU "
+                       "tensor (it is updated in place)")
+  assert ring_keys.numel() == B * window * hd == ring_values.numel()
+  assert num_tokens.dtype == torch.int32 and num_tokens.shape == (B,)
+  out = torch.empty_like(from_ring)
+  with torch.cuda.device(out.device):
+    _lib.check(_lib.lib().rg_attention_decode_finish(
+        _p(from_ring), _p(probs), _p(k_new), _p(v_new), _p(out),
+        _p(ring_keys), _p(ring_values), _p(num_tokens), B, heads, hd, window,
+        int(bool(update_cache)), _dtype_code(out), _stream(out)))
+  return out
+
+
 _packed_weights = {}  # (id(w_x), id(w_a)) -> (ref_x, ref_a, stamp, packed)
 
 

@@ -178,3 +178,87 @@ def test_captured_decode_step_equals_eager(model, which):
   # the modules are back to returning new cache tensors
   assert not any(b.recurrent_block.decode_in_place for b in m.blocks
                  if hasattr(b, "recurrent_block"))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hd", [16, 256])
+def test_rope_kernel(dtype, hd):
+  """rg_rope against the reference's tensor expression (modules.py:52-83)
+  evaluated by torch on the GPU in the same dtype: bit-identical (the same
+  float32 table, sin/cos of the same angles, the same roundings)."""
+  from recurrentgemma_amd import ops
+  gen = torch.Generator().manual_seed(hd)
+  x = torch.randn(3, 7, 2, hd, generator=gen).to(dtype).to(DEV)
+  pos = torch.tensor([[-1, -1, 0, 1, 2, 3, 4], [0, 1, 2, 0, 1, 2, 3],
+                      [2040, 2041, 2042, 2043, 2044, 2045, 2046]], device=DEV)
+  inv = G._inv_frequencies(hd, DEV)
+  half = hd // 2
+  rot, keep = x[..., :half], x[..., half:]
+  angle = pos.reshape(3, 7, 1, 1) * inv
+  sin, cos = torch.sin(angle).type_as(x), torch.cos(angle).type_as(x)
+  lo, hi = torch.chunk(rot, 2, dim=-1)
+  want = torch.cat([lo * cos - hi * sin, hi * cos + lo * sin, keep], dim=-1)
+  for p in (pos, pos.to(torch.int32)):
+    got = ops.rope(x, p, inv)
+    assert torch.equal(got, want), (got - want).abs().max()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,heads,hd,window", [(2, 2, 16, 6), (5, 10, 256, 64),
+                                               (3, 4, 64, 300)])
+def test_attention_decode_kernels(dtype, B, heads, hd, window):
+  """The decode step of the attention block (scores product + the two
+  kernels + values product) against the reference's formulation
+  (modules.py:440-474: concatenate the ring and the new key/value, mask from
+  the ring positions, float32 softmax) evaluated by torch on the GPU, for a
+  ring that is empty, partly filled, exactly full and wrapped.  fp32: 1e-5 of
+  the largest magnitude; bf16: 2e-2 (sum of the ring part and the new token's
+  part rounded separately).  Ring and token count must be updated exactly."""
+  from recurrentgemma_amd import ops
+  gen = torch.Generator().manual_seed(B * 1000 + window)
+  tol = 1e-5 if dtype == torch.float32 else 2e-2
+  nts = torch.tensor(([0, 3, window, 2 * window + 5, window - 1] * B)[:B],
+                     dtype=torch.int32, device=DEV)
+  q = torch.randn(B, heads, hd, generator=gen).to(dtype).to(DEV)
+  kn = torch.randn(B, hd, generator=gen).to(dtype).to(DEV)
+  vn = torch.randn(B, hd, generator=gen).to(dtype).to(DEV)
+  rk = torch.randn(B, window, hd, generator=gen).to(dtype).to(DEV)
+  rv = torch.randn(B, window, hd, generator=gen).to(dtype).to(DEV)
+  scale = hd ** -0.5
+  # reference formulation
+  n = nts[:, None].long()
+  slot = torch.arange(window, device=DEV)[None]
+  now = slot + (n // window) * window
+  k_pos = torch.where(now < n, now, now - window)
+  k_pos = torch.cat([k_pos, n], dim=-1)                       # [B, w+1]
+  mask = (n >= k_pos) & (n <= k_pos + window) & (k_pos >= 0)
+  keys = torch.cat([rk, kn[:, None]], dim=1)
+  vals = torch.cat([rv, vn[:, None]], dim=1)
+  logits = torch.einsum("bnh,bsh->bns", q, keys) * scale
+  logits = torch.where(mask[:, None], logits, -2.3819763e38).float()
+  p = torch.softmax(logits, dim=-1).type_as(q)
+  want = torch.einsum("bns,bsh->bnh", p, vals)
+  # kernels
+  k2, v2, nt2 = rk.clone(), rv.clone(), nts.clone()
+  scores = torch.bmm(q, k2.transpose(1, 2))
+  probs = ops.attention_decode_probs(scores, q, kn, nt2, scale)
+  assert helpers_max_rel(probs, p) < tol
+  out = ops.attention_decode_finish(torch.bmm(probs[..., :window], v2), probs,
+                                    kn, vn, k2, v2, nt2, update_cache=True)
+  assert helpers_max_rel(out, want) < tol
+  assert torch.equal(nt2, nts + 1)
+  rows = torch.arange(B, device=DEV)
+  exp_k, exp_v = rk.clone(), rv.clone()
+  exp_k[rows, (nts % window).long()] = kn
+  exp_v[rows, (nts % window).long()] = vn
+  assert torch.equal(k2, exp_k) and torch.equal(v2, exp_v)
+  # without the cache update nothing is written
+  k3, v3, nt3 = rk.clone(), rv.clone(), nts.clone()
+  out3 = ops.attention_decode_finish(torch.bmm(probs[..., :window], v3), probs,
+                                     kn, vn, k3, v3, nt3, update_cache=False)
+  assert torch.equal(out3, out) and torch.equal(k3, rk) and torch.equal(nt3, nts)
+
+
+def helpers_max_rel(got, want):
+  got, want = got.float(), want.float()
+  return ((got - want).abs().max() / want.abs().max().clamp_min(1e-30)).item()
