@@ -146,8 +146,15 @@ class _StackedLinear(nn.Module):
   def forward(self, x):
     lead = x.shape[:-1]
     x2 = x.reshape(-1, x.shape[-1])
-    gate = torch.addmm(self.b[0].reshape(-1), x2, self.w[0])
-    up = torch.addmm(self.b[1].reshape(-1), x2, self.w[1])
+    if x2.shape[0] <= 1024:
+      # few rows (decode): both projections as one batched product on the
+      # stacked parameters, half the launches
+      out = torch.baddbmm(self.b.reshape(2, 1, -1),
+                          x2[None].expand(2, -1, -1), self.w)
+      gate, up = out[0], out[1]
+    else:
+      gate = torch.addmm(self.b[0].reshape(-1), x2, self.w[0])
+      up = torch.addmm(self.b[1].reshape(-1), x2, self.w[1])
     return gate.reshape(*lead, -1), up.reshape(*lead, -1)
 
 
