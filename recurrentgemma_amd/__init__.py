@@ -2,6 +2,7 @@
 `recurrentgemma.torch` modules of the same names), and the residual stack and
 sampler that call it."""
 
+from recurrentgemma_amd import training
 from recurrentgemma_amd.layers import BlockDiagonalLinear
 from recurrentgemma_amd.layers import Conv1D
 from recurrentgemma_amd.layers import RGLRU
@@ -28,5 +29,5 @@ __all__ = [
     "Griffin", "GriffinConfig", "LocalAttentionBlock", "MLPBlock", "Preset",
     "RGLRU", "RMSNorm", "RecurrentBlock", "RecurrentBlockCache",
     "ResidualBlock", "Sampler", "SamplerOutput", "TemporalBlockType",
-    "recurrent_core", "rnn_param_init", "rnn_scan",
+    "recurrent_core", "rnn_param_init", "rnn_scan", "training",
 ]

@@ -8,7 +8,9 @@ recurrentgemma/torch/layers.py:
   rnn_param_init       layers.py:194-213
   RGLRU                layers.py:233-376
   Conv1D               layers.py:379-650
-Forward only (inference); the kernels are not differentiable.
+The kernels are forward only; inside `training.differentiable()` the modules
+run the reference's op sequence under autograd with the recurrence on the scan
+kernel in both directions (see training.py).
 
 Differences from the reference, on purpose:
   * Conv1D.forward does not modify its input (the reference multiplies slices
@@ -28,6 +30,7 @@ import torch
 from torch import nn
 
 from recurrentgemma_amd import ops
+from recurrentgemma_amd import training
 
 
 class BlockDiagonalLinear(nn.Module):
@@ -55,12 +58,13 @@ class BlockDiagonalLinear(nn.Module):
     std = math.sqrt(self.w_init_variance_scale / self.block_width)
     torch.nn.init.normal_(w, mean=0.0, std=std)
 
-  @torch.no_grad()
   def forward(self, x: torch.Tensor) -> torch.Tensor:
-    return ops.block_diag_linear(x, self.w, self.b)
+    if training.is_enabled():
+      return training.block_diag_linear(x, self.w, self.b)
+    with torch.no_grad():
+      return ops.block_diag_linear(x, self.w, self.b)
 
 
-@torch.no_grad()
 def rnn_scan(x, a, reset, h0, acc_dtype=torch.float32):
   """h_t = a_t h_{t-1} + x_t with a zeroed at resets; float32 state."""
   assert x.ndim == 3
@@ -70,9 +74,12 @@ def rnn_scan(x, a, reset, h0, acc_dtype=torch.float32):
   assert h0 is None or h0.dtype == acc_dtype
   if acc_dtype != torch.float32:
     raise NotImplementedError("the scan kernel keeps its state in float32")
+  if training.is_enabled():
+    return training.rnn_scan(x, a, reset, h0)
   if a.shape != x.shape:
     a = a.expand_as(x)
-  return ops.linear_scan(x, a, reset, h0)
+  with torch.no_grad():
+    return ops.linear_scan(x, a, reset, h0)
 
 
 def rnn_param_init(tensor, min_rad, max_rad, transform="softplus", eps=1e-8):
@@ -113,11 +120,19 @@ class RGLRU(nn.Module):
   def a_param_init(self, w: torch.Tensor) -> torch.Tensor:
     return rnn_param_init(w, min_rad=0.9, max_rad=0.999)
 
-  @torch.no_grad()
   def forward(self, x, segment_pos, cache=None, return_cache=True):
     """x [B,T,W] (the conv output), cache: previous state [B,W] float32."""
     bs, l, _ = x.shape
     assert segment_pos.shape == (bs, l)
+    if training.is_enabled():
+      y, last_h = training.rg_lru(
+          x, segment_pos, self.a_param, self.input_gate.w, self.input_gate.b,
+          self.a_gate.w, self.a_gate.b, h0=cache)
+      return y, (last_h if return_cache else None)
+    with torch.no_grad():
+      return self._forward_kernels(x, segment_pos, cache, return_cache)
+
+  def _forward_kernels(self, x, segment_pos, cache, return_cache):
     gx_pre, ga_pre = ops.gates_gemm(x, self.input_gate.w, self.input_gate.b,
                                     self.a_gate.w, self.a_gate.b)
     y, last_h, _ = ops.lru_scan_fused(x, gx_pre, ga_pre, self.a_param,
@@ -155,9 +170,22 @@ class Conv1D(nn.Module):
     std = math.sqrt(self.w_init_variance_scale / self.temporal_width)
     torch.nn.init.normal_(w, mean=0.0, std=std)
 
-  @torch.no_grad()
   def forward(self, x, segment_pos, cache=None, return_cache=True):
     """cache None: prefill over [B,T,W]; cache [B,K-1,W]: one decode token."""
+    if training.is_enabled():
+      if cache is not None:
+        raise NotImplementedError("the differentiable path is prefill only")
+      out = training.conv1d(x, segment_pos, self.w, self.b)
+      new_cache = None
+      if return_cache:  # the masked tail the kernels return, outside autograd
+        with torch.no_grad():
+          new_cache = ops.conv1d_prefill(x.detach(), segment_pos, self.w,
+                                         self.b, True)[1]
+      return out, new_cache
+    with torch.no_grad():
+      return self._forward_kernels(x, segment_pos, cache, return_cache)
+
+  def _forward_kernels(self, x, segment_pos, cache, return_cache):
     if cache is not None:
       b, num_tokens, d = x.shape
       assert cache.shape == (b, self.temporal_width - 1, d)

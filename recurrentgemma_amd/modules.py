@@ -19,6 +19,7 @@ from torch import nn
 
 from recurrentgemma_amd import layers
 from recurrentgemma_amd import ops
+from recurrentgemma_amd import training
 
 
 class RecurrentBlockCache(NamedTuple):
@@ -136,18 +137,33 @@ class RecurrentBlock(nn.Module):
     std = math.sqrt(self.final_w_init_variance_scale / self.lru_width)
     torch.nn.init.normal_(w, mean=0.0, std=std)
 
-  @torch.no_grad()
   def forward(self, x, segment_pos, cache=None, return_cache=True):
-    y = self.linear_y(x)
-    x = self.linear_x(x)
-    x, new_cache = recurrent_core(
-        self.conv_1d, self.rg_lru, x, segment_pos, cache, return_cache,
-        in_place=self.decode_in_place and cache is not None and return_cache)
-    x = ops.gelu_mul(x, y)  # x * gelu(y), one pass (modules.py:627-628, 644)
-    x = self.linear_out(x)
+    if training.is_enabled():
+      return self._forward_differentiable(x, segment_pos, cache, return_cache)
+    with torch.no_grad():
+      y = self.linear_y(x)
+      x = self.linear_x(x)
+      x, new_cache = recurrent_core(
+          self.conv_1d, self.rg_lru, x, segment_pos, cache, return_cache,
+          in_place=self.decode_in_place and cache is not None and return_cache)
+      x = ops.gelu_mul(x, y)  # x * gelu(y), one pass (modules.py:627-628, 644)
+      x = self.linear_out(x)
     if not return_cache:
       return x, None
     return x, new_cache
+
+  def _forward_differentiable(self, x, segment_pos, cache, return_cache):
+    """The reference's op sequence (modules.py:605-655) under autograd."""
+    if cache is not None:
+      raise NotImplementedError("the differentiable path is prefill only")
+    y = gelu(self.linear_y(x))
+    x = self.linear_x(x)
+    x, conv_state = self.conv_1d(x, segment_pos, None, return_cache)
+    x, h = self.rg_lru(x, segment_pos, None, return_cache)
+    x = self.linear_out(x * y)
+    if not return_cache:
+      return x, None
+    return x, RecurrentBlockCache(rg_lru_state=h, conv1d_state=conv_state)
 
   @classmethod
   def init_cache(cls, batch_size, lru_width, dtype, conv1d_temporal_width=4,

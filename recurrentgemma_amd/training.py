@@ -1,0 +1,143 @@
+"""Differentiable forward of the recurrent block, for fine-tuning.
+
+The inference kernels fuse conv, gates and recurrence and keep nothing for a
+backward pass.  Inside `with training.differentiable():` the drop-in modules
+(Conv1D, BlockDiagonalLinear, RGLRU, RecurrentBlock) instead run the
+reference's sequence of tensor ops (recurrentgemma/torch/layers.py:127-137,
+313-365, 447-529) on the GPU under autograd, except for the one part that is
+a Python loop over time there: the linear recurrence (layers.py:140-191),
+which is the scan kernel in both directions --
+
+  forward   h_t = a_t h_{t-1} + x_t
+  backward  g_t = dy_t + a_{t+1} g_{t+1}     (the same recurrence, time
+            dx_t = g_t                        reversed, coefficients shifted by
+            da_t = g_t h_{t-1}                one step)
+            dh_0 = a_0 g_0
+
+with a_t zeroed at document starts.  sqrt(1 - a^2) keeps the reference's
+clipped derivative (layers.py:216-230).  Prefill only (no decode cache).
+"""
+
+from __future__ import annotations
+
+import contextlib
+
+import torch
+
+from recurrentgemma_amd import ops
+
+_MAX_SQRT_GRADIENT = 1000.0
+_enabled = False
+
+
+def is_enabled() -> bool:
+  return _enabled
+
+
+@contextlib.contextmanager
+def differentiable():
+  """Within this context the modules of this package build an autograd
+  graph (and are correspondingly slower and hungrier for memory)."""
+  global _enabled
+  old, _enabled = _enabled, True
+  try:
+    yield
+  finally:
+    _enabled = old
+
+
+class _LinearScan(torch.autograd.Function):
+  """y_t = h_t = a'_t h_{t-1} + x_t in float32, a' = a with zeros at resets;
+  returns (y rounded to the activation dtype, h_last float32)."""
+
+  @staticmethod
+  def forward(ctx, x, a, reset, h0):
+    y, h_last = ops.linear_scan(x, a, reset, h0)
+    ctx.save_for_backward(a, reset, y, h0)
+    return y, h_last
+
+  @staticmethod
+  def backward(ctx, dy, dh_last):
+    a, reset, y, h0 = ctx.saved_tensors
+    B, T, W = y.shape
+    a_eff = a * (~reset)[..., None].to(a.dtype)
+    # time reversed, coefficient of step s = a'_{T-s} (s >= 1); step 0 takes
+    # dh_last in as the initial state with coefficient one
+    a_rev = torch.cat([torch.ones_like(a_eff[:, :1]),
+                       torch.flip(a_eff[:, 1:], dims=[1])], dim=1)
+    dy_rev = torch.flip(dy, dims=[1]).contiguous()
+    carry = (torch.zeros((B, W), dtype=torch.float32, device=y.device)
+             if dh_last is None else dh_last.float().contiguous())
+    no_reset = torch.zeros((B, T), dtype=torch.bool, device=y.device)
+    g_rev, g0 = ops.linear_scan(dy_rev, a_rev.contiguous(), no_reset, carry)
+    g = torch.flip(g_rev, dims=[1])
+    first = (torch.zeros_like(y[:, :1]) if h0 is None
+             else h0.to(y.dtype)[:, None])
+    h_prev = torch.cat([first, y[:, :-1]], dim=1)
+    da = g * h_prev * (~reset)[..., None].to(g.dtype)
+    dh0 = None if h0 is None else a_eff[:, 0].float() * g0
+    return g, da, None, dh0
+
+
+class _BoundedSqrt(torch.autograd.Function):
+  """sqrt with the derivative clipped at _MAX_SQRT_GRADIENT."""
+
+  @staticmethod
+  def forward(ctx, x):
+    ctx.save_for_backward(x)
+    return torch.sqrt(x)
+
+  @staticmethod
+  def backward(ctx, grad):
+    (x,) = ctx.saved_tensors
+    return grad / torch.sqrt(torch.clip(4.0 * x,
+                                        min=1 / (_MAX_SQRT_GRADIENT ** 2)))
+
+
+def rnn_scan(x, a, reset, h0=None):
+  if a.shape != x.shape:
+    a = a.expand_as(x)
+  return _LinearScan.apply(x.contiguous(), a.contiguous(), reset, h0)
+
+
+def block_diag_linear(x, w, b):
+  """y[..., h, :] = x[..., h, :] @ w[h] + b[h]  (layers.py:127-137)."""
+  h, bw, _ = w.shape
+  xs = x.reshape(*x.shape[:-1], h, bw)
+  y = torch.einsum("...hi,hij->...hj", xs, w) + b
+  return y.reshape(x.shape)
+
+
+def conv1d(x, segment_pos, w, b):
+  """Conv1D.forward without a cache (layers.py:447-529), functional: tap s of
+  token t is x[t - s] unless a document starts at one of t-s+1 .. t."""
+  K = w.shape[0]
+  T = x.shape[1]
+  not_start = (segment_pos != 0).to(x.dtype)  # [B, T]
+  keep = torch.ones_like(not_start)
+  out = None
+  for s in range(min(K, T)):
+    if s > 0:
+      # keep_s[t] = prod_{j < s} not_start[t - j]
+      shifted = torch.nn.functional.pad(not_start, (s - 1, 0), value=1.0)[:, :T]
+      keep = keep * shifted
+    xs = torch.nn.functional.pad(x, (0, 0, s, 0))[:, :T]
+    term = xs * keep[..., None] * w[K - 1 - s]
+    out = term if out is None else out + term
+  return out + b
+
+
+def rg_lru(x, segment_pos, a_param, w_x, b_x, w_a, b_a, h0=None):
+  """RGLRU.forward (layers.py:313-365) with the recurrence on the scan kernel.
+  Returns (y, h_last)."""
+  reset = segment_pos == 0
+  gate_x = torch.sigmoid(block_diag_linear(x, w_x, b_x))
+  gate_a = torch.sigmoid(block_diag_linear(x, w_a, b_a))
+  log_a = -8.0 * gate_a * torch.nn.functional.softplus(a_param)
+  a = torch.exp(log_a)
+  a_square = torch.exp(2 * log_a)
+  gated_x = x * gate_x
+  multiplier = _BoundedSqrt.apply(1 - a_square)
+  multiplier = reset[..., None] + ~reset[..., None] * multiplier
+  normalized_x = gated_x * multiplier.type(x.dtype)
+  return rnn_scan(normalized_x, a, reset, h0)

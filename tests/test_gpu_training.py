@@ -1,0 +1,117 @@
+"""The differentiable path (training.differentiable()) on the GPU against
+gradients written by the reference's own modules under torch autograd
+(tests/golden/make_grad_golden.py; float32, tiny shapes).  Tolerance 1e-4 of
+the largest reference magnitude per tensor (sums in a different order on a
+different device)."""
+
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import recurrentgemma_amd as rg
+from recurrentgemma_amd import training
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "grad_golden.npz")
+TOL = 1e-4
+
+
+@pytest.fixture(scope="module")
+def golden():
+  return np.load(GOLDEN)
+
+
+def close(got, want, what):
+  want = torch.from_numpy(np.asarray(want))
+  got = got.detach().cpu()
+  assert got.shape == want.shape, (what, got.shape, want.shape)
+  err = (got - want).abs().max().item()
+  scale = max(want.abs().max().item(), 1e-6)
+  assert err <= TOL * scale, (what, err, scale)
+
+
+def dev(a):
+  return torch.from_numpy(np.asarray(a)).to(DEV)
+
+
+def test_recurrent_block_gradients(golden):
+  blk = rg.RecurrentBlock(width=32, num_heads=2, lru_width=64,
+                          dtype=torch.float32)
+  sd = {k[len("blk/param/"):]: torch.from_numpy(golden[k])
+        for k in golden.files if k.startswith("blk/param/")}
+  blk.load_state_dict(sd)
+  blk = blk.to(DEV)
+  x = dev(golden["blk/x"]).requires_grad_(True)
+  seg = dev(golden["blk/seg"])
+  with training.differentiable():
+    y, cache = blk(x, seg)
+    loss = (y * dev(golden["blk/r"])).sum() + (
+        cache.rg_lru_state * dev(golden["blk/rh"])).sum()
+  loss.backward()
+  close(y, golden["blk/y"], "y")
+  close(cache.rg_lru_state, golden["blk/h"], "h")
+  close(x.grad, golden["blk/grad/x"], "dx")
+  for name, p in blk.named_parameters():
+    close(p.grad, golden[f"blk/grad/{name}"], "d" + name)
+  # outside the context the same module runs the inference kernels again and
+  # builds no graph
+  assert not training.is_enabled()
+  y2, _ = blk(x, seg)
+  assert not y2.requires_grad
+  close(y2, golden["blk/y"], "y (kernels)")
+  # the conv state returned in differentiable mode is the kernels' masked tail
+  _, cache2 = blk(x, seg)
+  assert torch.equal(cache.conv1d_state, cache2.conv1d_state)
+
+
+def test_rglru_gradients_with_initial_state(golden):
+  lru = rg.RGLRU(width=64, num_heads=2, dtype=torch.float32)
+  lru.load_state_dict({k[len("lru/param/"):]: torch.from_numpy(golden[k])
+                       for k in golden.files if k.startswith("lru/param/")})
+  lru = lru.to(DEV)
+  x = dev(golden["lru/x"]).requires_grad_(True)
+  h0 = dev(golden["lru/h0"]).requires_grad_(True)
+  seg = dev(golden["lru/seg"])
+  with training.differentiable():
+    y, h = lru(x, seg, h0)
+    loss = (y * dev(golden["lru/r"])).sum() + (h * dev(golden["lru/rh"])).sum()
+  loss.backward()
+  close(y, golden["lru/y"], "y")
+  close(h, golden["lru/h"], "h")
+  close(x.grad, golden["lru/grad/x"], "dx")
+  close(h0.grad, golden["lru/grad/h0"], "dh0")
+  for name, p in lru.named_parameters():
+    close(p.grad, golden[f"lru/grad/{name}"], "d" + name)
+
+
+@pytest.mark.parametrize("T", [1, 2, 65, 300])
+def test_scan_gradients_against_sequential_loop(T):
+  """The scan Function alone against autograd through a float64 Python loop
+  on the CPU, with resets and an initial state, at lengths that span one and
+  several steps of the scan kernel."""
+  gen = torch.Generator().manual_seed(T)
+  B, W = 3, 96
+  x = torch.randn(B, T, W, generator=gen)
+  a = torch.rand(B, T, W, generator=gen) * 0.5 + 0.5
+  h0 = torch.randn(B, W, generator=gen)
+  reset = torch.rand(B, T, generator=gen) < 0.1
+  r, rh = torch.randn(B, T, W, generator=gen), torch.randn(B, W, generator=gen)
+
+  xd, ad, hd = (t.double().requires_grad_(True) for t in (x, a, h0))
+  h, ys = hd, []
+  for t in range(T):
+    h = ad[:, t] * (~reset[:, t])[:, None] * h + xd[:, t]
+    ys.append(h)
+  ((torch.stack(ys, 1) * r).sum() + (h * rh).sum()).backward()
+
+  xg, ag, hg = (t.to(DEV).requires_grad_(True) for t in (x, a, h0))
+  with training.differentiable():
+    y, hl = rg.rnn_scan(xg, ag, reset.to(DEV), hg)
+  ((y * r.to(DEV)).sum() + (hl * rh.to(DEV)).sum()).backward()
+  close(y, torch.stack(ys, 1).float().detach().numpy(), "y")
+  close(xg.grad, xd.grad.float().numpy(), "dx")
+  close(ag.grad, ad.grad.float().numpy(), "da")
+  close(hg.grad, hd.grad.float().numpy(), "dh0")
