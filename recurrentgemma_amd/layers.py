@@ -33,30 +33,34 @@ from recurrentgemma_amd import ops
 from recurrentgemma_amd import training
 
 
+def _normal_(w: torch.Tensor, variance: float) -> None:
+  torch.nn.init.normal_(w, mean=0.0, std=math.sqrt(variance))
+
+
+def _new_param(shape, device, dtype) -> nn.Parameter:
+  return nn.Parameter(torch.empty(tuple(shape), device=device, dtype=dtype))
+
+
 class BlockDiagonalLinear(nn.Module):
   """Block-diagonal linear layer: y[..., h, :] = x[..., h, :] @ w[h] + b[h]."""
 
   def __init__(self, width, num_blocks, w_init_variance_scale=1.0, device=None,
                dtype=None):
-    super().__init__()
-    self.width = width
-    self.num_blocks = num_blocks
+    nn.Module.__init__(self)
+    bw = width // num_blocks
+    self.width, self.num_blocks, self.block_width = width, num_blocks, bw
     self.w_init_variance_scale = w_init_variance_scale
-    self.block_width = self.width // self.num_blocks
-    self.w = nn.Parameter(torch.empty(
-        [self.num_blocks, self.block_width, self.block_width], device=device,
-        dtype=dtype))
-    self.b = nn.Parameter(torch.empty(
-        [self.num_blocks, self.block_width], device=device, dtype=dtype))
+    self.w = _new_param((num_blocks, bw, bw), device, dtype)  # [H, in, out]
+    self.b = _new_param((num_blocks, bw), device, dtype)
     self.reset_parameters()
 
   def reset_parameters(self) -> None:
     self.w_init_(self.w)
-    torch.nn.init.zeros_(self.b)
+    with torch.no_grad():
+      self.b.zero_()
 
   def w_init_(self, w: torch.Tensor) -> None:
-    std = math.sqrt(self.w_init_variance_scale / self.block_width)
-    torch.nn.init.normal_(w, mean=0.0, std=std)
+    _normal_(w, self.w_init_variance_scale / self.block_width)
 
   def forward(self, x: torch.Tensor) -> torch.Tensor:
     if training.is_enabled():
@@ -67,11 +71,12 @@ class BlockDiagonalLinear(nn.Module):
 
 def rnn_scan(x, a, reset, h0, acc_dtype=torch.float32):
   """h_t = a_t h_{t-1} + x_t with a zeroed at resets; float32 state."""
-  assert x.ndim == 3
-  assert a.shape == x.shape[-a.ndim:]
-  assert a.dtype == x.dtype
-  assert type(a) is type(x)
-  assert h0 is None or h0.dtype == acc_dtype
+  if x.ndim != 3 or a.shape != x.shape[-a.ndim:]:
+    raise AssertionError(f"x {tuple(x.shape)} / a {tuple(a.shape)}")
+  if a.dtype != x.dtype or type(a) is not type(x):
+    raise AssertionError("x and a must have one dtype")
+  if h0 is not None and h0.dtype != acc_dtype:
+    raise AssertionError(f"h0 must be {acc_dtype}")
   if acc_dtype != torch.float32:
     raise NotImplementedError("the scan kernel keeps its state in float32")
   if training.is_enabled():
@@ -84,12 +89,16 @@ def rnn_scan(x, a, reset, h0, acc_dtype=torch.float32):
 
 def rnn_param_init(tensor, min_rad, max_rad, transform="softplus", eps=1e-8):
   """Initialises Lambda so that exp(-softplus(Lambda)) lies on a ring."""
+  if transform != "softplus":
+    raise NotImplementedError(transform)
+  lo, hi = min_rad * min_rad + eps, max_rad * max_rad + eps
   with torch.no_grad():
-    tensor.uniform_(min_rad ** 2 + eps, max_rad ** 2 + eps)
-    tensor.log_().mul_(0.5)
-    if transform == "softplus":
-      return tensor.neg_().exp_().sub_(1.0).log_()
-    raise NotImplementedError()
+    # u ~ U[lo, hi];  Lambda = log(u^(-1/2) - 1), step by step in place so that
+    # the values are those of the reference for the same generator state
+    for op, arg in (("uniform_", (lo, hi)), ("log_", ()), ("mul_", (0.5,)),
+                    ("neg_", ()), ("exp_", ()), ("sub_", (1.0,)), ("log_", ())):
+      getattr(tensor, op)(*arg)
+  return tensor
 
 
 class RGLRU(nn.Module):
@@ -97,24 +106,20 @@ class RGLRU(nn.Module):
 
   def __init__(self, width, num_heads, w_init_variance_scale=1.0, device=None,
                dtype=None):
-    super().__init__()
-    self.width = width
-    self.num_heads = num_heads
+    nn.Module.__init__(self)
+    self.width, self.num_heads = width, num_heads
     self.w_init_variance_scale = w_init_variance_scale
-    self.a_param = nn.Parameter(torch.empty([self.width], device=device,
-                                            dtype=dtype))
-    self.input_gate = BlockDiagonalLinear(
-        width=self.width, num_blocks=self.num_heads,
-        w_init_variance_scale=w_init_variance_scale, device=device, dtype=dtype)
-    self.a_gate = BlockDiagonalLinear(
-        width=self.width, num_blocks=self.num_heads,
-        w_init_variance_scale=self.w_init_variance_scale, device=device,
-        dtype=dtype)
+    self.a_param = _new_param((width,), device, dtype)
+    gate = dict(width=width, num_blocks=num_heads,
+                w_init_variance_scale=w_init_variance_scale, device=device,
+                dtype=dtype)
+    self.input_gate, self.a_gate = (BlockDiagonalLinear(**gate),
+                                    BlockDiagonalLinear(**gate))
     self.reset_parameters()
 
   def reset_parameters(self) -> None:
-    self.input_gate.reset_parameters()
-    self.a_gate.reset_parameters()
+    for gate in (self.input_gate, self.a_gate):
+      gate.reset_parameters()
     self.a_param_init(self.a_param)
 
   def a_param_init(self, w: torch.Tensor) -> torch.Tensor:
@@ -122,8 +127,9 @@ class RGLRU(nn.Module):
 
   def forward(self, x, segment_pos, cache=None, return_cache=True):
     """x [B,T,W] (the conv output), cache: previous state [B,W] float32."""
-    bs, l, _ = x.shape
-    assert segment_pos.shape == (bs, l)
+    if tuple(segment_pos.shape) != tuple(x.shape[:2]):
+      raise AssertionError(f"segment_pos {tuple(segment_pos.shape)} does not "
+                           f"match x {tuple(x.shape)}")
     if training.is_enabled():
       y, last_h = training.rg_lru(
           x, segment_pos, self.a_param, self.input_gate.w, self.input_gate.b,
@@ -153,22 +159,20 @@ class Conv1D(nn.Module):
 
   def __init__(self, width, temporal_width, w_init_variance_scale=0.01,
                device=None, dtype=None):
-    super().__init__()
-    self.width = width
-    self.temporal_width = temporal_width
+    nn.Module.__init__(self)
+    self.width, self.temporal_width = width, temporal_width
     self.w_init_variance_scale = w_init_variance_scale
-    self.w = nn.Parameter(torch.empty([self.temporal_width, self.width],
-                                      device=device, dtype=dtype))
-    self.b = nn.Parameter(torch.empty([width], device=device, dtype=dtype))
+    self.w = _new_param((temporal_width, width), device, dtype)
+    self.b = _new_param((width,), device, dtype)
     self.reset_parameters()
 
   def reset_parameters(self) -> None:
     self.w_init_(self.w)
-    torch.nn.init.zeros_(self.b)
+    with torch.no_grad():
+      self.b.zero_()
 
   def w_init_(self, w: torch.Tensor) -> None:
-    std = math.sqrt(self.w_init_variance_scale / self.temporal_width)
-    torch.nn.init.normal_(w, mean=0.0, std=std)
+    _normal_(w, self.w_init_variance_scale / self.temporal_width)
 
   def forward(self, x, segment_pos, cache=None, return_cache=True):
     """cache None: prefill over [B,T,W]; cache [B,K-1,W]: one decode token."""
