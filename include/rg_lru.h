@@ -183,6 +183,15 @@ int rg_gelu_mul(const void* a, const void* g, void* out, int64_t n, int dtype,
 int rg_rms_norm(const void* x, const void* scale, void* out, int64_t rows,
                 int width, float eps, int dtype, void* stream);
 
+/* The residual sum of a block and the norm that follows it in one pass
+ * (recurrentgemma/torch/modules.py:893-896 `residual = x + raw_x;
+ * x = self.channel_pre_norm(residual)`): sum_out = x + addend (rounded to
+ * `dtype`), out = rg_rms_norm(sum_out).  sum_out may alias x or addend; out
+ * must be a different buffer. */
+int rg_add_rms_norm(const void* x, const void* addend, const void* scale,
+                    void* sum_out, void* out, int64_t rows, int width,
+                    float eps, int dtype, void* stream);
+
 /* ---- the local-attention block around its matrix products ----------------
  * Not part of the recurrent path: the steps of the attention block that the
  * reference spells as dozens of elementwise tensor ops per block and decoded

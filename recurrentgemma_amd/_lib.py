@@ -44,6 +44,8 @@ SIGNATURES = {
     "rg_gelu_mul": (_i, [_vp, _vp, _vp, ctypes.c_int64, _i, _vp]),
     "rg_rms_norm": (_i, [_vp, _vp, _vp, ctypes.c_int64, _i, ctypes.c_float, _i,
                          _vp]),
+    "rg_add_rms_norm": (_i, [_vp, _vp, _vp, _vp, _vp, ctypes.c_int64, _i,
+                             ctypes.c_float, _i, _vp]),
     "rg_rope": (_i, [_vp, _vp, _i, _vp, _vp, ctypes.c_int64, _i, _i, _i, _vp]),
     "rg_attention_decode_probs": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i,
                                        ctypes.c_float, _i, _vp]),

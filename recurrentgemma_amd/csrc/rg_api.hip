@@ -376,9 +376,26 @@ int rg_rms_norm(const void* x, const void* scale, void* out, int64_t rows,
   RG_CHECK_PTR(x);
   RG_CHECK_PTR(scale);
   RG_CHECK_PTR(out);
-  return launch_status(__func__,
-                       rg::launch_rms_norm(x, scale, out, rows, width, eps,
-                                           dtype, (hipStream_t)stream));
+  return launch_status(
+      __func__, rg::launch_rms_norm(x, nullptr, scale, nullptr, out, rows,
+                                    width, eps, dtype, (hipStream_t)stream));
+}
+
+int rg_add_rms_norm(const void* x, const void* addend, const void* scale,
+                    void* sum_out, void* out, int64_t rows, int width,
+                    float eps, int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(rows > 0 && width > 0, "%s: rows=%lld width=%d must be positive",
+             __func__, (long long)rows, width);
+  RG_CHECK_PTR(x);
+  RG_CHECK_PTR(addend);
+  RG_CHECK_PTR(scale);
+  RG_CHECK_PTR(sum_out);
+  RG_CHECK_PTR(out);
+  RG_REQUIRE(out != sum_out, "%s: out must not alias sum_out", __func__);
+  return launch_status(
+      __func__, rg::launch_rms_norm(x, addend, scale, sum_out, out, rows, width,
+                                    eps, dtype, (hipStream_t)stream));
 }
 
 int rg_rope(const void* x, const void* positions, int positions_is_i64,

@@ -2,6 +2,8 @@
 // (recurrentgemma/torch/modules.py:627-628 `y = gelu(linear_y(x))`, :289-291
 // the tanh approximation, :644 `x = x * y`), one pass instead of torch's gelu
 // pass plus multiply pass.  `a` is the RG-LRU output, `g` the linear_y output.
+#include <type_traits>
+
 #include "rg_common.h"
 #include "rg_internal.h"
 
@@ -79,16 +81,25 @@ gelu_mul_f32_kernel(const f32x4* __restrict__ a, const f32x4* __restrict__ g,
 // of tensor ops (for bf16: x^2, the mean, var + eps, the rsqrt, x * rsqrt and
 // scale + 1 are each a bf16 tensor there; sums accumulate in float32).  One
 // workgroup per row; the row is read twice, the second time from cache.
-template <typename T>
+// ADD: the row normalised is x + addend (rounded to the activation dtype, the
+// residual sum of the block, recurrentgemma/torch/modules.py:893-896), which
+// is also written to `sum_out`.
+template <typename T, bool ADD>
 __global__ void __launch_bounds__(256)
-rms_norm_kernel(const T* __restrict__ x, const T* __restrict__ scale,
+rms_norm_kernel(const T* __restrict__ x, const T* __restrict__ addend,
+                const T* __restrict__ scale, T* __restrict__ sum_out,
                 T* __restrict__ out, int width, float eps) {
   __shared__ float partial[4];
-  const T* xr = x + (int64_t)blockIdx.x * width;
-  T* outr = out + (int64_t)blockIdx.x * width;
+  const int64_t row = (int64_t)blockIdx.x * width;
+  const T* xr = x + row;
+  T* outr = out + row;
   float sum = 0.0f;
   for (int i = threadIdx.x; i < width; i += 256) {
-    const float v = load_scalar<T>(xr + i);
+    float v = load_scalar<T>(xr + i);
+    if (ADD) {
+      v = round_act<T>(v + load_scalar<T>(addend + row + i));
+      store_scalar<T>(sum_out + row + i, v);
+    }
     sum += round_act<T>(v * v);
   }
 #pragma unroll
@@ -99,7 +110,8 @@ rms_norm_kernel(const T* __restrict__ x, const T* __restrict__ scale,
   const float var = round_act<T>(sum * (1.0f / (float)width));
   const float r = round_act<T>(1.0f / sqrtf(round_act<T>(var + eps)));
   for (int i = threadIdx.x; i < width; i += 256) {
-    const float v = load_scalar<T>(xr + i);
+    // (with ADD each thread re-reads the sums it stored itself)
+    const float v = load_scalar<T>((ADD ? sum_out + row : xr) + i);
     const float g = round_act<T>(load_scalar<T>(scale + i) + 1.0f);
     store_scalar<T>(outr + i, round_act<T>(v * r) * g);
   }
@@ -109,14 +121,18 @@ rms_norm_kernel(const T* __restrict__ x, const T* __restrict__ scale,
 // lanes, the row stays in registers between the two passes (one read, one
 // write; the scalar kernel above re-reads through the cache and moved
 // 1.7 TB/s on 131 072 rows of 2560).
+template <bool ADD>
 __global__ void __launch_bounds__(256)
 rms_norm_bf16_rows_kernel(const u32x4* __restrict__ x,
+                          const u32x4* __restrict__ addend,
                           const u32x4* __restrict__ scale,
+                          u32x4* __restrict__ sum_out,
                           u32x4* __restrict__ out, int chunks, float inv_width,
                           float eps) {
   __shared__ float partial[4];
-  const u32x4* xr = x + (int64_t)blockIdx.x * chunks;
-  u32x4* outr = out + (int64_t)blockIdx.x * chunks;
+  const int64_t row = (int64_t)blockIdx.x * chunks;
+  const u32x4* xr = x + row;
+  u32x4* outr = out + row;
   u32x4 v[2];
   float sum = 0.0f;
 #pragma unroll
@@ -124,6 +140,16 @@ rms_norm_bf16_rows_kernel(const u32x4* __restrict__ x,
     const int i = threadIdx.x + c * 256;
     v[c] = u32x4{0u, 0u, 0u, 0u};
     if (i < chunks) v[c] = __builtin_nontemporal_load(xr + i);
+    if (ADD && i < chunks) {
+      const u32x4 w = __builtin_nontemporal_load(addend + row + i);
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        v[c][k] = pack_bf16x2(
+            __uint_as_float(v[c][k] << 16) + __uint_as_float(w[k] << 16),
+            __uint_as_float(v[c][k] & 0xffff0000u) +
+                __uint_as_float(w[k] & 0xffff0000u));
+      sum_out[row + i] = v[c];
+    }
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const float lo = __uint_as_float(v[c][k] << 16);
@@ -181,22 +207,39 @@ hipError_t launch_gelu_mul(const void* a, const void* g, void* out, int64_t n,
   return hipGetLastError();
 }
 
-hipError_t launch_rms_norm(const void* x, const void* scale, void* out,
-                           int64_t rows, int width, float eps, int dtype,
-                           hipStream_t s) {
+hipError_t launch_rms_norm(const void* x, const void* addend, const void* scale,
+                           void* sum_out, void* out, int64_t rows, int width,
+                           float eps, int dtype, hipStream_t s) {
   if (rows > 0x7fffffff) return hipErrorInvalidValue;
-  const bool aligned =
-      (((uintptr_t)x | (uintptr_t)scale | (uintptr_t)out) & 15) == 0;
-  if (dtype == 0)
-    rms_norm_kernel<float><<<dim3((unsigned)rows), 256, 0, s>>>(
-        (const float*)x, (const float*)scale, (float*)out, width, eps);
-  else if (width % 8 == 0 && width <= 4096 && aligned)
-    rms_norm_bf16_rows_kernel<<<dim3((unsigned)rows), 256, 0, s>>>(
-        (const u32x4*)x, (const u32x4*)scale, (u32x4*)out, width / 8,
-        1.0f / (float)width, eps);
-  else
-    rms_norm_kernel<uint16_t><<<dim3((unsigned)rows), 256, 0, s>>>(
-        (const uint16_t*)x, (const uint16_t*)scale, (uint16_t*)out, width, eps);
+  const bool add = addend != nullptr;
+  const bool aligned = (((uintptr_t)x | (uintptr_t)addend | (uintptr_t)scale |
+                         (uintptr_t)sum_out | (uintptr_t)out) & 15) == 0;
+  const dim3 grid((unsigned)rows);
+  if (dtype != 0 && width % 8 == 0 && width <= 4096 && aligned) {
+    const int chunks = width / 8;
+    const float inv = 1.0f / (float)width;
+    if (add)
+      rms_norm_bf16_rows_kernel<true><<<grid, 256, 0, s>>>(
+          (const u32x4*)x, (const u32x4*)addend, (const u32x4*)scale,
+          (u32x4*)sum_out, (u32x4*)out, chunks, inv, eps);
+    else
+      rms_norm_bf16_rows_kernel<false><<<grid, 256, 0, s>>>(
+          (const u32x4*)x, nullptr, (const u32x4*)scale, nullptr, (u32x4*)out,
+          chunks, inv, eps);
+    return hipGetLastError();
+  }
+  auto run = [&](auto* tag) {
+    typedef std::remove_pointer_t<decltype(tag)> T;
+    if (add)
+      rms_norm_kernel<T, true><<<grid, 256, 0, s>>>(
+          (const T*)x, (const T*)addend, (const T*)scale, (T*)sum_out, (T*)out,
+          width, eps);
+    else
+      rms_norm_kernel<T, false><<<grid, 256, 0, s>>>(
+          (const T*)x, nullptr, (const T*)scale, nullptr, (T*)out, width, eps);
+  };
+  if (dtype == 0) run((float*)nullptr);
+  else run((uint16_t*)nullptr);
   return hipGetLastError();
 }
 

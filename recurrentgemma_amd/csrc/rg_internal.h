@@ -110,10 +110,11 @@ hipError_t launch_block_step_bf16(const StepArgs& a, hipStream_t s);
 // out[i] = a[i] * gelu_tanh(g[i]) over n elements (out may alias a or g).
 hipError_t launch_gelu_mul(const void* a, const void* g, void* out, int64_t n,
                            int dtype, hipStream_t s);
-// out[r, :] = x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * (scale + 1)
-hipError_t launch_rms_norm(const void* x, const void* scale, void* out,
-                           int64_t rows, int width, float eps, int dtype,
-                           hipStream_t s);
+// out[r, :] = v * rsqrt(mean(v^2) + eps) * (scale + 1) with v = x[r, :], or,
+// with an addend, v = x[r, :] + addend[r, :] (also written to sum_out)
+hipError_t launch_rms_norm(const void* x, const void* addend, const void* scale,
+                           void* sum_out, void* out, int64_t rows, int width,
+                           float eps, int dtype, hipStream_t s);
 // Steps of the local-attention block around its matrix products
 // (rg_attention.hip).
 hipError_t launch_rope(const void* x, const void* pos, int pos_kind,

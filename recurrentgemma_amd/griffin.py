@@ -123,6 +123,10 @@ class RMSNorm(nn.Module):
     # reference's chain of tensor ops
     return ops.rms_norm(x, self.scale, self.eps)
 
+  def add_then_norm(self, x, addend):
+    """(x + addend, forward(x + addend)) in one kernel."""
+    return ops.add_rms_norm(x, addend, self.scale, self.eps)
+
 
 class _StackedLinear(nn.Module):
   """Two width -> expanded projections with stacked parameters `w`
@@ -401,8 +405,8 @@ class ResidualBlock(nn.Module):
     mixed, new_cache = self.temporal_block(self.temporal_pre_norm(x),
                                            segment_pos, cache,
                                            return_cache=return_cache)
-    residual = mixed + x
-    return self.mlp_block(self.channel_pre_norm(residual)) + residual, new_cache
+    residual, normed = self.channel_pre_norm.add_then_norm(mixed, x)
+    return self.mlp_block(normed) + residual, new_cache
 
   @classmethod
   def init_cache(cls, batch_size, width, num_heads, attention_window_size,

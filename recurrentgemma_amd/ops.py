@@ -289,6 +289,22 @@ def rms_norm(x, scale, eps=1e-6):
   return out
 
 
+def add_rms_norm(x, addend, scale, eps=1e-6):
+  """(x + addend, rms_norm(x + addend)) in one pass."""
+  assert x.shape == addend.shape
+  x = _dev(x, "x")
+  _same(x.dtype, x.device, addend=addend, scale=scale)
+  addend, scale = _dev(addend, "addend"), _dev(scale, "scale")
+  width = x.shape[-1]
+  assert scale.shape == (width,)
+  total, out = torch.empty_like(x), torch.empty_like(x)
+  with torch.cuda.device(x.device):
+    _lib.check(_lib.lib().rg_add_rms_norm(
+        _p(x), _p(addend), _p(scale), _p(total), _p(out), x.numel() // width,
+        width, eps, _dtype_code(x), _stream(x)))
+  return total, out
+
+
 def rope(x, positions, inv_freq):
   """Rotary embedding on the first half of the last dimension of
   x [B, T, heads, head_dim]; positions [B, T]; inv_freq [head_dim / 4] f32."""

@@ -674,6 +674,12 @@ def test_rms_norm(dtype, rows, width):
     assert (err > 0).float().mean() < 0.35
   x3 = x.reshape(1, rows, width)  # leading dimensions are rows
   assert torch.equal(ops.rms_norm(_dev(x3), _dev(scale), eps).cpu()[0], got)
+  # the residual sum fused in front: identical to add, then norm
+  other = torch.randn(rows, width, generator=gen).to(dtype)
+  total, normed = ops.add_rms_norm(_dev(x), _dev(other), _dev(scale), eps)
+  want_total = _dev(x) + _dev(other)
+  assert torch.equal(total, want_total)
+  assert torch.equal(normed, ops.rms_norm(want_total, _dev(scale), eps))
 
 
 # --------------------------------- full-size, size-independent properties --

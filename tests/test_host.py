@@ -24,7 +24,7 @@ def _declared_symbols():
 
 def test_library_exports_every_declared_symbol():
   names = _declared_symbols()
-  assert len(names) == 19, names
+  assert len(names) == 20, names
   lib = ctypes.CDLL(_lib.LIB_PATH)
   for n in names:
     assert hasattr(lib, n), n
@@ -67,6 +67,10 @@ def test_c_side_validation_without_launch():
   assert rc == -1 and b"null" in lib.rg_last_error()
   rc = lib.rg_gelu_mul(ok, ok, ok, 8, 3, None)
   assert rc == -2 and b"dtype" in lib.rg_last_error()
+  rc = lib.rg_add_rms_norm(ok, ok, ok, y, y, 4, 64, 1e-6, 1, None)
+  assert rc == -1 and b"alias" in lib.rg_last_error()
+  rc = lib.rg_add_rms_norm(ok, None, ok, ok, y, 4, 64, 1e-6, 1, None)
+  assert rc == -1 and b"null" in lib.rg_last_error()
   args = [ok, ok, 1, ok, ok, ok, ok, ok, ok, None, ok, None, y, None, None]
   rc = lib.rg_recurrent_prefill(*args, 1, 8, 256, 1, 0, None)
   assert rc == -2 and b"unsupported" in lib.rg_last_error().lower()  # fp32
