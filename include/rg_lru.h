@@ -259,6 +259,41 @@ int rg_recurrent_step_packed(const void* x, const void* segpos,
                              const void* a_param, void* y, int B, int W, int H,
                              int dtype, void* stream);
 
+/* The linear layers around the recurrent and attention blocks for a decode
+ * step (at most 64 rows), bf16: torch.nn.Linear (modules.py:579-601 linear_y /
+ * linear_x / linear_out, :717-721 ffw_down, :334-352 the attention projections)
+ * and the stacked Einsum of the MLP (layers.py:76-101, modules.py:711-716).
+ * With so few rows a layer is one pass over its weight matrix, so the weights
+ * are repacked once, into the order the MFMA operand registers are filled
+ * (1 KB blocks per 32 weight rows x 16 inputs), and streamed from there.
+ *
+ * rg_linear_pack: w holds N weight rows of K inputs, `layout` 0 = [N, K]
+ *   (nn.Linear.weight), 1 = [groups, K, N / groups] (Einsum "cdD": weight row
+ *   g N/groups + j is w[g, :, j]).  gelu_pair != 0 interleaves tiles of the
+ *   first and the second half of the rows for the fused MLP epilogue below.
+ *   `packed`: rg_linear_packed_bytes(N, K) bytes (0 = shape unsupported:
+ *   needs K % 64 == 0 and N % 32 == 0; gelu_pair N % 64 == 0).  Pack again
+ *   whenever the weights change.
+ * rg_linear_rows: x [M, K], M <= 64; bias [N] or null;
+ *   out [groups, M, N / groups]  = x @ w^T + bias, rounded once; with
+ *       `residual` (same layout as out, may alias out): that plus residual,
+ *       rounded again (the separate add of modules.py:893-898);
+ *   gelu_pair: out [M, N / 2] = gelu(gate) * up with gate / up = rows j and
+ *       N/2 + j of x @ w^T + bias, each rounded (modules.py:752-757); groups
+ *       must be 1 and residual null.
+ *   workspace: rg_linear_rows_workspace_bytes(M, K, N) bytes (may be 0), for
+ *   the partial sums of shapes whose K is split over the grid; the sums are
+ *   added in a fixed order, results do not vary from run to run.
+ *   out must not alias x. */
+size_t rg_linear_packed_bytes(int N, int K, int gelu_pair);
+int rg_linear_pack(const void* w, int layout, int groups, int gelu_pair,
+                   void* packed, int N, int K, void* stream);
+size_t rg_linear_rows_workspace_bytes(int M, int K, int N);
+int rg_linear_rows(const void* x, const void* w_packed, const void* bias,
+                   const void* residual, void* out, void* workspace,
+                   size_t workspace_bytes, int M, int K, int N, int groups,
+                   int gelu_pair, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

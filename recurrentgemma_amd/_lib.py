@@ -44,6 +44,11 @@ SIGNATURES = {
     "rg_gelu_mul": (_i, [_vp, _vp, _vp, ctypes.c_int64, _i, _vp]),
     "rg_rms_norm": (_i, [_vp, _vp, _vp, ctypes.c_int64, _i, ctypes.c_float, _i,
                          _vp]),
+    "rg_linear_packed_bytes": (ctypes.c_size_t, [_i, _i, _i]),
+    "rg_linear_pack": (_i, [_vp, _i, _i, _i, _vp, _i, _i, _vp]),
+    "rg_linear_rows_workspace_bytes": (ctypes.c_size_t, [_i, _i, _i]),
+    "rg_linear_rows": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_size_t, _i,
+                            _i, _i, _i, _i, _vp]),
     "rg_add_rms_norm": (_i, [_vp, _vp, _vp, _vp, _vp, ctypes.c_int64, _i,
                              ctypes.c_float, _i, _vp]),
     "rg_rope": (_i, [_vp, _vp, _i, _vp, _vp, ctypes.c_int64, _i, _i, _i, _vp]),

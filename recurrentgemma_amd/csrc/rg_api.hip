@@ -491,6 +491,78 @@ int rg_pack_gate_weights(const void* w_x, const void* w_a, void* packed, int W,
                                      w_x, w_a, packed, H, (hipStream_t)stream));
 }
 
+size_t rg_linear_packed_bytes(int N, int K, int gelu_pair) {
+  if (N <= 0 || K <= 0 || K % 64 != 0 || N % 32 != 0) return 0;
+  if (gelu_pair && N % 64 != 0) return 0;
+  return (size_t)N * K * 2;
+}
+
+int rg_linear_pack(const void* w, int layout, int groups, int gelu_pair,
+                   void* packed, int N, int K, void* stream) {
+  RG_REQUIRE(N > 0 && K > 0, "%s: N=%d K=%d must be positive", __func__, N, K);
+  if (rg_linear_packed_bytes(N, K, gelu_pair) == 0)
+    return fail(RG_ERR_UNSUPPORTED,
+                "%s: needs K %% 64 == 0 and N %% 32 == 0 (64 for gelu pairs), "
+                "got N=%d K=%d", __func__, N, K);
+  RG_REQUIRE(layout == 0 || layout == 1, "%s: layout=%d", __func__, layout);
+  RG_REQUIRE(groups >= 1 && N % groups == 0,
+             "%s: N=%d is not a multiple of groups=%d", __func__, N, groups);
+  RG_CHECK_PTR(w);
+  RG_CHECK_PTR(packed);
+  RG_REQUIRE(packed != w, "%s: packed must not alias w", __func__);
+  return launch_status(
+      __func__, rg::launch_linear_pack(w, packed, N, K, layout, groups,
+                                       gelu_pair != 0, (hipStream_t)stream));
+}
+
+size_t rg_linear_rows_workspace_bytes(int M, int K, int N) {
+  if (M <= 0 || K <= 0 || N <= 0) return 0;
+  const int slices = rg::linear_rows_k_slices(K, N);
+  return slices > 1 ? (size_t)slices * M * N * sizeof(float) : 0;
+}
+
+int rg_linear_rows(const void* x, const void* w_packed, const void* bias,
+                   const void* residual, void* out, void* workspace,
+                   size_t workspace_bytes, int M, int K, int N, int groups,
+                   int gelu_pair, void* stream) {
+  RG_REQUIRE(M > 0 && K > 0 && N > 0, "%s: M=%d K=%d N=%d must be positive",
+             __func__, M, K, N);
+  if (M > 64 || rg_linear_packed_bytes(N, K, gelu_pair) == 0)
+    return fail(RG_ERR_UNSUPPORTED,
+                "%s: needs M <= 64, K %% 64 == 0, N %% 32 == 0 (64 for gelu "
+                "pairs), got M=%d K=%d N=%d", __func__, M, K, N);
+  RG_REQUIRE(groups >= 1 && N % groups == 0 && (N / groups) % 4 == 0,
+             "%s: N=%d / groups=%d must be a multiple of 4", __func__, N,
+             groups);
+  RG_REQUIRE(!gelu_pair || (groups == 1 && residual == nullptr),
+             "%s: gelu pairs take one group and no residual", __func__);
+  RG_CHECK_PTR(x);
+  RG_CHECK_PTR(w_packed);
+  RG_CHECK_PTR(out);
+  RG_CHECK_OPT_PTR(bias);
+  RG_CHECK_OPT_PTR(residual);
+  RG_REQUIRE(out != x, "%s: out must not alias x", __func__);
+  const size_t need = rg_linear_rows_workspace_bytes(M, K, N);
+  if (!gelu_pair && need > 0 &&
+      (workspace == nullptr || workspace_bytes < need || !aligned16(workspace)))
+    return fail(RG_ERR_WORKSPACE,
+                "%s: workspace of %zu bytes (16-byte aligned) required, got %zu",
+                __func__, need, workspace ? workspace_bytes : (size_t)0);
+  rg::LinearArgs a;
+  a.x = x;
+  a.w_packed = w_packed;
+  a.bias = bias;
+  a.residual = residual;
+  a.out = out;
+  a.partial = (float*)workspace;
+  a.M = M;
+  a.K = K;
+  a.N = N;
+  a.group_width = N / groups;
+  return launch_status(
+      __func__, rg::launch_linear_rows(a, gelu_pair != 0, (hipStream_t)stream));
+}
+
 int rg_recurrent_step_packed(const void* x, const void* segpos,
                              int segpos_is_i64, const void* conv_cache_in,
                              void* conv_cache_out, const void* h_in,

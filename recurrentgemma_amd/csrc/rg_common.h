@@ -236,5 +236,19 @@ __device__ __forceinline__ float sigmoid_fast(float v) {
   return __builtin_amdgcn_rcpf(1.0f + e);
 }
 
+
+// a * gelu_tanh(g) for bf16 operands held as floats (modules.py:289-291, :644):
+// gelu in fp32 as 0.5 g (1 + tanh u) with tanh u = 2 sigmoid(2u) - 1 rounded
+// to float32 first, so that the negative tail saturates to -0 exactly where a
+// float32 tanh does; gelu is rounded to bf16 like the module output it is in
+// the reference; the caller rounds the product.
+__device__ __forceinline__ float gelu_mul_bf16(float av, float gv) {
+  constexpr float c0 = 0.7978845608028654f;  // sqrt(2/pi)
+  constexpr float c1 = 0.044715f;
+  const float u = c0 * __builtin_fmaf(c1 * gv * gv, gv, gv);
+  const float t = __builtin_fmaf(2.0f, sigmoid_fast(2.0f * u), -1.0f);
+  return av * round_to_bf16(0.5f * gv * (1.0f + t));
+}
+
 }  // namespace rg
 #endif  // RG_COMMON_H_

@@ -13,10 +13,7 @@ namespace {
 constexpr float kGeluC0 = 0.7978845608028654f;  // sqrt(2/pi)
 constexpr float kGeluC1 = 0.044715f;
 
-// bf16: gelu in fp32 as 0.5 v (1 + tanh u) with tanh u = 2 sigmoid(2u) - 1
-// rounded to float32 first, so that the negative tail saturates to -0 exactly
-// where a float32 tanh does; gelu is rounded to bf16 like the module output it
-// is in the reference, then the product is rounded once.
+// bf16: gelu_mul_bf16 per element, the product rounded once.
 // One 16-byte item (eight elements) per thread, streaming loads and stores, no
 // loop: measured at 2^29 elements this shape (2^18 workgroups, each one
 // contiguous 4 KB of every operand) moves 6.4 TB/s, a grid-stride loop over
@@ -26,12 +23,7 @@ gelu_mul_bf16_kernel(const u32x4* __restrict__ a, const u32x4* __restrict__ g,
                      u32x4* __restrict__ out, int64_t n8,
                      const uint16_t* a_tail, const uint16_t* g_tail,
                      uint16_t* out_tail, int tail) {
-  auto one = [](float av, float gv) {
-    const float u = kGeluC0 * __builtin_fmaf(kGeluC1 * gv * gv, gv, gv);
-    const float t = __builtin_fmaf(2.0f, sigmoid_fast(2.0f * u), -1.0f);
-    const float y = round_to_bf16(0.5f * gv * (1.0f + t));
-    return av * y;
-  };
+  auto one = [](float av, float gv) { return gelu_mul_bf16(av, gv); };
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i < n8) {
     const u32x4 av = __builtin_nontemporal_load(a + i);

@@ -97,6 +97,17 @@ struct StepArgs {
   int B, W, H;
 };
 
+struct LinearArgs {
+  const void* x;         // [M, K] bf16
+  const void* w_packed;  // see launch_linear_pack
+  const void* bias;      // [N] or null
+  const void* residual;  // laid out like out, or null
+  void* out;             // [G, M, N / G]; gelu pairs: [M, N / 2]
+  float* partial;        // [slices, M, N] when K is split over the grid
+  int M, K, N;
+  int group_width;       // N / G
+};
+
 // Each returns hipSuccess or the launch error.  dtype: 0 = f32, 1 = bf16.
 hipError_t launch_conv1d_prefill(const ConvArgs& a, int dtype, hipStream_t s);
 hipError_t launch_conv1d_step(const ConvStepArgs& a, int dtype, hipStream_t s);
@@ -131,6 +142,12 @@ hipError_t launch_attn_decode_finish(const void* from_ring, const void* probs,
                                      int32_t* num_tokens, int B, int heads,
                                      int hd, int window, int update, int dtype,
                                      hipStream_t s);
+// Linear layers for at most 64 rows (rg_linear.hip).
+int linear_rows_k_slices(int K, int N);
+hipError_t launch_linear_pack(const void* w, void* packed, int N, int K,
+                              int layout, int groups, int pair, hipStream_t s);
+hipError_t launch_linear_rows(const LinearArgs& a, int gelu_pair,
+                              hipStream_t s);
 hipError_t launch_pack_gate_weights(const void* w_x, const void* w_a,
                                     void* packed, int H, hipStream_t s);
 

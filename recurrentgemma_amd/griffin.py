@@ -174,6 +174,10 @@ class MLPBlock(nn.Module):
     self.ffw_up = _StackedLinear(width, expanded_width, device=device,
                                  dtype=dtype)
     self.ffw_down = nn.Linear(expanded_width, width, device=device, dtype=dtype)
+    # for at most 64 rows (a decode step): up-projections, gelu and product in
+    # one pass over the stacked weight; down-projection with the residual add
+    self._rows_up = ops.PackedLinear(layout=1, gelu_pair=True)
+    self._rows_down = ops.PackedLinear()
     self.reset_parameters()
 
   def reset_parameters(self) -> None:
@@ -182,9 +186,17 @@ class MLPBlock(nn.Module):
     torch.nn.init.normal_(self.ffw_down.weight, mean=0.0, std=std)
     torch.nn.init.zeros_(self.ffw_down.bias)
 
-  def forward(self, x):
+  def forward(self, x, residual=None):
+    """residual: added to the result (the block's skip connection,
+    modules.py:897-898)."""
+    if (ops.PackedLinear.usable(x, self.width, 2 * self.expanded_width, True)
+        and ops.PackedLinear.usable(x, self.expanded_width, self.width)):
+      hidden = self._rows_up(x, (self.ffw_up.w,), (self.ffw_up.b,))
+      return self._rows_down(hidden, (self.ffw_down.weight,),
+                             (self.ffw_down.bias,), residual=residual)
     gate, up = self.ffw_up(x)
-    return self.ffw_down(ops.gelu_mul(up, gate))  # gelu(gate) * up, one pass
+    out = self.ffw_down(ops.gelu_mul(up, gate))  # gelu(gate) * up, one pass
+    return out if residual is None else out + residual
 
 
 def _inv_frequencies(head_dim, device, max_wavelength=_MAX_WAVELENGTH):
@@ -223,6 +235,10 @@ class LocalAttentionBlock(nn.Module):
     self.proj_k = nn.Linear(width, self.head_dim, bias=False, **kw)
     self.proj_v = nn.Linear(width, self.head_dim, bias=False, **kw)
     self.proj_final = nn.Linear(width, width, bias=True, **kw)
+    # the projections for at most 64 rows (a decode step)
+    self._rows_q = ops.PackedLinear()
+    self._rows_kv = ops.PackedLinear()
+    self._rows_final = ops.PackedLinear()
     self._inv_freq = None
     self.reset_parameters()
 
@@ -272,9 +288,16 @@ class LocalAttentionBlock(nn.Module):
   def forward(self, x, segment_pos, cache=None, return_cache=True):
     b, t, _ = x.shape
     assert segment_pos.shape == (b, t), segment_pos.shape
-    q = self.proj_q(x).reshape(b, t, self.num_heads, self.head_dim)
-    k = self.proj_k(x).reshape(b, t, 1, self.head_dim)
-    v = self.proj_v(x).reshape(b, t, 1, self.head_dim)
+    few_rows = (ops.PackedLinear.usable(x, self.width, self.width) and
+                ops.PackedLinear.usable(x, self.width, 2 * self.head_dim))
+    if few_rows:
+      q = self._rows_q(x, (self.proj_q.weight,))
+      k, v = self._rows_kv(x, (self.proj_k.weight, self.proj_v.weight))
+    else:
+      q, k, v = self.proj_q(x), self.proj_k(x), self.proj_v(x)
+    q = q.reshape(b, t, self.num_heads, self.head_dim)
+    k = k.reshape(b, t, 1, self.head_dim)
+    v = v.reshape(b, t, 1, self.head_dim)
     q, k = self._rope(q, segment_pos), self._rope(k, segment_pos)
 
     if cache is not None and t == 1:
@@ -309,7 +332,13 @@ class LocalAttentionBlock(nn.Module):
         v_all.transpose(1, 2).expand(-1, self.num_heads, -1, -1),
         attn_mask=mask[:, None])
     out = out.transpose(1, 2).reshape(b, t, self.width)
-    return self.proj_final(out), new_cache
+    return self._project_out(out), new_cache
+
+  def _project_out(self, x):
+    if ops.PackedLinear.usable(x, self.width, self.width):
+      return self._rows_final(x, (self.proj_final.weight,),
+                              (self.proj_final.bias,))
+    return self.proj_final(x)
 
   def _ring_positions(self, num_tokens, t):
     """Positions held by the ring (slot j keeps the largest position congruent
@@ -344,7 +373,7 @@ class LocalAttentionBlock(nn.Module):
     out = ops.attention_decode_finish(
         from_ring, probs, k[:, 0, 0], v[:, 0, 0], cache.keys, cache.values,
         cache.num_tokens, update_cache=return_cache)
-    out = self.proj_final(out.reshape(b, 1, self.width))
+    out = self._project_out(out.reshape(b, 1, self.width))
     return out, (cache if return_cache else None)
 
   @classmethod
@@ -406,7 +435,7 @@ class ResidualBlock(nn.Module):
                                            segment_pos, cache,
                                            return_cache=return_cache)
     residual, normed = self.channel_pre_norm.add_then_norm(mixed, x)
-    return self.mlp_block(normed) + residual, new_cache
+    return self.mlp_block(normed, residual=residual), new_cache
 
   @classmethod
   def init_cache(cls, batch_size, width, num_heads, attention_window_size,

@@ -118,6 +118,10 @@ class RecurrentBlock(nn.Module):
     # instead of returning new ones (set by callers that replay a captured
     # decode step on fixed buffers)
     self.decode_in_place = False
+    # the linear layers for at most 64 rows (a decode step): linear_y and
+    # linear_x as one pass over both weight matrices, linear_out as another
+    self._rows_yx = ops.PackedLinear()
+    self._rows_out = ops.PackedLinear()
     self.reset_parameters()
 
   def reset_parameters(self) -> None:
@@ -141,13 +145,24 @@ class RecurrentBlock(nn.Module):
     if training.is_enabled():
       return self._forward_differentiable(x, segment_pos, cache, return_cache)
     with torch.no_grad():
-      y = self.linear_y(x)
-      x = self.linear_x(x)
+      few_rows = (
+          ops.PackedLinear.usable(x, self.width, self.lru_width) and
+          ops.PackedLinear.usable(x, self.lru_width, self.width))
+      if few_rows:
+        y, x = self._rows_yx(x, (self.linear_y.weight, self.linear_x.weight),
+                             (self.linear_y.bias, self.linear_x.bias))
+      else:
+        y = self.linear_y(x)
+        x = self.linear_x(x)
       x, new_cache = recurrent_core(
           self.conv_1d, self.rg_lru, x, segment_pos, cache, return_cache,
           in_place=self.decode_in_place and cache is not None and return_cache)
       x = ops.gelu_mul(x, y)  # x * gelu(y), one pass (modules.py:627-628, 644)
-      x = self.linear_out(x)
+      if few_rows:
+        x = self._rows_out(x, (self.linear_out.weight,),
+                           (self.linear_out.bias,))
+      else:
+        x = self.linear_out(x)
     if not return_cache:
       return x, None
     return x, new_cache

@@ -399,6 +399,127 @@ def packed_gate_weights(w_x, w_a):
   return packed
 
 
+class PackedLinear:
+  """Linear layers that read the same few rows (a decode step), on the
+  weight-streaming kernel (rg_linear_rows).  Holds the weights in the kernel's
+  operand order, packed on first use and again whenever a parameter is written
+  to or re-pointed; the parameters themselves are passed with every call.
+
+  layout 0: `weights` are torch.nn.Linear weights [N_i, K] applied to the same
+    input; several of them (equal N_i) run as one launch and come back as a
+    tuple of outputs.
+  layout 1: one stacked Einsum weight [G, K, E] (layers.py:76-101) with bias
+    [G, 1, 1, E]; outputs as a tuple of G tensors, or, with gelu_pair (G = 2),
+    gelu(out[0]) * out[1] as one tensor (modules.py:752-757).
+  """
+
+  def __init__(self, layout=0, gelu_pair=False):
+    self.layout = layout
+    self.gelu_pair = gelu_pair
+    self._stamp = None
+    self._packed = None
+    self._bias = None
+    self._shape = None  # (N, K, groups)
+
+  def __deepcopy__(self, memo):
+    return PackedLinear(self.layout, self.gelu_pair)
+
+  @staticmethod
+  def usable(x, K, N, gelu_pair=False) -> bool:
+    """Whether x [..., K] qualifies: bf16 on the GPU, at most 64 rows, and a
+    weight shape the packed layout covers."""
+    return (x.is_cuda and x.dtype == torch.bfloat16 and
+            x.numel() // K <= 64 and
+            _lib.lib().rg_linear_packed_bytes(N, K, int(gelu_pair)) > 0)
+
+  def _prepare(self, weights, biases):
+    tensors = tuple(weights) + tuple(b for b in (biases or ()) if b is not None)
+    stamp = tuple((id(t), t.data_ptr(), t._version) for t in tensors)
+    if stamp == self._stamp:
+      return
+    w0 = weights[0]
+    lib = _lib.lib()
+    if self.layout == 0:
+      K = w0.shape[1]
+      rows = [w.shape[0] for w in weights]
+      if len(set(rows)) != 1 or any(w.shape[1] != K for w in weights):
+        raise ValueError("layers packed together must have equal shapes")
+      groups, N = len(weights), sum(rows)
+    else:
+      assert len(weights) == 1
+      groups, K, E = w0.shape
+      N = groups * E
+      if self.gelu_pair and groups != 2:
+        raise ValueError("gelu pairs need a weight stacked [2, K, E]")
+    nbytes = lib.rg_linear_packed_bytes(N, K, int(self.gelu_pair))
+    if nbytes == 0:
+      raise ValueError(f"unsupported linear shape N={N} K={K}")
+    packed = torch.empty(nbytes // 2, dtype=w0.dtype, device=w0.device)
+    with torch.cuda.device(w0.device):
+      if self.layout == 0:
+        at = 0
+        for w in weights:  # tile blocks of consecutive rows are consecutive
+          part = packed[at:at + w.numel()]
+          _lib.check(lib.rg_linear_pack(_p(_dev(w, "weight")), 0, 1, 0, _p(part),
+                                        w.shape[0], K, _stream(w)))
+          at += w.numel()
+      else:
+        _lib.check(lib.rg_linear_pack(_p(_dev(w0, "weight")), 1, groups,
+                                      int(self.gelu_pair), _p(packed), N, K,
+                                      _stream(w0)))
+    bias = None
+    if biases is not None and any(b is not None for b in biases):
+      if any(b is None for b in biases):
+        raise ValueError("either every layer has a bias or none")
+      bias = torch.cat([b.detach().reshape(-1) for b in biases])
+      assert bias.numel() == N
+    self._packed, self._bias = packed, bias
+    self._shape = (N, K, groups)
+    self._stamp = stamp
+
+  @torch.no_grad()
+  def __call__(self, x, weights, biases=None, residual=None):
+    """x [..., K].  Returns out [..., N] (one layer), a tuple of outputs
+    (several layers / a stacked weight), or the gelu pair product [..., N/2].
+    residual (one layer only): added after the output is rounded."""
+    x = _dev(x, "x")
+    _dtype_code(x)
+    self._prepare(weights, biases)
+    N, K, groups = self._shape
+    if x.shape[-1] != K:
+      raise ValueError(f"x has {x.shape[-1]} columns, the weights take {K}")
+    _same(x.dtype, x.device, weight=weights[0], residual=residual)
+    lead = x.shape[:-1]
+    M = x.numel() // K
+    lib = _lib.lib()
+    if self.gelu_pair:
+      out = torch.empty((*lead, N // 2), dtype=x.dtype, device=x.device)
+      g = 1
+    elif groups > 1:
+      out = torch.empty((groups, *lead, N // groups), dtype=x.dtype,
+                        device=x.device)
+      g = groups
+    else:
+      out = torch.empty((*lead, N), dtype=x.dtype, device=x.device)
+      g = 1
+    if residual is not None:
+      if g != 1 or self.gelu_pair:
+        raise ValueError("a residual goes with a single plain layer")
+      residual = _dev(residual, "residual")
+      assert residual.shape == out.shape
+    need = lib.rg_linear_rows_workspace_bytes(M, K, N)
+    ws = (torch.empty(need, dtype=torch.uint8, device=x.device)
+          if need and not self.gelu_pair else None)
+    with torch.cuda.device(x.device):
+      _lib.check(lib.rg_linear_rows(
+          _p(x), _p(self._packed), _p(self._bias), _p(residual), _p(out),
+          _p(ws), need if ws is not None else 0, M, K, N, g,
+          int(self.gelu_pair), _stream(x)))
+    if g > 1:
+      return tuple(out[i] for i in range(g))
+    return out
+
+
 def recurrent_step(x, segment_pos, conv_cache, h, conv_w, conv_b, w_x, b_x, w_a,
                    b_a, a_param, in_place=False):
   """One decode step of conv -> RG-LRU.  Returns (y, h_new, conv_cache_new).

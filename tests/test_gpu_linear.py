@@ -1,0 +1,176 @@
+"""The linear layers for few rows (rg_linear_pack / rg_linear_rows), on the GPU.
+
+Reference: the exact product in float64 on the host.  The kernel accumulates
+in float32 and rounds once to bf16, so a result may differ from the rounded
+exact value by the float32 accumulation error (bounded here by 2e-5 of the
+sum of absolute terms) plus one bf16 ulp where that error crosses a rounding
+boundary.  Residual add, gelu pairs and grouped outputs are checked bit for
+bit against the same kernel's plain output followed by the separate steps
+(torch's add, this package's rg_gelu_mul)."""
+
+import copy
+
+import pytest
+import torch
+
+from recurrentgemma_amd import griffin as G
+from recurrentgemma_amd import ops
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+BF = torch.bfloat16
+
+
+def _rand(gen, *shape, scale=1.0):
+  return (torch.randn(*shape, generator=gen) * scale).to(BF)
+
+
+def _check(got, x, w_rows, bias):
+  """got [M, N] against x [M, K] @ w_rows [N, K]^T + bias in float64."""
+  xd, wd = x.double(), w_rows.double()
+  exact = xd @ wd.T
+  bound = 2e-5 * (xd.abs() @ wd.abs().T)
+  if bias is not None:
+    exact = exact + bias.double()
+    bound = bound + 2e-5 * bias.double().abs()
+  ulp = torch.maximum(exact.abs(), torch.tensor(1e-30, dtype=torch.float64))
+  ulp = 2.0 ** (torch.floor(torch.log2(ulp)) - 7)
+  err = (got.cpu().double() - exact).abs()
+  worst = (err - bound - ulp).max().item()
+  assert worst <= 0, worst
+
+
+@pytest.mark.parametrize("M,K,N,with_bias", [
+    (64, 2560, 2560, True),    # one tile of 32 weight rows per workgroup
+    (5, 128, 64, False),       # fewer rows than a tile, two chunks of K
+    (33, 192, 96, True),       # second half-tile partly filled, odd chunk count
+    (64, 7680, 2560, True),    # K split over the grid, finished by a second pass
+    (1, 2560, 15360, True),    # two tiles per workgroup
+])
+def test_linear_rows(M, K, N, with_bias):
+  gen = torch.Generator().manual_seed(M * 7 + K + N)
+  x = _rand(gen, M, K)
+  w = _rand(gen, N, K, scale=K ** -0.5)
+  b = _rand(gen, N) if with_bias else None
+  layer = ops.PackedLinear()
+  xg, wg = x.to(DEV), w.to(DEV)
+  bg = None if b is None else b.to(DEV)
+  got = layer(xg, (wg,), None if bg is None else (bg,))
+  assert got.shape == (M, N) and got.dtype == BF
+  _check(got, x, w, b)
+  # leading dimensions are rows; same bits on a second run
+  again = layer(xg.reshape(1, M, K), (wg,), None if bg is None else (bg,))
+  assert torch.equal(again[0], got)
+  # residual: added after the product is rounded, like a separate add
+  res = _rand(gen, M, N).to(DEV)
+  with_res = layer(xg, (wg,), None if bg is None else (bg,), residual=res)
+  assert torch.equal(with_res, got + res)
+  # against the library product of the same operands: a few bf16 ulps
+  lib = torch.nn.functional.linear(xg, wg, bg)
+  scale = lib.float().abs().max().item()
+  assert (lib.float() - got.float()).abs().max().item() <= 2 ** -6 * scale
+
+
+def test_layers_packed_together():
+  """Two nn.Linear layers on the same input as one launch: each output equals
+  the layer run alone."""
+  gen = torch.Generator().manual_seed(11)
+  M, K, N = 64, 2560, 2560
+  x = _rand(gen, M, K).to(DEV)
+  w1, w2 = (_rand(gen, N, K, scale=K ** -0.5).to(DEV) for _ in range(2))
+  b1, b2 = (_rand(gen, N).to(DEV) for _ in range(2))
+  both = ops.PackedLinear()(x, (w1, w2), (b1, b2))
+  assert len(both) == 2
+  assert torch.equal(both[0], ops.PackedLinear()(x, (w1,), (b1,)))
+  assert torch.equal(both[1], ops.PackedLinear()(x, (w2,), (b2,)))
+  with pytest.raises(ValueError):
+    ops.PackedLinear()(x, (w1, w2[:64]), (b1, b2[:64]))
+
+
+@pytest.mark.parametrize("M,K,E", [(64, 2560, 7680), (3, 128, 96)])
+def test_stacked_weight_and_gelu_pairs(M, K, E):
+  """The MLP's stacked up-projection [2, K, E] (Einsum "cdD" layout): plain
+  outputs against float64, the fused gelu(gate) * up against rg_gelu_mul on
+  those outputs."""
+  gen = torch.Generator().manual_seed(E)
+  x = _rand(gen, M, K)
+  w = _rand(gen, 2, K, E, scale=K ** -0.5)
+  b = _rand(gen, 2, 1, 1, E)
+  xg, wg, bg = x.to(DEV), w.to(DEV), b.to(DEV)
+  gate, up = ops.PackedLinear(layout=1)(xg, (wg,), (bg,))
+  _check(gate, x, w[0].T, b[0].reshape(-1))
+  _check(up, x, w[1].T, b[1].reshape(-1))
+  if E % 32 == 0:
+    fused = ops.PackedLinear(layout=1, gelu_pair=True)(xg, (wg,), (bg,))
+    assert fused.shape == (M, E)
+    assert torch.equal(fused, ops.gelu_mul(up.contiguous(), gate.contiguous()))
+
+
+def test_repacks_when_a_weight_changes():
+  gen = torch.Generator().manual_seed(3)
+  x = _rand(gen, 8, 128).to(DEV)
+  w = _rand(gen, 64, 128).to(DEV)
+  layer = ops.PackedLinear()
+  first = layer(x, (w,))
+  w.mul_(2.0)  # exact in bf16
+  assert torch.equal(layer(x, (w,)), first * 2.0)
+  other = _rand(gen, 64, 128).to(DEV)
+  _check(layer(x, (other,)), x.cpu(), other.cpu(), None)
+  assert copy.deepcopy(layer)._packed is None
+
+
+def test_unsupported_shapes_are_refused():
+  x = torch.zeros(4, 100, dtype=BF, device=DEV)
+  assert not ops.PackedLinear.usable(x, 100, 64)         # K % 64
+  assert not ops.PackedLinear.usable(x.float(), 100, 64)
+  x = torch.zeros(65, 128, dtype=BF, device=DEV)
+  assert not ops.PackedLinear.usable(x, 128, 64)         # more than 64 rows
+  assert ops.PackedLinear.usable(x[:64], 128, 64)
+  with pytest.raises(ValueError):
+    ops.PackedLinear()(x[:4], (torch.zeros(48, 128, dtype=BF, device=DEV),))
+
+
+def test_decode_steps_with_and_without_the_row_kernels(monkeypatch):
+  """A small bf16 model: prompt, then three cached steps, once with the
+  linear layers of the steps on rg_linear_rows and once on the library
+  products.  Same weights, different summation order: logits agree to bf16
+  noise."""
+  R, A = G.TemporalBlockType.RECURRENT, G.TemporalBlockType.ATTENTION
+  cfg = G.GriffinConfig(
+      vocab_size=512, width=256, mlp_expanded_width=768, num_heads=2,
+      block_types=(R, A, R), embeddings_scale_by_sqrt_dim=True,
+      attention_window_size=16, logits_soft_cap=30.0, lru_width=256)
+  torch.manual_seed(5)
+  model = G.Griffin(cfg, dtype=BF).to(DEV).eval()
+  gen = torch.Generator().manual_seed(6)
+  B, T = 4, 20  # 80 rows: the prompt pass stays on the library products
+  tokens = torch.randint(0, 512, (B, T + 3), generator=gen).to(DEV)
+  pos = torch.arange(T + 3, device=DEV)[None].expand(B, -1).to(torch.int32)
+
+  def run():
+    _, cache = model(tokens[:, :T], pos[:, :T], None, return_logits=False,
+                     return_cache=True)
+    outs = []
+    for i in range(T, T + 3):
+      logits, cache = model(tokens[:, i:i + 1], pos[:, i:i + 1], cache,
+                            return_logits=True, return_cache=True)
+      outs.append(logits.float())
+    return torch.stack(outs)
+
+  calls = []
+  real = ops.PackedLinear.__call__
+
+  def counting(self, *a, **k):
+    calls.append(1)
+    return real(self, *a, **k)
+
+  monkeypatch.setattr(ops.PackedLinear, "__call__", counting)
+  with_rows = run()
+  # per step: recurrent 2 x (2 + 2 MLP) + attention (3 + 2 MLP)
+  assert len(calls) == 3 * 13, len(calls)
+  monkeypatch.setattr(ops.PackedLinear, "usable",
+                      staticmethod(lambda *a, **k: False))
+  library = run()
+  assert len(calls) == 3 * 13
+  scale = library.abs().max().item()
+  assert (with_rows - library).abs().max().item() <= 0.03 * scale

@@ -24,7 +24,7 @@ def _declared_symbols():
 
 def test_library_exports_every_declared_symbol():
   names = _declared_symbols()
-  assert len(names) == 20, names
+  assert len(names) == 24, names
   lib = ctypes.CDLL(_lib.LIB_PATH)
   for n in names:
     assert hasattr(lib, n), n
@@ -71,6 +71,30 @@ def test_c_side_validation_without_launch():
   assert rc == -1 and b"alias" in lib.rg_last_error()
   rc = lib.rg_add_rms_norm(ok, None, ok, ok, y, 4, 64, 1e-6, 1, None)
   assert rc == -1 and b"null" in lib.rg_last_error()
+  # linear layers for few rows
+  assert lib.rg_linear_packed_bytes(2560, 2560, 0) == 2560 * 2560 * 2
+  assert lib.rg_linear_packed_bytes(2560, 2500, 0) == 0   # K % 64
+  assert lib.rg_linear_packed_bytes(2576, 2560, 0) == 0   # N % 32
+  assert lib.rg_linear_packed_bytes(2592, 2560, 1) == 0   # pairs: N % 64
+  rc = lib.rg_linear_pack(ok, 0, 1, 0, y, 2576, 2560, None)
+  assert rc == -2 and b"N=2576" in lib.rg_last_error()
+  rc = lib.rg_linear_pack(ok, 2, 1, 0, y, 64, 64, None)
+  assert rc == -1 and b"layout" in lib.rg_last_error()
+  rc = lib.rg_linear_pack(ok, 0, 1, 0, ok, 64, 64, None)
+  assert rc == -1 and b"alias" in lib.rg_last_error()
+  assert lib.rg_linear_rows_workspace_bytes(64, 2560, 2560) == 0
+  assert lib.rg_linear_rows_workspace_bytes(64, 7680, 2560) == 3 * 64 * 2560 * 4
+  rc = lib.rg_linear_rows(ok, ok, None, None, y, None, 0, 65, 64, 64, 1, 0, None)
+  assert rc == -2 and b"M <= 64" in lib.rg_last_error()
+  rc = lib.rg_linear_rows(ok, ok, None, None, ok, None, 0, 4, 64, 64, 1, 0, None)
+  assert rc == -1 and b"alias" in lib.rg_last_error()
+  rc = lib.rg_linear_rows(ok, ok, None, ok, y, None, 0, 4, 64, 64, 1, 1, None)
+  assert rc == -1 and b"gelu pairs" in lib.rg_last_error()
+  rc = lib.rg_linear_rows(ok, ok, None, None, y, None, 0, 4, 64, 64, 3, 0, None)
+  assert rc == -1 and b"groups" in lib.rg_last_error()
+  rc = lib.rg_linear_rows(ok, ok, None, None, y, None, 0, 64, 7680, 2560, 1, 0,
+                          None)
+  assert rc == -4 and b"workspace" in lib.rg_last_error()
   args = [ok, ok, 1, ok, ok, ok, ok, ok, ok, None, ok, None, y, None, None]
   rc = lib.rg_recurrent_prefill(*args, 1, 8, 256, 1, 0, None)
   assert rc == -2 and b"unsupported" in lib.rg_last_error().lower()  # fp32
