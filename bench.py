@@ -218,7 +218,8 @@ def run_griffin(args, torch, rg, wl):
                             "as a captured HIP graph")
                          + "), recurrent blocks: "
                          "rg_recurrent_prefill / two-kernel form + "
-                         "rg_recurrent_step_packed + rg_gelu_mul"},
+                         "rg_recurrent_step_packed + rg_gelu_mul; linear "
+                         "layers of a decode step: rg_linear_rows"},
       "prompt_pass": {"ms": t_prompt * 1e3,
                       "tokens_per_s": B * T / t_prompt},
       "whole_generation": {"ms": t_full * 1e3,

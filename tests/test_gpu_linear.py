@@ -61,6 +61,8 @@ def test_linear_rows(M, K, N, with_bias):
   # leading dimensions are rows; same bits on a second run
   again = layer(xg.reshape(1, M, K), (wg,), None if bg is None else (bg,))
   assert torch.equal(again[0], got)
+  for _ in range(10):  # whichever workgroup adds the slices of K, same sum
+    assert torch.equal(layer(xg, (wg,), None if bg is None else (bg,)), got)
   # residual: added after the product is rounded, like a separate add
   res = _rand(gen, M, N).to(DEV)
   with_res = layer(xg, (wg,), None if bg is None else (bg,), residual=res)
