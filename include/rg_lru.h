@@ -284,7 +284,19 @@ int rg_recurrent_step_packed(const void* x, const void* segpos,
  *   workspace: rg_linear_rows_workspace_bytes(M, K, N) bytes (may be 0), for
  *   the partial sums of shapes whose K is split over the grid; the sums are
  *   added in a fixed order, results do not vary from run to run.
- *   out must not alias x. */
+ *   out must not alias x.
+ * rg_linear_rows_partial / rg_add_rms_norm_partial: a layer whose result goes
+ *   straight into a residual sum and an RMSNorm (linear_out and proj_final into
+ *   channel_pre_norm, modules.py:893-896; ffw_down into the next block's
+ *   temporal_pre_norm, modules.py:886-898) without being written in between.
+ *   The first writes only the fp32 partial sums `partial` [slices, M, N] of
+ *   x @ w^T with K split in `slices` (1..8) over the grid -- three times the
+ *   workgroups for the 2560-row layers, which alone fill a third of the CUs.
+ *   The second reads them instead of x: v = round(sum over slices, in slice
+ *   order, + bias); with addend, v = round(v + addend); sum_out = v,
+ *   out = rg_rms_norm(v).  bf16, width % 8 == 0, width <= 4096.  The same
+ *   values as those steps taken one by one (rg_linear_rows itself may split K
+ *   differently and then differs in the last bit of the fp32 sum). */
 size_t rg_linear_packed_bytes(int N, int K, int gelu_pair);
 int rg_linear_pack(const void* w, int layout, int groups, int gelu_pair,
                    void* packed, int N, int K, void* stream);
@@ -293,6 +305,12 @@ int rg_linear_rows(const void* x, const void* w_packed, const void* bias,
                    const void* residual, void* out, void* workspace,
                    size_t workspace_bytes, int M, int K, int N, int groups,
                    int gelu_pair, void* stream);
+int rg_linear_rows_partial(const void* x, const void* w_packed, void* partial,
+                           int M, int K, int N, int slices, void* stream);
+int rg_add_rms_norm_partial(const void* partial, int slices, const void* bias,
+                            const void* addend, const void* scale,
+                            void* sum_out, void* out, int rows, int width,
+                            float eps, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

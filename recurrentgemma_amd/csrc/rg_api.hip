@@ -563,6 +563,58 @@ int rg_linear_rows(const void* x, const void* w_packed, const void* bias,
       __func__, rg::launch_linear_rows(a, gelu_pair != 0, (hipStream_t)stream));
 }
 
+int rg_linear_rows_partial(const void* x, const void* w_packed, void* partial,
+                           int M, int K, int N, int slices, void* stream) {
+  RG_REQUIRE(M > 0 && K > 0 && N > 0, "%s: M=%d K=%d N=%d must be positive",
+             __func__, M, K, N);
+  if (M > 64 || rg_linear_packed_bytes(N, K, 0) == 0)
+    return fail(RG_ERR_UNSUPPORTED,
+                "%s: needs M <= 64, K %% 64 == 0, N %% 32 == 0, got M=%d K=%d "
+                "N=%d", __func__, M, K, N);
+  RG_REQUIRE(slices >= 1 && slices <= 8, "%s: slices=%d not in 1..8", __func__,
+             slices);
+  RG_CHECK_PTR(x);
+  RG_CHECK_PTR(w_packed);
+  RG_CHECK_PTR(partial);
+  RG_REQUIRE(partial != x, "%s: partial must not alias x", __func__);
+  rg::LinearArgs a{};
+  a.x = x;
+  a.w_packed = w_packed;
+  a.partial = (float*)partial;
+  a.M = M;
+  a.K = K;
+  a.N = N;
+  a.group_width = N;
+  return launch_status(__func__, rg::launch_linear_rows_partial(
+                                     a, slices, (hipStream_t)stream));
+}
+
+int rg_add_rms_norm_partial(const void* partial, int slices, const void* bias,
+                            const void* addend, const void* scale,
+                            void* sum_out, void* out, int rows, int width,
+                            float eps, int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(rows > 0 && width > 0, "%s: rows=%d width=%d must be positive",
+             __func__, rows, width);
+  if (dtype != RG_DTYPE_BF16 || width % 8 != 0 || width > 4096)
+    return fail(RG_ERR_UNSUPPORTED,
+                "%s: needs bf16 and width %% 8 == 0, width <= 4096 (dtype=%d "
+                "width=%d)", __func__, dtype, width);
+  RG_REQUIRE(slices >= 1 && slices <= 8, "%s: slices=%d not in 1..8", __func__,
+             slices);
+  RG_CHECK_PTR(partial);
+  RG_CHECK_PTR(scale);
+  RG_CHECK_PTR(sum_out);
+  RG_CHECK_PTR(out);
+  RG_CHECK_OPT_PTR(bias);
+  RG_CHECK_OPT_PTR(addend);
+  RG_REQUIRE(out != sum_out, "%s: out must not alias sum_out", __func__);
+  return launch_status(
+      __func__, rg::launch_rms_norm_partial((const float*)partial, slices, bias,
+                                            addend, scale, sum_out, out, rows,
+                                            width, eps, (hipStream_t)stream));
+}
+
 int rg_recurrent_step_packed(const void* x, const void* segpos,
                              int segpos_is_i64, const void* conv_cache_in,
                              void* conv_cache_out, const void* h_in,

@@ -113,9 +113,18 @@ rms_norm_kernel(const T* __restrict__ x, const T* __restrict__ addend,
 // lanes, the row stays in registers between the two passes (one read, one
 // write; the scalar kernel above re-reads through the cache and moved
 // 1.7 TB/s on 131 072 rows of 2560).
-template <bool ADD>
+// The row a linear layer left as fp32 partial sums over slices of its K
+// (rg_linear.hip): x = round(sum of the slices, in slice order, + bias).
+struct PartialRows {
+  const f32x4* sums;     // [slices][rows][width]
+  int slices;
+  int64_t slice_stride;  // rows * width / 4
+  const u32x4* bias;     // [width] or null
+};
+
+template <bool ADD, bool FROM_PARTIAL>
 __global__ void __launch_bounds__(256)
-rms_norm_bf16_rows_kernel(const u32x4* __restrict__ x,
+rms_norm_bf16_rows_kernel(const u32x4* __restrict__ x, PartialRows part,
                           const u32x4* __restrict__ addend,
                           const u32x4* __restrict__ scale,
                           u32x4* __restrict__ sum_out,
@@ -131,7 +140,29 @@ rms_norm_bf16_rows_kernel(const u32x4* __restrict__ x,
   for (int c = 0; c < 2; ++c) {
     const int i = threadIdx.x + c * 256;
     v[c] = u32x4{0u, 0u, 0u, 0u};
-    if (i < chunks) v[c] = __builtin_nontemporal_load(xr + i);
+    if (!FROM_PARTIAL && i < chunks) v[c] = __builtin_nontemporal_load(xr + i);
+    if (FROM_PARTIAL && i < chunks) {
+      f32x4 lo = {0.0f, 0.0f, 0.0f, 0.0f}, hi = lo;
+      const f32x4* src = part.sums + (row + i) * 2;
+      for (int s = 0; s < part.slices; ++s) {
+        lo += src[s * part.slice_stride];
+        hi += src[s * part.slice_stride + 1];
+      }
+      if (part.bias) {
+        const u32x4 b = part.bias[i];
+        lo += f32x4{__uint_as_float(b[0] << 16),
+                    __uint_as_float(b[0] & 0xffff0000u),
+                    __uint_as_float(b[1] << 16),
+                    __uint_as_float(b[1] & 0xffff0000u)};
+        hi += f32x4{__uint_as_float(b[2] << 16),
+                    __uint_as_float(b[2] & 0xffff0000u),
+                    __uint_as_float(b[3] << 16),
+                    __uint_as_float(b[3] & 0xffff0000u)};
+      }
+      v[c] = u32x4{pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]),
+                   pack_bf16x2(hi[0], hi[1]), pack_bf16x2(hi[2], hi[3])};
+      if (!ADD) sum_out[row + i] = v[c];
+    }
     if (ADD && i < chunks) {
       const u32x4 w = __builtin_nontemporal_load(addend + row + i);
 #pragma unroll
@@ -210,14 +241,15 @@ hipError_t launch_rms_norm(const void* x, const void* addend, const void* scale,
   if (dtype != 0 && width % 8 == 0 && width <= 4096 && aligned) {
     const int chunks = width / 8;
     const float inv = 1.0f / (float)width;
+    const PartialRows none{};
     if (add)
-      rms_norm_bf16_rows_kernel<true><<<grid, 256, 0, s>>>(
-          (const u32x4*)x, (const u32x4*)addend, (const u32x4*)scale,
+      rms_norm_bf16_rows_kernel<true, false><<<grid, 256, 0, s>>>(
+          (const u32x4*)x, none, (const u32x4*)addend, (const u32x4*)scale,
           (u32x4*)sum_out, (u32x4*)out, chunks, inv, eps);
     else
-      rms_norm_bf16_rows_kernel<false><<<grid, 256, 0, s>>>(
-          (const u32x4*)x, nullptr, (const u32x4*)scale, nullptr, (u32x4*)out,
-          chunks, inv, eps);
+      rms_norm_bf16_rows_kernel<false, false><<<grid, 256, 0, s>>>(
+          (const u32x4*)x, none, nullptr, (const u32x4*)scale, nullptr,
+          (u32x4*)out, chunks, inv, eps);
     return hipGetLastError();
   }
   auto run = [&](auto* tag) {
@@ -232,6 +264,32 @@ hipError_t launch_rms_norm(const void* x, const void* addend, const void* scale,
   };
   if (dtype == 0) run((float*)nullptr);
   else run((uint16_t*)nullptr);
+  return hipGetLastError();
+}
+
+// bf16 rows given as partial sums; the caller has checked width % 8 == 0,
+// width <= 4096 and 16-byte alignment.
+hipError_t launch_rms_norm_partial(const float* sums, int slices,
+                                   const void* bias, const void* addend,
+                                   const void* scale, void* sum_out, void* out,
+                                   int rows, int width, float eps,
+                                   hipStream_t s) {
+  const int chunks = width / 8;
+  const float inv = 1.0f / (float)width;
+  PartialRows part;
+  part.sums = (const f32x4*)sums;
+  part.slices = slices;
+  part.slice_stride = (int64_t)rows * width / 4;
+  part.bias = (const u32x4*)bias;
+  const dim3 grid((unsigned)rows);
+  if (addend)
+    rms_norm_bf16_rows_kernel<true, true><<<grid, 256, 0, s>>>(
+        nullptr, part, (const u32x4*)addend, (const u32x4*)scale,
+        (u32x4*)sum_out, (u32x4*)out, chunks, inv, eps);
+  else
+    rms_norm_bf16_rows_kernel<false, true><<<grid, 256, 0, s>>>(
+        nullptr, part, nullptr, (const u32x4*)scale, (u32x4*)sum_out,
+        (u32x4*)out, chunks, inv, eps);
   return hipGetLastError();
 }
 

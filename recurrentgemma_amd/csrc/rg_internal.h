@@ -148,6 +148,15 @@ hipError_t launch_linear_pack(const void* w, void* packed, int N, int K,
                               int layout, int groups, int pair, hipStream_t s);
 hipError_t launch_linear_rows(const LinearArgs& a, int gelu_pair,
                               hipStream_t s);
+// Only the fp32 partial sums a.partial[slices][M][N] of x @ W^T, K split in
+// `slices`; rg_elementwise.hip's norm kernel takes them from there.
+hipError_t launch_linear_rows_partial(const LinearArgs& a, int slices,
+                                      hipStream_t s);
+hipError_t launch_rms_norm_partial(const float* sums, int slices,
+                                   const void* bias, const void* addend,
+                                   const void* scale, void* sum_out, void* out,
+                                   int rows, int width, float eps,
+                                   hipStream_t s);
 hipError_t launch_pack_gate_weights(const void* w_x, const void* w_a,
                                     void* packed, int H, hipStream_t s);
 

@@ -328,6 +328,11 @@ hipError_t launch_linear_pack(const void* w, void* packed, int N, int K,
   return hipGetLastError();
 }
 
+hipError_t launch_linear_rows_partial(const LinearArgs& a, int slices,
+                                      hipStream_t s) {
+  return launch_rows<1, kPartial>(a, dim3(a.N / 32, slices), s);
+}
+
 hipError_t launch_linear_rows(const LinearArgs& a, int gelu_pair,
                               hipStream_t s) {
   const int tiles = a.N / 32;

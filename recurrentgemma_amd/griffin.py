@@ -124,7 +124,9 @@ class RMSNorm(nn.Module):
     return ops.rms_norm(x, self.scale, self.eps)
 
   def add_then_norm(self, x, addend):
-    """(x + addend, forward(x + addend)) in one kernel."""
+    """(x + addend, forward(x + addend)) in one kernel.  x may be an
+    ops.PartialSums (a layer output not added up yet; addend may then be None
+    or ride in x)."""
     return ops.add_rms_norm(x, addend, self.scale, self.eps)
 
 
@@ -186,12 +188,17 @@ class MLPBlock(nn.Module):
     torch.nn.init.normal_(self.ffw_down.weight, mean=0.0, std=std)
     torch.nn.init.zeros_(self.ffw_down.bias)
 
-  def forward(self, x, residual=None):
+  def forward(self, x, residual=None, defer_out=False):
     """residual: added to the result (the block's skip connection,
-    modules.py:897-898)."""
+    modules.py:897-898).  defer_out: the caller normalises the result next and
+    accepts it as ops.PartialSums (returned where that saves a pass)."""
     if (ops.PackedLinear.usable(x, self.width, 2 * self.expanded_width, True)
         and ops.PackedLinear.usable(x, self.expanded_width, self.width)):
       hidden = self._rows_up(x, (self.ffw_up.w,), (self.ffw_up.b,))
+      if defer_out and ops.PackedLinear.partial_slices(
+          hidden, self.expanded_width, self.width):
+        return self._rows_down.partial(hidden, (self.ffw_down.weight,),
+                                       (self.ffw_down.bias,), addend=residual)
       return self._rows_down(hidden, (self.ffw_down.weight,),
                              (self.ffw_down.bias,), residual=residual)
     gate, up = self.ffw_up(x)
@@ -285,7 +292,9 @@ class LocalAttentionBlock(nn.Module):
                                num_tokens=num_tokens)
 
   @torch.no_grad()
-  def forward(self, x, segment_pos, cache=None, return_cache=True):
+  def forward(self, x, segment_pos, cache=None, return_cache=True,
+              defer_out=False):
+    """defer_out: as for RecurrentBlock.forward."""
     b, t, _ = x.shape
     assert segment_pos.shape == (b, t), segment_pos.shape
     few_rows = (ops.PackedLinear.usable(x, self.width, self.width) and
@@ -301,7 +310,7 @@ class LocalAttentionBlock(nn.Module):
     q, k = self._rope(q, segment_pos), self._rope(k, segment_pos)
 
     if cache is not None and t == 1:
-      return self._decode_step(x, q, k, v, cache, return_cache)
+      return self._decode_step(x, q, k, v, cache, return_cache, defer_out)
 
     new_cache = None
     if cache is not None:
@@ -332,12 +341,14 @@ class LocalAttentionBlock(nn.Module):
         v_all.transpose(1, 2).expand(-1, self.num_heads, -1, -1),
         attn_mask=mask[:, None])
     out = out.transpose(1, 2).reshape(b, t, self.width)
-    return self._project_out(out), new_cache
+    return self._project_out(out, defer_out), new_cache
 
-  def _project_out(self, x):
+  def _project_out(self, x, defer_out=False):
+    weights, biases = (self.proj_final.weight,), (self.proj_final.bias,)
+    if defer_out and ops.PackedLinear.partial_slices(x, self.width, self.width):
+      return self._rows_final.partial(x, weights, biases)
     if ops.PackedLinear.usable(x, self.width, self.width):
-      return self._rows_final(x, (self.proj_final.weight,),
-                              (self.proj_final.bias,))
+      return self._rows_final(x, weights, biases)
     return self.proj_final(x)
 
   def _ring_positions(self, num_tokens, t):
@@ -351,7 +362,7 @@ class LocalAttentionBlock(nn.Module):
     q_pos = torch.arange(t, device=n.device)[None] + n
     return k_pos, q_pos
 
-  def _decode_step(self, x, q, k, v, cache, return_cache):
+  def _decode_step(self, x, q, k, v, cache, return_cache, defer_out=False):
     """One new token against the ring and itself, without concatenating or
     expanding the cached keys and values: all heads share them, so the scores
     are one batched [heads, head_dim] x [head_dim, window] product per row on
@@ -373,7 +384,7 @@ class LocalAttentionBlock(nn.Module):
     out = ops.attention_decode_finish(
         from_ring, probs, k[:, 0, 0], v[:, 0, 0], cache.keys, cache.values,
         cache.num_tokens, update_cache=return_cache)
-    out = self._project_out(out.reshape(b, 1, self.width))
+    out = self._project_out(out.reshape(b, 1, self.width), defer_out)
     return out, (cache if return_cache else None)
 
   @classmethod
@@ -430,12 +441,22 @@ class ResidualBlock(nn.Module):
     self.mlp_block.reset_parameters()
 
   @torch.no_grad()
-  def forward(self, x, segment_pos, cache=None, return_cache=True):
-    mixed, new_cache = self.temporal_block(self.temporal_pre_norm(x),
-                                           segment_pos, cache,
-                                           return_cache=return_cache)
+  def forward(self, x, segment_pos, cache=None, return_cache=True,
+              defer_out=False):
+    """x and, with defer_out, the result may be ops.PartialSums: the output of
+    the previous block's last layer before its slices of K are added, which
+    the norm kernel that reads it next does (Griffin.forward chains the blocks
+    that way for a decode step)."""
+    if isinstance(x, ops.PartialSums):
+      x, normed = self.temporal_pre_norm.add_then_norm(x, None)
+    else:
+      normed = self.temporal_pre_norm(x)
+    mixed, new_cache = self.temporal_block(normed, segment_pos, cache,
+                                           return_cache=return_cache,
+                                           defer_out=True)
     residual, normed = self.channel_pre_norm.add_then_norm(mixed, x)
-    return self.mlp_block(normed, residual=residual), new_cache
+    return (self.mlp_block(normed, residual=residual, defer_out=defer_out),
+            new_cache)
 
   @classmethod
   def init_cache(cls, batch_size, width, num_heads, attention_window_size,
@@ -521,10 +542,16 @@ class Griffin(nn.Module):
       name = f"blocks.{i}"
       x, new_cache[name] = block(x, segment_pos,
                                  None if cache is None else cache[name],
-                                 return_cache=return_cache)
+                                 return_cache=return_cache,
+                                 defer_out=return_logits or
+                                 i + 1 < len(self.blocks))
     if not return_logits:
       return None, new_cache
-    logits = self.embedder.decode(self.final_norm(x))
+    if isinstance(x, ops.PartialSums):
+      x = self.final_norm.add_then_norm(x, None)[1]
+    else:
+      x = self.final_norm(x)
+    logits = self.embedder.decode(x)
     cap = self.config.logits_soft_cap
     if cap:
       logits = torch.tanh(logits / cap) * cap

@@ -141,7 +141,11 @@ class RecurrentBlock(nn.Module):
     std = math.sqrt(self.final_w_init_variance_scale / self.lru_width)
     torch.nn.init.normal_(w, mean=0.0, std=std)
 
-  def forward(self, x, segment_pos, cache=None, return_cache=True):
+  def forward(self, x, segment_pos, cache=None, return_cache=True,
+              defer_out=False):
+    """defer_out: the caller adds the result to a residual and normalises it
+    next (ops.add_rms_norm) and accepts it as ops.PartialSums, which is what
+    it gets where that saves a pass (a few rows, bf16)."""
     if training.is_enabled():
       return self._forward_differentiable(x, segment_pos, cache, return_cache)
     with torch.no_grad():
@@ -158,7 +162,11 @@ class RecurrentBlock(nn.Module):
           self.conv_1d, self.rg_lru, x, segment_pos, cache, return_cache,
           in_place=self.decode_in_place and cache is not None and return_cache)
       x = ops.gelu_mul(x, y)  # x * gelu(y), one pass (modules.py:627-628, 644)
-      if few_rows:
+      if few_rows and defer_out and ops.PackedLinear.partial_slices(
+          x, self.lru_width, self.width):
+        x = self._rows_out.partial(x, (self.linear_out.weight,),
+                                   (self.linear_out.bias,))
+      elif few_rows:
         x = self._rows_out(x, (self.linear_out.weight,),
                            (self.linear_out.bias,))
       else:

@@ -290,7 +290,10 @@ def rms_norm(x, scale, eps=1e-6):
 
 
 def add_rms_norm(x, addend, scale, eps=1e-6):
-  """(x + addend, rms_norm(x + addend)) in one pass."""
+  """(x + addend, rms_norm(x + addend)) in one pass.  x may be a PartialSums
+  (then addend may be None: the sum is the layer output itself)."""
+  if isinstance(x, PartialSums):
+    return _add_rms_norm_partial(x, addend, scale, eps)
   assert x.shape == addend.shape
   x = _dev(x, "x")
   _same(x.dtype, x.device, addend=addend, scale=scale)
@@ -302,6 +305,27 @@ def add_rms_norm(x, addend, scale, eps=1e-6):
     _lib.check(_lib.lib().rg_add_rms_norm(
         _p(x), _p(addend), _p(scale), _p(total), _p(out), x.numel() // width,
         width, eps, _dtype_code(x), _stream(x)))
+  return total, out
+
+
+def _add_rms_norm_partial(ps, addend, scale, eps):
+  if ps.addend is not None:
+    if addend is not None:
+      raise ValueError("the partial sums already carry an addend")
+    addend = ps.addend
+  slices, rows, width = ps.sums.shape
+  scale = _dev(scale, "scale")
+  assert scale.shape == (width,) and scale.dtype == ps.dtype
+  if addend is not None:
+    assert tuple(addend.shape) == tuple(ps.shape)
+    _same(ps.dtype, ps.sums.device, addend=addend)
+    addend = _dev(addend, "addend")
+  total = torch.empty(ps.shape, dtype=ps.dtype, device=ps.sums.device)
+  out = torch.empty_like(total)
+  with torch.cuda.device(total.device):
+    _lib.check(_lib.lib().rg_add_rms_norm_partial(
+        _p(ps.sums), slices, _p(ps.bias), _p(addend), _p(scale), _p(total),
+        _p(out), rows, width, eps, _DTYPES[ps.dtype], _stream(total)))
   return total, out
 
 
@@ -399,6 +423,25 @@ def packed_gate_weights(w_x, w_a):
   return packed
 
 
+class PartialSums:
+  """The output of a linear layer that has not been added up yet: fp32 partial
+  sums over slices of K (PackedLinear.partial), its bias, and optionally a
+  tensor still to be added (a skip connection).  `add_rms_norm` takes it in
+  place of a tensor; `materialize()` gives the tensor it stands for."""
+
+  def __init__(self, sums, bias, shape, dtype, addend=None):
+    self.sums, self.bias = sums, bias    # [slices, M, N] float32, [N] | None
+    self.shape, self.dtype = shape, dtype  # of the tensor this stands for
+    self.addend = addend
+
+  def materialize(self):
+    N = self.shape[-1]
+    out = (self.sums.sum(0) if self.bias is None
+           else self.sums.sum(0) + self.bias.float())
+    out = out.to(self.dtype).reshape(self.shape)
+    return out if self.addend is None else out + self.addend
+
+
 class PackedLinear:
   """Linear layers that read the same few rows (a decode step), on the
   weight-streaming kernel (rg_linear_rows).  Holds the weights in the kernel's
@@ -476,6 +519,34 @@ class PackedLinear:
     self._packed, self._bias = packed, bias
     self._shape = (N, K, groups)
     self._stamp = stamp
+
+  @staticmethod
+  def partial_slices(x, K, N) -> int:
+    """In how many slices of K `partial` would run this shape; 0 = not worth
+    it (enough weight rows to fill the GPU without splitting K, or a width the
+    norm kernel that adds the slices does not take)."""
+    if not PackedLinear.usable(x, K, N) or N % 8 or N > 4096:
+      return 0
+    tiles = N // 32
+    return 3 if tiles <= 85 else 2 if tiles <= 128 else 0
+
+  @torch.no_grad()
+  def partial(self, x, weights, biases=None, addend=None) -> PartialSums:
+    """One layer, left as partial sums for the norm that follows it
+    (add_rms_norm): K is split over the grid, so three times as many
+    workgroups stream the weights, and no separate pass adds the slices."""
+    x = _dev(x, "x")
+    self._prepare(weights, biases)
+    N, K, groups = self._shape
+    assert groups == 1 and not self.gelu_pair
+    slices = self.partial_slices(x, K, N)
+    assert slices > 0
+    M = x.numel() // K
+    sums = torch.empty((slices, M, N), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+      _lib.check(_lib.lib().rg_linear_rows_partial(
+          _p(x), _p(self._packed), _p(sums), M, K, N, slices, _stream(x)))
+    return PartialSums(sums, self._bias, (*x.shape[:-1], N), x.dtype, addend)
 
   @torch.no_grad()
   def __call__(self, x, weights, biases=None, residual=None):

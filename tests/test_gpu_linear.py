@@ -108,6 +108,41 @@ def test_stacked_weight_and_gelu_pairs(M, K, E):
     assert torch.equal(fused, ops.gelu_mul(up.contiguous(), gate.contiguous()))
 
 
+@pytest.mark.parametrize("M,K,N,with_addend", [
+    (64, 2560, 2560, True), (64, 7680, 2560, True), (7, 256, 256, False)])
+def test_partial_sums_into_the_norm(M, K, N, with_addend):
+  """A layer left as partial sums over slices of K and the norm kernel that
+  adds them: the values of adding the slices in order, bias, rounding, the
+  addend, rounding and rg_rms_norm as separate steps."""
+  gen = torch.Generator().manual_seed(K + N + M)
+  x = _rand(gen, M, K)
+  w = _rand(gen, N, K, scale=K ** -0.5)
+  b = _rand(gen, N)
+  scale = _rand(gen, N, scale=0.3).to(DEV)
+  addend = _rand(gen, 1, M, N).to(DEV) if with_addend else None
+  layer = ops.PackedLinear()
+  xg = x.to(DEV).reshape(1, M, K)
+  assert ops.PackedLinear.partial_slices(xg, K, N) == 3
+  ps = layer.partial(xg, (w.to(DEV),), (b.to(DEV),))
+  assert ps.sums.shape == (3, M, N) and ps.shape == (1, M, N)
+  plain = ps.materialize()
+  _check(plain[0], x, w, b)
+  want_total = plain if addend is None else plain + addend
+  total, normed = ops.add_rms_norm(ps, addend, scale)
+  assert torch.equal(total, want_total)
+  assert torch.equal(normed, ops.rms_norm(want_total, scale))
+  # the addend may also ride in the partial sums (a skip connection)
+  if addend is not None:
+    ps.addend = addend
+    assert torch.equal(ps.materialize(), want_total)
+    total2, normed2 = ops.add_rms_norm(ps, None, scale)
+    assert torch.equal(total2, total) and torch.equal(normed2, normed)
+    with pytest.raises(ValueError):
+      ops.add_rms_norm(ps, addend, scale)
+  # many weight rows: splitting K is not worth it
+  assert ops.PackedLinear.partial_slices(xg, K, 15360) == 0
+
+
 def test_repacks_when_a_weight_changes():
   gen = torch.Generator().manual_seed(3)
   x = _rand(gen, 8, 128).to(DEV)
@@ -166,10 +201,21 @@ def test_decode_steps_with_and_without_the_row_kernels(monkeypatch):
     calls.append(1)
     return real(self, *a, **k)
 
+  partials = []
+  real_partial = ops.PackedLinear.partial
+
+  def counting_partial(self, *a, **k):
+    partials.append(1)
+    calls.append(1)
+    return real_partial(self, *a, **k)
+
   monkeypatch.setattr(ops.PackedLinear, "__call__", counting)
+  monkeypatch.setattr(ops.PackedLinear, "partial", counting_partial)
   with_rows = run()
   # per step: recurrent 2 x (2 + 2 MLP) + attention (3 + 2 MLP)
   assert len(calls) == 3 * 13, len(calls)
+  # 6 of the 13 feed a norm next and are left as partial sums for it
+  assert len(partials) == 3 * 6, len(partials)
   monkeypatch.setattr(ops.PackedLinear, "usable",
                       staticmethod(lambda *a, **k: False))
   library = run()

@@ -24,7 +24,7 @@ def _declared_symbols():
 
 def test_library_exports_every_declared_symbol():
   names = _declared_symbols()
-  assert len(names) == 24, names
+  assert len(names) == 26, names
   lib = ctypes.CDLL(_lib.LIB_PATH)
   for n in names:
     assert hasattr(lib, n), n
@@ -95,6 +95,19 @@ def test_c_side_validation_without_launch():
   rc = lib.rg_linear_rows(ok, ok, None, None, y, None, 0, 64, 7680, 2560, 1, 0,
                           None)
   assert rc == -4 and b"workspace" in lib.rg_last_error()
+  rc = lib.rg_linear_rows_partial(ok, ok, y, 64, 2560, 2560, 9, None)
+  assert rc == -1 and b"slices" in lib.rg_last_error()
+  rc = lib.rg_linear_rows_partial(ok, ok, y, 64, 2560, 2570, 3, None)
+  assert rc == -2
+  rc = lib.rg_add_rms_norm_partial(ok, 3, None, None, ok, y, y, 4, 64, 1e-6, 1,
+                                   None)
+  assert rc == -1 and b"alias" in lib.rg_last_error()
+  rc = lib.rg_add_rms_norm_partial(ok, 3, None, None, ok, ok, y, 4, 64, 1e-6, 0,
+                                   None)
+  assert rc == -2 and b"bf16" in lib.rg_last_error()
+  rc = lib.rg_add_rms_norm_partial(ok, 3, None, None, ok, ok, y, 4, 60, 1e-6, 1,
+                                   None)
+  assert rc == -2
   args = [ok, ok, 1, ok, ok, ok, ok, ok, ok, None, ok, None, y, None, None]
   rc = lib.rg_recurrent_prefill(*args, 1, 8, 256, 1, 0, None)
   assert rc == -2 and b"unsupported" in lib.rg_last_error().lower()  # fp32
