@@ -259,6 +259,18 @@ int rg_recurrent_step_packed(const void* x, const void* segpos,
                              const void* a_param, void* y, int B, int W, int H,
                              int dtype, void* stream);
 
+/* The two steps between the last linear layer and the next token id:
+ * rg_soft_cap: out = tanh(x / cap) * cap over n elements (griffin.py:203-206),
+ *   one pass with the roundings of torch's three (quotient as x * (1 / cap),
+ *   tanh, product); out may alias x.
+ * rg_argmax_rows: out[r] = index of the largest of x[r, 0..n), the first among
+ *   equals, NaN above everything (torch.argmax, greedy sampling,
+ *   sampler.py:126-128); x [rows, n] contiguous, out int64. */
+int rg_soft_cap(const void* x, void* out, int64_t n, float cap, int dtype,
+                void* stream);
+int rg_argmax_rows(const void* x, int64_t* out, int rows, int n, int dtype,
+                   void* stream);
+
 /* The linear layers around the recurrent and attention blocks for a decode
  * step (at most 64 rows), bf16: torch.nn.Linear (modules.py:579-601 linear_y /
  * linear_x / linear_out, :717-721 ffw_down, :334-352 the attention projections)

@@ -368,6 +368,30 @@ int rg_gelu_mul(const void* a, const void* g, void* out, int64_t n, int dtype,
       __func__, rg::launch_gelu_mul(a, g, out, n, dtype, (hipStream_t)stream));
 }
 
+int rg_soft_cap(const void* x, void* out, int64_t n, float cap, int dtype,
+                void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(n > 0, "%s: n=%lld must be positive", __func__, (long long)n);
+  RG_REQUIRE(cap > 0.0f, "%s: cap=%g must be positive", __func__, (double)cap);
+  RG_CHECK_PTR(x);
+  RG_CHECK_PTR(out);
+  return launch_status(
+      __func__, rg::launch_soft_cap(x, out, n, cap, dtype, (hipStream_t)stream));
+}
+
+int rg_argmax_rows(const void* x, int64_t* out, int rows, int n, int dtype,
+                   void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(rows > 0 && n > 0, "%s: rows=%d n=%d must be positive", __func__,
+             rows, n);
+  RG_CHECK_PTR(x);
+  RG_REQUIRE(out != nullptr && ((uintptr_t)out & 7) == 0,
+             "%s: out is null or not 8-byte aligned", __func__);
+  return launch_status(__func__,
+                       rg::launch_argmax_rows(x, out, rows, n, dtype,
+                                              (hipStream_t)stream));
+}
+
 int rg_rms_norm(const void* x, const void* scale, void* out, int64_t rows,
                 int width, float eps, int dtype, void* stream) {
   RG_CHECK_DTYPE(dtype);

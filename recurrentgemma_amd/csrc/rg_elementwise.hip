@@ -207,7 +207,127 @@ rms_norm_bf16_rows_kernel(const u32x4* __restrict__ x, PartialRows part,
   }
 }
 
+// Soft cap of the logits (recurrentgemma/torch/griffin.py:203-206
+// `logits = tanh(logits / cap) * cap`): torch's three kernels in one, with
+// their roundings (the quotient -- torch multiplies by the reciprocal of a
+// scalar divisor --, the tanh and the product each rounded to the dtype).
+template <typename T>
+__global__ void __launch_bounds__(256)
+soft_cap_kernel(const T* __restrict__ x, T* __restrict__ out, int64_t n,
+                float inv_cap, float cap) {
+  constexpr int kPer = 16 / sizeof(T);
+  const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * kPer;
+  auto one = [&](float v) {
+    v = round_act<T>(v * inv_cap);
+    v = round_act<T>(tanhf(v));
+    return round_act<T>(v * cap);
+  };
+  if (i0 + kPer <= n) {
+    alignas(16) T in[kPer];
+    alignas(16) T o[kPer];
+    *reinterpret_cast<u32x4*>(in) =
+        __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x + i0));
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) store_scalar<T>(o + k, one(load_scalar<T>(in + k)));
+    __builtin_nontemporal_store(*reinterpret_cast<u32x4*>(o),
+                                reinterpret_cast<u32x4*>(out + i0));
+  } else {
+    for (int64_t i = i0; i < n; ++i)
+      store_scalar<T>(out + i, one(load_scalar<T>(x + i)));
+  }
+}
+
+// Index of the largest element of every row (the first one among equals, a NaN
+// counts as larger than everything: torch.argmax's rule; greedy sampling,
+// recurrentgemma/torch/sampler.py:126-128).  One workgroup per row.
+template <typename T>
+__global__ void __launch_bounds__(1024)
+argmax_rows_kernel(const T* __restrict__ x, int64_t* __restrict__ out, int n) {
+  __shared__ float best_v[16];
+  __shared__ int best_i[16];
+  const T* row = x + (int64_t)blockIdx.x * n;
+  float bv = 0.0f;
+  int bi = 0x7fffffff;
+  // a beats b: larger, or NaN where b is not; equal values keep the lower index
+  auto better = [](float v, int i, float w, int j) {
+    if (j == 0x7fffffff) return true;
+    const bool vn = v != v, wn = w != w;
+    if (vn || wn) return vn && (!wn || i < j);
+    return v > w || (v == w && i < j);
+  };
+  constexpr int kPer = 16 / sizeof(T);
+  const int vec_n = ((reinterpret_cast<uintptr_t>(row) & 15) == 0) ? n / kPer : 0;
+  for (int c = threadIdx.x; c < vec_n; c += 1024) {
+    alignas(16) T in[kPer];
+    *reinterpret_cast<u32x4*>(in) =
+        __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(row) + c);
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+      const float v = load_scalar<T>(in + k);
+      if (better(v, c * kPer + k, bv, bi)) {
+        bv = v;
+        bi = c * kPer + k;
+      }
+    }
+  }
+  for (int i = vec_n * kPer + threadIdx.x; i < n; i += 1024) {
+    const float v = load_scalar<T>(row + i);
+    if (better(v, i, bv, bi)) {
+      bv = v;
+      bi = i;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, 64);
+    const int oi = __shfl_xor(bi, off, 64);
+    if (oi != 0x7fffffff && better(ov, oi, bv, bi)) {
+      bv = ov;
+      bi = oi;
+    }
+  }
+  if ((threadIdx.x & 63) == 0) {
+    best_v[threadIdx.x >> 6] = bv;
+    best_i[threadIdx.x >> 6] = bi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 16; ++w)
+      if (best_i[w] != 0x7fffffff && better(best_v[w], best_i[w], bv, bi)) {
+        bv = best_v[w];
+        bi = best_i[w];
+      }
+    out[blockIdx.x] = bi;
+  }
+}
+
 }  // namespace
+
+hipError_t launch_soft_cap(const void* x, void* out, int64_t n, float cap,
+                           int dtype, hipStream_t s) {
+  const int per = dtype == 0 ? 4 : 8;
+  const int64_t blocks = ((n + per - 1) / per + 255) / 256;
+  if (blocks > 0x7fffffff) return hipErrorInvalidValue;
+  const float inv = 1.0f / cap;
+  if (dtype == 0)
+    soft_cap_kernel<float><<<dim3((unsigned)blocks), 256, 0, s>>>(
+        (const float*)x, (float*)out, n, inv, cap);
+  else
+    soft_cap_kernel<uint16_t><<<dim3((unsigned)blocks), 256, 0, s>>>(
+        (const uint16_t*)x, (uint16_t*)out, n, inv, cap);
+  return hipGetLastError();
+}
+
+hipError_t launch_argmax_rows(const void* x, int64_t* out, int rows, int n,
+                              int dtype, hipStream_t s) {
+  if (dtype == 0)
+    argmax_rows_kernel<float><<<dim3((unsigned)rows), 1024, 0, s>>>(
+        (const float*)x, out, n);
+  else
+    argmax_rows_kernel<uint16_t><<<dim3((unsigned)rows), 1024, 0, s>>>(
+        (const uint16_t*)x, out, n);
+  return hipGetLastError();
+}
 
 hipError_t launch_gelu_mul(const void* a, const void* g, void* out, int64_t n,
                            int dtype, hipStream_t s) {

@@ -121,6 +121,11 @@ hipError_t launch_block_step_bf16(const StepArgs& a, hipStream_t s);
 // out[i] = a[i] * gelu_tanh(g[i]) over n elements (out may alias a or g).
 hipError_t launch_gelu_mul(const void* a, const void* g, void* out, int64_t n,
                            int dtype, hipStream_t s);
+// out = tanh(x / cap) * cap, n elements; out[r] = argmax(x[r, :n])
+hipError_t launch_soft_cap(const void* x, void* out, int64_t n, float cap,
+                           int dtype, hipStream_t s);
+hipError_t launch_argmax_rows(const void* x, int64_t* out, int rows, int n,
+                              int dtype, hipStream_t s);
 // out[r, :] = v * rsqrt(mean(v^2) + eps) * (scale + 1) with v = x[r, :], or,
 // with an addend, v = x[r, :] + addend[r, :] (also written to sum_out)
 hipError_t launch_rms_norm(const void* x, const void* addend, const void* scale,

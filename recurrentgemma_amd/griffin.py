@@ -554,7 +554,7 @@ class Griffin(nn.Module):
     logits = self.embedder.decode(x)
     cap = self.config.logits_soft_cap
     if cap:
-      logits = torch.tanh(logits / cap) * cap
+      logits = ops.soft_cap(logits, cap)
     return logits, (new_cache if return_cache else None)
 
   def init_cache(self, batch_size, dtype, device=None) -> Cache:

@@ -308,6 +308,27 @@ def add_rms_norm(x, addend, scale, eps=1e-6):
   return total, out
 
 
+def soft_cap(x, cap):
+  """tanh(x / cap) * cap, one pass."""
+  x = _dev(x, "x")
+  out = torch.empty_like(x)
+  with torch.cuda.device(x.device):
+    _lib.check(_lib.lib().rg_soft_cap(_p(x), _p(out), x.numel(), float(cap),
+                                      _dtype_code(x), _stream(x)))
+  return out
+
+
+def argmax_last(x):
+  """torch.argmax(x, dim=-1) (first index among equals), one pass."""
+  x = _dev(x, "x")
+  n = x.shape[-1]
+  out = torch.empty(x.shape[:-1], dtype=torch.int64, device=x.device)
+  with torch.cuda.device(x.device):
+    _lib.check(_lib.lib().rg_argmax_rows(_p(x), _p(out), x.numel() // n, n,
+                                         _dtype_code(x), _stream(x)))
+  return out
+
+
 def _add_rms_norm_partial(ps, addend, scale, eps):
   if ps.addend is not None:
     if addend is not None:

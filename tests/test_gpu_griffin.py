@@ -262,3 +262,45 @@ def test_attention_decode_kernels(dtype, B, heads, hd, window):
 def helpers_max_rel(got, want):
   got, want = got.float(), want.float()
   return ((got - want).abs().max() / want.abs().max().clamp_min(1e-30)).item()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_soft_cap_kernel(dtype):
+  """rg_soft_cap against torch's own three kernels on the GPU (quotient by a
+  scalar, tanh, product): same roundings; one unit in the last place is left
+  for the tanh of two builds of the device math library."""
+  from recurrentgemma_amd import ops
+  gen = torch.Generator().manual_seed(77)
+  x = (torch.randn(3, 5, 1003, generator=gen) * 40).to(dtype).to(DEV)
+  got = ops.soft_cap(x, 30.0)
+  want = torch.tanh(x / 30.0) * 30.0
+  assert got.dtype == dtype and got.shape == x.shape
+  ulp = torch.finfo(dtype).eps * want.float().abs().clamp_min(1e-30)
+  assert ((got.float() - want.float()).abs() <= ulp).all()
+  assert (got.float().abs() <= 30.0).all()
+  mism = (got != want).float().mean().item()
+  assert mism < 0.02, mism
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_argmax_kernel(dtype):
+  """rg_argmax_rows against torch.argmax: bf16 rows of a vocabulary's length
+  are full of equal maxima (first index wins), plus rows with a NaN, a row
+  whose maximum is its last element, negative rows."""
+  from recurrentgemma_amd import ops
+  gen = torch.Generator().manual_seed(78)
+  x = torch.randn(9, 25601, generator=gen).to(dtype)
+  x[1] = -x[1].abs() - 1.0
+  x[2, -1] = 100.0
+  x[3, 17] = float("nan")
+  x[4, 5] = x[4, 20000] = 50.0
+  x[5] = 0.0
+  x = x.to(DEV)
+  got = ops.argmax_last(x)
+  assert got.dtype == torch.int64
+  assert torch.equal(got, torch.argmax(x, dim=-1))
+  assert got[2].item() == 25600 and got[3].item() == 17 and got[4].item() == 5
+  x3 = x[:8].reshape(2, 4, -1)
+  assert torch.equal(ops.argmax_last(x3), torch.argmax(x3, dim=-1))
+  odd = x[:, 1:100]  # rows that are neither contiguous nor 16-byte aligned
+  assert torch.equal(ops.argmax_last(odd), torch.argmax(odd, dim=-1))
