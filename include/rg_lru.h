@@ -207,6 +207,13 @@ int rg_add_rms_norm(const void* x, const void* addend, const void* scale,
 int rg_rope(const void* x, const void* positions, int positions_is_i64,
             const float* inv_freq, void* out, int64_t rows, int heads,
             int head_dim, int dtype, void* stream);
+/* The same for queries and keys in one launch (modules.py:431-432 applies it
+ * to both with the same positions): q [rows, q_heads, head_dim],
+ * k [rows, k_heads, head_dim]. */
+int rg_rope_pair(const void* q, const void* k, const void* positions,
+                 int positions_is_i64, const float* inv_freq, void* q_out,
+                 void* k_out, int64_t rows, int q_heads, int k_heads,
+                 int head_dim, int dtype, void* stream);
 
 /* Masked softmax of one decoded token against the ring cache and itself
  * (modules.py:152-183 `_compute_cache_mask`, :462-470): scores

@@ -49,6 +49,8 @@ SIGNATURES = {
     "rg_linear_rows_workspace_bytes": (ctypes.c_size_t, [_i, _i, _i]),
     "rg_linear_rows": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_size_t, _i,
                             _i, _i, _i, _i, _vp]),
+    "rg_rope_pair": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, ctypes.c_int64, _i,
+                          _i, _i, _i, _vp]),
     "rg_soft_cap": (_i, [_vp, _vp, ctypes.c_int64, ctypes.c_float, _i, _vp]),
     "rg_argmax_rows": (_i, [_vp, _vp, _i, _i, _i, _vp]),
     "rg_linear_rows_partial": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),

@@ -438,8 +438,32 @@ int rg_rope(const void* x, const void* positions, int positions_is_i64,
   RG_REQUIRE(out != x, "%s: out must not alias x", __func__);
   return launch_status(
       __func__, rg::launch_rope(x, positions, positions_is_i64 ? 1 : 0,
-                                inv_freq, out, rows, heads, head_dim, dtype,
-                                (hipStream_t)stream));
+                                inv_freq, out, rows, heads, head_dim, nullptr,
+                                nullptr, 0, dtype, (hipStream_t)stream));
+}
+
+int rg_rope_pair(const void* q, const void* k, const void* positions,
+                 int positions_is_i64, const float* inv_freq, void* q_out,
+                 void* k_out, int64_t rows, int q_heads, int k_heads,
+                 int head_dim, int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(rows > 0 && q_heads > 0 && k_heads > 0 && head_dim > 0,
+             "%s: rows=%lld q_heads=%d k_heads=%d head_dim=%d must be positive",
+             __func__, (long long)rows, q_heads, k_heads, head_dim);
+  RG_REQUIRE(head_dim % 4 == 0, "%s: head_dim=%d is not a multiple of 4",
+             __func__, head_dim);
+  RG_CHECK_PTR(q);
+  RG_CHECK_PTR(k);
+  RG_CHECK_PTR(positions);
+  RG_CHECK_PTR(inv_freq);
+  RG_CHECK_PTR(q_out);
+  RG_CHECK_PTR(k_out);
+  RG_REQUIRE(q_out != q && k_out != k, "%s: outputs must not alias inputs",
+             __func__);
+  return launch_status(
+      __func__, rg::launch_rope(q, positions, positions_is_i64 ? 1 : 0,
+                                inv_freq, q_out, rows, q_heads, head_dim, k,
+                                k_out, k_heads, dtype, (hipStream_t)stream));
 }
 
 int rg_attention_decode_probs(const void* scores, const void* q,

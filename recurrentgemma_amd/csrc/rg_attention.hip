@@ -20,16 +20,26 @@ __device__ __forceinline__ float position_as_float(const void* pos, int kind,
 // x, out [rows, n, hd]; positions [rows]; inv_freq [hd / 4] float32.
 // First half of the head dimension: element i pairs with element i + hd/4,
 // rotated by position * inv_freq[i]; second half copied.
+// A second tensor (x2, out2 [rows, n2, hd], same positions: the keys beside
+// the queries) takes the elements from `total` up to `total + total2`.
 template <typename T>
 __global__ void __launch_bounds__(256)
 rope_kernel(const T* __restrict__ x, const void* __restrict__ pos,
             int pos_kind, const float* __restrict__ inv_freq,
-            T* __restrict__ out, int64_t total, int n, int hd) {
+            T* __restrict__ out, int64_t total, int n, int hd,
+            const T* __restrict__ x2, T* __restrict__ out2, int64_t total2,
+            int n2) {
   // products and their sum are separate tensors in the reference: no fused
   // multiply-add (matters in float32, where nothing is rounded in between)
 #pragma clang fp contract(off)
-  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (e >= total) return;
+  int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) {
+    e -= total;
+    if (e >= total2) return;
+    x = x2;
+    out = out2;
+    n = n2;
+  }
   const int d = (int)(e % hd);
   const int half = hd / 2, quarter = hd / 4;
   if (d >= half) {
@@ -157,14 +167,17 @@ hipError_t by_dtype(int dtype, F&& f) {
 
 hipError_t launch_rope(const void* x, const void* pos, int pos_kind,
                        const float* inv_freq, void* out, int64_t rows, int n,
-                       int hd, int dtype, hipStream_t s) {
+                       int hd, const void* x2, void* out2, int n2, int dtype,
+                       hipStream_t s) {
   const int64_t total = rows * n * hd;
-  const int64_t blocks = (total + 255) / 256;
+  const int64_t total2 = x2 ? rows * n2 * hd : 0;
+  const int64_t blocks = (total + total2 + 255) / 256;
   if (blocks > 0x7fffffff) return hipErrorInvalidValue;
   return by_dtype(dtype, [&](auto* tag) {
     typedef std::remove_pointer_t<decltype(tag)> T;
     rope_kernel<T><<<dim3((unsigned)blocks), 256, 0, s>>>(
-        (const T*)x, pos, pos_kind, inv_freq, (T*)out, total, n, hd);
+        (const T*)x, pos, pos_kind, inv_freq, (T*)out, total, n, hd,
+        (const T*)x2, (T*)out2, total2, n2);
   });
 }
 

@@ -135,7 +135,8 @@ hipError_t launch_rms_norm(const void* x, const void* addend, const void* scale,
 // (rg_attention.hip).
 hipError_t launch_rope(const void* x, const void* pos, int pos_kind,
                        const float* inv_freq, void* out, int64_t rows, int n,
-                       int hd, int dtype, hipStream_t s);
+                       int hd, const void* x2, void* out2, int n2, int dtype,
+                       hipStream_t s);
 hipError_t launch_attn_decode_probs(const void* scores, const void* q,
                                     const void* k_new,
                                     const int32_t* num_tokens, void* probs,

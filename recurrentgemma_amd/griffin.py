@@ -249,13 +249,6 @@ class LocalAttentionBlock(nn.Module):
     self._inv_freq = None
     self.reset_parameters()
 
-  def _rope(self, x, positions):
-    """Rotary embedding on the first half of the head dimension
-    (modules.py:52-83), one kernel."""
-    if self._inv_freq is None or self._inv_freq.device != x.device:
-      self._inv_freq = _inv_frequencies(self.head_dim, x.device)
-    return ops.rope(x, positions, self._inv_freq)
-
   @property
   def head_dim(self) -> int:
     return self.width // self.num_heads
@@ -307,7 +300,10 @@ class LocalAttentionBlock(nn.Module):
     q = q.reshape(b, t, self.num_heads, self.head_dim)
     k = k.reshape(b, t, 1, self.head_dim)
     v = v.reshape(b, t, 1, self.head_dim)
-    q, k = self._rope(q, segment_pos), self._rope(k, segment_pos)
+    if self._inv_freq is None or self._inv_freq.device != x.device:
+      self._inv_freq = _inv_frequencies(self.head_dim, x.device)
+    # rotary embedding of queries and keys (modules.py:431-432), one kernel
+    q, k = ops.rope_pair(q, k, segment_pos, self._inv_freq)
 
     if cache is not None and t == 1:
       return self._decode_step(x, q, k, v, cache, return_cache, defer_out)

@@ -365,6 +365,24 @@ def rope(x, positions, inv_freq):
   return out
 
 
+def rope_pair(q, k, positions, inv_freq):
+  """rope(q), rope(k) in one launch: q [B, T, heads, hd], k [B, T, kv_heads,
+  hd], same positions."""
+  B, T, n, hd = q.shape
+  assert k.shape[:2] == (B, T) and k.shape[3] == hd
+  q, k = _dev(q, "q"), _dev(k, "k")
+  _same(q.dtype, q.device, k=k)
+  pos, is64 = _segpos(positions, B, T)
+  inv = _dev(inv_freq, "inv_freq")
+  assert inv.dtype == torch.float32 and inv.shape == (hd // 4,)
+  q_out, k_out = torch.empty_like(q), torch.empty_like(k)
+  with torch.cuda.device(q.device):
+    _lib.check(_lib.lib().rg_rope_pair(
+        _p(q), _p(k), _p(pos), is64, _p(inv), _p(q_out), _p(k_out), B * T, n,
+        k.shape[2], hd, _dtype_code(q), _stream(q)))
+  return q_out, k_out
+
+
 def attention_decode_probs(scores, q, k_new, num_tokens, scale):
   """softmax over the written ring slots and the new token: scores
   [B, heads, window] (unscaled), q [B, heads, hd], k_new [B, hd], num_tokens

@@ -201,6 +201,10 @@ def test_rope_kernel(dtype, hd):
   for p in (pos, pos.to(torch.int32)):
     got = ops.rope(x, p, inv)
     assert torch.equal(got, want), (got - want).abs().max()
+  # queries and keys in one launch: each as on its own
+  k = torch.randn(3, 7, 1, hd, generator=gen).to(dtype).to(DEV)
+  q2, k2 = ops.rope_pair(x, k, pos, inv)
+  assert torch.equal(q2, want) and torch.equal(k2, ops.rope(k, pos, inv))
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
