@@ -17,6 +17,7 @@ from __future__ import annotations
 import enum
 import itertools
 import math
+import weakref
 from typing import Any, NamedTuple
 
 import torch
@@ -226,6 +227,23 @@ def _visible(q_pos, k_pos, window, q_doc=None, k_doc=None):
   return mask & (k >= 0)
 
 
+_one_document = [None, None, False]  # tensor (weak), its version, answer
+
+
+def _rows_are_one_document(segment_pos) -> bool:
+  """True if no row starts a document after its first token: every row is then
+  one document (or the tail of one) and its mask is the plain causal one.
+  Asking costs a host synchronisation, so the answer is kept for the tensor
+  object it was given for (the blocks of a model all ask about the same one)."""
+  ref, version, answer = _one_document
+  if (ref is not None and ref() is segment_pos and
+      version == segment_pos._version):
+    return answer
+  answer = bool((segment_pos[:, 1:] != 0).all())
+  _one_document[:] = [weakref.ref(segment_pos), segment_pos._version, answer]
+  return answer
+
+
 class LocalAttentionBlock(nn.Module):
   """Sliding-window multi-query attention with a ring KV cache
   (modules.py:294-493)."""
@@ -322,13 +340,26 @@ class LocalAttentionBlock(nn.Module):
           raise NotImplementedError(
               "a cached call takes one token or at least a window of them")
     else:
-      doc = torch.cumsum(segment_pos == 0, dim=-1)
-      pos = torch.arange(t, device=x.device)[None].expand(b, t)
-      mask = _visible(pos, pos, self.window_size, doc, doc)
       k_all, v_all = k, v
       if return_cache:
         new_cache = self._cache_from_prompt(k, v, segment_pos,
                                             self.window_size)
+      if (x.is_cuda and 1 < t <= self.window_size + 1 and
+          _rows_are_one_document(segment_pos)):
+        # one document per row, all of it inside the window: the mask of
+        # modules.py:86-127 is the causal one, which the library's attention
+        # kernel applies by itself (4 ms instead of 17 ms per block at
+        # 64 x 2047 tokens, where the mask is 268 MB to build and to read)
+        out = nn.functional.scaled_dot_product_attention(
+            q.transpose(1, 2),
+            k.transpose(1, 2).expand(-1, self.num_heads, -1, -1),
+            v.transpose(1, 2).expand(-1, self.num_heads, -1, -1),
+            is_causal=True)
+        out = out.transpose(1, 2).reshape(b, t, self.width)
+        return self._project_out(out, defer_out), new_cache
+      doc = torch.cumsum(segment_pos == 0, dim=-1)
+      pos = torch.arange(t, device=x.device)[None].expand(b, t)
+      mask = _visible(pos, pos, self.window_size, doc, doc)
 
     # [B, heads, T, head_dim] against one shared key/value head
     out = nn.functional.scaled_dot_product_attention(

@@ -308,3 +308,55 @@ def test_argmax_kernel(dtype):
   assert torch.equal(ops.argmax_last(x3), torch.argmax(x3, dim=-1))
   odd = x[:, 1:100]  # rows that are neither contiguous nor 16-byte aligned
   assert torch.equal(ops.argmax_last(odd), torch.argmax(odd, dim=-1))
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-4),
+                                       (torch.bfloat16, 3e-2)])
+def test_prompt_attention_causal_shortcut(monkeypatch, dtype, tol):
+  """Rows that are one document inside the window take the library's causal
+  attention instead of the explicit mask: same logits and cache (to the
+  tolerance of the dtype); a row with a second document start, or a prompt
+  longer than the window, keeps the mask."""
+  R, A = G.TemporalBlockType.RECURRENT, G.TemporalBlockType.ATTENTION
+  cfg = G.GriffinConfig(
+      vocab_size=64, width=64, mlp_expanded_width=96, num_heads=2,
+      block_types=(A, R, A), embeddings_scale_by_sqrt_dim=True,
+      attention_window_size=16, logits_soft_cap=30.0, lru_width=64)
+  torch.manual_seed(9)
+  m = G.Griffin(cfg, dtype=dtype).to(DEV).eval()
+  gen = torch.Generator().manual_seed(10)
+  B, T = 3, 12
+  tokens = torch.randint(0, 64, (B, T), generator=gen).to(DEV)
+  asked = []
+  real = G._rows_are_one_document
+
+  def spy(segment_pos):
+    asked.append(real(segment_pos))
+    return asked[-1]
+
+  def forced_off(segment_pos):
+    return False
+
+  def run(pos, fn):
+    monkeypatch.setattr(G, "_rows_are_one_document", fn)
+    return m(tokens[:, :pos.shape[1]], pos, None, return_logits=True,
+             return_cache=True)
+
+  one_doc = torch.arange(T, device=DEV)[None].expand(B, -1).contiguous()
+  one_doc[1] += 5  # a row that continues a document
+  logits, cache = run(one_doc, spy)
+  assert asked == [True, True]
+  want, want_cache = run(one_doc, forced_off)
+  scale = want.float().abs().max().item()
+  assert (logits.float() - want.float()).abs().max().item() <= tol * scale
+  for name in cache:
+    for got_t, want_t in zip(cache[name], want_cache[name]):
+      s = max(want_t.float().abs().max().item(), 1e-6)
+      assert (got_t.float() - want_t.float()).abs().max().item() <= tol * s
+  # a second document start in one row: the mask path, bit for bit
+  two_docs = one_doc.clone()
+  two_docs[2, 7:] = torch.arange(T - 7, device=DEV)
+  asked.clear()
+  got2, _ = run(two_docs, spy)
+  assert asked == [False, False]
+  assert torch.equal(got2, run(two_docs, forced_off)[0])
