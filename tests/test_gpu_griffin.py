@@ -181,7 +181,7 @@ def test_captured_decode_step_equals_eager(model, which):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("hd", [16, 256])
+@pytest.mark.parametrize("hd", [16, 64, 256])
 def test_rope_kernel(dtype, hd):
   """rg_rope against the reference's tensor expression (modules.py:52-83)
   evaluated by torch on the GPU in the same dtype: bit-identical (the same
