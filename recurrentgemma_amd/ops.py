@@ -474,7 +474,6 @@ class PartialSums:
     self.addend = addend
 
   def materialize(self):
-    N = self.shape[-1]
     out = (self.sums.sum(0) if self.bias is None
            else self.sums.sum(0) + self.bias.float())
     out = out.to(self.dtype).reshape(self.shape)
