@@ -125,6 +125,34 @@ int rg_linear_scan(const void* x, const void* a, const void* reset,
                    const void* h0, void* y, void* h_last, int B, int T, int W,
                    int dtype, void* stream);
 
+/* The two scans above for few rows and channels: one workgroup per (row, slab
+ * of 256 or 128 channels) leaves most of the GPU idle when B * W / 256 is
+ * small (a single prompt: 10 to 16 workgroups).  These variants cut every
+ * sequence into chunks that run as workgroups of their own: a first pass
+ * reduces each chunk to (product of its a_t, its state from a zero start), a
+ * small kernel chains those into every chunk's incoming state, a second pass
+ * runs each chunk from there and writes y -- the scan operator is associative
+ * (recurrentgemma/jax/scan.py:161-187), this is the kernel's own cross-wave
+ * carry one level up.  Twice the reads, none of the idling.
+ * rg_scan_split_workspace_bytes is 0 for shapes
+ * that gain nothing (then the calls behave exactly like the plain ones and
+ * workspace may be null); otherwise workspace (16-byte aligned, that many
+ * bytes) is required.  Same arguments and results otherwise (fp32 1e-5, the
+ * float32 state is combined in a different order). */
+size_t rg_scan_split_workspace_bytes(int B, int T, int W);
+int rg_lru_scan_fused_split(const void* x, int apply_conv, const void* conv_w,
+                            const void* conv_b, const void* gx_pre,
+                            const void* ga_pre, const void* a_param,
+                            const void* segpos, int segpos_is_i64,
+                            const void* h0, void* y, void* h_last,
+                            void* conv_cache_out, void* workspace,
+                            size_t workspace_bytes, int B, int T, int W,
+                            int dtype, void* stream);
+int rg_linear_scan_split(const void* x, const void* a, const void* reset,
+                         const void* h0, void* y, void* h_last, void* workspace,
+                         size_t workspace_bytes, int B, int T, int W, int dtype,
+                         void* stream);
+
 /* Prefill of the conv -> RG-LRU core in ONE launch, as RecurrentBlock.forward
  * chains the two modules without a cache (recurrentgemma/torch/modules.py:
  * 632-643: Conv1D.forward layers.py:447-529, then RGLRU.forward :313-365 with

@@ -40,6 +40,12 @@ SIGNATURES = {
                                   _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i,
                                   _i, _vp]),
     "rg_linear_scan": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "rg_scan_split_workspace_bytes": (_sz, [_i, _i, _i]),
+    "rg_lru_scan_fused_split": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i,
+                                     _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i,
+                                     _i, _vp]),
+    "rg_linear_scan_split": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i,
+                                  _i, _i, _i, _vp]),
     "rg_recurrent_step_workspace_bytes": (_sz, [_i, _i, _i]),
     "rg_gelu_mul": (_i, [_vp, _vp, _vp, ctypes.c_int64, _i, _vp]),
     "rg_rms_norm": (_i, [_vp, _vp, _vp, ctypes.c_int64, _i, ctypes.c_float, _i,

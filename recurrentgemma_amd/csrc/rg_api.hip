@@ -26,6 +26,10 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 size_t esize(int dtype) { return dtype == RG_DTYPE_F32 ? 4 : 2; }
 
+// The entry point named in error messages: the function itself, or, in a body
+// shared by two entry points, the one that was called.
+#define RG_WHO __func__
+
 #define RG_REQUIRE(cond, ...) \
   do {                        \
     if (!(cond)) return fail(RG_ERR_BAD_ARG, __VA_ARGS__); \
@@ -35,17 +39,17 @@ size_t esize(int dtype) { return dtype == RG_DTYPE_F32 ? 4 : 2; }
   do {                                                                   \
     if ((dtype) != RG_DTYPE_F32 && (dtype) != RG_DTYPE_BF16)             \
       return fail(RG_ERR_UNSUPPORTED, "%s: dtype %d is not f32/bf16",    \
-                  __func__, (dtype));                                    \
+                  RG_WHO, (dtype));                                    \
   } while (0)
 
 #define RG_CHECK_PTR(p)                                                     \
   do {                                                                      \
-    RG_REQUIRE((p) != nullptr, "%s: %s is null", __func__, #p);             \
-    RG_REQUIRE(aligned16(p), "%s: %s is not 16-byte aligned", __func__, #p); \
+    RG_REQUIRE((p) != nullptr, "%s: %s is null", RG_WHO, #p);             \
+    RG_REQUIRE(aligned16(p), "%s: %s is not 16-byte aligned", RG_WHO, #p); \
   } while (0)
 
 #define RG_CHECK_OPT_PTR(p) \
-  RG_REQUIRE(aligned16(p), "%s: %s is not 16-byte aligned", __func__, #p)
+  RG_REQUIRE(aligned16(p), "%s: %s is not 16-byte aligned", RG_WHO, #p)
 
 }  // namespace
 
@@ -174,15 +178,45 @@ int rg_gates_gemm(const void* x, int apply_conv, const void* segpos,
   return launch_status(__func__, e);
 }
 
-int rg_lru_scan_fused(const void* x, int apply_conv, const void* conv_w,
-                      const void* conv_b, const void* gx_pre,
-                      const void* ga_pre, const void* a_param,
-                      const void* segpos, int segpos_is_i64, const void* h0,
-                      void* y, void* h_last, void* conv_cache_out, int B, int T,
-                      int W, int dtype, void* stream) {
+size_t rg_scan_split_workspace_bytes(int B, int T, int W) {
+  if (B <= 0 || T <= 0 || W <= 0) return 0;
+  int chunks, t_chunk;
+  rg::scan_split_plan(B, T, W, &chunks, &t_chunk);
+  return chunks > 1 ? (size_t)3 * B * chunks * W * sizeof(float) : 0;
+}
+
+// Points the scan at its workspace if the shape is one that is cut into
+// chunks; RG_OK or the error for a workspace that is missing or too small.
+static int plan_scan_split(const char* who, rg::ScanArgs* a, void* workspace,
+                           size_t workspace_bytes) {
+  const size_t need = rg_scan_split_workspace_bytes(a->B, a->T, a->W);
+  if (need == 0) return RG_OK;
+  if (workspace == nullptr || workspace_bytes < need || !aligned16(workspace))
+    return fail(RG_ERR_WORKSPACE,
+                "%s: workspace of %zu bytes (16-byte aligned) required, got %zu",
+                who, need, workspace ? workspace_bytes : (size_t)0);
+  rg::scan_split_plan(a->B, a->T, a->W, &a->chunks, &a->t_chunk);
+  const size_t one = (size_t)a->B * a->chunks * a->W;
+  a->ws_p = (float*)workspace;
+  a->ws_h = a->ws_p + one;
+  a->ws_h_in = a->ws_h + one;
+  return RG_OK;
+}
+
+#undef RG_WHO
+#define RG_WHO who
+static int lru_scan_fused_impl(const char* who, const void* x, int apply_conv,
+                               const void* conv_w, const void* conv_b,
+                               const void* gx_pre, const void* ga_pre,
+                               const void* a_param, const void* segpos,
+                               int segpos_is_i64, const void* h0, void* y,
+                               void* h_last, void* conv_cache_out,
+                               void* workspace, size_t workspace_bytes,
+                               bool split, int B, int T, int W, int dtype,
+                               void* stream) {
   RG_CHECK_DTYPE(dtype);
   RG_REQUIRE(B > 0 && T > 0 && W > 0, "%s: B=%d T=%d W=%d must be positive",
-             __func__, B, T, W);
+             who, B, T, W);
   RG_CHECK_PTR(x);
   RG_CHECK_PTR(gx_pre);
   RG_CHECK_PTR(ga_pre);
@@ -193,13 +227,13 @@ int rg_lru_scan_fused(const void* x, int apply_conv, const void* conv_w,
   RG_CHECK_OPT_PTR(h_last);
   RG_CHECK_OPT_PTR(conv_cache_out);
   RG_REQUIRE(y != x && y != gx_pre && y != ga_pre,
-             "%s: y must not alias an input", __func__);
+             "%s: y must not alias an input", who);
   if (apply_conv) {
     RG_CHECK_PTR(conv_w);
     RG_CHECK_PTR(conv_b);
   } else {
     RG_REQUIRE(conv_cache_out == nullptr,
-               "%s: conv_cache_out needs apply_conv", __func__);
+               "%s: conv_cache_out needs apply_conv", who);
   }
   rg::ScanArgs a{};
   a.x = x;
@@ -218,8 +252,40 @@ int rg_lru_scan_fused(const void* x, int apply_conv, const void* conv_w,
   a.B = B;
   a.T = T;
   a.W = W;
-  return launch_status(__func__,
-                       rg::launch_lru_scan(a, dtype, (hipStream_t)stream));
+  if (split) {
+    const int rc = plan_scan_split(who, &a, workspace, workspace_bytes);
+    if (rc != RG_OK) return rc;
+  }
+  return launch_status(who, rg::launch_lru_scan(a, dtype, (hipStream_t)stream));
+}
+
+#undef RG_WHO
+#define RG_WHO __func__
+
+int rg_lru_scan_fused(const void* x, int apply_conv, const void* conv_w,
+                      const void* conv_b, const void* gx_pre,
+                      const void* ga_pre, const void* a_param,
+                      const void* segpos, int segpos_is_i64, const void* h0,
+                      void* y, void* h_last, void* conv_cache_out, int B, int T,
+                      int W, int dtype, void* stream) {
+  return lru_scan_fused_impl(__func__, x, apply_conv, conv_w, conv_b, gx_pre,
+                             ga_pre, a_param, segpos, segpos_is_i64, h0, y,
+                             h_last, conv_cache_out, nullptr, 0, false, B, T, W,
+                             dtype, stream);
+}
+
+int rg_lru_scan_fused_split(const void* x, int apply_conv, const void* conv_w,
+                            const void* conv_b, const void* gx_pre,
+                            const void* ga_pre, const void* a_param,
+                            const void* segpos, int segpos_is_i64,
+                            const void* h0, void* y, void* h_last,
+                            void* conv_cache_out, void* workspace,
+                            size_t workspace_bytes, int B, int T, int W,
+                            int dtype, void* stream) {
+  return lru_scan_fused_impl(__func__, x, apply_conv, conv_w, conv_b, gx_pre,
+                             ga_pre, a_param, segpos, segpos_is_i64, h0, y,
+                             h_last, conv_cache_out, workspace, workspace_bytes,
+                             true, B, T, W, dtype, stream);
 }
 
 int rg_recurrent_prefill(const void* x, const void* segpos, int segpos_is_i64,
@@ -282,19 +348,23 @@ int rg_recurrent_prefill(const void* x, const void* segpos, int segpos_is_i64,
                        rg::launch_block_fused_bf16(a, (hipStream_t)stream));
 }
 
-int rg_linear_scan(const void* x, const void* a, const void* reset,
-                   const void* h0, void* y, void* h_last, int B, int T, int W,
-                   int dtype, void* stream) {
+#undef RG_WHO
+#define RG_WHO who
+static int linear_scan_impl(const char* who, const void* x, const void* a,
+                            const void* reset, const void* h0, void* y,
+                            void* h_last, void* workspace,
+                            size_t workspace_bytes, bool split, int B, int T,
+                            int W, int dtype, void* stream) {
   RG_CHECK_DTYPE(dtype);
   RG_REQUIRE(B > 0 && T > 0 && W > 0, "%s: B=%d T=%d W=%d must be positive",
-             __func__, B, T, W);
+             who, B, T, W);
   RG_CHECK_PTR(x);
   RG_CHECK_PTR(a);
   RG_CHECK_PTR(reset);
   RG_CHECK_PTR(y);
   RG_CHECK_OPT_PTR(h0);
   RG_CHECK_OPT_PTR(h_last);
-  RG_REQUIRE(y != x && y != a, "%s: y must not alias an input", __func__);
+  RG_REQUIRE(y != x && y != a, "%s: y must not alias an input", who);
   rg::ScanArgs s{};
   s.plain = 1;
   s.x = x;
@@ -308,8 +378,29 @@ int rg_linear_scan(const void* x, const void* a, const void* reset,
   s.B = B;
   s.T = T;
   s.W = W;
-  return launch_status(__func__,
-                       rg::launch_lru_scan(s, dtype, (hipStream_t)stream));
+  if (split) {
+    const int rc = plan_scan_split(who, &s, workspace, workspace_bytes);
+    if (rc != RG_OK) return rc;
+  }
+  return launch_status(who, rg::launch_lru_scan(s, dtype, (hipStream_t)stream));
+}
+
+#undef RG_WHO
+#define RG_WHO __func__
+
+int rg_linear_scan(const void* x, const void* a, const void* reset,
+                   const void* h0, void* y, void* h_last, int B, int T, int W,
+                   int dtype, void* stream) {
+  return linear_scan_impl(__func__, x, a, reset, h0, y, h_last, nullptr, 0,
+                          false, B, T, W, dtype, stream);
+}
+
+int rg_linear_scan_split(const void* x, const void* a, const void* reset,
+                         const void* h0, void* y, void* h_last, void* workspace,
+                         size_t workspace_bytes, int B, int T, int W, int dtype,
+                         void* stream) {
+  return linear_scan_impl(__func__, x, a, reset, h0, y, h_last, workspace,
+                          workspace_bytes, true, B, T, W, dtype, stream);
 }
 
 size_t rg_recurrent_step_workspace_bytes(int B, int W, int dtype) {

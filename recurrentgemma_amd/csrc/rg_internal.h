@@ -61,6 +61,13 @@ struct ScanArgs {
   float* h_last;
   void* cache_out;
   int B, T, W;
+  // sequences cut into `chunks` chunks of t_chunk tokens (chunks <= 1: not
+  // cut), with three [B][chunks][W] float rows of workspace: every chunk's
+  // product of a_t, its state from a zero start, its incoming state
+  int chunks, t_chunk;
+  float* ws_p;
+  float* ws_h;
+  float* ws_h_in;
 };
 
 struct FusedArgs {
@@ -114,6 +121,7 @@ hipError_t launch_conv1d_step(const ConvStepArgs& a, int dtype, hipStream_t s);
 hipError_t launch_gemm_generic(const GemmArgs& a, int dtype, hipStream_t s);
 hipError_t launch_gemm_mfma_bf16(const GemmArgs& a, hipStream_t s);
 hipError_t launch_lru_scan(const ScanArgs& a, int dtype, hipStream_t s);
+void scan_split_plan(int B, int T, int W, int* chunks, int* t_chunk);
 hipError_t launch_block_fused_bf16(const FusedArgs& a, hipStream_t s);
 hipError_t launch_block_step_bf16(const StepArgs& a, hipStream_t s);
 // bf16 [H,256,256] x 2 -> one buffer of the same total size in MFMA operand

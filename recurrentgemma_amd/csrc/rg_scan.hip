@@ -470,7 +470,17 @@ __device__ __forceinline__ void phase2(__amdgpu_buffer_rsrc_t ry, uint32_t voff,
   }
 }
 
-template <typename T, int CH, int KL, bool CONV, bool FAST, bool PLAIN>
+// SPLIT: a row's sequence cut into chunks that run as workgroups of their own
+// (blockIdx.y), for few rows and channel slabs: 0 = the whole row in one
+// workgroup; 1 = summary of a chunk: its state from a zero start and the
+// product of its a_t, nothing else written; 2 = the chunk again from its true
+// incoming state (h_in, computed from the summaries), writing y.  The scan
+// operator is associative, so this is the kernel's own cross-wave carry one
+// level up.
+enum ScanSplit { kWholeRow = 0, kChunkSummary = 1, kChunkReplay = 2 };
+
+template <typename T, int CH, int KL, bool CONV, bool FAST, bool PLAIN,
+          int SPLIT>
 __global__ void __launch_bounds__(kMaxNW* kWave, (sizeof(T) == 2 ? 4 : 2))
 lru_scan_kernel(ScanArgs p) {
   // LDS (sized at launch): per buffer and wave the lanes' (P.., Hloc..)
@@ -485,7 +495,13 @@ lru_scan_kernel(ScanArgs p) {
   AggRow* const agg0 = reinterpret_cast<AggRow*>(lds_f);   // [2][nw]
   CarryRow* const carry_s =
       reinterpret_cast<CarryRow*>(lds_f + 2 * nw * kWave * 2 * CH);  // [2]
-  const int T_len = p.T;
+  // tokens [t_lo, T_len) of the row are this workgroup's; everything below
+  // treats T_len as the end of the sequence
+  const int chunk = SPLIT == kWholeRow ? 0 : (int)blockIdx.y;
+  const int t_lo = SPLIT == kWholeRow ? 0 : chunk * p.t_chunk;
+  const int T_len =
+      SPLIT == kWholeRow ? p.T : (t_lo + p.t_chunk < p.T ? t_lo + p.t_chunk : p.T);
+  const bool last_chunk = T_len == p.T;
   const int64_t W = p.W;
   const int nslab = (p.W + kWave * CH - 1) / (kWave * CH);
   const int b = blockIdx.x / nslab;
@@ -516,7 +532,7 @@ lru_scan_kernel(ScanArgs p) {
     }
   }
 
-  const int64_t row0 = (int64_t)b * T_len;
+  const int64_t row0 = (int64_t)b * p.T;
   const uint32_t row_bytes = (uint32_t)p.W * (uint32_t)sizeof(T);
   const uint32_t voff =
       active ? (uint32_t)c_raw * (uint32_t)sizeof(T) : kOutOfRange;
@@ -527,10 +543,17 @@ lru_scan_kernel(ScanArgs p) {
   const char* garow = (const char*)p.ga + row0 * row_bytes;
   char* yrow = (char*)p.y + row0 * row_bytes;
 
+  // per-chunk rows of the workspace: [B][chunks][W] each
+  const int64_t ws_row = ((int64_t)b * p.chunks + chunk) * W + c;
   float h[CH];
+  float chunk_p[CH];  // kChunkSummary: product of every a_t seen so far
 #pragma unroll
-  for (int ch = 0; ch < CH; ++ch)
-    h[ch] = p.h0 ? p.h0[(int64_t)b * W + c + ch] : 0.0f;
+  for (int ch = 0; ch < CH; ++ch) {
+    if (SPLIT == kChunkSummary) h[ch] = 0.0f;
+    else if (SPLIT == kChunkReplay) h[ch] = p.ws_h_in[ws_row + ch];
+    else h[ch] = p.h0 ? p.h0[(int64_t)b * W + c + ch] : 0.0f;
+    chunk_p[ch] = 1.0f;
+  }
 
   const int span = nw * KL;
 
@@ -544,16 +567,17 @@ lru_scan_kernel(ScanArgs p) {
   Tile<T, CH, KL> tl;
   uint32_t starts;
   {
-    const SegRaw seg = load_seg<KL, CONV>(p, row0, wave * KL, T_len, lane);
+    const SegRaw seg =
+        load_seg<KL, CONV>(p, row0, t_lo + wave * KL, T_len, lane);
     const StepAddr<KL> a0 =
-        step_addr<KL>(xrow, gxrow, garow, wave * KL, T_len, row_bytes);
+        step_addr<KL>(xrow, gxrow, garow, t_lo + wave * KL, T_len, row_bytes);
     load_halo<T, CH, KL, CONV>(tl, a0, voff);
 #pragma unroll
     for (int i = 0; i < KL; ++i) load_token<T, CH, KL, PLAIN>(tl, i, a0, voff);
     starts = doc_starts(seg);
   }
 
-  for (int step = 0, tb = 0; tb < T_len; ++step, tb += span) {
+  for (int step = 0, tb = t_lo; tb < T_len; ++step, tb += span) {
     const int buf = step & 1;
     const int t0 = tb + wave * KL;
     const bool any = t0 < T_len;
@@ -587,18 +611,27 @@ lru_scan_kernel(ScanArgs p) {
     }
     for (int v = 0; v < wave; ++v) {
 #pragma unroll
-      for (int ch = 0; ch < CH; ++ch)
+      for (int ch = 0; ch < CH; ++ch) {
         h[ch] = __builtin_fmaf(agg[v][lane][ch], h[ch], agg[v][lane][CH + ch]);
+        if (SPLIT == kChunkSummary) chunk_p[ch] *= agg[v][lane][ch];
+      }
+    }
+    if (SPLIT == kChunkSummary) {  // complete in the last wave only
+#pragma unroll
+      for (int ch = 0; ch < CH; ++ch) chunk_p[ch] *= any ? P[ch] : 1.0f;
     }
 
     {
+      // (a summary writes no y: a descriptor of no bytes drops every store)
       const __amdgpu_buffer_rsrc_t ry = make_rsrc(
-          yrow + (int64_t)(any ? t0 : T_len - 1) * row_bytes, span_bytes);
+          yrow + (int64_t)(any ? t0 : T_len - 1) * row_bytes,
+          SPLIT == kChunkSummary ? 0u : span_bytes);
       // this wave holds token T-1 iff its valid tokens end the sequence
+      float* h_end = p.h_last ? p.h_last + (int64_t)b * W + c : nullptr;
+      if (SPLIT == kChunkSummary) h_end = p.ws_h + ws_row;
+      if (SPLIT == kChunkReplay && !last_chunk) h_end = nullptr;
       float* const h_last_lane =
-          (p.h_last && active && any && t0 + n_valid == T_len)
-              ? p.h_last + (int64_t)b * W + c
-              : nullptr;
+          (h_end && active && any && t0 + n_valid == T_len) ? h_end : nullptr;
       float hw[CH];  // replay on a copy: a wave without tokens must hand the
 #pragma unroll       // carry on unchanged
       for (int ch = 0; ch < CH; ++ch) hw[ch] = h[ch];
@@ -612,6 +645,15 @@ lru_scan_kernel(ScanArgs p) {
     }
     starts = doc_starts(seg_next);
   }
+
+  if (SPLIT == kChunkSummary) {
+    if (wave == nw - 1 && active) {
+#pragma unroll
+      for (int ch = 0; ch < CH; ++ch) p.ws_p[ws_row + ch] = chunk_p[ch];
+    }
+    return;
+  }
+  if (SPLIT == kChunkReplay && !last_chunk) return;
 
   // Masked conv state: rows T-3..T-1 of x, each zeroed if a document starts in
   // a later position of the row; rows before the sequence start are zero.
@@ -633,38 +675,106 @@ lru_scan_kernel(ScanArgs p) {
   }
 }
 
-template <typename T, int CH, int KL, bool CONV, bool FAST, bool PLAIN>
+// h_in of every chunk from the summaries: h_in[0] = h0, h_in[k+1] =
+// P[k] h_in[k] + H[k].  One thread per (row, channel).
+__global__ void __launch_bounds__(256)
+scan_chunk_carry_kernel(ScanArgs p) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (int64_t)p.B * p.W) return;
+  const int64_t b = i / p.W, c = i - b * p.W;
+  float h = p.h0 ? p.h0[i] : 0.0f;
+  for (int k0 = 0; k0 < p.chunks; k0 += 8) {
+    float pk[8], hk[8];  // eight chunks' summaries in flight at a time
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int k = k0 + j < p.chunks ? k0 + j : p.chunks - 1;
+      const int64_t at = (b * p.chunks + k) * p.W + c;
+      pk[j] = p.ws_p[at];
+      hk[j] = p.ws_h[at];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (k0 + j < p.chunks) {
+        p.ws_h_in[(b * p.chunks + k0 + j) * p.W + c] = h;
+        h = __builtin_fmaf(pk[j], h, hk[j]);
+      }
+    }
+  }
+}
+
+template <typename T, int CH, int KL, bool CONV, bool FAST, bool PLAIN,
+          int SPLIT>
 hipError_t launch_t(const ScanArgs& a, hipStream_t s) {
   const int nslab = (a.W + kWave * CH - 1) / (kWave * CH);
   const int64_t blocks = (int64_t)a.B * nslab;
+  const int chunks = SPLIT == kWholeRow ? 1 : a.chunks;
+  const int t_run = SPLIT == kWholeRow ? a.T : a.t_chunk;
   // Waves per workgroup: enough to cover the sequence, and 16 rather than 8
   // when the grid alone would leave most of the 256 CUs' wave slots empty.
-  int max_nw = blocks * 8 >= 4096 ? 8 : kMaxNW;
+  int max_nw = blocks * chunks * 8 >= 4096 ? 8 : kMaxNW;
   int nw = 1;
-  while (nw < max_nw && nw * KL < a.T) nw *= 2;
+  while (nw < max_nw && nw * KL < t_run) nw *= 2;
+  if (SPLIT != kWholeRow && (a.t_chunk % (nw * KL) != 0 || chunks > 65535))
+    return hipErrorInvalidValue;
   // a wave's rows of one step must fit a descriptor's 32-bit offsets
   if (blocks > 0x7fffffff ||
       (int64_t)a.W * sizeof(T) * (KL + 3) >= (int64_t)kOutOfRange)
     return hipErrorInvalidValue;
   const size_t lds = sizeof(float) * (2 * nw * kWave * 2 * CH + 2 * kWave * CH);
-  auto kern = lru_scan_kernel<T, CH, KL, CONV, FAST, PLAIN>;
+  auto kern = lru_scan_kernel<T, CH, KL, CONV, FAST, PLAIN, SPLIT>;
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(
         (const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
   }
-  kern<<<dim3((unsigned)blocks), dim3(nw * kWave), lds, s>>>(a);
+  kern<<<dim3((unsigned)blocks, (unsigned)chunks), dim3(nw * kWave), lds, s>>>(
+      a);
   return hipGetLastError();
+}
+
+template <typename T, int CH, int KL, bool CONV, bool FAST, bool PLAIN>
+hipError_t launch_split(const ScanArgs& a, hipStream_t s) {
+  if (a.chunks <= 1)
+    return launch_t<T, CH, KL, CONV, FAST, PLAIN, kWholeRow>(a, s);
+  hipError_t e = launch_t<T, CH, KL, CONV, FAST, PLAIN, kChunkSummary>(a, s);
+  if (e != hipSuccess) return e;
+  const int64_t n = (int64_t)a.B * a.W;
+  scan_chunk_carry_kernel<<<dim3((unsigned)((n + 255) / 256)), 256, 0, s>>>(a);
+  e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  return launch_t<T, CH, KL, CONV, FAST, PLAIN, kChunkReplay>(a, s);
 }
 
 template <typename T, int CH, int KL, bool FAST>
 hipError_t launch_mode(const ScanArgs& a, hipStream_t s) {
-  if (a.plain) return launch_t<T, CH, KL, false, FAST, true>(a, s);
-  if (a.apply_conv) return launch_t<T, CH, KL, true, FAST, false>(a, s);
-  return launch_t<T, CH, KL, false, FAST, false>(a, s);
+  if (a.plain) return launch_split<T, CH, KL, false, FAST, true>(a, s);
+  if (a.apply_conv) return launch_split<T, CH, KL, true, FAST, false>(a, s);
+  return launch_split<T, CH, KL, false, FAST, false>(a, s);
 }
 
 }  // namespace
+
+// Whether, and how, to cut the sequences of this shape into chunks.  One
+// workgroup walks a row at about 2.5 us per 64-token step however few of them
+// run (a row of 8192 tokens: 0.32 ms).  Cut into chunks the rows are read
+// twice, but every CU works: the aim is one workgroup per CU (more would queue
+// for a second round on the CUs that finish first), chunk lengths in multiples
+// of 128 tokens (a step of 16 waves at 8 tokens each, the longest step in
+// use).  Worth it up to about 32 (row, 256-channel slab) pairs and from about
+// a thousand tokens on; measured, bf16, T = 8192: 10 pairs 321 -> 75 us,
+// 80 pairs no gain.
+void scan_split_plan(int B, int T, int W, int* chunks, int* t_chunk) {
+  *chunks = 1;
+  *t_chunk = T;
+  const int64_t wide_blocks = (int64_t)B * ((W + 255) / 256);
+  if (wide_blocks > 32 || T < 1024) return;
+  const int want = (int)(256 / wide_blocks);
+  const int len = ((T + want - 1) / want + 127) / 128 * 128;
+  const int n = (T + len - 1) / len;
+  if (n < 2) return;
+  *t_chunk = len;
+  *chunks = n;
+}
 
 hipError_t launch_lru_scan(const ScanArgs& a, int dtype, hipStream_t s) {
   // Channels per lane: 8 bytes per lane where the width allows it (every row
@@ -676,7 +786,8 @@ hipError_t launch_lru_scan(const ScanArgs& a, int dtype, hipStream_t s) {
   }
   // 8-byte lanes halve the number of workgroups (B * ceil(W/256)); below
   // about 200 of them too many of the 256 CUs idle and 4-byte lanes win.
-  const int64_t wide_blocks = (int64_t)a.B * ((a.W + 255) / 256);
+  const int64_t wide_blocks =
+      (int64_t)a.B * ((a.W + 255) / 256) * (a.chunks > 1 ? a.chunks : 1);
   if (a.W % 4 == 0 && wide_blocks >= 200)
     return launch_mode<uint16_t, 4, 4, true>(a, s);
   if (a.W % 2 == 0) return launch_mode<uint16_t, 2, 8, true>(a, s);

@@ -147,8 +147,16 @@ def gates_gemm(x, w_x, b_x, w_a, b_a, conv=None):
   return gx, ga
 
 
+def _scan_workspace(B, T, W, device, split):
+  """Workspace for a scan whose sequences are cut into chunks that run side
+  by side (few rows and channels, long sequences), or None for the one-pass
+  form (split=False forces that one)."""
+  need = _lib.lib().rg_scan_split_workspace_bytes(B, T, W) if split else 0
+  return torch.empty(need, dtype=torch.uint8, device=device) if need else None
+
+
 def lru_scan_fused(x, gx_pre, ga_pre, a_param, segment_pos, h0=None, conv=None,
-                   return_h=True, return_conv_cache=False):
+                   return_h=True, return_conv_cache=False, split=True):
   """conv = None or (conv_w, conv_b): apply the width-4 conv to x first."""
   B, T, W = x.shape
   assert gx_pre.shape == x.shape and ga_pre.shape == x.shape
@@ -175,11 +183,18 @@ def lru_scan_fused(x, gx_pre, ga_pre, a_param, segment_pos, h0=None, conv=None,
   if return_conv_cache:
     assert conv is not None
     cache = x.new_empty((B, 3, W))
+  ws = _scan_workspace(B, T, W, x.device, split)
   with torch.cuda.device(x.device):
-    _lib.check(_lib.lib().rg_lru_scan_fused(
-        _p(x), int(conv is not None), _p(cw), _p(cb), _p(gx_pre), _p(ga_pre),
-        _p(a_param), _p(seg), is64, _p(h0), _p(y), _p(h_last), _p(cache), B, T,
-        W, _dtype_code(x), _stream(x)))
+    if ws is None:
+      _lib.check(_lib.lib().rg_lru_scan_fused(
+          _p(x), int(conv is not None), _p(cw), _p(cb), _p(gx_pre), _p(ga_pre),
+          _p(a_param), _p(seg), is64, _p(h0), _p(y), _p(h_last), _p(cache), B,
+          T, W, _dtype_code(x), _stream(x)))
+    else:
+      _lib.check(_lib.lib().rg_lru_scan_fused_split(
+          _p(x), int(conv is not None), _p(cw), _p(cb), _p(gx_pre), _p(ga_pre),
+          _p(a_param), _p(seg), is64, _p(h0), _p(y), _p(h_last), _p(cache),
+          _p(ws), ws.numel(), B, T, W, _dtype_code(x), _stream(x)))
   return y, h_last, cache
 
 
@@ -229,7 +244,7 @@ def recurrent_prefill(x, segment_pos, conv_w, conv_b, w_x, b_x, w_a, b_a,
   return y, h_last, cache
 
 
-def linear_scan(x, a, reset, h0=None):
+def linear_scan(x, a, reset, h0=None, split=True):
   B, T, W = x.shape
   x = _dev(x, "x")
   _same(x.dtype, x.device, a=a)
@@ -240,10 +255,16 @@ def linear_scan(x, a, reset, h0=None):
     h0 = _dev(h0, "h0")
   y = torch.empty_like(x)
   h_last = torch.empty((B, W), dtype=torch.float32, device=x.device)
+  ws = _scan_workspace(B, T, W, x.device, split)
   with torch.cuda.device(x.device):
-    _lib.check(_lib.lib().rg_linear_scan(
-        _p(x), _p(a), _p(reset), _p(h0), _p(y), _p(h_last), B, T, W,
-        _dtype_code(x), _stream(x)))
+    if ws is None:
+      _lib.check(_lib.lib().rg_linear_scan(
+          _p(x), _p(a), _p(reset), _p(h0), _p(y), _p(h_last), B, T, W,
+          _dtype_code(x), _stream(x)))
+    else:
+      _lib.check(_lib.lib().rg_linear_scan_split(
+          _p(x), _p(a), _p(reset), _p(h0), _p(y), _p(h_last), _p(ws),
+          ws.numel(), B, T, W, _dtype_code(x), _stream(x)))
   return y, h_last
 
 

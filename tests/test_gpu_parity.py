@@ -173,6 +173,57 @@ def test_rnn_scan(dtype, T):
     assert h.dtype == torch.float32
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,T,W,mean_doc", [
+    (1, 2048, 512, 0),      # one document, chunks of equal length
+    (1, 4097, 256, 300),    # ragged end, document starts in and between chunks
+    (3, 1100, 130, 40),     # narrow slab, last chunk shorter than the others
+    (3, 8192, 2560, 1500),  # the 2B width, long rows
+])
+def test_scans_cut_into_chunks(dtype, B, T, W, mean_doc):
+  """rg_lru_scan_fused_split / rg_linear_scan_split (sequences cut into chunks
+  that run side by side, for few rows) against the one-pass kernels on the
+  same inputs: the float32 state is combined in a different order, nothing
+  else differs -- fp32 1e-5, bf16 outputs within one rounding of the state;
+  conv cache bit for bit.  Oracle parity of the split path itself: the
+  few-row cases of test_core_vs_oracle, test_rnn_scan and
+  test_config1_fp32_parity run through it."""
+  from recurrentgemma_amd import _lib
+  assert _lib.lib().rg_scan_split_workspace_bytes(B, T, W) > 0
+  _announce("split scan", dtype, B, T, W, mean_doc)
+  g = torch.Generator().manual_seed(T + W)
+  x = _dev(torch.randn(B, T, W, generator=g).to(dtype))
+  gx = _dev(torch.randn(B, T, W, generator=g).to(dtype))
+  ga = _dev((torch.randn(B, T, W, generator=g) * 2).to(dtype))
+  a_param = _dev(R.make_params(W, 1, dtype, seed=5)["a_param"])
+  cw = _dev((torch.randn(4, W, generator=g) * 0.3).to(dtype))
+  cb = _dev((torch.randn(W, generator=g) * 0.1).to(dtype))
+  h0 = _dev(torch.randn(B, W, generator=g))
+  seg = (helpers.document_positions(B, T, mean_doc, seed=T) if mean_doc
+         else torch.arange(T)[None].expand(B, T).contiguous())
+  seg = _dev(seg)
+  tol_y = F32_TOL if dtype == torch.float32 else 2.0 ** -7
+  for conv in (None, (cw, cb)):
+    for start in (None, h0):
+      kw = dict(h0=start, conv=conv, return_conv_cache=conv is not None)
+      y1, h1, c1 = ops.lru_scan_fused(x, gx, ga, a_param, seg, split=False, **kw)
+      y2, h2, c2 = ops.lru_scan_fused(x, gx, ga, a_param, seg, split=True, **kw)
+      assert helpers.max_rel(y2, y1) < tol_y
+      assert helpers.max_rel(h2, h1) < F32_TOL
+      if conv is not None:
+        assert torch.equal(c1, c2)
+      if dtype == torch.bfloat16:  # almost every output rounds the same way
+        assert (y1 != y2).float().mean().item() < 0.01
+  # plain recurrence with resets
+  a = _dev(torch.rand(B, T, W, generator=g).to(dtype))
+  reset = seg == 0
+  for start in (None, h0):
+    y1, h1 = ops.linear_scan(x, a, reset, start, split=False)
+    y2, h2 = ops.linear_scan(x, a, reset, start, split=True)
+    assert helpers.max_rel(y2, y1) < tol_y
+    assert helpers.max_rel(h2, h1) < F32_TOL
+
+
 def test_rnn_scan_closed_forms():
   T, W = 3000, 64
   one = torch.ones(1, T, W, device=DEV)

@@ -24,7 +24,7 @@ def _declared_symbols():
 
 def test_library_exports_every_declared_symbol():
   names = _declared_symbols()
-  assert len(names) == 29, names
+  assert len(names) == 32, names
   lib = ctypes.CDLL(_lib.LIB_PATH)
   for n in names:
     assert hasattr(lib, n), n
@@ -95,6 +95,16 @@ def test_c_side_validation_without_launch():
   rc = lib.rg_linear_rows(ok, ok, None, None, y, None, 0, 64, 7680, 2560, 1, 0,
                           None)
   assert rc == -4 and b"workspace" in lib.rg_last_error()
+  # scans cut into chunks: only for few rows and long sequences
+  assert lib.rg_scan_split_workspace_bytes(16, 8192, 4096) == 0
+  assert lib.rg_scan_split_workspace_bytes(1, 1000, 2560) == 0
+  assert lib.rg_scan_split_workspace_bytes(1, 8192, 2560) == 3 * 22 * 2560 * 4
+  rc = lib.rg_lru_scan_fused_split(ok, 0, None, None, ok, ok, ok, ok, 1, None, y,
+                                   None, None, None, 0, 1, 8192, 2560, 1, None)
+  assert rc == -4 and b"rg_lru_scan_fused_split: workspace" in lib.rg_last_error()
+  rc = lib.rg_linear_scan_split(ok, ok, ok, None, None, None, None, 0, 1, 8192,
+                                2560, 1, None)
+  assert rc == -1 and b"rg_linear_scan_split: y is null" in lib.rg_last_error()
   rc = lib.rg_linear_rows_partial(ok, ok, y, 64, 2560, 2560, 9, None)
   assert rc == -1 and b"slices" in lib.rg_last_error()
   rc = lib.rg_linear_rows_partial(ok, ok, y, 64, 2560, 2570, 3, None)
