@@ -55,6 +55,10 @@ WORKLOADS = {
                    dtype="f32"),
     "9b_decode": dict(B=256, T=1, W=4096, H=16, mean_doc=None, seed=1004,
                       decode=True),
+    # one long prompt: 10 (row, channel slab) pairs, the scan runs its
+    # sequence as chunks side by side
+    "2b_single_prompt": dict(B=1, T=8192, W=2560, H=10, mean_doc=None,
+                             seed=1006),
     # random-init 2B residual stack, greedy decoding: 64 prompts of 2048 random
     # token ids, 256 new tokens each (--steps sets the number of new tokens)
     "2b_griffin_decode": dict(B=64, T=2048, new_tokens=256, seed=1005,
@@ -430,6 +434,8 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
   elapsed, first_ms, second_ms = timed(step, steps, warmup)
 
   tokens = B * T
+  from recurrentgemma_amd import _lib
+  in_chunks = _lib.lib().rg_scan_split_workspace_bytes(B, T, W) > 0
   seg_bytes = seg.element_size()
   scan_algo = scan_algorithmic_bytes(B, T, W, esize, seg_bytes, has_h0=False)
   gemm_flops = 1024.0 * W * tokens
@@ -494,7 +500,9 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
                         else f"geometric mean {wl['mean_doc']}"),
           "path": ("rg_recurrent_prefill (single launch)" if path == "single"
                    else "rg_gates_gemm(conv on load) + "
-                        "rg_lru_scan_fused(conv)")},
+                        + ("rg_lru_scan_fused_split(conv): sequences in chunks "
+                           "side by side" if in_chunks
+                           else "rg_lru_scan_fused(conv)"))},
       "roofline": roofline,
   }
   if path == "split":
