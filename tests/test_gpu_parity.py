@@ -185,9 +185,9 @@ def test_scans_cut_into_chunks(dtype, B, T, W, mean_doc):
   that run side by side, for few rows) against the one-pass kernels on the
   same inputs: the float32 state is combined in a different order, nothing
   else differs -- fp32 1e-5, bf16 outputs within one rounding of the state;
-  conv cache bit for bit.  Oracle parity of the split path itself: the
-  few-row cases of test_core_vs_oracle, test_rnn_scan and
-  test_config1_fp32_parity run through it."""
+  conv cache bit for bit.  Against the oracle: the plain recurrence below
+  (all but the largest shape), and the long single row of
+  test_core_vs_oracle, which runs through the split path."""
   from recurrentgemma_amd import _lib
   assert _lib.lib().rg_scan_split_workspace_bytes(B, T, W) > 0
   _announce("split scan", dtype, B, T, W, mean_doc)
@@ -222,6 +222,12 @@ def test_scans_cut_into_chunks(dtype, B, T, W, mean_doc):
     y2, h2 = ops.linear_scan(x, a, reset, start, split=True)
     assert helpers.max_rel(y2, y1) < tol_y
     assert helpers.max_rel(h2, h1) < F32_TOL
+    if B * T * W <= 4097 * 256:
+      yo, ho = R.rnn_scan(x.cpu(), a.cpu(), reset.cpu(),
+                          None if start is None else start.cpu())
+      assert helpers.max_rel(y2, yo) < (F32_TOL if dtype == torch.float32
+                                        else BF16_TOL)
+      assert helpers.max_rel(h2, ho) < F32_TOL
 
 
 def test_rnn_scan_closed_forms():
