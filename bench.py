@@ -14,7 +14,7 @@ ABI on torch's current stream.  Two forms of the path exist (--path):
           pre-activations go through HBM
 Prints ONE JSON line.
 
-Workloads (BASELINE.json configs):
+Workloads (the benchmark configurations this build is measured on):
   9b_prefill  B16 T8192 W4096 H16 bf16 / fp32 state, one document per row
               (the configuration the >= 70 % HBM-roofline target is stated on;
               default)

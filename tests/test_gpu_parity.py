@@ -1,6 +1,6 @@
 """GPU parity: the HIP path (through the C ABI) against the CPU oracle.
 
-Tolerances (BASELINE north_star): float32 max|d|/max|ref| <= 1e-5 on y and h;
+Tolerances (the bars this build is held to): float32 max|d|/max|ref| <= 1e-5 on y and h;
 bfloat16-in / float32-state <= 1e-2 against the widened oracle (reference
 semantics evaluated in float32 on the bfloat16 values, outputs rounded once).
 """
@@ -322,7 +322,7 @@ def _core_case(dtype, B, T, W, H, seg, seed, bias_std=0.2):
 
 
 def test_config1_fp32_parity():
-  """BASELINE config 1: B1 T512 W2560 H10 fp32, segment_pos = arange."""
+  """Benchmark configuration 1: B1 T512 W2560 H10 fp32, segment_pos = arange."""
   B, T, W, H = 1, 512, 2560, 10
   seg = torch.arange(T)[None]
   p = R.make_params(W, H, torch.float32, seed=1101)
@@ -820,7 +820,7 @@ def _full_size_properties(B, T, W, H, seg, seed):
 
 
 def test_config2_full_size_properties():
-  """BASELINE config 2: B8 T4096 W2560 H10 bf16, documents ~ Geometric(1024)."""
+  """Benchmark configuration 2: B8 T4096 W2560 H10 bf16, documents ~ Geometric(1024)."""
   B, T, W, H = 8, 4096, 2560, 10
   seg = helpers.document_positions(B, T, 1024, seed=1002)
   _announce("config2 full size")
@@ -828,7 +828,7 @@ def test_config2_full_size_properties():
 
 
 def test_config3_full_size_properties():
-  """BASELINE config 3: B16 T8192 W4096 H16 bf16, one document per row."""
+  """Benchmark configuration 3: B16 T8192 W4096 H16 bf16, one document per row."""
   B, T, W, H = 16, 8192, 4096, 16
   seg = torch.arange(T).expand(B, T).contiguous()
   _announce("config3 full size")
