@@ -73,6 +73,27 @@ def test_linear_rows(M, K, N, with_bias):
   assert (lib.float() - got.float()).abs().max().item() <= 2 ** -6 * scale
 
 
+def test_linear_rows_shape_sweep():
+  """Seeded sweep over row counts, depths and widths the packed layout takes
+  (every M from 1 to 64 occurs among the tile boundaries 31/32/33/63/64; odd
+  numbers of K chunks; widths that leave the last workgroups short)."""
+  rng = torch.Generator().manual_seed(2024)
+  shapes = [(1, 64, 32), (31, 64, 32), (32, 128, 96), (33, 320, 160),
+            (63, 448, 32), (64, 704, 416), (17, 1088, 64), (48, 64, 2048)]
+  for _ in range(12):
+    M = int(torch.randint(1, 65, (1,), generator=rng))
+    K = 64 * int(torch.randint(1, 24, (1,), generator=rng))
+    N = 32 * int(torch.randint(1, 40, (1,), generator=rng))
+    shapes.append((M, K, N))
+  for M, K, N in shapes:
+    x = _rand(rng, M, K)
+    w = _rand(rng, N, K, scale=K ** -0.5)
+    b = _rand(rng, N) if (M + N) % 2 else None
+    got = ops.PackedLinear()(x.to(DEV), (w.to(DEV),),
+                             None if b is None else (b.to(DEV),))
+    _check(got, x, w, b)
+
+
 def test_layers_packed_together():
   """Two nn.Linear layers on the same input as one launch: each output equals
   the layer run alone."""
