@@ -143,6 +143,24 @@ def test_sample_tokens_without_vocab(model, golden):
     assert torch.equal(single[0], out[r])
 
 
+def test_sampling_from_the_distribution(model):
+  """greedy_sampling=False draws from the categorical distribution of the
+  logits (sampler.py:129-131): reproducible under a seed, tokens in range, and
+  with one logit far above the rest the draw is that token."""
+  smp = S.Sampler(model, greedy_sampling=False)
+  toks = torch.tensor([[2, 7, 40, 3]], device=DEV, dtype=torch.int32)
+  lens = torch.tensor([4], device=DEV, dtype=torch.int32)
+  torch.manual_seed(123)
+  a, _ = smp.sample_tokens(toks, lens, 6)
+  torch.manual_seed(123)
+  b, _ = smp.sample_tokens(toks, lens, 6)
+  assert torch.equal(a, b)
+  assert a.shape == (1, 6) and int(a.min()) >= 0 and int(a.max()) < 48
+  peaked = torch.full((3, 48), -50.0, device=DEV)
+  peaked[0, 5] = peaked[1, 47] = peaked[2, 0] = 50.0
+  assert smp._pick(peaked).tolist() == [5, 47, 0]
+
+
 def _bf16_model():
   """Three blocks with 256-wide heads in bf16: the shapes that take the
   single-launch decode kernel on packed weights."""
