@@ -635,7 +635,21 @@ lru_scan_kernel(ScanArgs p) {
       float hw[CH];  // replay on a copy: a wave without tokens must hand the
 #pragma unroll       // carry on unchanged
       for (int ch = 0; ch < CH; ++ch) hw[ch] = h[ch];
-      phase2<T, CH, KL>(ry, voff, row_bytes, n_valid, h_last_lane, a_, xn_, hw);
+      if (SPLIT == kChunkSummary) {
+        // no outputs to replay for: the wave's pair applied to its incoming
+        // state is its final state (summaries are taken of whole steps only:
+        // the last chunk of a row, which may end inside a step, has none)
+#pragma unroll
+        for (int ch = 0; ch < CH; ++ch)
+          hw[ch] = __builtin_fmaf(P[ch], h[ch], H[ch]);
+        if (h_last_lane) {
+#pragma unroll
+          for (int ch = 0; ch < CH; ++ch) h_last_lane[ch] = hw[ch];
+        }
+      } else {
+        phase2<T, CH, KL>(ry, voff, row_bytes, n_valid, h_last_lane, a_, xn_,
+                          hw);
+      }
 #pragma unroll
       for (int ch = 0; ch < CH; ++ch) h[ch] = any ? hw[ch] : h[ch];
     }
@@ -683,11 +697,12 @@ scan_chunk_carry_kernel(ScanArgs p) {
   if (i >= (int64_t)p.B * p.W) return;
   const int64_t b = i / p.W, c = i - b * p.W;
   float h = p.h0 ? p.h0[i] : 0.0f;
+  // summaries exist for chunks 0 .. chunks-2
   for (int k0 = 0; k0 < p.chunks; k0 += 8) {
     float pk[8], hk[8];  // eight chunks' summaries in flight at a time
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const int k = k0 + j < p.chunks ? k0 + j : p.chunks - 1;
+      const int k = k0 + j < p.chunks - 1 ? k0 + j : p.chunks - 2;
       const int64_t at = (b * p.chunks + k) * p.W + c;
       pk[j] = p.ws_p[at];
       hk[j] = p.ws_h[at];
@@ -707,7 +722,10 @@ template <typename T, int CH, int KL, bool CONV, bool FAST, bool PLAIN,
 hipError_t launch_t(const ScanArgs& a, hipStream_t s) {
   const int nslab = (a.W + kWave * CH - 1) / (kWave * CH);
   const int64_t blocks = (int64_t)a.B * nslab;
-  const int chunks = SPLIT == kWholeRow ? 1 : a.chunks;
+  // (the last chunk's summary would feed no other chunk: not computed)
+  const int chunks = SPLIT == kWholeRow
+                         ? 1
+                         : (SPLIT == kChunkSummary ? a.chunks - 1 : a.chunks);
   const int t_run = SPLIT == kWholeRow ? a.T : a.t_chunk;
   // Waves per workgroup: enough to cover the sequence, and 16 rather than 8
   // when the grid alone would leave most of the 256 CUs' wave slots empty.
