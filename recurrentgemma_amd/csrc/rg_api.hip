@@ -150,6 +150,10 @@ int rg_gates_gemm(const void* x, int apply_conv, const void* segpos,
     RG_CHECK_PTR(segpos);
     RG_CHECK_PTR(conv_w);
     RG_CHECK_PTR(conv_b);
+    // the kernels address segpos through a 32-bit buffer descriptor
+    RG_REQUIRE((int64_t)B * T * (segpos_is_i64 ? 8 : 4) < ((int64_t)1 << 32),
+               "%s: B*T=%lld positions exceed the 4 GiB a segpos descriptor "
+               "covers", __func__, (long long)B * T);
   }
   rg::GemmArgs a{};
   a.x = x;

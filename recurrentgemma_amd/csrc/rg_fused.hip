@@ -486,9 +486,9 @@ __global__ void __launch_bounds__(512) block_fused_bf16_kernel(FusedArgs p) {
   };
 
   // ---- tile loop ------------------------------------------------------------
-  // Phases of one tile `it` (staged in buffer it % 3):
+  // Phases of one tile `it` (staged in buffer it % 2):
   //   A   MFMA of tokens 0-31, with the conv of tile it+1 (into buffer
-  //       (it+1) % 3) between the matrix instructions
+  //       (it+1) % 2) between the matrix instructions
   //   E0  gates + recurrence of tokens 0-31, with the MFMA of tokens 32-63
   //       and the row loads of tile it+2 spread through it
   //   E1  gates + recurrence of tokens 32-63
@@ -854,9 +854,9 @@ hipError_t launch_block_fused_bf16(const FusedArgs& a, hipStream_t s) {
   // (checked by the caller)
   const int64_t blocks = (int64_t)a.B * a.H;
   if (blocks <= 0 || blocks > 0x7fffffff) return hipErrorInvalidValue;
-  hipError_t e = hipFuncSetAttribute(
-      (const void*)block_fused_bf16_kernel,
-      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFusedLdsBytes);
+  static OncePerDevice once;
+  hipError_t e = set_max_dynamic_lds(
+      once, (const void*)block_fused_bf16_kernel, kFusedLdsBytes);
   if (e != hipSuccess) return e;
   block_fused_bf16_kernel<<<dim3((unsigned)blocks), 512, kFusedLdsBytes, s>>>(a);
   return hipGetLastError();

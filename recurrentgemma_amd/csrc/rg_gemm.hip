@@ -533,15 +533,15 @@ hipError_t launch_gemm_mfma_bf16(const GemmArgs& a, hipStream_t s) {
   dim3 grid((unsigned)per_head, (unsigned)a.H);
   hipError_t e;
   if (a.apply_conv) {
-    e = hipFuncSetAttribute((const void*)gates_mfma_bf16_kernel<true>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)kMfmaLdsBytes);
+    static OncePerDevice once;
+    e = set_max_dynamic_lds(once, (const void*)gates_mfma_bf16_kernel<true>,
+                            kMfmaLdsBytes);
     if (e != hipSuccess) return e;
     gates_mfma_bf16_kernel<true><<<grid, 512, kMfmaLdsBytes, s>>>(a);
   } else {
-    e = hipFuncSetAttribute((const void*)gates_mfma_bf16_kernel<false>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)kMfmaLdsBytes);
+    static OncePerDevice once;
+    e = set_max_dynamic_lds(once, (const void*)gates_mfma_bf16_kernel<false>,
+                            kMfmaLdsBytes);
     if (e != hipSuccess) return e;
     gates_mfma_bf16_kernel<false><<<grid, 512, kMfmaLdsBytes, s>>>(a);
   }

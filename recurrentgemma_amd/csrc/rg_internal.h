@@ -6,7 +6,30 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace rg {
+
+// Raises a kernel's dynamic LDS limit the first time it is launched on a
+// device; later launches on that device only read the flag (the attribute is a
+// property of the loaded function, it does not have to be set per launch).
+struct OncePerDevice {
+  std::atomic<uint64_t> done{0};  // bit d: set on device d (d < 64)
+};
+inline hipError_t set_max_dynamic_lds(OncePerDevice& once, const void* fn,
+                                      size_t bytes) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (dev < 64 && (once.done.load(std::memory_order_acquire) & bit))
+    return hipSuccess;
+  e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                          (int)bytes);
+  if (e == hipSuccess && dev < 64)
+    once.done.fetch_or(bit, std::memory_order_release);
+  return e;
+}
 
 struct ConvArgs {
   const void* x;

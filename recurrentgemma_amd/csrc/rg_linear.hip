@@ -302,9 +302,9 @@ linear_pack_kernel(const uint16_t* __restrict__ w, u32x4* __restrict__ packed,
 template <int NT, int MODE>
 hipError_t launch_rows(const LinearArgs& a, dim3 grid, hipStream_t s) {
   constexpr int lds = kWaves * wave_lds_bytes(NT);
-  hipError_t e =
-      hipFuncSetAttribute((const void*)linear_rows_kernel<NT, MODE>,
-                          hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+  static OncePerDevice once;  // one per instantiation of this launcher
+  hipError_t e = set_max_dynamic_lds(
+      once, (const void*)linear_rows_kernel<NT, MODE>, lds);
   if (e != hipSuccess) return e;
   linear_rows_kernel<NT, MODE><<<grid, kWaves * 64, lds, s>>>(a);
   return hipGetLastError();

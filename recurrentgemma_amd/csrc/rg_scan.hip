@@ -740,9 +740,13 @@ hipError_t launch_t(const ScanArgs& a, hipStream_t s) {
     return hipErrorInvalidValue;
   const size_t lds = sizeof(float) * (2 * nw * kWave * 2 * CH + 2 * kWave * CH);
   auto kern = lru_scan_kernel<T, CH, KL, CONV, FAST, PLAIN, SPLIT>;
-  if (lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(
-        (const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  // the limit is raised once, to what the largest workgroup of this
+  // instantiation needs
+  constexpr size_t lds_max =
+      sizeof(float) * (2 * kMaxNW * kWave * 2 * CH + 2 * kWave * CH);
+  if (lds_max > 48 * 1024) {
+    static OncePerDevice once;  // one per instantiation of this launcher
+    hipError_t e = set_max_dynamic_lds(once, (const void*)kern, lds_max);
     if (e != hipSuccess) return e;
   }
   kern<<<dim3((unsigned)blocks, (unsigned)chunks), dim3(nw * kWave), lds, s>>>(

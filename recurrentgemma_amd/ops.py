@@ -21,12 +21,21 @@ def _dtype_code(t: torch.Tensor) -> int:
   return _DTYPES[t.dtype]
 
 
-def _dev(t: torch.Tensor, name: str) -> torch.Tensor:
-  """Contiguous, 16-byte aligned, on a GPU; raises instead of computing on CPU."""
+def _dev(t: torch.Tensor, name: str, in_place: bool = False) -> torch.Tensor:
+  """Contiguous, 16-byte aligned, on a GPU; raises instead of computing on CPU.
+
+  A tensor that is not contiguous or not aligned is copied -- unless the call
+  updates it in place (in_place): the kernel would then write to the copy and
+  the caller's tensor would go stale, so that case raises."""
   if not t.is_cuda:
     raise RuntimeError(
         f"{name} is on {t.device}: recurrentgemma_amd runs on the GPU only "
         "(there is no CPU fallback)")
+  if in_place:
+    if not t.is_contiguous() or t.data_ptr() % 16:
+      raise ValueError(f"{name} must be a contiguous, 16-byte aligned GPU "
+                       "tensor (it is updated in place)")
+    return t
   t = t.contiguous()
   if t.data_ptr() % 16:
     t = t.clone(memory_format=torch.contiguous_format)
@@ -268,18 +277,12 @@ def linear_scan(x, a, reset, h0=None, split=True):
   return y, h_last
 
 
-_workspaces = {}
-
-
 def _workspace(B, W, dtype, device):
-  key = (B, W, dtype, device)
-  ws = _workspaces.get(key)
-  if ws is None:
-    n = _lib.lib().rg_recurrent_step_workspace_bytes(B, W, _DTYPES[dtype])
-    ws = torch.empty(n, dtype=torch.uint8, device=device)
-    _workspaces.clear()  # keep one workspace alive at a time
-    _workspaces[key] = ws
-  return ws
+  """Scratch of one rg_recurrent_step call, allocated per call: under graph
+  capture it then comes from the graph's own pool and stays valid for the
+  replays, and calls on different streams do not share it."""
+  n = _lib.lib().rg_recurrent_step_workspace_bytes(B, W, _DTYPES[dtype])
+  return torch.empty(n, dtype=torch.uint8, device=device)
 
 
 def gelu_mul(a, g):
@@ -665,8 +668,12 @@ def recurrent_step(x, segment_pos, conv_cache, h, conv_w, conv_b, w_x, b_x, w_a,
   x = _dev(x, "x")
   _same(x.dtype, x.device, conv_w=conv_w, conv_b=conv_b, w_x=w_x, b_x=b_x,
         w_a=w_a, b_a=b_a, a_param=a_param)
-  cache_in = _dev(conv_cache.to(x.dtype), "conv_cache")
-  h_in = _dev(h, "h")
+  if in_place and conv_cache.dtype != x.dtype:
+    raise ValueError(
+        f"in-place decode needs a conv state in the activation dtype "
+        f"{x.dtype}, got {conv_cache.dtype}")
+  cache_in = _dev(conv_cache.to(x.dtype), "conv_cache", in_place)
+  h_in = _dev(h, "h", in_place)
   seg, is64 = _segpos(segment_pos, B, 1)
   args = [_dev(t, n) for t, n in ((conv_w, "conv_w"), (conv_b, "conv_b"),
                                   (w_x, "w_x"), (b_x, "b_x"), (w_a, "w_a"),

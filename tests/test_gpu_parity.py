@@ -833,3 +833,194 @@ def test_config3_full_size_properties():
   seg = torch.arange(T).expand(B, T).contiguous()
   _announce("config3 full size")
   _full_size_properties(B, T, W, H, seg, seed=1103)
+
+
+# ------------------------------------------------- config 4 at full size --
+
+
+def test_config4_full_size_decode():
+  """Benchmark configuration 4 at its full shape: B256 W4096 H16 bf16, a
+  2048-token prefill through recurrent_core, then 64 chained single-token
+  steps.  Every step: single launch == three-launch form bit for bit (8 row
+  tiles x 16 heads, the grid of this shape); at the end: the state and the
+  last y equal those of one prefill over all 2112 tokens up to the fp32
+  association of the recurrence; a few rows against the oracle end to end."""
+  from recurrentgemma_amd import _lib
+  B, T, W, H, steps = 256, 2048, 4096, 16, 64
+  dtype = torch.bfloat16
+  p = R.make_params(W, H, dtype, seed=1104 + 100)
+  P = {k: _dev(v) for k, v in p.items()}
+  blk = _block(p, W, H, dtype)
+  g = torch.Generator().manual_seed(1104)
+  x = torch.randn(B, T + steps, W, generator=g).to(dtype)
+  xd = _dev(x)
+  seg = torch.arange(T + steps).expand(B, -1).contiguous()
+  segd = _dev(seg)
+  _announce("config4 full size: prefill")
+  y, cache = rg.recurrent_core(blk.conv_1d, blk.rg_lru,
+                               xd[:, :T].contiguous(),
+                               segd[:, :T].contiguous())
+  lib = _lib.lib()
+  ws = torch.empty(lib.rg_recurrent_step_workspace_bytes(B, W, 1),
+                   dtype=torch.uint8, device=DEV)
+  ptr = lambda t: t.data_ptr()
+  h3, cc3 = cache.rg_lru_state.clone(), cache.conv1d_state.clone()
+  ys = []
+  for i in range(steps):
+    if i % 16 == 0:
+      _announce("config4 full size: step", i)
+    xi = xd[:, T + i:T + i + 1].contiguous()
+    pos = segd[:, T + i:T + i + 1].contiguous()
+    y1, cache = rg.recurrent_core(blk.conv_1d, blk.rg_lru, xi, pos, cache)
+    y3 = torch.empty_like(xi)
+    h3n, cc3n = torch.empty_like(h3), torch.empty_like(cc3)
+    _lib.check(lib.rg_recurrent_step(
+        ptr(xi), ptr(pos), 1, ptr(cc3), ptr(cc3n), ptr(h3), ptr(h3n),
+        ptr(P["conv_w"]), ptr(P["conv_b"]), ptr(P["w_x"]), ptr(P["b_x"]),
+        ptr(P["w_a"]), ptr(P["b_a"]), ptr(P["a_param"]), ptr(y3), ptr(ws),
+        ws.numel(), B, W, H, 1, torch.cuda.current_stream().cuda_stream))
+    h3, cc3 = h3n, cc3n
+    assert torch.equal(y1, y3), i
+    assert torch.equal(cache.rg_lru_state, h3), i
+    assert torch.equal(cache.conv1d_state, cc3), i
+    ys.append(y1)
+  _announce("config4 full size: one prefill over all tokens")
+  y_full, c_full = rg.recurrent_core(blk.conv_1d, blk.rg_lru, xd, segd)
+  torch.cuda.synchronize()
+  assert helpers.max_rel(cache.rg_lru_state, c_full.rg_lru_state) < 1e-4
+  assert torch.equal(cache.conv1d_state, c_full.conv1d_state)
+  y_steps = torch.cat(ys, dim=1)
+  d = (y_steps.float() - y_full[:, T:].float()).abs()
+  assert d.max().item() <= 0.0625
+  assert (y_steps != y_full[:, T:]).float().mean().item() < 2e-3
+  # oracle, end to end, on three rows (prefill + 64 steps)
+  rows = [0, 131, 255]
+  xo, sego = x[rows], seg[rows]
+  yo, co = R.widened_recurrent_core(xo[:, :T], sego[:, :T], p)
+  assert helpers.max_rel(y[rows], yo) < BF16_TOL
+  for i in range(steps):
+    yo, co = R.widened_recurrent_core(xo[:, T + i:T + i + 1],
+                                      sego[:, T + i:T + i + 1], p, co)
+    assert helpers.max_rel(ys[i][rows], yo) < BF16_TOL, i
+  assert helpers.max_rel(cache.rg_lru_state[rows], co.rg_lru_state) < BF16_TOL
+  assert torch.equal(cache.conv1d_state[rows].cpu(), co.conv1d_state)
+
+
+# ------------------------------------ repeated launches are bit-identical --
+
+
+@pytest.mark.parametrize("B,T,W,H,mean_doc", [
+    (40, 512, 1024, 4, None),    # 160 workgroups, full tiles
+    (9, 1000, 512, 2, 120),      # ragged last tile, document starts
+    (300, 70, 256, 1, 20),       # more workgroups than CUs, short rows
+])
+def test_repeated_launches_are_bit_identical(B, T, W, H, mean_doc):
+  """200 launches each of rg_recurrent_prefill and rg_gates_gemm on the same
+  inputs give the same bits every time.  Regression test for 16-byte buffer
+  stores whose data registers were overwritten by the next vector instruction
+  before the store had read them (0-64 wrong elements per launch, not
+  deterministic): every such store goes through buffer_store_16() now."""
+  _announce("repeat launches", B, T, W, H, mean_doc)
+  seed = 9100 + B
+  p = R.make_params(W, H, torch.bfloat16, seed=seed, gate_bias_std=0.5)
+  P = {k: _dev(v) for k, v in p.items()}
+  g = torch.Generator().manual_seed(seed + 1)
+  x = _dev(torch.randn(B, T, W, generator=g).to(torch.bfloat16))
+  seg = (torch.arange(T).expand(B, T).contiguous() if mean_doc is None
+         else helpers.document_positions(B, T, mean_doc, seed=seed))
+  seg = _dev(seg)
+
+  def prefill():
+    return ops.recurrent_prefill(x, seg, P["conv_w"], P["conv_b"], P["w_x"],
+                                 P["b_x"], P["w_a"], P["b_a"], P["a_param"])
+
+  def gemm():
+    return ops.gates_gemm(x, P["w_x"], P["b_x"], P["w_a"], P["b_a"],
+                          conv=(seg, P["conv_w"], P["conv_b"]))
+
+  for fn in (prefill, gemm):
+    first = fn()
+    bad = torch.zeros((), dtype=torch.int64, device=DEV)
+    for _ in range(200):
+      out = fn()
+      for a, b in zip(out, first):
+        bad += (a != b).sum()
+    torch.cuda.synchronize()
+    assert bad.item() == 0, (fn.__name__, bad.item())
+
+
+# ------------------------------------------- scratch of the decode step --
+
+
+def test_step_scratch_survives_other_shapes_under_graph():
+  """The three-launch decode step (fp32, or heads that are not 256 wide)
+  exchanges its intermediates through scratch memory.  A captured step keeps
+  that memory's address: an eager step of another shape in between must not
+  take it away.  Capture at one shape, run eager steps of other shapes, replay,
+  and compare every replay with the same step run eagerly, bit for bit."""
+  W, H = 256, 2
+  dtype = torch.float32
+  p = R.make_params(W, H, dtype, seed=123, gate_bias_std=0.5)
+  P = {k: _dev(v) for k, v in p.items()}
+  g = torch.Generator().manual_seed(124)
+
+  def make(B, Wd):
+    return (_dev(torch.randn(B, 1, Wd, generator=g)),
+            _dev(torch.full((B, 1), 5, dtype=torch.int64)),
+            _dev(torch.randn(B, 3, Wd, generator=g)),
+            _dev(torch.randn(B, Wd, generator=g)))
+
+  def step(x, seg, cc, h, prm=P, in_place=True):
+    return ops.recurrent_step(x, seg, cc, h, prm["conv_w"], prm["conv_b"],
+                              prm["w_x"], prm["b_x"], prm["w_a"], prm["b_a"],
+                              prm["a_param"], in_place=in_place)
+
+  x, seg, cc_g, h_g = make(3, W)
+  cc_e, h_e = cc_g.clone(), h_g.clone()
+  side = torch.cuda.Stream()
+  side.wait_stream(torch.cuda.current_stream())
+  with torch.cuda.stream(side):
+    step(x, seg, cc_g.clone(), h_g.clone())  # warm-up off the capture
+  torch.cuda.current_stream().wait_stream(side)
+  torch.cuda.synchronize()
+  graph = torch.cuda.CUDAGraph()
+  with torch.cuda.graph(graph):
+    y_g, _, _ = step(x, seg, cc_g, h_g)
+  W2, H2 = 512, 4
+  P2 = {k: _dev(v) for k, v in
+        R.make_params(W2, H2, dtype, seed=125, gate_bias_std=0.5).items()}
+  for i in range(3):
+    # eager steps of other shapes: their scratch must be other memory
+    junk = [step(*make(7 + i, W2), prm=P2, in_place=False) for _ in range(2)]
+    x.copy_(torch.randn(3, 1, W, generator=g))
+    torch.cuda.synchronize()
+    graph.replay()
+    y_e, h_e, cc_e = step(x, seg, cc_e, h_e)
+    torch.cuda.synchronize()
+    assert torch.equal(y_g, y_e), i
+    assert torch.equal(h_g, h_e) and torch.equal(cc_g, cc_e), i
+    del junk
+
+
+def test_in_place_step_refuses_tensors_it_would_have_to_copy():
+  """An in-place decode step on a misaligned or non-contiguous cache tensor
+  would update a private copy: it raises instead."""
+  B, W, H = 4, 256, 1
+  p = {k: _dev(v) for k, v in
+       R.make_params(W, H, torch.bfloat16, seed=3).items()}
+  x = _dev(torch.zeros(B, 1, W, dtype=torch.bfloat16))
+  seg = _dev(torch.full((B, 1), 3, dtype=torch.int64))
+  cc = _dev(torch.zeros(B, 3, W, dtype=torch.bfloat16))
+  h_odd = _dev(torch.zeros(B * W + 1))[1:].view(B, W)  # 4-byte aligned only
+  args = (p["conv_w"], p["conv_b"], p["w_x"], p["b_x"], p["w_a"], p["b_a"],
+          p["a_param"])
+  with pytest.raises(ValueError):
+    ops.recurrent_step(x, seg, cc, h_odd, *args, in_place=True)
+  cc_t = _dev(torch.zeros(3, B, W, dtype=torch.bfloat16)).transpose(0, 1)
+  h = _dev(torch.zeros(B, W))
+  with pytest.raises(ValueError):
+    ops.recurrent_step(x, seg, cc_t, h, *args, in_place=True)
+  with pytest.raises(ValueError):  # a conv state that needs a dtype cast
+    ops.recurrent_step(x, seg, cc.float(), h, *args, in_place=True)
+  y, h2, cc2 = ops.recurrent_step(x, seg, cc, h, *args, in_place=True)
+  assert h2.data_ptr() == h.data_ptr() and cc2.data_ptr() == cc.data_ptr()
