@@ -191,6 +191,31 @@ int rg_recurrent_step(const void* x, const void* segpos, int segpos_is_i64,
                       void* y, void* workspace, size_t workspace_bytes, int B,
                       int W, int H, int dtype, void* stream);
 
+/* rg_recurrent_step without a workspace argument and without any allocation.
+ * It has no counterpart in the reference: it is for callers that cannot
+ * allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  The three launches of rg_recurrent_step
+ * (conv step, gate projections, scan step) exchange the conv output and the
+ * two gate pre-activations through a buffer of RG_STEP_STATIC_SCRATCH_BYTES
+ * that is part of the library's code object: every GPU the library runs on
+ * holds one copy until the process ends.  Shapes whose
+ * rg_recurrent_step_workspace_bytes(B, W, dtype) exceeds that size are
+ * rejected with RG_ERR_WORKSPACE.  Every call on a GPU uses that GPU's one
+ * buffer: calls that overlap on one GPU (two streams, two threads) race;
+ * calls in stream order do not, and nothing is carried from one call to the
+ * next.  The buffer's address is looked up on the first call on each device
+ * (hipGetSymbolAddress); make that call outside a graph capture.  All other
+ * arguments and results are those of rg_recurrent_step. */
+#define RG_STEP_STATIC_SCRATCH_BYTES (8u << 20)
+int rg_recurrent_step_static(const void* x, const void* segpos,
+                             int segpos_is_i64, const void* conv_cache_in,
+                             void* conv_cache_out, const void* h_in,
+                             void* h_out, const void* conv_w,
+                             const void* conv_b, const void* w_x,
+                             const void* b_x, const void* w_a, const void* b_a,
+                             const void* a_param, void* y, int B, int W, int H,
+                             int dtype, void* stream);
+
 /* The join of RecurrentBlock.forward's two branches in one pass:
  * out = a * gelu(g) with the tanh approximation, for recurrentgemma/torch/
  * modules.py:627-628 (`y = gelu(linear_y(x))`, gelu at :289-291) and :644

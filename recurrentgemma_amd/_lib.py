@@ -17,6 +17,7 @@ CSRC = os.path.join(_HERE, "csrc")
 RG_OK = 0
 RG_DTYPE_F32 = 0
 RG_DTYPE_BF16 = 1
+RG_STEP_STATIC_SCRATCH_BYTES = 8 << 20
 ABI_VERSION = 1
 
 _vp = ctypes.c_void_p
@@ -47,6 +48,9 @@ SIGNATURES = {
     "rg_linear_scan_split": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i,
                                   _i, _i, _i, _vp]),
     "rg_recurrent_step_workspace_bytes": (_sz, [_i, _i, _i]),
+    "rg_recurrent_step_static": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp,
+                                      _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i,
+                                      _i, _vp]),
     "rg_gelu_mul": (_i, [_vp, _vp, _vp, ctypes.c_int64, _i, _vp]),
     "rg_rms_norm": (_i, [_vp, _vp, _vp, ctypes.c_int64, _i, ctypes.c_float, _i,
                          _vp]),

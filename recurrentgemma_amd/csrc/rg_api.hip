@@ -2,6 +2,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <mutex>
+
 #include "../../include/rg_lru.h"
 #include "rg_internal.h"
 
@@ -20,6 +22,35 @@ int fail(int code, const char* fmt, ...) {
 int launch_status(const char* what, hipError_t e) {
   if (e == hipSuccess) return RG_OK;
   return fail(RG_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+}
+
+// Scratch of rg_recurrent_step_static: lives in the code object, one copy per
+// GPU the library is loaded on, for as long as the process runs.  In host code
+// the array's name is only a handle for hipGetSymbolAddress; kernels and
+// copies get the per-device address kept in g_step_scratch.
+static __device__ __align__(256) unsigned char scratch[RG_STEP_STATIC_SCRATCH_BYTES];
+constexpr int kMaxDevices = 64;
+void* g_step_scratch[kMaxDevices];  // device id -> address of its `scratch`
+std::mutex g_step_scratch_mutex;
+
+// The calling thread's current device's copy of `scratch` (looked up once per
+// device), or null with *err set.
+void* step_scratch(hipError_t* err) {
+  int dev = 0;
+  *err = hipGetDevice(&dev);
+  if (*err != hipSuccess) return nullptr;
+  if (dev < 0 || dev >= kMaxDevices) {
+    *err = hipErrorInvalidDevice;
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_step_scratch_mutex);
+  if (g_step_scratch[dev] == nullptr) {
+    void* ptr = nullptr;
+    *err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (*err != hipSuccess) return nullptr;
+    g_step_scratch[dev] = ptr;
+  }
+  return g_step_scratch[dev];
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -448,6 +479,35 @@ int rg_recurrent_step(const void* x, const void* segpos, int segpos_is_i64,
   return rg_lru_scan_fused(xc, 0, nullptr, nullptr, gx, ga, a_param, segpos,
                            segpos_is_i64, h_in, y, h_out, nullptr, B, 1, W,
                            dtype, stream);
+}
+
+int rg_recurrent_step_static(const void* x, const void* segpos,
+                             int segpos_is_i64, const void* conv_cache_in,
+                             void* conv_cache_out, const void* h_in,
+                             void* h_out, const void* conv_w,
+                             const void* conv_b, const void* w_x,
+                             const void* b_x, const void* w_a, const void* b_a,
+                             const void* a_param, void* y, int B, int W, int H,
+                             int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(B > 0 && W > 0 && H > 0, "%s: B=%d W=%d H=%d must be positive",
+             __func__, B, W, H);
+  const size_t need = rg_recurrent_step_workspace_bytes(B, W, dtype);
+  if (need > (size_t)RG_STEP_STATIC_SCRATCH_BYTES)
+    return fail(RG_ERR_WORKSPACE,
+                "%s: B=%d W=%d needs %zu bytes of scratch, the built-in buffer "
+                "holds %zu: use rg_recurrent_step with a workspace",
+                __func__, B, W, need, (size_t)RG_STEP_STATIC_SCRATCH_BYTES);
+  hipError_t e;
+  void* ws = step_scratch(&e);
+  if (ws == nullptr) return launch_status(__func__, e);
+  // the three launches write every scratch element they later read: nothing
+  // has to be cleared between calls
+  return rg_recurrent_step(x, segpos, segpos_is_i64, conv_cache_in,
+                           conv_cache_out, h_in, h_out, conv_w, conv_b, w_x,
+                           b_x, w_a, b_a, a_param, y, ws,
+                           (size_t)RG_STEP_STATIC_SCRATCH_BYTES, B, W, H, dtype,
+                           stream);
 }
 
 int rg_gelu_mul(const void* a, const void* g, void* out, int64_t n, int dtype,
