@@ -176,6 +176,30 @@ int rg_recurrent_prefill(const void* x, const void* segpos, int segpos_is_i64,
                          void* h_last, void* conv_cache_out, int B, int T,
                          int W, int H, int dtype, void* stream);
 
+/* rg_recurrent_prefill for few (row, head) pairs: one workgroup per pair
+ * leaves most of the GPU idle below 256 pairs, so the sequences are cut into
+ * chunks of whole 64-token tiles that run as workgroups of their own.  Pass 1
+ * runs every chunk but the last from a zero state and keeps (prod a_t, h_end)
+ * per chunk and channel, a small kernel chains them into every chunk's
+ * incoming state (h_in[k+1] = P[k] h_in[k] + H[k]: the scan operator of
+ * recurrentgemma/jax/scan.py:161-187, the algebra of multi_shard_correction,
+ * jax/pallas.py:73-195, across workgroups instead of devices), pass 2 runs
+ * every chunk from its incoming state and writes y.  `workspace` must hold
+ * rg_recurrent_prefill_split_workspace_bytes(B, T, W, H) bytes; that is 0 for
+ * shapes that are not cut, where the call is rg_recurrent_prefill itself.
+ * Results equal rg_recurrent_prefill's up to the float32 association of the
+ * recurrence across chunk boundaries. */
+size_t rg_recurrent_prefill_split_workspace_bytes(int B, int T, int W, int H);
+int rg_recurrent_prefill_split(const void* x, const void* segpos,
+                               int segpos_is_i64, const void* conv_w,
+                               const void* conv_b, const void* w_x,
+                               const void* b_x, const void* w_a,
+                               const void* b_a, const void* w_packed,
+                               const void* a_param, const void* h0, void* y,
+                               void* h_last, void* conv_cache_out,
+                               void* workspace, size_t workspace_bytes, int B,
+                               int T, int W, int H, int dtype, void* stream);
+
 /* One decode step of the conv -> RG-LRU core, as RecurrentBlock.forward chains
  * them with a cache (recurrentgemma/torch/modules.py:632-643 with
  * layers.py:469-474 and :170-177): x [B,1,W], segpos [B,1],

@@ -323,17 +323,31 @@ int rg_lru_scan_fused_split(const void* x, int apply_conv, const void* conv_w,
                              true, B, T, W, dtype, stream);
 }
 
-int rg_recurrent_prefill(const void* x, const void* segpos, int segpos_is_i64,
-                         const void* conv_w, const void* conv_b,
-                         const void* w_x, const void* b_x, const void* w_a,
-                         const void* b_a, const void* w_packed,
-                         const void* a_param, const void* h0, void* y,
-                         void* h_last, void* conv_cache_out, int B, int T,
-                         int W, int H, int dtype, void* stream) {
+size_t rg_recurrent_prefill_split_workspace_bytes(int B, int T, int W, int H) {
+  if (B <= 0 || T <= 0 || W <= 0 || H <= 0 || W % H != 0 || W / H != 256)
+    return 0;
+  int chunks, per;
+  rg::prefill_chunk_plan(B, H, T, &chunks, &per);
+  return chunks > 1 ? (size_t)3 * B * chunks * W * sizeof(float) : 0;
+}
+
+#undef RG_WHO
+#define RG_WHO who
+static int recurrent_prefill_impl(const char* who, const void* x,
+                                  const void* segpos, int segpos_is_i64,
+                                  const void* conv_w, const void* conv_b,
+                                  const void* w_x, const void* b_x,
+                                  const void* w_a, const void* b_a,
+                                  const void* w_packed, const void* a_param,
+                                  const void* h0, void* y, void* h_last,
+                                  void* conv_cache_out, void* workspace,
+                                  size_t workspace_bytes, bool split, int B,
+                                  int T, int W, int H, int dtype,
+                                  void* stream) {
   RG_CHECK_DTYPE(dtype);
   RG_REQUIRE(B > 0 && T > 0 && W > 0 && H > 0,
-             "%s: B=%d T=%d W=%d H=%d must be positive", __func__, B, T, W, H);
-  RG_REQUIRE(W % H == 0, "%s: W=%d is not a multiple of H=%d", __func__, W, H);
+             "%s: B=%d T=%d W=%d H=%d must be positive", who, B, T, W, H);
+  RG_REQUIRE(W % H == 0, "%s: W=%d is not a multiple of H=%d", who, W, H);
   RG_CHECK_PTR(x);
   RG_CHECK_PTR(segpos);
   RG_CHECK_PTR(conv_w);
@@ -348,7 +362,7 @@ int rg_recurrent_prefill(const void* x, const void* segpos, int segpos_is_i64,
   RG_CHECK_OPT_PTR(h0);
   RG_CHECK_OPT_PTR(h_last);
   RG_CHECK_OPT_PTR(conv_cache_out);
-  RG_REQUIRE(y != x, "%s: y must not alias x", __func__);
+  RG_REQUIRE(y != x, "%s: y must not alias x", who);
   // The single-launch kernel exists for bf16 with 256-wide heads and
   // sequences whose byte offsets fit 31 bits; everything else is served by
   // rg_gates_gemm + rg_lru_scan_fused.
@@ -357,7 +371,7 @@ int rg_recurrent_prefill(const void* x, const void* segpos, int segpos_is_i64,
     return fail(RG_ERR_UNSUPPORTED,
                 "%s: unsupported shape or dtype (needs bf16, W/H == 256, "
                 "T*W*2 < 2^31): dtype=%d W=%d H=%d T=%d",
-                __func__, dtype, W, H, T);
+                who, dtype, W, H, T);
   }
   rg::FusedArgs a{};
   a.x = x;
@@ -379,8 +393,56 @@ int rg_recurrent_prefill(const void* x, const void* segpos, int segpos_is_i64,
   a.T = T;
   a.W = W;
   a.H = H;
-  return launch_status(__func__,
-                       rg::launch_block_fused_bf16(a, (hipStream_t)stream));
+  a.chunks = 1;
+  a.tiles_per_chunk = (T + 63) / 64;
+  if (split) {
+    const size_t need = rg_recurrent_prefill_split_workspace_bytes(B, T, W, H);
+    if (need > 0) {
+      if (workspace == nullptr || workspace_bytes < need ||
+          !aligned16(workspace))
+        return fail(RG_ERR_WORKSPACE,
+                    "%s: workspace of %zu bytes (16-byte aligned) required, "
+                    "got %zu", who, need, workspace ? workspace_bytes : (size_t)0);
+      rg::prefill_chunk_plan(B, H, T, &a.chunks, &a.tiles_per_chunk);
+      const size_t one = (size_t)B * a.chunks * W;
+      a.ws_p = (float*)workspace;
+      a.ws_h = a.ws_p + one;
+      a.ws_h_in = a.ws_h + one;
+    }
+  }
+  return launch_status(who,
+                       rg::launch_block_prefill_bf16(a, (hipStream_t)stream));
+}
+#undef RG_WHO
+#define RG_WHO __func__
+
+int rg_recurrent_prefill(const void* x, const void* segpos, int segpos_is_i64,
+                         const void* conv_w, const void* conv_b,
+                         const void* w_x, const void* b_x, const void* w_a,
+                         const void* b_a, const void* w_packed,
+                         const void* a_param, const void* h0, void* y,
+                         void* h_last, void* conv_cache_out, int B, int T,
+                         int W, int H, int dtype, void* stream) {
+  return recurrent_prefill_impl(__func__, x, segpos, segpos_is_i64, conv_w,
+                                conv_b, w_x, b_x, w_a, b_a, w_packed, a_param,
+                                h0, y, h_last, conv_cache_out, nullptr, 0,
+                                false, B, T, W, H, dtype, stream);
+}
+
+int rg_recurrent_prefill_split(const void* x, const void* segpos,
+                               int segpos_is_i64, const void* conv_w,
+                               const void* conv_b, const void* w_x,
+                               const void* b_x, const void* w_a,
+                               const void* b_a, const void* w_packed,
+                               const void* a_param, const void* h0, void* y,
+                               void* h_last, void* conv_cache_out,
+                               void* workspace, size_t workspace_bytes, int B,
+                               int T, int W, int H, int dtype, void* stream) {
+  return recurrent_prefill_impl(__func__, x, segpos, segpos_is_i64, conv_w,
+                                conv_b, w_x, b_x, w_a, b_a, w_packed, a_param,
+                                h0, y, h_last, conv_cache_out, workspace,
+                                workspace_bytes, true, B, T, W, H, dtype,
+                                stream);
 }
 
 #undef RG_WHO

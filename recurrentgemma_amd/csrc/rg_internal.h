@@ -108,6 +108,14 @@ struct FusedArgs {
   float* h_last;       // [B, W] or null
   void* cache_out;     // [B, 3, W] or null
   int B, T, W, H;
+  // sequences cut into `chunks` chunks of tiles_per_chunk 64-token tiles
+  // (chunks <= 1: not cut), with three [B][chunks][W] float rows of
+  // workspace: every chunk's product of a_t, its state from a zero start, its
+  // incoming state
+  int chunks, tiles_per_chunk;
+  float* ws_p;
+  float* ws_h;
+  float* ws_h_in;
 };
 
 struct StepArgs {
@@ -145,7 +153,8 @@ hipError_t launch_gemm_generic(const GemmArgs& a, int dtype, hipStream_t s);
 hipError_t launch_gemm_mfma_bf16(const GemmArgs& a, hipStream_t s);
 hipError_t launch_lru_scan(const ScanArgs& a, int dtype, hipStream_t s);
 void scan_split_plan(int B, int T, int W, int* chunks, int* t_chunk);
-hipError_t launch_block_fused_bf16(const FusedArgs& a, hipStream_t s);
+hipError_t launch_block_prefill_bf16(const FusedArgs& a, hipStream_t s);
+void prefill_chunk_plan(int B, int H, int T, int* chunks, int* tiles_per_chunk);
 hipError_t launch_block_step_bf16(const StepArgs& a, hipStream_t s);
 // bf16 [H,256,256] x 2 -> one buffer of the same total size in MFMA operand
 // order (head, wave, k-step, gate, lane, 8 values).

@@ -35,8 +35,20 @@ def gelu(x: torch.Tensor) -> torch.Tensor:
 # does not shrink below 256 groups, while the two-kernel form scales with the
 # number of tokens.  Measured on MI355X (T = 1024 and 4096, 256-wide heads) the
 # two cross between 128 groups (two kernels 5 % ahead) and 160 (single launch
-# 25 % ahead).
+# 25 % ahead).  With few groups and long rows the sequences are cut into
+# chunks that run as workgroups of their own (rg_recurrent_prefill_split).
 _MIN_GROUPS_FOR_SINGLE_LAUNCH = 144
+
+
+def _single_launch_pays(x, num_heads) -> bool:
+  """Whether prefill goes to the single-launch kernel (whole rows or rows cut
+  into chunks) rather than to the gate GEMM + scan kernel pair."""
+  if not ops.recurrent_prefill_supported(x, num_heads):
+    return False
+  bs, l, w = x.shape
+  if bs * num_heads >= _MIN_GROUPS_FOR_SINGLE_LAUNCH:
+    return True
+  return ops.recurrent_prefill_chunked(bs, l, w, num_heads)
 
 
 @torch.no_grad()
@@ -71,10 +83,10 @@ def recurrent_core(conv_1d: layers.Conv1D, rg_lru: layers.RGLRU, x,
                              return_cache)
     y, h = rg_lru(xc, segment_pos,
                   None if cache is None else cache.rg_lru_state, return_cache)
-  elif (ops.recurrent_prefill_supported(x, rg_lru.num_heads) and
-        bs * rg_lru.num_heads >= _MIN_GROUPS_FOR_SINGLE_LAUNCH):
-    # one workgroup per (row, head): pays once there are enough of them to
-    # fill the GPU; below that the two-kernel form spreads over more CUs
+  elif _single_launch_pays(x, rg_lru.num_heads):
+    # one workgroup per (row, head) -- or per chunk of one -- pays once there
+    # are enough of them to fill the GPU; otherwise the two-kernel form
+    # spreads over more CUs
     y, h, conv_state = ops.recurrent_prefill(
         x, segment_pos, conv_1d.w, conv_1d.b, rg_lru.input_gate.w,
         rg_lru.input_gate.b, rg_lru.a_gate.w, rg_lru.a_gate.b, rg_lru.a_param,

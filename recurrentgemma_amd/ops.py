@@ -214,13 +214,23 @@ def recurrent_prefill_supported(x, num_heads):
           W // num_heads == 256 and T * W * 2 < 2**31 - 1)
 
 
+def recurrent_prefill_chunked(B, T, W, num_heads) -> bool:
+  """Whether rg_recurrent_prefill_split cuts the sequences of this shape into
+  chunks (few (row, head) pairs, long rows)."""
+  return _lib.lib().rg_recurrent_prefill_split_workspace_bytes(
+      B, T, W, num_heads) > 0
+
+
 def recurrent_prefill(x, segment_pos, conv_w, conv_b, w_x, b_x, w_a, b_a,
-                      a_param, h0=None, return_h=True, return_conv_cache=True):
+                      a_param, h0=None, return_h=True, return_conv_cache=True,
+                      split=True):
   """conv -> gates -> recurrence of a whole prefill in one launch.
 
   Returns (y, h_last | None, conv_cache | None).  Only for the shapes
   recurrent_prefill_supported() accepts; other shapes go through gates_gemm +
-  lru_scan_fused.
+  lru_scan_fused.  split: with few (row, head) pairs the sequences are cut
+  into chunks that run side by side (rg_recurrent_prefill_split); False forces
+  one workgroup per pair.
   """
   B, T, W = x.shape
   H = w_x.shape[0]
@@ -245,11 +255,21 @@ def recurrent_prefill(x, segment_pos, conv_w, conv_b, w_x, b_x, w_a, b_a,
   cache = x.new_empty((B, 3, W)) if return_conv_cache else None
   cw, cb, wx_, bx_, wa_, ba_, ap_ = args
   packed = packed_gate_weights(w_x, w_a)  # cached per weight version
+  lib = _lib.lib()
+  need = (lib.rg_recurrent_prefill_split_workspace_bytes(B, T, W, H)
+          if split else 0)
   with torch.cuda.device(x.device):
-    _lib.check(_lib.lib().rg_recurrent_prefill(
-        _p(x), _p(seg), is64, _p(cw), _p(cb), _p(wx_), _p(bx_), _p(wa_),
-        _p(ba_), _p(packed), _p(ap_), _p(h0), _p(y), _p(h_last), _p(cache), B,
-        T, W, H, _dtype_code(x), _stream(x)))
+    if need:
+      ws = torch.empty(need, dtype=torch.uint8, device=x.device)
+      _lib.check(lib.rg_recurrent_prefill_split(
+          _p(x), _p(seg), is64, _p(cw), _p(cb), _p(wx_), _p(bx_), _p(wa_),
+          _p(ba_), _p(packed), _p(ap_), _p(h0), _p(y), _p(h_last), _p(cache),
+          _p(ws), need, B, T, W, H, _dtype_code(x), _stream(x)))
+    else:
+      _lib.check(lib.rg_recurrent_prefill(
+          _p(x), _p(seg), is64, _p(cw), _p(cb), _p(wx_), _p(bx_), _p(wa_),
+          _p(ba_), _p(packed), _p(ap_), _p(h0), _p(y), _p(h_last), _p(cache),
+          B, T, W, H, _dtype_code(x), _stream(x)))
   return y, h_last, cache
 
 

@@ -58,3 +58,19 @@ def max_rel(got, want):
   want = want.detach().double().cpu()
   denom = want.abs().max().item()
   return (got - want).abs().max().item() / max(denom, 1e-30)
+
+
+def assert_close_elementwise(got, want, rtol=1e-2, atol_of_max=2e-3, what=""):
+  """Element by element: |got - want| <= rtol |want| + atol_of_max max|want|
+  (the reference's tests compare with rtol/atol per element,
+  torch/layers_test.py:131; the absolute term is scaled to the tensor so that
+  it stays a small fraction of typical magnitudes).  max_rel() alone would let
+  small elements be wrong by many of their own ulps."""
+  got = got.detach().double().cpu()
+  want = want.detach().double().cpu()
+  bound = rtol * want.abs() + atol_of_max * want.abs().max()
+  excess = (got - want).abs() - bound
+  worst = excess.max().item()
+  assert worst <= 0, (
+      f"{what}: {int((excess > 0).sum())} of {excess.numel()} elements outside "
+      f"rtol={rtol} atol={atol_of_max}*max; worst excess {worst:.3e}")

@@ -460,11 +460,19 @@ def test_recurrent_block_module():
     (1, 130, 256, 1, 3, torch.int64, False),   # documents of a few tokens
     (130, 70, 256, 1, 20, torch.int64, False),  # more workgroups than CUs/2
     (2, 100, 256, 1, -7, torch.int32, False),   # left padding: positions < 0
+    # few (row, head) pairs, long rows: the sequences run as chunks
+    (1, 1000, 512, 2, 200, torch.int64, True),
+    (2, 2048, 256, 1, None, torch.int64, False),
+    (1, 777, 768, 3, 100, torch.int32, True),
+    (3, 1500, 256, 1, 7, torch.int64, False),
 ])
 def test_recurrent_prefill_single_launch(B, T, W, H, mean_doc, seg_dtype,
                                          with_h0):
-  """rg_recurrent_prefill against the oracle (bf16 tolerance) and against the
-  two-kernel form (same arithmetic up to the association of the recurrence)."""
+  """rg_recurrent_prefill(_split) against the oracle (bf16 tolerance, also
+  element by element) and against the two-kernel form.  The single-launch
+  kernel keeps the gate pre-activations in float32 where the two-kernel form
+  rounds them to bf16 on their way through memory (as the reference's modules
+  do), so the two agree to a bf16 ulp or two, not bit for bit."""
   _announce("recurrent_prefill", B, T, W, H, mean_doc, seg_dtype, with_h0)
   seed = 7000 + T
   p = R.make_params(W, H, torch.bfloat16, seed=seed, gate_bias_std=0.5)
@@ -489,16 +497,28 @@ def test_recurrent_prefill_single_launch(B, T, W, H, mean_doc, seg_dtype,
   y2, h2, cache2 = ops.lru_scan_fused(
       xd, gx, ga, P["a_param"], segd, h0=h0d,
       conv=(P["conv_w"], P["conv_b"]), return_conv_cache=True)
-  assert (y != y2).float().mean().item() < 1e-3
-  assert (y.float() - y2.float()).abs().max().item() <= 0.0625
-  assert helpers.max_rel(h, h2) < 1e-5
+  assert helpers.max_rel(y, y2) < BF16_TOL
+  assert helpers.max_rel(h, h2) < BF16_TOL
   assert torch.equal(cache, cache2)
   xc, cc = R.widened_conv1d_forward(x, seg, p["conv_w"], p["conv_b"])
   yo, ho = R.widened_rglru_forward(xc, seg, p["a_param"], p["w_x"], p["b_x"],
                                    p["w_a"], p["b_a"], cache=h0)
   assert helpers.max_rel(y, yo) < BF16_TOL
   assert helpers.max_rel(h, ho) < BF16_TOL
+  helpers.assert_close_elementwise(y, yo, what="y")
+  helpers.assert_close_elementwise(h, ho, what="h")
   assert torch.equal(cache.cpu(), cc)
+  # whole rows and rows cut into chunks: the same arithmetic per token, the
+  # state crosses chunk boundaries in another float32 association
+  y1, h1, cache1 = ops.recurrent_prefill(
+      xd, segd, P["conv_w"], P["conv_b"], P["w_x"], P["b_x"], P["w_a"],
+      P["b_a"], P["a_param"], h0=h0d, split=False)
+  assert torch.equal(cache1, cache)
+  assert helpers.max_rel(h1, h) < 1e-5
+  assert (y1 != y).float().mean().item() < 2e-3
+  assert (y1.float() - y.float()).abs().max().item() <= 0.0625
+  if not ops.recurrent_prefill_chunked(B, T, W, H):
+    assert torch.equal(y1, y) and torch.equal(h1, h)
 
 
 @pytest.mark.parametrize("B,W,H,in_place", [(1, 256, 1, False),
@@ -762,18 +782,22 @@ def _full_size_properties(B, T, W, H, seg, seed):
   y1, h1, c1 = ops.lru_scan_fused(x, gx, ga, blk.rg_lru.a_param, segd,
                                   conv=(blk.conv_1d.w, blk.conv_1d.b),
                                   return_conv_cache=True)
-  assert (y1 != y).float().mean().item() < 1e-3
-  assert (y1.float() - y.float()).abs().max().item() <= 0.0625
-  assert helpers.max_rel(cache.rg_lru_state, h1) < 1e-5
+  # (the single-launch kernel keeps the pre-activations in float32, the
+  # two-kernel form rounds them to bf16: a bf16 ulp or two apart)
+  assert (y1 != y).float().mean().item() < 0.15
+  assert (y1.float() - y.float()).abs().max().item() <= 0.125
+  assert helpers.max_rel(y1, y) < BF16_TOL
+  assert helpers.max_rel(cache.rg_lru_state, h1) < BF16_TOL
   assert torch.equal(c1, cache.conv1d_state)
   if ops.recurrent_prefill_supported(x, H):
     yf, hf, cf = ops.recurrent_prefill(
         x, segd, blk.conv_1d.w, blk.conv_1d.b, blk.rg_lru.input_gate.w,
         blk.rg_lru.input_gate.b, blk.rg_lru.a_gate.w, blk.rg_lru.a_gate.b,
         blk.rg_lru.a_param)
-    assert (y1 != yf).float().mean().item() < 1e-3
-    assert (y1.float() - yf.float()).abs().max().item() <= 0.0625
-    assert helpers.max_rel(hf, h1) < 1e-5
+    assert (y1 != yf).float().mean().item() < 0.15
+    assert (y1.float() - yf.float()).abs().max().item() <= 0.125
+    assert helpers.max_rel(yf, y1) < BF16_TOL
+    assert helpers.max_rel(hf, h1) < BF16_TOL
     assert torch.equal(cf, c1)
   y_core, y = y, y1  # the exact statements below are about the two-kernel form
   cache_core, cache = cache, rg.RecurrentBlockCache(rg_lru_state=h1,
@@ -808,9 +832,9 @@ def _full_size_properties(B, T, W, H, seg, seed):
                                    segd[:1].contiguous())
   # (a one-row launch may use another lane width / step length, i.e. another
   # fp32 association of the carry: equal up to rare 1-ulp bf16 flips)
-  assert (y_row != y[:1]).float().mean().item() < 1e-3
-  assert (y_row.float() - y[:1].float()).abs().max().item() <= 0.0625
-  assert helpers.max_rel(c_row.rg_lru_state, cache.rg_lru_state[:1]) < 1e-5
+  assert (y_row != y[:1]).float().mean().item() < 0.15
+  assert (y_row.float() - y[:1].float()).abs().max().item() <= 0.125
+  assert helpers.max_rel(c_row.rg_lru_state, cache.rg_lru_state[:1]) < BF16_TOL
   assert torch.equal(c_row.conv1d_state, cache.conv1d_state[:1])
   # (6) spot parity against the oracle on one row's first tokens
   n = 300
@@ -887,12 +911,15 @@ def test_config4_full_size_decode():
   _announce("config4 full size: one prefill over all tokens")
   y_full, c_full = rg.recurrent_core(blk.conv_1d, blk.rg_lru, xd, segd)
   torch.cuda.synchronize()
-  assert helpers.max_rel(cache.rg_lru_state, c_full.rg_lru_state) < 1e-4
+  # (the decode step rounds the gate pre-activations to bf16 like the
+  # reference's modules, the prefill kernel keeps them in float32)
+  assert helpers.max_rel(cache.rg_lru_state, c_full.rg_lru_state) < 2e-3
   assert torch.equal(cache.conv1d_state, c_full.conv1d_state)
   y_steps = torch.cat(ys, dim=1)
   d = (y_steps.float() - y_full[:, T:].float()).abs()
-  assert d.max().item() <= 0.0625
-  assert (y_steps != y_full[:, T:]).float().mean().item() < 2e-3
+  assert d.max().item() <= 0.125
+  assert helpers.max_rel(y_steps, y_full[:, T:]) < BF16_TOL
+  assert (y_steps != y_full[:, T:]).float().mean().item() < 0.15
   # oracle, end to end, on three rows (prefill + 64 steps)
   rows = [0, 131, 255]
   xo, sego = x[rows], seg[rows]

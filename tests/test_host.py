@@ -24,7 +24,7 @@ def _declared_symbols():
 
 def test_library_exports_every_declared_symbol():
   names = _declared_symbols()
-  assert len(names) == 33, names
+  assert len(names) == 35, names
   lib = ctypes.CDLL(_lib.LIB_PATH)
   for n in names:
     assert hasattr(lib, n), n
@@ -58,6 +58,19 @@ def test_c_side_validation_without_launch():
   rc = lib.rg_recurrent_step(ok, ok, 1, ok, ok, ok, ok, ok, ok, ok, ok, ok, ok,
                              ok, ok, None, 0, 2, 256, 1, 1, None)
   assert rc == -4 and b"workspace" in lib.rg_last_error()
+  # rows cut into chunks for the single-launch prefill kernel
+  assert lib.rg_recurrent_prefill_split_workspace_bytes(16, 8192, 4096, 16) == 0
+  assert lib.rg_recurrent_prefill_split_workspace_bytes(1, 320, 2560, 10) == 0  # < 6 tiles
+  need = lib.rg_recurrent_prefill_split_workspace_bytes(1, 8192, 2560, 10)
+  assert need > 0 and need % (3 * 2560 * 4) == 0
+  rc = lib.rg_recurrent_prefill_split(ok, ok, 1, ok, ok, ok, ok, ok, ok, None,
+                                      ok, None, y, None, None, None, 0, 1, 8192,
+                                      2560, 10, 1, None)
+  assert rc == -4 and b"workspace" in lib.rg_last_error()
+  rc = lib.rg_recurrent_prefill_split(ok, ok, 1, ok, ok, ok, ok, ok, ok, None,
+                                      ok, None, y, None, None, None, 0, 1, 8192,
+                                      2560, 10, 0, None)
+  assert rc == -2 and b"unsupported" in lib.rg_last_error()
   # the entries added for the whole block
   rc = lib.rg_gelu_mul(ok, ok, ok, 0, 1, None)
   assert rc == -1 and b"positive" in lib.rg_last_error()
