@@ -6,9 +6,11 @@ A "step" is one pass of the hot path (Conv1D -> RG-LRU of the recurrent block)
 over one synthetic batch that is already resident in HBM, called through the C
 ABI on torch's current stream.  Two forms of the path exist (--path):
   single  rg_recurrent_prefill: conv, gate projections (bf16 MFMA), gate
-          arithmetic and recurrence in ONE launch, nothing but x and y moves
-          through HBM (default where one workgroup per row and head fills the
-          GPU)
+          arithmetic and recurrence in ONE kernel, nothing but x and y moves
+          through HBM.  Default where one workgroup per row and head fills the
+          GPU, and where rows are long enough to be cut into time chunks that
+          do (rg_recurrent_prefill_split: a summary pass, a carry pass and a
+          replay pass, x read twice)
   split   rg_gates_gemm (conv on load, both gate projections on bf16 MFMA)
           followed by rg_lru_scan_fused (conv + gates + chunked scan); the gate
           pre-activations go through HBM
@@ -65,13 +67,24 @@ WORKLOADS = {
                               griffin=True),
 }
 
-# HBM bytes per scan launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# (scaled by a copy kernel of known size); None until measured for a workload.
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (scaled
+# by a copy kernel of known size).  These are constants taken from the named
+# summary file, not something a bench run measures: the JSON says so in
+# `traffic_source`.  No entry = not measured for that workload (traffic null).
 MEASURED_TRAFFIC_BYTES = {
-    # profiles/hbm_traffic_9b_prefill.txt
-    ("9b_prefill", "single"): 2.164e9,   # 1.088 GB read + 1.076 GB written
-    ("9b_prefill", "scan"): 4.40e9,      # 3.33 GB read + 1.074 GB written
+    ("9b_prefill", "single"): (2.164e9, "profiles/hbm_traffic_9b_prefill.txt"),
+    ("9b_prefill", "scan"): (4.40e9, "profiles/hbm_traffic_9b_prefill.txt"),
 }
+
+
+def measured_traffic(workload, kernel):
+  """(bytes, source) of the committed counter summary for a kernel, or
+  (None, None)."""
+  return MEASURED_TRAFFIC_BYTES.get((workload, kernel), (None, None))
+
+
+METRIC = ("RG-LRU block tokens/s + scan HBM GB/s (% of roofline) at 2B and 9B "
+          "widths")
 
 
 def single_algorithmic_bytes(B, T, W, H, esize, seg_bytes, has_h0):
@@ -274,7 +287,7 @@ def run_decode(args, torch, rg, R, ops, wl):
   algo = decode_algorithmic_bytes(B, W, H, 2)
   achieved = algo / (dev_ms * 1e-3) / 1e9
   result = {
-      "metric": "RG-LRU block tokens/s + scan HBM GB/s (% of roofline)",
+      "metric": METRIC,
       "value": B / (elapsed / args.steps), "unit": "tokens/s", "n_gpus": 1,
       "steps": args.steps, "warmup": args.warmup,
       "ms_per_step": elapsed * 1e3 / args.steps, "higher_is_better": True,
@@ -356,14 +369,16 @@ def main():
                      max(10, args.steps // 2), 5, extras=False)
     result["at_2b_width"] = {
         k: r2[k] for k in ("value", "unit", "steps", "warmup", "ms_per_step",
-                           "config", "roofline", "gate_gemm")}
+                           "config", "roofline", "gate_gemm",
+                           "two_kernel_path") if k in r2}
   print(json.dumps(result))
 
 
 def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
   """One prefill workload: `warmup` untimed steps, `steps` timed ones; returns
-  the result line as a dict.  extras: also the two-kernel form of a
-  single-launch workload, the calibration copy and the CPU baseline."""
+  the result line as a dict; with the default path also the two-kernel form
+  of a single-kernel workload, after the timed region.  extras: the
+  calibration copy and the CPU baseline too."""
   wl = WORKLOADS[workload]
   B, T, W, H = wl["B"], wl["T"], wl["W"], wl["H"]
   dev = torch.device("cuda:0")
@@ -409,10 +424,13 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
       events[2].record()
     return out
 
+  # the choice RecurrentBlock makes: the single kernel where its workgroups
+  # (one per row, head and time chunk) fill the GPU
+  chunked = esize == 2 and ops.recurrent_prefill_chunked(B, T, W, H)
   path = args.path
   if path == "auto":
-    path = ("single" if ops.recurrent_prefill_supported(x, H) and B * H >= 144
-            else "split")
+    path = ("single" if ops.recurrent_prefill_supported(x, H)
+            and (B * H >= 144 or chunked) else "split")
   step = step_single if path == "single" else step_split
 
   def timed(fn, steps, warmup):
@@ -443,12 +461,13 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
 
   def split_figures(gemm_ms, scan_ms):
     achieved = scan_algo / (scan_ms * 1e-3) / 1e9
+    traffic, source = measured_traffic(workload, "scan")
     return {
         "scan": {
             "kernel": "lru_scan_kernel (conv + gates + scan)",
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
             "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get((workload, "scan")),
+            "traffic": traffic, "traffic_source": source,
             "algorithmic_bytes": scan_algo, "avg_launch_ms": scan_ms},
         "gate_gemm": {
             "kernel": ("gates_mfma_bf16_kernel" if esize == 2
@@ -463,11 +482,15 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
   if path == "single":
     algo = single_algorithmic_bytes(B, T, W, H, 2, seg_bytes, has_h0=False)
     achieved = algo / (first_ms * 1e-3) / 1e9
+    traffic, source = measured_traffic(workload, "single")
     roofline = {
-        "kernel": "block_fused_bf16_kernel (conv + gate GEMMs + gates + scan)",
+        "kernel": ("block_prefill_bf16_kernel (conv + gate GEMMs + gates + scan)"
+                   + (": summary pass over all chunks but the last, carry "
+                      "kernel, replay pass; avg_launch_ms covers the three"
+                      if chunked else "")),
         "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
         "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-        "traffic": MEASURED_TRAFFIC_BYTES.get((workload, "single")),
+        "traffic": traffic, "traffic_source": source,
         "algorithmic_bytes": algo, "avg_launch_ms": first_ms,
         "mfma_tflops": gemm_flops / (first_ms * 1e-3) / 1e12,
         "frac_of_bf16_mfma_peak": gemm_flops / (first_ms * 1e-3) / 2.5e15}
@@ -480,7 +503,7 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
     torch.cuda.synchronize()
 
   result = {
-      "metric": "RG-LRU block tokens/s + scan HBM GB/s (% of roofline)",
+      "metric": METRIC,
       "value": tokens / (elapsed / steps),
       "unit": "tokens/s",
       "n_gpus": 1,
@@ -498,7 +521,10 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
           "state": "f32",
           "documents": ("one per row" if wl["mean_doc"] is None
                         else f"geometric mean {wl['mean_doc']}"),
-          "path": ("rg_recurrent_prefill (single launch)" if path == "single"
+          "path": ("rg_recurrent_prefill_split (single kernel, rows in time "
+                   "chunks side by side)" if path == "single" and chunked
+                   else "rg_recurrent_prefill (single launch)"
+                   if path == "single"
                    else "rg_gates_gemm(conv on load) + "
                         + ("rg_lru_scan_fused_split(conv): sequences in chunks "
                            "side by side" if in_chunks
@@ -507,7 +533,7 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
   }
   if path == "split":
     result["gate_gemm"] = figs["gate_gemm"]
-  elif extras and args.path == "auto":
+  elif args.path == "auto":
     # the two-kernel form of the same step, measured after the timed region
     n2 = max(5, steps // 2)
     e2, g_ms, s_ms = timed(step_split, n2, 3)

@@ -328,7 +328,7 @@ size_t rg_recurrent_prefill_split_workspace_bytes(int B, int T, int W, int H) {
     return 0;
   int chunks, per;
   rg::prefill_chunk_plan(B, H, T, &chunks, &per);
-  return chunks > 1 ? (size_t)3 * B * chunks * W * sizeof(float) : 0;
+  return chunks > 1 ? (size_t)2 * B * chunks * W * sizeof(float) : 0;
 }
 
 #undef RG_WHO
@@ -407,7 +407,7 @@ static int recurrent_prefill_impl(const char* who, const void* x,
       const size_t one = (size_t)B * a.chunks * W;
       a.ws_p = (float*)workspace;
       a.ws_h = a.ws_p + one;
-      a.ws_h_in = a.ws_h + one;
+      a.ws_h_in = nullptr;
     }
   }
   return launch_status(who,

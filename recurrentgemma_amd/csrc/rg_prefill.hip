@@ -65,10 +65,15 @@ union Frag {
   f32x4 q;
 };
 
+// What one workgroup does with its tiles.  A row cut into chunks takes two
+// launches: the first runs chunk 0 as kChunkHead and chunks 1 .. n-2 as
+// kChunkSummary side by side, the second chunks 1 .. n-1 as kChunkReplay,
+// each starting from the summaries of the chunks before it.
 enum PrefillMode {
-  kWholeRow = 0,      // one workgroup per (row, head): y, h_last, conv state
-  kChunkSummary = 1,  // one per (row, head, chunk), zero start: (prod a, h_end)
-  kChunkReplay = 2    // the same chunks from their incoming state: y, ...
+  kWholeRow = 0,      // a whole row of one head: y, h_last, conv state
+  kChunkSummary = 1,  // a chunk from a zero state: (prod a, h_end), no y
+  kChunkReplay = 2,   // a chunk from its incoming state: y, ...
+  kChunkHead = 3      // chunk 0 from h0: y, and its end state as a summary
 };
 
 // s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding:
@@ -188,8 +193,8 @@ struct BlockAcc {
 };
 
 template <int MODE>
-__global__ void __launch_bounds__(kThreads) block_prefill_bf16_kernel(
-    FusedArgs p) {
+__device__ __forceinline__ void prefill_body(const FusedArgs& p,
+                                             const int chunk) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   lds_byte* const lds3 = (lds_byte*)lds_raw;
 
@@ -198,7 +203,6 @@ __global__ void __launch_bounds__(kThreads) block_prefill_bf16_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int b = blockIdx.x / p.H;
   const int h = blockIdx.x % p.H;
-  const int chunk = MODE == kWholeRow ? 0 : (int)blockIdx.y;
   const int T_len = p.T;
   const int64_t W = p.W;
   const int ntiles_all = (T_len + kTM - 1) / kTM;
@@ -215,16 +219,29 @@ __global__ void __launch_bounds__(kThreads) block_prefill_bf16_kernel(
   // (per 32-channel group: k-step, gate, lane, 8 values), or they are
   // transposed through LDS here, 128 k-rows of one gate at a time.
   if (p.w_packed) {
+    // 32 fragments at a time: all their loads are in flight before the first
+    // is moved (left to itself the compiler waits for every load in turn)
 #pragma unroll
     for (int nb = 0; nb < kNB; ++nb) {
       const f32x4* src = reinterpret_cast<const f32x4*>(p.w_packed) +
                          ((int64_t)(h * 8 + wave * kNB + nb) * 16 * 2) * 64 +
                          lane;
+      f32x4 w[32];
+#pragma unroll
+      for (int i = 0; i < 32; ++i) w[i] = src[i * 64];
+#pragma unroll
+      for (int i = 0; i < 32; i += 16)
+        asm volatile("" ::"v"(w[i]), "v"(w[i + 1]), "v"(w[i + 2]),
+                     "v"(w[i + 3]), "v"(w[i + 4]), "v"(w[i + 5]),
+                     "v"(w[i + 6]), "v"(w[i + 7]), "v"(w[i + 8]),
+                     "v"(w[i + 9]), "v"(w[i + 10]), "v"(w[i + 11]),
+                     "v"(w[i + 12]), "v"(w[i + 13]), "v"(w[i + 14]),
+                     "v"(w[i + 15]));
 #pragma unroll
       for (int ks = 0; ks < 16; ++ks)
 #pragma unroll
         for (int g = 0; g < 2; ++g)
-          set_weight_frag(4 * ks + 2 * nb + g, src[(ks * 2 + g) * 64]);
+          set_weight_frag(4 * ks + 2 * nb + g, w[ks * 2 + g]);
     }
   } else {
     uint16_t* const lds = reinterpret_cast<uint16_t*>(lds_raw);
@@ -650,10 +667,20 @@ __global__ void __launch_bounds__(kThreads) block_prefill_bf16_kernel(
     decay[nb] =
         (-8.0f * kLog2e) *
         softplus_precise(bf16_bits_to_f32(((const uint16_t*)p.a_param)[ch]));
-    if (MODE == kChunkReplay)
-      hc[nb] = p.ws_h_in[((int64_t)b * p.chunks + chunk) * W + ch];
-    else if (MODE == kWholeRow && p.h0)
+    if (MODE == kChunkReplay) {
+      // state at the start of this chunk from the summaries of the chunks
+      // before it: h <- P[k] h + H[k] (the scan operator of
+      // recurrentgemma/jax/scan.py:161-187 over chunks); chunk 0 has P = 0
+      // and H = its end state
+      float hin = 0.0f;
+      const float* sp = p.ws_p + (int64_t)b * p.chunks * W + ch;
+      const float* sh = p.ws_h + (int64_t)b * p.chunks * W + ch;
+      for (int k = 0; k < chunk; ++k)
+        hin = __builtin_fmaf(sp[(int64_t)k * W], hin, sh[(int64_t)k * W]);
+      hc[nb] = hin;
+    } else if ((MODE == kWholeRow || MODE == kChunkHead) && p.h0) {
       hc[nb] = p.h0[(int64_t)b * W + ch];
+    }
   }
   uint64_t m_before, m_cur;
   fetch_seg(tile_begin - 1);
@@ -784,6 +811,20 @@ __global__ void __launch_bounds__(kThreads) block_prefill_bf16_kernel(
     }
     return;
   }
+  if (MODE == kChunkHead) {
+    // whatever came before the row is in hc already: a summary with a zero
+    // product makes the carry kernel take hc as the next chunk's start
+    if (!upper) {
+#pragma unroll
+      for (int nb = 0; nb < kNB; ++nb) {
+        const int ch = h * kBW + n0 + 32 * nb + (lane & 31);
+        const int64_t at = (int64_t)b * p.chunks * W + ch;
+        p.ws_p[at] = 0.0f;
+        p.ws_h[at] = hc[nb];
+      }
+    }
+    return;
+  }
   if (!last_chunk) return;
   if (p.h_last && !upper) {
 #pragma unroll
@@ -811,29 +852,33 @@ __global__ void __launch_bounds__(kThreads) block_prefill_bf16_kernel(
   }
 }
 
-// h_in of every chunk from the summaries: h_in[0] = h0, h_in[k+1] =
-// P[k] h_in[k] + H[k] (the scan operator of recurrentgemma/jax/scan.py:161-187
-// over chunks).  One thread per (row, channel).
-__global__ void __launch_bounds__(256) prefill_chunk_carry_kernel(FusedArgs p) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= (int64_t)p.B * p.W) return;
-  const int64_t b = i / p.W, c = i - b * p.W;
-  float hcar = p.h0 ? p.h0[i] : 0.0f;
-  for (int k = 0; k < p.chunks; ++k) {
-    const int64_t at = (b * p.chunks + k) * p.W + c;
-    p.ws_h_in[at] = hcar;
-    if (k + 1 < p.chunks) hcar = __builtin_fmaf(p.ws_p[at], hcar, p.ws_h[at]);
+enum PrefillPass { kPassWholeRows = 0, kPassFirst = 1, kPassReplay = 2 };
+
+// blockIdx.x: (row, head); blockIdx.y: which chunk (kPassFirst: chunk 0 with
+// its outputs beside the summaries of chunks 1 .. n-2; kPassReplay: chunks
+// 1 .. n-1).
+template <int PASS>
+__global__ void __launch_bounds__(kThreads) block_prefill_bf16_kernel(
+    FusedArgs p) {
+  if (PASS == kPassWholeRows) {
+    prefill_body<kWholeRow>(p, 0);
+  } else if (PASS == kPassReplay) {
+    prefill_body<kChunkReplay>(p, (int)blockIdx.y + 1);
+  } else if (blockIdx.y == 0) {
+    prefill_body<kChunkHead>(p, 0);
+  } else {
+    prefill_body<kChunkSummary>(p, (int)blockIdx.y);
   }
 }
 
-template <int MODE>
-hipError_t launch_mode(const FusedArgs& a, int chunks, hipStream_t s) {
+template <int PASS>
+hipError_t launch_pass(const FusedArgs& a, int grid_y, hipStream_t s) {
   static OncePerDevice once;
   hipError_t e = set_max_dynamic_lds(
-      once, (const void*)block_prefill_bf16_kernel<MODE>, kPrefillLdsBytes);
+      once, (const void*)block_prefill_bf16_kernel<PASS>, kPrefillLdsBytes);
   if (e != hipSuccess) return e;
-  block_prefill_bf16_kernel<MODE>
-      <<<dim3((unsigned)(a.B * a.H), (unsigned)chunks), kThreads,
+  block_prefill_bf16_kernel<PASS>
+      <<<dim3((unsigned)(a.B * a.H), (unsigned)grid_y), kThreads,
          kPrefillLdsBytes, s>>>(a);
   return hipGetLastError();
 }
@@ -842,20 +887,23 @@ hipError_t launch_mode(const FusedArgs& a, int chunks, hipStream_t s) {
 
 // Into how many chunks of whole tiles the sequences of this shape are cut
 // (1: not cut).  One workgroup per (row, head) leaves CUs idle below 256
-// groups; cut into chunks every token is computed twice (summary pass, replay
-// pass), so it pays from three chunks per row on.
+// groups.  Cut into n chunks a row takes two launches of n-1 workgroups, each
+// as long as one chunk (every chunk but the first and the last is computed
+// twice): 2/n of the uncut time, which pays from n = 3 on.
 void prefill_chunk_plan(int B, int H, int T, int* chunks, int* tiles_per_chunk) {
   const int ntiles = (T + kTM - 1) / kTM;
   *chunks = 1;
   *tiles_per_chunk = ntiles;
   const int64_t groups = (int64_t)B * H;
-  if (groups * 3 > 256 || ntiles < 6) return;
-  int want = (int)(256 / groups);
+  if (groups * 2 > 256 || ntiles < 6) return;
+  int want = (int)(256 / groups) + 1;  // workgroups per launch and row, + 1
   if (want > ntiles / 2) want = ntiles / 2;
   if (want < 3) return;
   const int per = (ntiles + want - 1) / want;
+  const int n = (ntiles + per - 1) / per;
+  if (n < 3) return;
   *tiles_per_chunk = per;
-  *chunks = (ntiles + per - 1) / per;
+  *chunks = n;
 }
 
 hipError_t launch_block_prefill_bf16(const FusedArgs& a, hipStream_t s) {
@@ -863,15 +911,11 @@ hipError_t launch_block_prefill_bf16(const FusedArgs& a, hipStream_t s) {
   // (checked by the caller)
   const int64_t blocks = (int64_t)a.B * a.H;
   if (blocks <= 0 || blocks > 0x7fffffff) return hipErrorInvalidValue;
-  if (a.chunks <= 1) return launch_mode<kWholeRow>(a, 1, s);
-  if (a.chunks > 65535) return hipErrorInvalidValue;
-  hipError_t e = launch_mode<kChunkSummary>(a, a.chunks - 1, s);
+  if (a.chunks <= 1) return launch_pass<kPassWholeRows>(a, 1, s);
+  if (a.chunks < 3 || a.chunks > 65535) return hipErrorInvalidValue;
+  hipError_t e = launch_pass<kPassFirst>(a, a.chunks - 1, s);
   if (e != hipSuccess) return e;
-  const int64_t n = (int64_t)a.B * a.W;
-  prefill_chunk_carry_kernel<<<dim3((unsigned)((n + 255) / 256)), 256, 0, s>>>(a);
-  e = hipGetLastError();
-  if (e != hipSuccess) return e;
-  return launch_mode<kChunkReplay>(a, a.chunks, s);
+  return launch_pass<kPassReplay>(a, a.chunks - 1, s);
 }
 
 }  // namespace rg

@@ -62,7 +62,7 @@ def test_c_side_validation_without_launch():
   assert lib.rg_recurrent_prefill_split_workspace_bytes(16, 8192, 4096, 16) == 0
   assert lib.rg_recurrent_prefill_split_workspace_bytes(1, 320, 2560, 10) == 0  # < 6 tiles
   need = lib.rg_recurrent_prefill_split_workspace_bytes(1, 8192, 2560, 10)
-  assert need > 0 and need % (3 * 2560 * 4) == 0
+  assert need > 0 and need % (2 * 2560 * 4) == 0
   rc = lib.rg_recurrent_prefill_split(ok, ok, 1, ok, ok, ok, ok, ok, ok, None,
                                       ok, None, y, None, None, None, 0, 1, 8192,
                                       2560, 10, 1, None)
