@@ -18,6 +18,14 @@ soft cap, the sampler's left padding and split prompt processing):
   * Sampler.__call__ (greedy) on prompts of different lengths, with logits.
 All float32, tiny shapes.  The model's parameters are stored too, under the
 reference's state-dict keys.
+
+With --bf16 it writes tests/golden/griffin_bf16_golden.npz instead: the
+reference model in bfloat16 with 256-wide RG-LRU heads (the shapes that take
+this package's bf16 kernels), its parameters regenerated from a seed by
+tests/helpers.seeded_state_dict instead of stored, and beside every bf16
+result the same computation by the reference in float32 on the same
+(bf16-valued) parameters: the distance between the two is the yardstick for a
+third bf16 implementation.
 """
 
 import importlib.util
@@ -164,5 +172,90 @@ def main():
   print("wrote", OUT, len(out), "arrays,", os.path.getsize(OUT), "bytes")
 
 
+BF16_OUT = os.path.join(os.path.dirname(os.path.abspath(__file__)),
+                        "griffin_bf16_golden.npz")
+BF16_SEED = 77
+
+
+def bf16_config(common):
+  R, A = common.TemporalBlockType.RECURRENT, common.TemporalBlockType.ATTENTION
+  return common.GriffinConfig(
+      vocab_size=512, width=512, mlp_expanded_width=768, num_heads=2,
+      block_types=(R, R, A), embeddings_scale_by_sqrt_dim=True,
+      attention_window_size=16, logits_soft_cap=30.0, lru_width=512)
+
+
+def main_bf16():
+  sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.dirname(
+      os.path.abspath(__file__)))))
+  from tests import helpers
+  common, griffin, sampler = load_reference()
+  config = bf16_config(common)
+  models = {}
+  for tag, dtype in (("bf16", torch.bfloat16), ("f32", torch.float32)):
+    m = griffin.Griffin(config, gradient_checkpointing=False, dtype=dtype)
+    shapes = {k: tuple(v.shape) for k, v in m.state_dict().items()}
+    sd = helpers.seeded_state_dict(shapes, BF16_SEED, torch.bfloat16)
+    m.load_state_dict({k: v.to(dtype) for k, v in sd.items()})
+    models[tag] = m.eval()
+  out = {"param_checksum": np.float64(helpers.state_dict_checksum(sd)),
+         "param_seed": np.int64(BF16_SEED)}
+
+  def f32(t):
+    return t.detach().float().cpu().numpy().copy()
+
+  gen = torch.Generator().manual_seed(9)
+  with torch.no_grad():
+    # ---- case 1: left-padded prompts longer than the window + 4 steps ------
+    T, steps = 24, 4
+    tokens = torch.randint(3, config.vocab_size, (2, T), generator=gen)
+    pos = torch.stack([torch.arange(T),
+                       torch.cat([torch.full((5,), -1), torch.arange(T - 5)])])
+    step_tokens = torch.randint(3, config.vocab_size, (2, steps), generator=gen)
+    out["c1/tokens"], out["c1/pos"] = tokens.numpy(), pos.numpy()
+    out["c1/step_tokens"] = step_tokens.numpy()
+    for tag, m in models.items():
+      logits, cache = m(tokens, pos, None, return_logits=True,
+                        return_cache=True)
+      out[f"c1/{tag}/logits"] = f32(logits)
+      for name, c in cache.items():
+        for field, value in c._asdict().items():
+          out[f"c1/{tag}/cache/{name}/{field}"] = f32(value) if (
+              value.is_floating_point()) else value.numpy().copy()
+      p = pos[:, -1:] + 1
+      for i in range(steps):
+        lg, cache = m(step_tokens[:, i:i + 1], p, cache, return_logits=True,
+                      return_cache=True)
+        out[f"c1/{tag}/step{i}_logits"] = f32(lg)
+        p = p + 1
+      for name, c in cache.items():
+        for field, value in c._asdict().items():
+          out[f"c1/{tag}/final_cache/{name}/{field}"] = f32(value) if (
+              value.is_floating_point()) else value.numpy().copy()
+
+    # ---- case 2: the sampler, greedy, prompts of different lengths ---------
+    prompts = ["5 9 13 21 8 30 11 400 17 250 31 77 19 23 101 202 303 404 55",
+               "7 40 3", "12 500 6 88 91"]
+    out["c2/prompts"] = np.array(prompts)
+    for tag, m in models.items():
+      smp = sampler.Sampler(m, ToyVocab(), greedy_sampling=True)
+      res = smp(prompts, total_generation_steps=12, echo=True,
+                return_logits=True, end_sampling_at_eos_token=False)
+      for i, (t, lg) in enumerate(zip(res.tokens, res.logits)):
+        out[f"c2/{tag}/tokens{i}"] = t.numpy().copy()
+        out[f"c2/{tag}/logits{i}"] = f32(lg)
+
+  np.savez_compressed(BF16_OUT, **out)
+  print("wrote", BF16_OUT, len(out), "arrays,", os.path.getsize(BF16_OUT),
+        "bytes")
+  for k in ("c1/%s/logits", "c1/%s/step3_logits", "c2/%s/logits0"):
+    a, b = out[k % "bf16"], out[k % "f32"]
+    print(k, "max |bf16 - f32| =", np.abs(a - b).max(), "rms",
+          np.sqrt(np.mean((a - b) ** 2)), "max |f32| =", np.abs(b).max())
+
+
 if __name__ == "__main__":
-  main()
+  if "--bf16" in sys.argv[1:]:
+    main_bf16()
+  else:
+    main()

@@ -74,3 +74,41 @@ def assert_close_elementwise(got, want, rtol=1e-2, atol_of_max=2e-3, what=""):
   assert worst <= 0, (
       f"{what}: {int((excess > 0).sum())} of {excess.numel()} elements outside "
       f"rtol={rtol} atol={atol_of_max}*max; worst excess {worst:.3e}")
+
+
+def seeded_state_dict(shapes, seed, dtype=torch.bfloat16):
+  """A state dict that a seed fixes: {name: shape} -> {name: tensor}, every
+  value rounded to `dtype` and returned in it.  The golden vectors of the bf16
+  residual stack were written by the reference model holding exactly these
+  parameters (tests/golden/make_griffin_golden.py), so that a few MB of
+  weights need not be stored; `param_checksum` in the fixture guards the
+  regeneration.  Matrices ~ N(0, 1/fan_in), biases and norm scales ~ N(0, 0.1),
+  a_param such that the base decay is uniform in [0.9, 0.999]."""
+  out = {}
+  for i, name in enumerate(sorted(shapes)):
+    shape = tuple(shapes[name])
+    g = torch.Generator().manual_seed(seed * 1000 + i)
+    if name.endswith("a_param"):
+      u = torch.rand(shape, generator=g) * 0.099 + 0.9
+      t = torch.log(torch.expm1(-0.5 * torch.log(u)))
+    elif name.endswith((".b", ".bias", ".scale")) or len(shape) < 2:
+      t = torch.randn(shape, generator=g) * 0.1
+    else:
+      # nn.Linear and the embedding table are [out, in]; the block-diagonal,
+      # einsum and conv weights [..., in, out]
+      fan_in = (shape[-1] if name.endswith((".weight", "input_embedding"))
+                else shape[-2])
+      t = torch.randn(shape, generator=g) / fan_in ** 0.5
+    out[name] = t.to(dtype)
+  return out
+
+
+def state_dict_checksum(sd):
+  """Sum of |value| * (1 + position mod 7) over all tensors in name order, in
+  float64: moves if any value, shape or order differs."""
+  total = 0.0
+  for name in sorted(sd):
+    v = sd[name].detach().double().flatten().abs()
+    w = (torch.arange(v.numel(), dtype=torch.float64) % 7) + 1.0
+    total += float((v * w).sum())
+  return total
