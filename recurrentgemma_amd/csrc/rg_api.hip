@@ -155,6 +155,9 @@ int rg_block_diag_linear(const void* x, const void* w, const void* b, void* y,
   a.W = H * bw;
   a.H = H;
   a.bw = bw;
+  if (dtype == RG_DTYPE_F32 && bw == 256)
+    return launch_status(__func__,
+                         rg::launch_gemm_mfma_f32(a, (hipStream_t)stream));
   return launch_status(__func__,
                        rg::launch_gemm_generic(a, dtype, (hipStream_t)stream));
 }
@@ -208,6 +211,8 @@ int rg_gates_gemm(const void* x, int apply_conv, const void* segpos,
   hipError_t e;
   if (dtype == RG_DTYPE_BF16 && a.bw == 256)
     e = rg::launch_gemm_mfma_bf16(a, (hipStream_t)stream);
+  else if (dtype == RG_DTYPE_F32 && a.bw == 256)
+    e = rg::launch_gemm_mfma_f32(a, (hipStream_t)stream);
   else
     e = rg::launch_gemm_generic(a, dtype, (hipStream_t)stream);
   return launch_status(__func__, e);
@@ -215,26 +220,28 @@ int rg_gates_gemm(const void* x, int apply_conv, const void* segpos,
 
 size_t rg_scan_split_workspace_bytes(int B, int T, int W) {
   if (B <= 0 || T <= 0 || W <= 0) return 0;
+  // (the size does not know the dtype: the finest cut, float32's, is the
+  // largest)
   int chunks, t_chunk;
-  rg::scan_split_plan(B, T, W, &chunks, &t_chunk);
-  return chunks > 1 ? (size_t)3 * B * chunks * W * sizeof(float) : 0;
+  rg::scan_split_plan(B, T, W, 64, &chunks, &t_chunk);
+  return chunks > 1 ? (size_t)2 * B * chunks * W * sizeof(float) : 0;
 }
 
 // Points the scan at its workspace if the shape is one that is cut into
 // chunks; RG_OK or the error for a workspace that is missing or too small.
-static int plan_scan_split(const char* who, rg::ScanArgs* a, void* workspace,
-                           size_t workspace_bytes) {
+static int plan_scan_split(const char* who, rg::ScanArgs* a, int dtype,
+                           void* workspace, size_t workspace_bytes) {
   const size_t need = rg_scan_split_workspace_bytes(a->B, a->T, a->W);
   if (need == 0) return RG_OK;
   if (workspace == nullptr || workspace_bytes < need || !aligned16(workspace))
     return fail(RG_ERR_WORKSPACE,
                 "%s: workspace of %zu bytes (16-byte aligned) required, got %zu",
                 who, need, workspace ? workspace_bytes : (size_t)0);
-  rg::scan_split_plan(a->B, a->T, a->W, &a->chunks, &a->t_chunk);
+  rg::scan_split_plan(a->B, a->T, a->W, rg::scan_split_granule(dtype, a->W),
+                      &a->chunks, &a->t_chunk);
   const size_t one = (size_t)a->B * a->chunks * a->W;
   a->ws_p = (float*)workspace;
   a->ws_h = a->ws_p + one;
-  a->ws_h_in = a->ws_h + one;
   return RG_OK;
 }
 
@@ -288,7 +295,7 @@ static int lru_scan_fused_impl(const char* who, const void* x, int apply_conv,
   a.T = T;
   a.W = W;
   if (split) {
-    const int rc = plan_scan_split(who, &a, workspace, workspace_bytes);
+    const int rc = plan_scan_split(who, &a, dtype, workspace, workspace_bytes);
     if (rc != RG_OK) return rc;
   }
   return launch_status(who, rg::launch_lru_scan(a, dtype, (hipStream_t)stream));
@@ -407,7 +414,6 @@ static int recurrent_prefill_impl(const char* who, const void* x,
       const size_t one = (size_t)B * a.chunks * W;
       a.ws_p = (float*)workspace;
       a.ws_h = a.ws_p + one;
-      a.ws_h_in = nullptr;
     }
   }
   return launch_status(who,
@@ -476,7 +482,7 @@ static int linear_scan_impl(const char* who, const void* x, const void* a,
   s.T = T;
   s.W = W;
   if (split) {
-    const int rc = plan_scan_split(who, &s, workspace, workspace_bytes);
+    const int rc = plan_scan_split(who, &s, dtype, workspace, workspace_bytes);
     if (rc != RG_OK) return rc;
   }
   return launch_status(who, rg::launch_lru_scan(s, dtype, (hipStream_t)stream));

@@ -501,6 +501,161 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
   }
 }
 
+
+// ======================================================= fp32 MFMA kernel ==
+//
+// float32, block width 256, on v_mfma_f32_32x32x2_f32: true float32 products
+// and sums (no reduced-precision operand formats), so the 1e-5 bar of the
+// float32 path holds.  One workgroup of four waves per (32-row tile of x, half
+// of a head's 256 outputs, head and gate); wave w owns 32 output columns and
+// keeps their 256 x 32 weights in 128 registers for all the row tiles it
+// walks.  The row tile (optionally convolved on load) is staged through LDS.
+// Small tiles on purpose: the shapes that come here in float32 are small, and
+// 32 x 128 outputs per workgroup spread them over every CU, three workgroups
+// to a CU.
+//
+// Operand layout of the instruction: lane l supplies A[row l % 32][k = l / 32]
+// and B[k = l / 32][col l % 32] of a 32 x 2 by 2 x 32 product.  Which two k go
+// together is free as long as A and B agree, so each lane reads four
+// consecutive k of its row with one 16-byte LDS read (k = 8 j + 4 (l / 32) + i,
+// i = 0..3) and holds the weights of the same k.
+constexpr int kF32TM = 32;          // rows per tile
+constexpr int kF32Stride = kBW + 4; // floats per LDS row (16 rows: 64 banks)
+constexpr size_t kF32LdsBytes = (size_t)kF32TM * kF32Stride * sizeof(float);
+
+template <bool CONV>
+__global__ void __launch_bounds__(256, 2) gates_mfma_f32_kernel(GemmArgs p) {
+  extern __shared__ __align__(16) unsigned char f32_lds[];
+  float* const As = reinterpret_cast<float*>(f32_lds);
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int z = blockIdx.z;
+  const int gate = z / p.H;
+  const int h = z - gate * p.H;
+  const int col = lane & 31, g = lane >> 5;
+  const int n = blockIdx.y * 128 + wave * 32 + col;  // output column in head
+  const float* x = (const float*)p.x;
+  const float* w = (const float*)p.w[gate] + (int64_t)h * kBW * kBW;
+  float* out = (float*)p.out[gate];
+  const int64_t W = p.W;
+
+  // this lane's weights: k = 8 j + 4 g + i at register 4 j + i
+  float bw_[128];
+  {
+    const __amdgpu_buffer_rsrc_t rw = make_rsrc(w, kBW * kBW * 4);
+    const uint32_t woff = (uint32_t)((4 * g) * kBW + n) * 4u;
+#pragma unroll
+    for (int j = 0; j < 32; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        bw_[4 * j + i] = __builtin_bit_cast(
+            float, __builtin_amdgcn_raw_buffer_load_b32(
+                       rw, woff, (uint32_t)((8 * j + i) * kBW * 4), 0));
+  }
+  const float bias = ((const float*)p.b[gate])[h * kBW + n];
+
+  // staging: thread = channel of the head
+  const int c = h * kBW + tid;
+  float cw0 = 0, cw1 = 0, cw2 = 0, cw3 = 0, cb = 0;
+  if (CONV) {
+    const float* cw = (const float*)p.conv_w;
+    cw0 = cw[c]; cw1 = cw[W + c]; cw2 = cw[2 * W + c]; cw3 = cw[3 * W + c];
+    cb = ((const float*)p.conv_b)[c];
+  }
+
+  const int64_t ntiles = (p.M + kF32TM - 1) / kF32TM;
+  for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+    const int64_t m0 = tile * kF32TM;
+    if (CONV) {
+      // bit 2 + r of starts: a document or a sequence begins at row m0 + r
+      // (every wave works the mask out for itself: it stays in scalar
+      // registers)
+      bool st = false;
+      if (lane < kF32TM + 2) {
+        const int64_t m = m0 + lane - 2;
+        st = true;
+        if (m >= 0 && m < p.M)
+          st = (m % p.T == 0) || is_doc_start(p.segpos, p.seg_kind, m);
+      }
+      const uint64_t starts = __ballot(st);
+      // Rows m0-3 .. m0+31 through a descriptor over just these rows (rows
+      // before the first and after the last read as zero), eight at a time:
+      // beside the weights there is no room for the values of a whole tile.
+      const int64_t first = m0 >= 3 ? m0 - 3 : 0;
+      const int64_t last = m0 + kF32TM < p.M ? m0 + kF32TM : p.M;
+      const __amdgpu_buffer_rsrc_t rx = make_rsrc(
+          x + first * W, (uint32_t)((last - first) * W * sizeof(float)));
+      const uint32_t row_bytes = (uint32_t)W * 4u;
+      const uint32_t voff = (uint32_t)c * 4u;
+      const int skip = (int)(first - (m0 - 3));  // rows before row 0: 0..3
+      float h1, h2, h3;  // x[m-1], x[m-2], x[m-3] of the next row
+      {
+        float hv[3];
+#pragma unroll
+        for (int r = 0; r < 3; ++r)
+          hv[r] = r < skip ? 0.0f
+                           : __builtin_bit_cast(
+                                 float, __builtin_amdgcn_raw_buffer_load_b32(
+                                            rx, voff,
+                                            (uint32_t)(r - skip) * row_bytes, 0));
+        h3 = hv[0]; h2 = hv[1]; h1 = hv[2];
+      }
+#pragma unroll
+      for (int part = 0; part < kF32TM / 8; ++part) {
+        float xv[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
+          xv[r] = __builtin_bit_cast(
+              float, __builtin_amdgcn_raw_buffer_load_b32(
+                         rx, voff,
+                         (uint32_t)(8 * part + r + 3 - skip) * row_bytes, 0));
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          // taps older than the newest document start of rows m-2 .. m are cut
+          const int rr = 8 * part + r;
+          const bool a1 = !((starts >> (2 + rr)) & 1);
+          const bool a2 = a1 && !((starts >> (1 + rr)) & 1);
+          const bool a3 = a2 && !((starts >> rr) & 1);
+          As[rr * kF32Stride + tid] =
+              conv4(xv[r], a1 ? h1 : 0.0f, a2 ? h2 : 0.0f, a3 ? h3 : 0.0f, cw0,
+                    cw1, cw2, cw3, cb);
+          h3 = h2; h2 = h1; h1 = xv[r];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
+#pragma unroll 8
+      for (int r = 0; r < kF32TM; ++r) {
+        const int64_t m = m0 + r;
+        As[r * kF32Stride + tid] = m < p.M ? x[m * W + c] : 0.0f;
+      }
+    }
+    __syncthreads();
+
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    const float* a_lane = As + col * kF32Stride + 4 * g;
+#pragma unroll
+    for (int j = 0; j < 32; ++j) {
+      const f32x4 a = *reinterpret_cast<const f32x4*>(a_lane + 8 * j);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], bw_[4 * j + i], acc, 0,
+                                                   0, 0);
+    }
+    // result register r of lane l: row 8 (r / 4) + 4 (l / 32) + r % 4, column
+    // l % 32
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int64_t m = m0 + 8 * (r >> 2) + 4 * g + (r & 3);
+      if (m < p.M) out[m * W + h * kBW + n] = acc[r] + bias;
+    }
+    __syncthreads();  // the tile is overwritten by the next round
+  }
+}
+
 }  // namespace
 
 hipError_t launch_gemm_generic(const GemmArgs& a, int dtype, hipStream_t s) {
@@ -519,6 +674,34 @@ hipError_t launch_gemm_generic(const GemmArgs& a, int dtype, hipStream_t s) {
       bdl_generic_kernel<uint16_t, true><<<grid, 256, 0, s>>>(a);
     else
       bdl_generic_kernel<uint16_t, false><<<grid, 256, 0, s>>>(a);
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_gemm_mfma_f32(const GemmArgs& a, hipStream_t s) {
+  // needs float32 and bw == 256 (checked by the caller); one or two gates
+  const int64_t ntiles = (a.M + kF32TM - 1) / kF32TM;
+  // enough workgroups for every CU three times over; beyond that a workgroup
+  // walks several row tiles with its weights in place
+  const int64_t per_tile = 2 * (int64_t)a.H * a.ngates;
+  int64_t gx = (768 + per_tile - 1) / per_tile;
+  if (gx > ntiles) gx = ntiles;
+  if (gx < 1) gx = 1;
+  if ((int64_t)a.H * a.ngates > 65535) return hipErrorInvalidValue;
+  dim3 grid((unsigned)gx, 2, (unsigned)(a.H * a.ngates));
+  hipError_t e;
+  if (a.apply_conv) {
+    static OncePerDevice once;
+    e = set_max_dynamic_lds(once, (const void*)gates_mfma_f32_kernel<true>,
+                            kF32LdsBytes);
+    if (e != hipSuccess) return e;
+    gates_mfma_f32_kernel<true><<<grid, 256, kF32LdsBytes, s>>>(a);
+  } else {
+    static OncePerDevice once;
+    e = set_max_dynamic_lds(once, (const void*)gates_mfma_f32_kernel<false>,
+                            kF32LdsBytes);
+    if (e != hipSuccess) return e;
+    gates_mfma_f32_kernel<false><<<grid, 256, kF32LdsBytes, s>>>(a);
   }
   return hipGetLastError();
 }

@@ -90,7 +90,6 @@ struct ScanArgs {
   int chunks, t_chunk;
   float* ws_p;
   float* ws_h;
-  float* ws_h_in;
 };
 
 struct FusedArgs {
@@ -115,7 +114,6 @@ struct FusedArgs {
   int chunks, tiles_per_chunk;
   float* ws_p;
   float* ws_h;
-  float* ws_h_in;
 };
 
 struct StepArgs {
@@ -151,8 +149,12 @@ hipError_t launch_conv1d_prefill(const ConvArgs& a, int dtype, hipStream_t s);
 hipError_t launch_conv1d_step(const ConvStepArgs& a, int dtype, hipStream_t s);
 hipError_t launch_gemm_generic(const GemmArgs& a, int dtype, hipStream_t s);
 hipError_t launch_gemm_mfma_bf16(const GemmArgs& a, hipStream_t s);
+hipError_t launch_gemm_mfma_f32(const GemmArgs& a, hipStream_t s);
 hipError_t launch_lru_scan(const ScanArgs& a, int dtype, hipStream_t s);
-void scan_split_plan(int B, int T, int W, int* chunks, int* t_chunk);
+void scan_split_plan(int B, int T, int W, int granule, int* chunks,
+                     int* t_chunk);
+// Chunk lengths are multiples of this for the kernel that handles (dtype, W).
+int scan_split_granule(int dtype, int W);
 hipError_t launch_block_prefill_bf16(const FusedArgs& a, hipStream_t s);
 void prefill_chunk_plan(int B, int H, int T, int* chunks, int* tiles_per_chunk);
 hipError_t launch_block_step_bf16(const StepArgs& a, hipStream_t s);

@@ -550,7 +550,16 @@ lru_scan_kernel(ScanArgs p) {
 #pragma unroll
   for (int ch = 0; ch < CH; ++ch) {
     if (SPLIT == kChunkSummary) h[ch] = 0.0f;
-    else if (SPLIT == kChunkReplay) h[ch] = p.ws_h_in[ws_row + ch];
+    else if (SPLIT == kChunkReplay) {
+      // state at the start of this chunk: h <- P[k] h + H[k] over the chunks
+      // before it (the scan operator one level up)
+      float hin = p.h0 ? p.h0[(int64_t)b * W + c + ch] : 0.0f;
+      const int64_t ws0 = (int64_t)b * p.chunks * W + c + ch;
+      for (int kc = 0; kc < chunk; ++kc)
+        hin = __builtin_fmaf(p.ws_p[ws0 + (int64_t)kc * W], hin,
+                             p.ws_h[ws0 + (int64_t)kc * W]);
+      h[ch] = hin;
+    }
     else h[ch] = p.h0 ? p.h0[(int64_t)b * W + c + ch] : 0.0f;
     chunk_p[ch] = 1.0f;
   }
@@ -689,34 +698,6 @@ lru_scan_kernel(ScanArgs p) {
   }
 }
 
-// h_in of every chunk from the summaries: h_in[0] = h0, h_in[k+1] =
-// P[k] h_in[k] + H[k].  One thread per (row, channel).
-__global__ void __launch_bounds__(256)
-scan_chunk_carry_kernel(ScanArgs p) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= (int64_t)p.B * p.W) return;
-  const int64_t b = i / p.W, c = i - b * p.W;
-  float h = p.h0 ? p.h0[i] : 0.0f;
-  // summaries exist for chunks 0 .. chunks-2
-  for (int k0 = 0; k0 < p.chunks; k0 += 8) {
-    float pk[8], hk[8];  // eight chunks' summaries in flight at a time
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int k = k0 + j < p.chunks - 1 ? k0 + j : p.chunks - 2;
-      const int64_t at = (b * p.chunks + k) * p.W + c;
-      pk[j] = p.ws_p[at];
-      hk[j] = p.ws_h[at];
-    }
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      if (k0 + j < p.chunks) {
-        p.ws_h_in[(b * p.chunks + k0 + j) * p.W + c] = h;
-        h = __builtin_fmaf(pk[j], h, hk[j]);
-      }
-    }
-  }
-}
-
 template <typename T, int CH, int KL, bool CONV, bool FAST, bool PLAIN,
           int SPLIT>
 hipError_t launch_t(const ScanArgs& a, hipStream_t s) {
@@ -760,10 +741,6 @@ hipError_t launch_split(const ScanArgs& a, hipStream_t s) {
     return launch_t<T, CH, KL, CONV, FAST, PLAIN, kWholeRow>(a, s);
   hipError_t e = launch_t<T, CH, KL, CONV, FAST, PLAIN, kChunkSummary>(a, s);
   if (e != hipSuccess) return e;
-  const int64_t n = (int64_t)a.B * a.W;
-  scan_chunk_carry_kernel<<<dim3((unsigned)((n + 255) / 256)), 256, 0, s>>>(a);
-  e = hipGetLastError();
-  if (e != hipSuccess) return e;
   return launch_t<T, CH, KL, CONV, FAST, PLAIN, kChunkReplay>(a, s);
 }
 
@@ -781,21 +758,27 @@ hipError_t launch_mode(const ScanArgs& a, hipStream_t s) {
 // run (a row of 8192 tokens: 0.32 ms).  Cut into chunks the rows are read
 // twice, but every CU works: the aim is one workgroup per CU (more would queue
 // for a second round on the CUs that finish first), chunk lengths in multiples
-// of 128 tokens (a step of 16 waves at 8 tokens each, the longest step in
-// use).  Worth it up to about 32 (row, 256-channel slab) pairs and from about
-// a thousand tokens on; measured, bf16, T = 8192: 10 pairs 321 -> 75 us,
-// 80 pairs no gain.
-void scan_split_plan(int B, int T, int W, int* chunks, int* t_chunk) {
+// of `granule` tokens, the longest step of the kernel that will run (16 waves
+// at 8 tokens each: 128; float32 with two channels per lane: 16 x 4 = 64).
+// Worth it up to about 32 (row, 256-channel slab) pairs and from about five
+// hundred tokens on; measured, bf16, T = 8192: 10 pairs 321 -> 75 us, 80 pairs
+// no gain.
+void scan_split_plan(int B, int T, int W, int granule, int* chunks,
+                     int* t_chunk) {
   *chunks = 1;
   *t_chunk = T;
   const int64_t wide_blocks = (int64_t)B * ((W + 255) / 256);
-  if (wide_blocks > 32 || T < 1024) return;
+  if (wide_blocks > 32 || T < 512) return;
   const int want = (int)(256 / wide_blocks);
-  const int len = ((T + want - 1) / want + 127) / 128 * 128;
+  const int len = ((T + want - 1) / want + granule - 1) / granule * granule;
   const int n = (T + len - 1) / len;
   if (n < 2) return;
   *t_chunk = len;
   *chunks = n;
+}
+
+int scan_split_granule(int dtype, int W) {
+  return dtype == 0 && W % 2 == 0 ? 64 : 128;
 }
 
 hipError_t launch_lru_scan(const ScanArgs& a, int dtype, hipStream_t s) {

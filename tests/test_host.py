@@ -110,8 +110,8 @@ def test_c_side_validation_without_launch():
   assert rc == -4 and b"workspace" in lib.rg_last_error()
   # scans cut into chunks: only for few rows and long sequences
   assert lib.rg_scan_split_workspace_bytes(16, 8192, 4096) == 0
-  assert lib.rg_scan_split_workspace_bytes(1, 1000, 2560) == 0
-  assert lib.rg_scan_split_workspace_bytes(1, 8192, 2560) == 3 * 22 * 2560 * 4
+  assert lib.rg_scan_split_workspace_bytes(1, 500, 2560) == 0
+  assert lib.rg_scan_split_workspace_bytes(1, 8192, 2560) == 2 * 22 * 2560 * 4
   rc = lib.rg_lru_scan_fused_split(ok, 0, None, None, ok, ok, ok, ok, 1, None, y,
                                    None, None, None, 0, 1, 8192, 2560, 1, None)
   assert rc == -4 and b"rg_lru_scan_fused_split: workspace" in lib.rg_last_error()
