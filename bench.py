@@ -276,14 +276,36 @@ def run_decode(args, torch, rg, R, ops, wl):
   torch.cuda.synchronize()
   e0 = torch.cuda.Event(enable_timing=True)
   e1 = torch.cuda.Event(enable_timing=True)
-  t0 = time.perf_counter()
-  e0.record()
-  for _ in range(args.steps):
-    step()
-  e1.record()
-  torch.cuda.synchronize()
-  elapsed = time.perf_counter() - t0
-  dev_ms = e0.elapsed_time(e1) / args.steps
+
+  def eager_loop():
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+      step()
+    e1.record()
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0, e0.elapsed_time(e1) / args.steps
+
+  eager_elapsed, eager_dev_ms = eager_loop()
+  if args.eager:
+    elapsed, dev_ms = eager_elapsed, eager_dev_ms
+  else:
+    # The K consecutive steps as one captured HIP graph (what the sampler does
+    # with its decode step): the launches cost no host time, the device sees
+    # the kernels back to back.
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+      for _ in range(args.steps):
+        step()
+    graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    dev_ms = e0.elapsed_time(e1) / args.steps
   algo = decode_algorithmic_bytes(B, W, H, 2)
   achieved = algo / (dev_ms * 1e-3) / 1e9
   result = {
@@ -295,7 +317,12 @@ def run_decode(args, torch, rg, R, ops, wl):
       "data": "synthetic",
       "config": {"workload": args.workload, "batch": B, "seq_len": 1,
                  "lru_width": W, "heads": H, "activations": "bf16",
-                 "state": "f32", "path": "rg_recurrent_step, caches in place"},
+                 "state": "f32",
+                 "path": "rg_recurrent_step, caches in place, "
+                         + ("launched from Python step by step" if args.eager
+                            else "the steps captured as one HIP graph")},
+      "eager_loop": {"ms_per_step": eager_elapsed * 1e3 / args.steps,
+                     "device_ms_per_step": eager_dev_ms},
       "roofline": {"kernel": "rg_recurrent_step (all launches of one step)",
                    "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
                    "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
@@ -334,8 +361,9 @@ def main():
                   help="lean run for the profiler: no CPU leg and no "
                        "additional 2B-width measurement")
   ap.add_argument("--eager", action="store_true",
-                  help="2b_griffin_decode: launch every kernel of a decode "
-                       "step from Python instead of replaying a captured graph")
+                  help="2b_griffin_decode, 9b_decode: launch every kernel of a "
+                       "decode step from Python instead of replaying a "
+                       "captured graph")
   ap.add_argument("--calibration-copy", action="store_true",
                   help="after the timed steps, run one plain device copy of x "
                        "(known size) so that a counter run of this command "
@@ -471,10 +499,11 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
             "algorithmic_bytes": scan_algo, "avg_launch_ms": scan_ms},
         "gate_gemm": {
             "kernel": ("gates_mfma_bf16_kernel" if esize == 2
-                       else "bdl_generic_kernel (fp32 FMA)"),
+                       else "gates_mfma_f32_kernel (v_mfma_f32_32x32x2_f32)"),
             "avg_launch_ms": gemm_ms,
             "tflops": gemm_flops / (gemm_ms * 1e-3) / 1e12,
-            "frac_of_bf16_mfma_peak": gemm_flops / (gemm_ms * 1e-3) / 2.5e15,
+            "frac_of_mfma_peak": gemm_flops / (gemm_ms * 1e-3)
+                                 / (2.5e15 if esize == 2 else 157.3e12),
             "gbs": gemm_bytes / (gemm_ms * 1e-3) / 1e9,
             "frac_of_hbm_peak": gemm_bytes / (gemm_ms * 1e-3) / 1e9
                                 / HBM_PEAK_GBS}}
@@ -497,6 +526,24 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
   else:
     figs = split_figures(first_ms, second_ms)
     roofline = figs["scan"]
+
+  cold = None
+  if extras and x.numel() * esize * 4 < (256 << 20):
+    # The whole working set fits the caches (4 MB of L2 per XCD, 256 MB behind
+    # them): the timed loop above is a warm-cache figure.  Cold: 1 GiB is
+    # written between the steps and each step is timed on its own.
+    flush = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    n_cold = min(steps, 20)
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)]
+           for _ in range(n_cold)]
+    for i in range(n_cold):
+      flush.fill_(i & 1)
+      step(evs[i])
+    torch.cuda.synchronize()
+    cold = {"ms_per_step": sum(e[0].elapsed_time(e[2]) for e in evs) / n_cold,
+            "steps": n_cold,
+            "how": "1 GiB written between steps; HIP events around each step"}
+    del flush
 
   if extras and args.calibration_copy:
     torch.empty_like(x).copy_(x)  # reads and writes x.numel()*2 bytes
@@ -531,6 +578,8 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
                            else "rg_lru_scan_fused(conv)"))},
       "roofline": roofline,
   }
+  if cold:
+    result["cold_caches"] = cold
   if path == "split":
     result["gate_gemm"] = figs["gate_gemm"]
   elif args.path == "auto":

@@ -51,7 +51,7 @@ pack_gate_weights_kernel(const uint16_t* __restrict__ w_x,
 // Replaces Conv1D.forward's decode branch (layers.py:469-474, 491-529) and
 // RGLRU.forward / rnn_scan with T == 1 (layers.py:313-365, 170-177).
 constexpr int kStepRows = 32;
-constexpr int kStepRowsPerThread = 8;  // 32 rows x 128 channel pairs / 512
+constexpr int kStepRowsPerThread = 4;  // 32 rows x 64 channel quads / 512
 
 __global__ void __launch_bounds__(512) block_step_bf16_kernel(StepArgs p) {
   __shared__ __align__(16) uint16_t stage[kStepRows * kLdsStride];
@@ -59,16 +59,106 @@ __global__ void __launch_bounds__(512) block_step_bf16_kernel(StepArgs p) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int b0 = blockIdx.x * kStepRows;
-  const int h = blockIdx.y;
+  // Workgroups go to the eight XCDs in turn (linear id modulo 8), each with
+  // an L2 of its own: the (head, row tile) pairs are dealt out so that one
+  // XCD gets a contiguous run of pairs in head-major order, i.e. all row
+  // tiles of a head fetch its weights through the same L2 (the plain order
+  // sends the tiles of a head to eight different ones, and every L2 then
+  // pulls in every head's weights).
+  const int tiles = (p.B + kStepRows - 1) / kStepRows;
+  int pair = blockIdx.x;
+  {
+    const int per_xcd = (int)gridDim.x / 8;
+    if (pair < 8 * per_xcd) pair = (pair & 7) * per_xcd + (pair >> 3);
+  }
+  const int h = pair / tiles;
+  const int b0 = (pair - h * tiles) * kStepRows;
   const int B = p.B;
   const int64_t W = p.W;
   const bool upper = lane >= 32;
   const int n0 = wave * 32;
   const int ch = h * kBW + n0 + (lane & 31);
 
-  // ---- loads first: this wave's weights (32 x 16 bytes per lane), the state
-  //      of this lane's 16 (row, channel) elements ---------------------------
+  // Everything per row goes through descriptors over this tile's rows only:
+  // rows past the end of the batch read as zero and their stores are dropped,
+  // without a branch around any access.
+  const int rows_here = B - b0 < kStepRows ? B - b0 : kStepRows;
+  const uint32_t row_bytes = (uint32_t)W * 2u;
+  const __amdgpu_buffer_rsrc_t rx = make_rsrc(
+      (const uint16_t*)p.x + (int64_t)b0 * W, (uint32_t)rows_here * row_bytes);
+  const __amdgpu_buffer_rsrc_t rcin =
+      make_rsrc((const uint16_t*)p.cache_in + (int64_t)b0 * 3 * W,
+                (uint32_t)rows_here * 3u * row_bytes);
+  const __amdgpu_buffer_rsrc_t rcout =
+      make_rsrc((uint16_t*)p.cache_out + (int64_t)b0 * 3 * W,
+                (uint32_t)rows_here * 3u * row_bytes);
+  const __amdgpu_buffer_rsrc_t rhin = make_rsrc(
+      p.h_in + (int64_t)b0 * W, (uint32_t)rows_here * 2u * row_bytes);
+  const __amdgpu_buffer_rsrc_t rhout = make_rsrc(
+      p.h_out + (int64_t)b0 * W, (uint32_t)rows_here * 2u * row_bytes);
+  const __amdgpu_buffer_rsrc_t ry = make_rsrc(
+      (uint16_t*)p.y + (int64_t)b0 * W, (uint32_t)rows_here * row_bytes);
+  // ---- loads, in the order they are needed: the conv step's rows (thread =
+  //      four channels of four rows: 8-byte accesses, a wave per access covers
+  //      the head's 512 bytes of a row), the small per-channel and per-row
+  //      values, this lane's 16 state elements, this wave's weights (32 x 16
+  //      bytes per lane).  Loads return in order, so the conv step runs while
+  //      the weights are still on their way.
+  const int cq = lane;
+  const int rg = wave;
+  const uint32_t c = h * kBW + cq * 4;
+  u32x2 xr[kStepRowsPerThread], s0[kStepRowsPerThread], s1[kStepRowsPerThread],
+      s2[kStepRowsPerThread];  // state oldest first
+#pragma unroll
+  for (int j = 0; j < kStepRowsPerThread; ++j) {
+    const uint32_t row = rg * kStepRowsPerThread + j;
+    xr[j] = __builtin_amdgcn_raw_buffer_load_b64(rx, 2u * c, row * row_bytes, 0);
+    s0[j] = __builtin_amdgcn_raw_buffer_load_b64(
+        rcin, 2u * c, (row * 3u + 0u) * row_bytes, 0);
+    s1[j] = __builtin_amdgcn_raw_buffer_load_b64(
+        rcin, 2u * c, (row * 3u + 1u) * row_bytes, 0);
+    s2[j] = __builtin_amdgcn_raw_buffer_load_b64(
+        rcin, 2u * c, (row * 3u + 2u) * row_bytes, 0);
+  }
+  const uint16_t* cw = (const uint16_t*)p.conv_w + c;
+  const u32x2 u0 = *reinterpret_cast<const u32x2*>(cw);
+  const u32x2 u1 = *reinterpret_cast<const u32x2*>(cw + W);
+  const u32x2 u2 = *reinterpret_cast<const u32x2*>(cw + 2 * W);
+  const u32x2 u3 = *reinterpret_cast<const u32x2*>(cw + 3 * W);
+  const u32x2 ub =
+      *reinterpret_cast<const u32x2*>((const uint16_t*)p.conv_b + c);
+  __builtin_amdgcn_sched_barrier(0);
+  // (the small per-channel and per-row values are requested here, with
+  // everything else: asked for where they are used they would cost a memory
+  // round trip of their own after the conv step)
+  const uint16_t bias_x_raw = ((const uint16_t*)p.b[0])[ch];
+  const uint16_t bias_a_raw = ((const uint16_t*)p.b[1])[ch];
+  const uint16_t a_param_raw = ((const uint16_t*)p.a_param)[ch];
+  // position of row lane % 32: two unconditional 32-bit loads (for int32
+  // positions the high half is sent out of range and reads as zero)
+  uint32_t seg_lo, seg_hi;
+  {
+    const bool is64 = p.seg_kind == kSegI64;
+    const uint32_t esize = is64 ? 8u : 4u;
+    const __amdgpu_buffer_rsrc_t rseg =
+        make_rsrc((const char*)p.segpos + (int64_t)b0 * esize,
+                  (uint32_t)rows_here * esize);
+    const uint32_t off = (uint32_t)(lane & 31) * esize;
+    seg_lo = __builtin_amdgcn_raw_buffer_load_b32(rseg, off, 0, 0);
+    seg_hi = __builtin_amdgcn_raw_buffer_load_b32(
+        rseg, is64 ? off + 4u : kBufferOutOfRange, 0, 0);
+  }
+  float hv[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    // row 8 (r / 4) + r % 4 (+ 4 in the upper half-wave)
+    hv[r] = __builtin_bit_cast(
+        float,
+        __builtin_amdgcn_raw_buffer_load_b32(
+            rhin, (uint32_t)ch * 4u + (upper ? 8u * row_bytes : 0u),
+            (uint32_t)(8 * (r >> 2) + (r & 3)) * 2u * row_bytes, 0));
+  }
+
   Frag bfrag[16][2];
   {
     const f32x4* src = reinterpret_cast<const f32x4*>(p.w_packed) +
@@ -78,78 +168,49 @@ __global__ void __launch_bounds__(512) block_step_bf16_kernel(StepArgs p) {
 #pragma unroll
       for (int g = 0; g < 2; ++g) bfrag[ks][g].q = src[(ks * 2 + g) * 64];
   }
-  float hv[16];
-#pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int64_t b = b0 + 8 * (r >> 2) + (r & 3) + (upper ? 4 : 0);
-    hv[r] = b < B ? p.h_in[b * W + ch] : 0.0f;
-  }
+  // (nothing above may sink below this line: left alone the compiler moves
+  // most of the weight and state loads behind the conv step, whose own loads
+  // it waits for first, and the kernel pays two memory round trips in a row)
+  __builtin_amdgcn_sched_barrier(0);
 
   // ---- conv step of this tile's rows -> LDS (bf16), new conv state ---------
   {
-    const int cp = tid & 127;
-    const int rg = tid >> 7;
-    const uint32_t c = h * kBW + cp * 2;
-    const uint16_t* xin = (const uint16_t*)p.x;
-    const uint16_t* cin = (const uint16_t*)p.cache_in;
-    uint16_t* cout = (uint16_t*)p.cache_out;
-    uint32_t xr[kStepRowsPerThread], s0[kStepRowsPerThread],
-        s1[kStepRowsPerThread], s2[kStepRowsPerThread];  // state oldest first
 #pragma unroll
     for (int j = 0; j < kStepRowsPerThread; ++j) {
-      const int64_t b = b0 + rg * kStepRowsPerThread + j;
-      xr[j] = s0[j] = s1[j] = s2[j] = 0u;
-      if (b < B) {
-        xr[j] = *reinterpret_cast<const uint32_t*>(xin + b * W + c);
-        s0[j] = *reinterpret_cast<const uint32_t*>(cin + (b * 3 + 0) * W + c);
-        s1[j] = *reinterpret_cast<const uint32_t*>(cin + (b * 3 + 1) * W + c);
-        s2[j] = *reinterpret_cast<const uint32_t*>(cin + (b * 3 + 2) * W + c);
-      }
-    }
-    const uint16_t* cw = (const uint16_t*)p.conv_w + c;
-    const uint32_t u0 = *reinterpret_cast<const uint32_t*>(cw);
-    const uint32_t u1 = *reinterpret_cast<const uint32_t*>(cw + W);
-    const uint32_t u2 = *reinterpret_cast<const uint32_t*>(cw + 2 * W);
-    const uint32_t u3 = *reinterpret_cast<const uint32_t*>(cw + 3 * W);
-    const uint32_t ub =
-        *reinterpret_cast<const uint32_t*>((const uint16_t*)p.conv_b + c);
+      const uint32_t row = rg * kStepRowsPerThread + j;
+      u32x2 packed;
 #pragma unroll
-    for (int j = 0; j < kStepRowsPerThread; ++j) {
-      const int row = rg * kStepRowsPerThread + j;
-      const int64_t b = b0 + row;
-      float o[2];
+      for (int w2 = 0; w2 < 2; ++w2) {
+        float o[2];
 #pragma unroll
-      for (int k = 0; k < 2; ++k) {
-        auto unpack = [&](uint32_t v) {
-          return k == 0 ? __uint_as_float(v << 16)
-                        : __uint_as_float(v & 0xffff0000u);
-        };
-        o[k] = conv4(unpack(xr[j]), unpack(s2[j]), unpack(s1[j]), unpack(s0[j]),
-                     unpack(u0), unpack(u1), unpack(u2), unpack(u3), unpack(ub));
+        for (int k = 0; k < 2; ++k) {
+          auto unpack = [&](const u32x2& v) {
+            return k == 0 ? __uint_as_float(v[w2] << 16)
+                          : __uint_as_float(v[w2] & 0xffff0000u);
+          };
+          o[k] = conv4(unpack(xr[j]), unpack(s2[j]), unpack(s1[j]),
+                       unpack(s0[j]), unpack(u0), unpack(u1), unpack(u2),
+                       unpack(u3), unpack(ub));
+        }
+        packed[w2] = pack_bf16x2(o[0], o[1]);
       }
-      *reinterpret_cast<uint32_t*>(stage + (size_t)row * kLdsStride + cp * 2) =
-          pack_bf16x2(o[0], o[1]);
-      if (b < B) {
-        *reinterpret_cast<uint32_t*>(cout + (b * 3 + 0) * W + c) = s1[j];
-        *reinterpret_cast<uint32_t*>(cout + (b * 3 + 1) * W + c) = s2[j];
-        *reinterpret_cast<uint32_t*>(cout + (b * 3 + 2) * W + c) = xr[j];
-      }
+      *reinterpret_cast<u32x2*>(stage + (size_t)row * kLdsStride + cq * 4) =
+          packed;
+      __builtin_amdgcn_raw_buffer_store_b64(s1[j], rcout, 2u * c,
+                                            (row * 3u + 0u) * row_bytes, 0);
+      __builtin_amdgcn_raw_buffer_store_b64(s2[j], rcout, 2u * c,
+                                            (row * 3u + 1u) * row_bytes, 0);
+      __builtin_amdgcn_raw_buffer_store_b64(xr[j], rcout, 2u * c,
+                                            (row * 3u + 2u) * row_bytes, 0);
     }
   }
 
-  const float bias_x = bf16_bits_to_f32(((const uint16_t*)p.b[0])[ch]);
-  const float bias_a = bf16_bits_to_f32(((const uint16_t*)p.b[1])[ch]);
+  const float bias_x = bf16_bits_to_f32(bias_x_raw);
+  const float bias_a = bf16_bits_to_f32(bias_a_raw);
   const float decay =
-      (-8.0f * kLog2e) *
-      softplus_precise(bf16_bits_to_f32(((const uint16_t*)p.a_param)[ch]));
+      (-8.0f * kLog2e) * softplus_precise(bf16_bits_to_f32(a_param_raw));
   // rows of this tile whose position is 0 (document start: forget the state)
-  uint32_t m_start;
-  {
-    const int64_t b = (int64_t)b0 + (lane & 31);
-    bool st = false;
-    if (b < B) st = is_doc_start(p.segpos, p.seg_kind, b);
-    m_start = (uint32_t)__ballot(st);
-  }
+  const uint32_t m_start = (uint32_t)__ballot((seg_lo | seg_hi) == 0u);
   __syncthreads();  // the staged tile is complete
 
   f32x16 acc_x, acc_a;
@@ -171,19 +232,23 @@ __global__ void __launch_bounds__(512) block_step_bf16_kernel(StepArgs p) {
   }
   const uint16_t* xcp =
       stage + (size_t)(4 * (lane >> 5)) * kLdsStride + n0 + (lane & 31);
-  float* h_out = p.h_out;
-  uint16_t* yout = (uint16_t*)p.y;
+  // Outputs: neighbouring lanes hold neighbouring channels of the same rows.
+  // Lanes swap in pairs so that the even lane stores both channels of the even
+  // row of a row pair and the odd lane both channels of the odd row: 8-byte
+  // state and 4-byte y stores, half as many as one store per element.
+  const bool odd = lane & 1;
+  const uint32_t pair_ch = (uint32_t)(ch & ~1);
 #pragma unroll
   for (int r = 0; r < 16; r += 2) {
     // pre-activations are a bf16 module output in the reference
     const uint32_t px2 = pack_bf16x2(acc_x[r], acc_x[r + 1]);
     const uint32_t pa2 = pack_bf16x2(acc_a[r], acc_a[r + 1]);
+    float hn[2];
 #pragma unroll
     for (int e = 0; e < 2; ++e) {
       const int rr = r + e;
       const int i = 8 * (rr >> 2) + (rr & 3);
       const int row = i + (upper ? 4 : 0);
-      const int64_t b = (int64_t)b0 + row;
       const float xc = bf16_bits_to_f32(xcp[(size_t)i * kLdsStride]);
       const float px = e == 0 ? __uint_as_float(px2 << 16)
                               : __uint_as_float(px2 & 0xffff0000u);
@@ -195,12 +260,25 @@ __global__ void __launch_bounds__(512) block_step_bf16_kernel(StepArgs p) {
       if ((m_start >> row) & 1u) a = 0.0f;  // the input scale becomes 1 below
       const float mult = __builtin_amdgcn_sqrtf(__builtin_fmaf(-a, a, 1.0f));
       const float xn = (xc * gate_x) * mult;
-      const float hn = __builtin_fmaf(a, hv[rr], xn);
-      if (b < B) {
-        h_out[b * W + ch] = hn;
-        yout[b * W + ch] = f32_to_bf16_bits(hn);
-      }
+      hn[e] = __builtin_fmaf(a, hv[rr], xn);
     }
+    // what the partner lane stores of mine: the even lane keeps row r, the
+    // odd lane row r + 1
+    const float give = odd ? hn[0] : hn[1];
+    const float got = __uint_as_float(__builtin_amdgcn_mov_dpp(
+        __float_as_uint(give), 0xB1 /* quad_perm [1,0,3,2] */, 0xf, 0xf, true));
+    const float mine = odd ? hn[1] : hn[0];
+    const float lo = odd ? got : mine;  // channel pair_ch
+    const float hi = odd ? mine : got;  // channel pair_ch + 1
+    // row 8 (r / 4) + r % 4, + 1 in the odd lane, + 4 in the upper half-wave
+    const uint32_t lane_rows = (odd ? 1u : 0u) + (upper ? 4u : 0u);
+    const uint32_t tile_row = (uint32_t)(8 * (r >> 2) + (r & 3));
+    __builtin_amdgcn_raw_buffer_store_b64(
+        u32x2{__float_as_uint(lo), __float_as_uint(hi)}, rhout,
+        pair_ch * 4u + lane_rows * 2u * row_bytes, tile_row * 2u * row_bytes, 0);
+    __builtin_amdgcn_raw_buffer_store_b32(pack_bf16x2(lo, hi), ry,
+                                          pair_ch * 2u + lane_rows * row_bytes,
+                                          tile_row * row_bytes, 0);
   }
 }
 
@@ -217,8 +295,9 @@ hipError_t launch_pack_gate_weights(const void* w_x, const void* w_a,
 hipError_t launch_block_step_bf16(const StepArgs& a, hipStream_t s) {
   // needs head width 256 (checked by the caller)
   const int tiles = (a.B + kStepRows - 1) / kStepRows;
-  if (tiles <= 0 || a.H > 65535) return hipErrorInvalidValue;
-  block_step_bf16_kernel<<<dim3((unsigned)tiles, (unsigned)a.H), 512, 0, s>>>(a);
+  if (tiles <= 0 || (int64_t)tiles * a.H > 0x7fffffff)
+    return hipErrorInvalidValue;
+  block_step_bf16_kernel<<<dim3((unsigned)(tiles * a.H)), 512, 0, s>>>(a);
   return hipGetLastError();
 }
 
