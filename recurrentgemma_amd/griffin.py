@@ -17,6 +17,7 @@ from __future__ import annotations
 import enum
 import itertools
 import math
+import functools
 import weakref
 from typing import Any, NamedTuple
 
@@ -227,6 +228,27 @@ def _visible(q_pos, k_pos, window, q_doc=None, k_doc=None):
   return mask & (k >= 0)
 
 
+def _inference_only(forward):
+  """The residual stack around the recurrent block runs without an autograd
+  graph (its few-row linear layers, attention and normalisation kernels have
+  no backward pass).  A caller that would expect gradients -- inside
+  training.differentiable(), or with gradients enabled on a module in
+  training mode -- gets an error instead of silently detached tensors."""
+
+  @functools.wraps(forward)
+  def wrapper(self, *args, **kwargs):
+    from recurrentgemma_amd import training
+    if training.is_enabled() or (torch.is_grad_enabled() and self.training):
+      raise NotImplementedError(
+          f"{type(self).__name__} is forward only: call .eval() or run it "
+          "under torch.no_grad() (only RecurrentBlock, Conv1D and RGLRU have "
+          "a differentiable path, inside training.differentiable())")
+    with torch.no_grad():
+      return forward(self, *args, **kwargs)
+
+  return wrapper
+
+
 _one_document = [None, None, False]  # tensor (weak), its version, answer
 
 
@@ -236,11 +258,13 @@ def _rows_are_one_document(segment_pos) -> bool:
   Asking costs a host synchronisation, so the answer is kept for the tensor
   object it was given for (the blocks of a model all ask about the same one)."""
   ref, version, answer = _one_document
-  if (ref is not None and ref() is segment_pos and
-      version == segment_pos._version):
+  # (inference-mode tensors keep no version counter: asked again every time)
+  now = None if segment_pos.is_inference() else segment_pos._version
+  if (ref is not None and ref() is segment_pos and now is not None and
+      version == now):
     return answer
   answer = bool((segment_pos[:, 1:] != 0).all())
-  _one_document[:] = [weakref.ref(segment_pos), segment_pos._version, answer]
+  _one_document[:] = [weakref.ref(segment_pos), now, answer]
   return answer
 
 
@@ -302,7 +326,7 @@ class LocalAttentionBlock(nn.Module):
     return AttentionBlockCache(keys=place(keys), values=place(values),
                                num_tokens=num_tokens)
 
-  @torch.no_grad()
+  @_inference_only
   def forward(self, x, segment_pos, cache=None, return_cache=True,
               defer_out=False):
     """defer_out: as for RecurrentBlock.forward."""
@@ -467,7 +491,7 @@ class ResidualBlock(nn.Module):
     self.channel_pre_norm.reset_parameters()
     self.mlp_block.reset_parameters()
 
-  @torch.no_grad()
+  @_inference_only
   def forward(self, x, segment_pos, cache=None, return_cache=True,
               defer_out=False):
     """x and, with defer_out, the result may be ops.PartialSums: the output of
@@ -558,7 +582,7 @@ class Griffin(nn.Module):
       block.reset_parameters()
     self.final_norm.reset_parameters()
 
-  @torch.no_grad()
+  @_inference_only
   def forward(self, tokens, segment_pos, cache: Cache | None = None,
               return_logits=True, return_cache=True):
     if not return_logits and not return_cache:

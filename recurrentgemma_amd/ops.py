@@ -478,16 +478,30 @@ def attention_decode_finish(from_ring, probs, k_new, v_new, ring_keys,
 _packed_weights = {}  # (id(w_x), id(w_a)) -> (ref_x, ref_a, stamp, packed)
 
 
+def tensor_stamp(t):
+  """(storage address, version counter) of a tensor: changes when the tensor
+  is written in place or re-pointed.  Inference-mode tensors keep no version
+  counter; None then stands in, and callers treat such a stamp as never equal
+  to a kept one (they recompute)."""
+  if t.is_inference():
+    return (t.data_ptr(), None)
+  return (t.data_ptr(), t._version)
+
+
+def stamps_match(old, new):
+  return old == new and not any(v is None for _, v in new)
+
+
 def packed_gate_weights(w_x, w_a):
   """Both gate matrices in MFMA operand order (rg_pack_gate_weights), cached per
   pair of tensor objects until either is written to, re-pointed or dies."""
   import weakref
   key = (id(w_x), id(w_a))
-  stamp = (w_x.data_ptr(), w_x._version, w_a.data_ptr(), w_a._version)
+  stamp = (tensor_stamp(w_x), tensor_stamp(w_a))
   hit = _packed_weights.get(key)
   if hit is not None:
     ref_x, ref_a, old_stamp, packed = hit
-    if ref_x() is w_x and ref_a() is w_a and old_stamp == stamp:
+    if ref_x() is w_x and ref_a() is w_a and stamps_match(old_stamp, stamp):
       return packed
   H, bw, _ = w_x.shape
   W = H * bw
@@ -559,8 +573,8 @@ class PackedLinear:
 
   def _prepare(self, weights, biases):
     tensors = tuple(weights) + tuple(b for b in (biases or ()) if b is not None)
-    stamp = tuple((id(t), t.data_ptr(), t._version) for t in tensors)
-    if stamp == self._stamp:
+    stamp = tuple((id(t),) + tensor_stamp(t) for t in tensors)
+    if stamp == self._stamp and not any(v[2] is None for v in stamp):
       return
     w0 = weights[0]
     lib = _lib.lib()

@@ -28,6 +28,14 @@ class SamplerOutput(NamedTuple):
   tokens: list[torch.Tensor]
 
 
+def _parameter_stamp(model):
+  """Address, version counter and dtype of every parameter: a captured step
+  reads re-laid-out copies of the weights made when it was captured, so it is
+  only good for as long as this stays the same (no load_state_dict, optimizer
+  step, .to() since)."""
+  return tuple(ops.tensor_stamp(p) + (p.dtype,) for p in model.parameters())
+
+
 class _CapturedStep:
   """One cached single-token pass through the model, captured once as a HIP
   graph on fixed buffers (token ids, positions, every block's cache, logits)
@@ -39,6 +47,7 @@ class _CapturedStep:
 
   def __init__(self, model, batch_size, dtype, device):
     self.model = model
+    self.stamp = _parameter_stamp(model)
     ints = dict(device=device, dtype=torch.int32)
     self.tokens = torch.zeros((batch_size, 1), **ints)
     self.pos = torch.ones((batch_size, 1), **ints)
@@ -182,7 +191,9 @@ class Sampler:
     captured = None
     if self.use_graph and total_generation_steps > 2:
       captured = self._captured.get(bsz)
-      if captured is None:
+      stamp = _parameter_stamp(model)
+      if (captured is None or captured.stamp != stamp or
+          any(s[1] is None for s in stamp)):  # (no version counter: recapture)
         captured = self._captured[bsz] = _CapturedStep(model, bsz, self.dtype,
                                                        dev)
       captured.load(cache, pos)

@@ -198,6 +198,49 @@ def test_captured_decode_step_equals_eager(model, which):
                  if hasattr(b, "recurrent_block"))
 
 
+def test_captured_step_is_redone_after_a_weight_update():
+  """A captured step reads re-laid-out copies of the weights taken at capture
+  time: after the parameters are written in place the sampler must capture
+  again, not replay a graph that mixes old packed and new plain weights."""
+  m = _bf16_model()
+  g = torch.Generator().manual_seed(5)
+  toks = torch.randint(3, 512, (2, 7), generator=g).to(DEV, torch.int32)
+  lens = torch.tensor([7, 7], device=DEV, dtype=torch.int32)
+  graphed = S.Sampler(m, use_graph=True)
+  _, before = graphed.sample_tokens(toks, lens, 10, return_logits=True)
+  first = graphed._captured[2]
+  with torch.no_grad():
+    for p in m.parameters():
+      if p.dim() >= 2:
+        p.mul_(0.5)  # the logits change
+  want_t, want_l = S.Sampler(m).sample_tokens(toks, lens, 10, return_logits=True)
+  got_t, got_l = graphed.sample_tokens(toks, lens, 10, return_logits=True)
+  assert graphed._captured[2] is not first
+  assert torch.equal(got_t, want_t) and torch.equal(got_l, want_l)
+  assert not torch.equal(got_l, before)
+  # inference-mode tensors (no version counter) are accepted everywhere
+  with torch.inference_mode():
+    toks_i = toks.clone()
+    out_i, _ = S.Sampler(m).sample_tokens(toks_i, lens.clone(), 4)
+  assert torch.equal(out_i, want_t[:, :4])
+
+
+def test_stack_refuses_to_run_where_gradients_are_expected():
+  m = _bf16_model()
+  toks = torch.randint(3, 512, (1, 4)).to(DEV, torch.int32)
+  pos = torch.arange(4, device=DEV)[None]
+  m.train()
+  with pytest.raises(NotImplementedError, match="forward only"):
+    m(toks, pos)
+  with torch.no_grad():
+    m(toks, pos)  # fine without gradients
+  m.eval()
+  from recurrentgemma_amd import training
+  with training.differentiable():
+    with pytest.raises(NotImplementedError, match="forward only"):
+      m(toks, pos)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("hd", [16, 64, 256])
 def test_rope_kernel(dtype, hd):
