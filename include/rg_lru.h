@@ -130,8 +130,8 @@ int rg_linear_scan(const void* x, const void* a, const void* reset,
  * small (a single prompt: 10 to 16 workgroups).  These variants cut every
  * sequence into chunks that run as workgroups of their own: a first pass
  * reduces each chunk to (product of its a_t, its state from a zero start), a
- * small kernel chains those into every chunk's incoming state, a second pass
- * runs each chunk from there and writes y -- the scan operator is associative
+ * second pass chains those into its chunk's incoming state, runs the chunk
+ * from there and writes y -- the scan operator is associative
  * (recurrentgemma/jax/scan.py:161-187), this is the kernel's own cross-wave
  * carry one level up.  Twice the reads, none of the idling.
  * rg_scan_split_workspace_bytes is 0 for shapes
@@ -161,9 +161,12 @@ int rg_linear_scan_split(const void* x, const void* a, const void* reset,
  * h_last (nullable) float32 [B,W]; conv_cache_out (nullable) [B,3,W], the
  * masked tail described at rg_conv1d_prefill.  Same arithmetic as
  * rg_gates_gemm(apply_conv) followed by rg_lru_scan_fused(apply_conv), but the
- * conv output and the gate pre-activations stay on chip: one persistent
- * workgroup per (b, head) walks the sequence in 64-token tiles (conv -> LDS ->
- * bf16 MFMA -> gates -> in-register recurrence).  w_packed (nullable) is the
+ * conv output and the gate pre-activations stay on chip, the latter in
+ * float32 (the two-call form rounds them to bf16 on their way through memory,
+ * so the two agree to a bf16 unit or two, not bit for bit): one workgroup of
+ * four waves, one per SIMD, per (b, head) walks the sequence in 64-token tiles
+ * (x -> LDS by the memory pipe, conv -> LDS, bf16 MFMA on weights resident in
+ * accumulation registers, gates, in-register recurrence).  w_packed (nullable) is the
  * output of rg_pack_gate_weights for the same w_x / w_a (see below): with it
  * the kernel skips its own re-layout of the weights.  Returns RG_ERR_UNSUPPORTED
  * unless dtype is bf16, W/H == 256 and T*W*2 < 2^31; callers then use the
@@ -178,13 +181,14 @@ int rg_recurrent_prefill(const void* x, const void* segpos, int segpos_is_i64,
 
 /* rg_recurrent_prefill for few (row, head) pairs: one workgroup per pair
  * leaves most of the GPU idle below 256 pairs, so the sequences are cut into
- * chunks of whole 64-token tiles that run as workgroups of their own.  Pass 1
- * runs every chunk but the last from a zero state and keeps (prod a_t, h_end)
- * per chunk and channel, a small kernel chains them into every chunk's
- * incoming state (h_in[k+1] = P[k] h_in[k] + H[k]: the scan operator of
- * recurrentgemma/jax/scan.py:161-187, the algebra of multi_shard_correction,
- * jax/pallas.py:73-195, across workgroups instead of devices), pass 2 runs
- * every chunk from its incoming state and writes y.  `workspace` must hold
+ * chunks of whole 64-token tiles that run as workgroups of their own, in two
+ * launches.  The first runs chunk 0 for real (from h0, writing y) beside
+ * chunks 1 .. n-2 from a zero state, of which only (prod a_t, h_end) per
+ * channel is kept; the second runs chunks 1 .. n-1, each from the state it
+ * chains out of the summaries before it (h_in[k+1] = P[k] h_in[k] + H[k]: the
+ * scan operator of recurrentgemma/jax/scan.py:161-187, the algebra of
+ * multi_shard_correction, jax/pallas.py:73-195, across workgroups instead of
+ * devices), and writes y.  `workspace` (16-byte aligned) must hold
  * rg_recurrent_prefill_split_workspace_bytes(B, T, W, H) bytes; that is 0 for
  * shapes that are not cut, where the call is rg_recurrent_prefill itself.
  * Results equal rg_recurrent_prefill's up to the float32 association of the
