@@ -506,13 +506,14 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
 //
 // float32, block width 256, on v_mfma_f32_32x32x2_f32: true float32 products
 // and sums (no reduced-precision operand formats), so the 1e-5 bar of the
-// float32 path holds.  One workgroup of four waves per (32-row tile of x, half
-// of a head's 256 outputs, head and gate); wave w owns 32 output columns and
-// keeps their 256 x 32 weights in 128 registers for all the row tiles it
-// walks.  The row tile (optionally convolved on load) is staged through LDS.
-// Small tiles on purpose: the shapes that come here in float32 are small, and
-// 32 x 128 outputs per workgroup spread them over every CU, three workgroups
-// to a CU.
+// float32 path holds.  One workgroup of four waves per (32-row tile of x, a
+// quarter of a head's 256 outputs, head and gate); a wave owns 32 output
+// columns and one half of K and keeps its 128 x 32 weights in 64 registers for
+// all the row tiles it walks; the two halves of K meet in LDS.  The row tile
+// (optionally convolved on load) is staged through LDS.  Small work items on
+// purpose: the shapes that come here in float32 are small, and 32 x 64 outputs
+// per workgroup with K in halves make 64 matrix instructions per wave, which
+// spread evenly over the SIMDs (config 1: 1280 workgroups, five to a CU).
 //
 // Operand layout of the instruction: lane l supplies A[row l % 32][k = l / 32]
 // and B[k = l / 32][col l % 32] of a 32 x 2 by 2 x 32 product.  Which two k go
@@ -524,7 +525,7 @@ constexpr int kF32Stride = kBW + 4; // floats per LDS row (16 rows: 64 banks)
 constexpr size_t kF32LdsBytes = (size_t)kF32TM * kF32Stride * sizeof(float);
 
 template <bool CONV>
-__global__ void __launch_bounds__(256, 2) gates_mfma_f32_kernel(GemmArgs p) {
+__global__ void __launch_bounds__(256, 3) gates_mfma_f32_kernel(GemmArgs p) {
   extern __shared__ __align__(16) unsigned char f32_lds[];
   float* const As = reinterpret_cast<float*>(f32_lds);
   const int tid = threadIdx.x;
@@ -534,19 +535,20 @@ __global__ void __launch_bounds__(256, 2) gates_mfma_f32_kernel(GemmArgs p) {
   const int gate = z / p.H;
   const int h = z - gate * p.H;
   const int col = lane & 31, g = lane >> 5;
-  const int n = blockIdx.y * 128 + wave * 32 + col;  // output column in head
+  const int nb = wave & 1, kh = wave >> 1;  // column block, half of K
+  const int n = blockIdx.y * 64 + nb * 32 + col;  // output column in head
   const float* x = (const float*)p.x;
   const float* w = (const float*)p.w[gate] + (int64_t)h * kBW * kBW;
   float* out = (float*)p.out[gate];
   const int64_t W = p.W;
 
-  // this lane's weights: k = 8 j + 4 g + i at register 4 j + i
-  float bw_[128];
+  // this lane's weights: k = 128 kh + 8 j + 4 g + i at register 4 j + i
+  float bw_[64];
   {
     const __amdgpu_buffer_rsrc_t rw = make_rsrc(w, kBW * kBW * 4);
-    const uint32_t woff = (uint32_t)((4 * g) * kBW + n) * 4u;
+    const uint32_t woff = (uint32_t)((128 * kh + 4 * g) * kBW + n) * 4u;
 #pragma unroll
-    for (int j = 0; j < 32; ++j)
+    for (int j = 0; j < 16; ++j)
 #pragma unroll
       for (int i = 0; i < 4; ++i)
         bw_[4 * j + i] = __builtin_bit_cast(
@@ -578,10 +580,9 @@ __global__ void __launch_bounds__(256, 2) gates_mfma_f32_kernel(GemmArgs p) {
         if (m >= 0 && m < p.M)
           st = (m % p.T == 0) || is_doc_start(p.segpos, p.seg_kind, m);
       }
-      const uint64_t starts = __ballot(st);
       // Rows m0-3 .. m0+31 through a descriptor over just these rows (rows
-      // before the first and after the last read as zero), eight at a time:
-      // beside the weights there is no room for the values of a whole tile.
+      // before the first and after the last read as zero), all requested
+      // before the first is used: one memory round trip per tile.
       const int64_t first = m0 >= 3 ? m0 - 3 : 0;
       const int64_t last = m0 + kF32TM < p.M ? m0 + kF32TM : p.M;
       const __amdgpu_buffer_rsrc_t rx = make_rsrc(
@@ -589,40 +590,24 @@ __global__ void __launch_bounds__(256, 2) gates_mfma_f32_kernel(GemmArgs p) {
       const uint32_t row_bytes = (uint32_t)W * 4u;
       const uint32_t voff = (uint32_t)c * 4u;
       const int skip = (int)(first - (m0 - 3));  // rows before row 0: 0..3
-      float h1, h2, h3;  // x[m-1], x[m-2], x[m-3] of the next row
-      {
-        float hv[3];
+      float xv[kF32TM + 3];
 #pragma unroll
-        for (int r = 0; r < 3; ++r)
-          hv[r] = r < skip ? 0.0f
-                           : __builtin_bit_cast(
-                                 float, __builtin_amdgcn_raw_buffer_load_b32(
-                                            rx, voff,
-                                            (uint32_t)(r - skip) * row_bytes, 0));
-        h3 = hv[0]; h2 = hv[1]; h1 = hv[2];
-      }
+      for (int r = 0; r < kF32TM + 3; ++r)
+        xv[r] = r < skip ? 0.0f
+                         : __builtin_bit_cast(
+                               float, __builtin_amdgcn_raw_buffer_load_b32(
+                                          rx, voff,
+                                          (uint32_t)(r - skip) * row_bytes, 0));
+      const uint64_t starts = __ballot(st);  // (after the row loads are out)
 #pragma unroll
-      for (int part = 0; part < kF32TM / 8; ++part) {
-        float xv[8];
-#pragma unroll
-        for (int r = 0; r < 8; ++r)
-          xv[r] = __builtin_bit_cast(
-              float, __builtin_amdgcn_raw_buffer_load_b32(
-                         rx, voff,
-                         (uint32_t)(8 * part + r + 3 - skip) * row_bytes, 0));
-#pragma unroll
-        for (int r = 0; r < 8; ++r) {
-          // taps older than the newest document start of rows m-2 .. m are cut
-          const int rr = 8 * part + r;
-          const bool a1 = !((starts >> (2 + rr)) & 1);
-          const bool a2 = a1 && !((starts >> (1 + rr)) & 1);
-          const bool a3 = a2 && !((starts >> rr) & 1);
-          As[rr * kF32Stride + tid] =
-              conv4(xv[r], a1 ? h1 : 0.0f, a2 ? h2 : 0.0f, a3 ? h3 : 0.0f, cw0,
-                    cw1, cw2, cw3, cb);
-          h3 = h2; h2 = h1; h1 = xv[r];
-        }
-        __builtin_amdgcn_sched_barrier(0);
+      for (int r = 0; r < kF32TM; ++r) {
+        // taps older than the newest document start of rows m-2 .. m are cut
+        const bool a1 = !((starts >> (2 + r)) & 1);
+        const bool a2 = a1 && !((starts >> (1 + r)) & 1);
+        const bool a3 = a2 && !((starts >> r) & 1);
+        As[r * kF32Stride + tid] =
+            conv4(xv[r + 3], a1 ? xv[r + 2] : 0.0f, a2 ? xv[r + 1] : 0.0f,
+                  a3 ? xv[r] : 0.0f, cw0, cw1, cw2, cw3, cb);
       }
     } else {
 #pragma unroll 8
@@ -636,21 +621,33 @@ __global__ void __launch_bounds__(256, 2) gates_mfma_f32_kernel(GemmArgs p) {
     f32x16 acc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
-    const float* a_lane = As + col * kF32Stride + 4 * g;
+    const float* a_lane = As + col * kF32Stride + 128 * kh + 4 * g;
 #pragma unroll
-    for (int j = 0; j < 32; ++j) {
+    for (int j = 0; j < 16; ++j) {
       const f32x4 a = *reinterpret_cast<const f32x4*>(a_lane + 8 * j);
 #pragma unroll
       for (int i = 0; i < 4; ++i)
         acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], bw_[4 * j + i], acc, 0,
                                                    0, 0);
     }
-    // result register r of lane l: row 8 (r / 4) + 4 (l / 32) + r % 4, column
-    // l % 32
+    // the upper half of K hands its sums over through LDS (the staged tile is
+    // done with): [register][column block][lane], lanes next to each other
+    __syncthreads();
+    float* const red = As + nb * 64 + lane;
+    if (kh == 1) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int64_t m = m0 + 8 * (r >> 2) + 4 * g + (r & 3);
-      if (m < p.M) out[m * W + h * kBW + n] = acc[r] + bias;
+      for (int r = 0; r < 16; ++r) red[r * 128] = acc[r];
+    }
+    __syncthreads();
+    if (kh == 0) {
+      // result register r of lane l: row 8 (r / 4) + 4 (l / 32) + r % 4,
+      // column l % 32
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int64_t m = m0 + 8 * (r >> 2) + 4 * g + (r & 3);
+        if (m < p.M)
+          out[m * W + h * kBW + n] = (acc[r] + red[r * 128]) + bias;
+      }
     }
     __syncthreads();  // the tile is overwritten by the next round
   }
@@ -681,14 +678,14 @@ hipError_t launch_gemm_generic(const GemmArgs& a, int dtype, hipStream_t s) {
 hipError_t launch_gemm_mfma_f32(const GemmArgs& a, hipStream_t s) {
   // needs float32 and bw == 256 (checked by the caller); one or two gates
   const int64_t ntiles = (a.M + kF32TM - 1) / kF32TM;
-  // enough workgroups for every CU three times over; beyond that a workgroup
+  // enough workgroups for every CU five times over; beyond that a workgroup
   // walks several row tiles with its weights in place
-  const int64_t per_tile = 2 * (int64_t)a.H * a.ngates;
-  int64_t gx = (768 + per_tile - 1) / per_tile;
+  const int64_t per_tile = 4 * (int64_t)a.H * a.ngates;
+  int64_t gx = (1280 + per_tile - 1) / per_tile;
   if (gx > ntiles) gx = ntiles;
   if (gx < 1) gx = 1;
   if ((int64_t)a.H * a.ngates > 65535) return hipErrorInvalidValue;
-  dim3 grid((unsigned)gx, 2, (unsigned)(a.H * a.ngates));
+  dim3 grid((unsigned)gx, 4, (unsigned)(a.H * a.ngates));
   hipError_t e;
   if (a.apply_conv) {
     static OncePerDevice once;
