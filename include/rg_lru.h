@@ -204,6 +204,28 @@ int rg_recurrent_prefill_split(const void* x, const void* segpos,
                                void* workspace, size_t workspace_bytes, int B,
                                int T, int W, int H, int dtype, void* stream);
 
+/* The recurrent block between its linear layers in one kernel
+ * (RecurrentBlock.forward, recurrentgemma/torch/modules.py:627-644):
+ *   out = rglru(conv1d(x)) * gelu_tanh(gate_branch)
+ * x is the output of linear_x, gate_branch the output of linear_y before its
+ * activation, both [B,T,W]; out feeds linear_out.  rg_recurrent_prefill_split
+ * (whole rows or rows in chunks: same workspace rule, workspace may be null
+ * when rg_recurrent_prefill_split_workspace_bytes is 0) with the join of the
+ * two branches applied where y is stored: same values, bit for bit, as that
+ * call followed by rg_gelu_mul(y, gate_branch) (gelu rounded to `dtype` like
+ * the tensor it is in the reference, then the product rounded), without the
+ * pass over y in between.  out may alias gate_branch (every element is read
+ * before it is written, by the same lane); neither may alias x.  h_last and
+ * conv_cache_out as in rg_recurrent_prefill.  RG_ERR_UNSUPPORTED for the
+ * shapes rg_recurrent_prefill refuses: callers then use the separate calls. */
+int rg_recurrent_prefill_gelu_mul(
+    const void* x, const void* gate_branch, const void* segpos,
+    int segpos_is_i64, const void* conv_w, const void* conv_b, const void* w_x,
+    const void* b_x, const void* w_a, const void* b_a, const void* w_packed,
+    const void* a_param, const void* h0, void* out, void* h_last,
+    void* conv_cache_out, void* workspace, size_t workspace_bytes, int B, int T,
+    int W, int H, int dtype, void* stream);
+
 /* One decode step of the conv -> RG-LRU core, as RecurrentBlock.forward chains
  * them with a cache (recurrentgemma/torch/modules.py:632-643 with
  * layers.py:469-474 and :170-177): x [B,1,W], segpos [B,1],

@@ -346,7 +346,8 @@ static int recurrent_prefill_impl(const char* who, const void* x,
                                   const void* w_x, const void* b_x,
                                   const void* w_a, const void* b_a,
                                   const void* w_packed, const void* a_param,
-                                  const void* h0, void* y, void* h_last,
+                                  const void* h0, const void* gate_branch,
+                                  void* y, void* h_last,
                                   void* conv_cache_out, void* workspace,
                                   size_t workspace_bytes, bool split, int B,
                                   int T, int W, int H, int dtype,
@@ -369,6 +370,7 @@ static int recurrent_prefill_impl(const char* who, const void* x,
   RG_CHECK_OPT_PTR(h0);
   RG_CHECK_OPT_PTR(h_last);
   RG_CHECK_OPT_PTR(conv_cache_out);
+  RG_CHECK_OPT_PTR(gate_branch);
   RG_REQUIRE(y != x, "%s: y must not alias x", who);
   // The single-launch kernel exists for bf16 with 256-wide heads and
   // sequences whose byte offsets fit 31 bits; everything else is served by
@@ -394,6 +396,7 @@ static int recurrent_prefill_impl(const char* who, const void* x,
   a.a_param = a_param;
   a.h0 = (const float*)h0;
   a.y = y;
+  a.gate_branch = gate_branch;
   a.h_last = (float*)h_last;
   a.cache_out = conv_cache_out;
   a.B = B;
@@ -431,8 +434,8 @@ int rg_recurrent_prefill(const void* x, const void* segpos, int segpos_is_i64,
                          int W, int H, int dtype, void* stream) {
   return recurrent_prefill_impl(__func__, x, segpos, segpos_is_i64, conv_w,
                                 conv_b, w_x, b_x, w_a, b_a, w_packed, a_param,
-                                h0, y, h_last, conv_cache_out, nullptr, 0,
-                                false, B, T, W, H, dtype, stream);
+                                h0, nullptr, y, h_last, conv_cache_out,
+                                nullptr, 0, false, B, T, W, H, dtype, stream);
 }
 
 int rg_recurrent_prefill_split(const void* x, const void* segpos,
@@ -446,9 +449,25 @@ int rg_recurrent_prefill_split(const void* x, const void* segpos,
                                int T, int W, int H, int dtype, void* stream) {
   return recurrent_prefill_impl(__func__, x, segpos, segpos_is_i64, conv_w,
                                 conv_b, w_x, b_x, w_a, b_a, w_packed, a_param,
-                                h0, y, h_last, conv_cache_out, workspace,
-                                workspace_bytes, true, B, T, W, H, dtype,
-                                stream);
+                                h0, nullptr, y, h_last, conv_cache_out,
+                                workspace, workspace_bytes, true, B, T, W, H,
+                                dtype, stream);
+}
+
+int rg_recurrent_prefill_gelu_mul(
+    const void* x, const void* gate_branch, const void* segpos,
+    int segpos_is_i64, const void* conv_w, const void* conv_b, const void* w_x,
+    const void* b_x, const void* w_a, const void* b_a, const void* w_packed,
+    const void* a_param, const void* h0, void* out, void* h_last,
+    void* conv_cache_out, void* workspace, size_t workspace_bytes, int B, int T,
+    int W, int H, int dtype, void* stream) {
+  RG_CHECK_PTR(gate_branch);
+  RG_REQUIRE(gate_branch != x, "%s: gate_branch must not alias x", __func__);
+  return recurrent_prefill_impl(__func__, x, segpos, segpos_is_i64, conv_w,
+                                conv_b, w_x, b_x, w_a, b_a, w_packed, a_param,
+                                h0, gate_branch, out, h_last, conv_cache_out,
+                                workspace, workspace_bytes, true, B, T, W, H,
+                                dtype, stream);
 }
 
 #undef RG_WHO

@@ -104,13 +104,15 @@ struct FusedArgs {
   const void* a_param; // [W]
   const float* h0;     // [B, W] or null
   void* y;             // [B, T, W]
+  // or null: [B, T, W] bf16, the other branch of the recurrent block before
+  // its activation; y is then the block's join y * gelu(gate_branch)
+  const void* gate_branch;
   float* h_last;       // [B, W] or null
   void* cache_out;     // [B, 3, W] or null
   int B, T, W, H;
   // sequences cut into `chunks` chunks of tiles_per_chunk 64-token tiles
-  // (chunks <= 1: not cut), with three [B][chunks][W] float rows of
-  // workspace: every chunk's product of a_t, its state from a zero start, its
-  // incoming state
+  // (chunks <= 1: not cut), with two [B][chunks][W] float rows of workspace:
+  // every chunk's product of a_t and its state from a zero start
   int chunks, tiles_per_chunk;
   float* ws_p;
   float* ws_h;

@@ -192,7 +192,7 @@ struct BlockAcc {
   f32x16 v[kNB][2];
 };
 
-template <int MODE>
+template <int MODE, bool GELU>
 __device__ __forceinline__ void prefill_body(const FusedArgs& p,
                                              const int chunk) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
@@ -299,6 +299,10 @@ __device__ __forceinline__ void prefill_body(const FusedArgs& p,
       make_rsrc((const char*)p.x + (int64_t)b * seq_bytes, seq_bytes);
   const __amdgpu_buffer_rsrc_t ry = make_rsrc(
       (char*)p.y + (int64_t)b * seq_bytes, MODE == kChunkSummary ? 0 : seq_bytes);
+  // GELU: the block's other branch, read where y is written
+  const __amdgpu_buffer_rsrc_t rgate = make_rsrc(
+      (const char*)p.gate_branch + (int64_t)b * seq_bytes,
+      GELU && MODE != kChunkSummary ? seq_bytes : 0);
   const bool seg_is64 = p.seg_kind == kSegI64;
   const uint32_t seg_esize = seg_is64 ? 8u : 4u;
   const __amdgpu_buffer_rsrc_t rseg =
@@ -510,8 +514,26 @@ __device__ __forceinline__ void prefill_body(const FusedArgs& p,
   float hc[kNB] = {0.0f, 0.0f};    // carried state of this lane's channels
   float prod[kNB] = {1.0f, 1.0f};  // kChunkSummary: product of a, own tokens
   u32x4 y_pending[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+  u32x4 g_pending[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};  // GELU: same positions
   uint32_t y_pending_row = kBufferOutOfRange;  // byte offset of its first row
   auto flush_y = [&]() {
+    if (GELU) {
+      // y * gelu(gate branch), each factor a bf16 tensor as in the reference
+      // (recurrentgemma/torch/modules.py:627-628, 644): the arithmetic and
+      // roundings of the stand-alone gelu_mul pass
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const float lo =
+              gelu_mul_bf16(__uint_as_float(y_pending[j][k] << 16),
+                            __uint_as_float(g_pending[j][k] << 16));
+          const float hi =
+              gelu_mul_bf16(__uint_as_float(y_pending[j][k] & 0xffff0000u),
+                            __uint_as_float(g_pending[j][k] & 0xffff0000u));
+          y_pending[j][k] = pack_bf16x2(lo, hi);
+        }
+    }
     buffer_store_16(y_pending[0], ry, y_lane_bytes, y_pending_row);
     buffer_store_16(y_pending[1], ry, y_lane_bytes,
                     y_pending_row + 8u * row_bytes);
@@ -653,6 +675,12 @@ __device__ __forceinline__ void prefill_body(const FusedArgs& p,
                                                      8 * kPatchStride);
         __builtin_amdgcn_wave_barrier();
         y_pending_row = (uint32_t)(t_blk + 16 * (g >> 1)) * row_bytes;
+        if (GELU) {
+          g_pending[0] = __builtin_amdgcn_raw_buffer_load_b128(
+              rgate, y_lane_bytes + y_pending_row, 0, 0);
+          g_pending[1] = __builtin_amdgcn_raw_buffer_load_b128(
+              rgate, y_lane_bytes + y_pending_row + 8u * row_bytes, 0, 0);
+        }
       }
       pinned(8 * r + 7);
     }
@@ -857,30 +885,39 @@ enum PrefillPass { kPassWholeRows = 0, kPassFirst = 1, kPassReplay = 2 };
 // blockIdx.x: (row, head); blockIdx.y: which chunk (kPassFirst: chunk 0 with
 // its outputs beside the summaries of chunks 1 .. n-2; kPassReplay: chunks
 // 1 .. n-1).
-template <int PASS>
+// GELU: y is written as y * gelu(gate_branch), the join of the recurrent
+// block's two branches, instead of the plain RG-LRU output.
+template <int PASS, bool GELU>
 __global__ void __launch_bounds__(kThreads) block_prefill_bf16_kernel(
     FusedArgs p) {
   if (PASS == kPassWholeRows) {
-    prefill_body<kWholeRow>(p, 0);
+    prefill_body<kWholeRow, GELU>(p, 0);
   } else if (PASS == kPassReplay) {
-    prefill_body<kChunkReplay>(p, (int)blockIdx.y + 1);
+    prefill_body<kChunkReplay, GELU>(p, (int)blockIdx.y + 1);
   } else if (blockIdx.y == 0) {
-    prefill_body<kChunkHead>(p, 0);
+    prefill_body<kChunkHead, GELU>(p, 0);
   } else {
-    prefill_body<kChunkSummary>(p, (int)blockIdx.y);
+    prefill_body<kChunkSummary, false>(p, (int)blockIdx.y);
   }
+}
+
+template <int PASS, bool GELU>
+hipError_t launch_pass_as(const FusedArgs& a, int grid_y, hipStream_t s) {
+  static OncePerDevice once;
+  hipError_t e = set_max_dynamic_lds(
+      once, (const void*)block_prefill_bf16_kernel<PASS, GELU>,
+      kPrefillLdsBytes);
+  if (e != hipSuccess) return e;
+  block_prefill_bf16_kernel<PASS, GELU>
+      <<<dim3((unsigned)(a.B * a.H), (unsigned)grid_y), kThreads,
+         kPrefillLdsBytes, s>>>(a);
+  return hipGetLastError();
 }
 
 template <int PASS>
 hipError_t launch_pass(const FusedArgs& a, int grid_y, hipStream_t s) {
-  static OncePerDevice once;
-  hipError_t e = set_max_dynamic_lds(
-      once, (const void*)block_prefill_bf16_kernel<PASS>, kPrefillLdsBytes);
-  if (e != hipSuccess) return e;
-  block_prefill_bf16_kernel<PASS>
-      <<<dim3((unsigned)(a.B * a.H), (unsigned)grid_y), kThreads,
-         kPrefillLdsBytes, s>>>(a);
-  return hipGetLastError();
+  if (a.gate_branch) return launch_pass_as<PASS, true>(a, grid_y, s);
+  return launch_pass_as<PASS, false>(a, grid_y, s);
 }
 
 }  // namespace

@@ -54,12 +54,16 @@ def _single_launch_pays(x, num_heads) -> bool:
 @torch.no_grad()
 def recurrent_core(conv_1d: layers.Conv1D, rg_lru: layers.RGLRU, x,
                    segment_pos, cache: RecurrentBlockCache | None = None,
-                   return_cache: bool = True, in_place: bool = False):
+                   return_cache: bool = True, in_place: bool = False,
+                   gate_branch=None):
   """conv_1d -> rg_lru exactly as RecurrentBlock.forward chains them
   (modules.py:632-643), fused.  Returns (y, RecurrentBlockCache | None).
   in_place (decode only): the step overwrites the tensors of `cache` and
   returns them, for callers that replay a captured step on fixed buffers; the
-  default returns new tensors like the reference."""
+  default returns new tensors like the reference.
+  gate_branch: the block's linear_y output; the result is then the join
+  y * gelu(gate_branch) of modules.py:627-628, 644 -- inside the prefill
+  kernel where that runs, as a pass of its own (ops.gelu_mul) elsewhere."""
   bs, l, _ = x.shape
   assert segment_pos.shape == (bs, l)
   fused = conv_1d.temporal_width == 4
@@ -72,6 +76,8 @@ def recurrent_core(conv_1d: layers.Conv1D, rg_lru: layers.RGLRU, x,
           x, segment_pos, cache.conv1d_state, cache.rg_lru_state, conv_1d.w,
           conv_1d.b, rg_lru.input_gate.w, rg_lru.input_gate.b, rg_lru.a_gate.w,
           rg_lru.a_gate.b, rg_lru.a_param, in_place=in_place)
+      if gate_branch is not None:
+        y = ops.gelu_mul(y, gate_branch)
       if not return_cache:
         return y, None
       return y, RecurrentBlockCache(rg_lru_state=h, conv1d_state=conv_state)
@@ -86,11 +92,20 @@ def recurrent_core(conv_1d: layers.Conv1D, rg_lru: layers.RGLRU, x,
   elif _single_launch_pays(x, rg_lru.num_heads):
     # one workgroup per (row, head) -- or per chunk of one -- pays once there
     # are enough of them to fill the GPU; otherwise the two-kernel form
-    # spreads over more CUs
+    # spreads over more CUs.  The join with the gate branch goes into the
+    # kernel for whole rows (measured at B16 T8192 W4096: 1.15 ms against
+    # 0.91 + 0.40 ms apart); with rows in chunks it would lengthen the one
+    # workgroup per row that produces outputs in the first launch while the
+    # others only summarise, and the separate pass is as fast (0.33 ms both
+    # ways at B8 T4096 W2560).
+    chunked = ops.recurrent_prefill_chunked(bs, l, x.shape[2], rg_lru.num_heads)
     y, h, conv_state = ops.recurrent_prefill(
         x, segment_pos, conv_1d.w, conv_1d.b, rg_lru.input_gate.w,
         rg_lru.input_gate.b, rg_lru.a_gate.w, rg_lru.a_gate.b, rg_lru.a_param,
-        h0=None, return_h=return_cache, return_conv_cache=return_cache)
+        h0=None, return_h=return_cache, return_conv_cache=return_cache,
+        gate_branch=None if chunked else gate_branch)
+    if not chunked:
+      gate_branch = None  # joined inside the kernel
   else:
     gx_pre, ga_pre = ops.gates_gemm(
         x, rg_lru.input_gate.w, rg_lru.input_gate.b, rg_lru.a_gate.w,
@@ -99,6 +114,8 @@ def recurrent_core(conv_1d: layers.Conv1D, rg_lru: layers.RGLRU, x,
         x, gx_pre, ga_pre, rg_lru.a_param, segment_pos, h0=None,
         conv=(conv_1d.w, conv_1d.b), return_h=return_cache,
         return_conv_cache=return_cache)
+  if gate_branch is not None:
+    y = ops.gelu_mul(y, gate_branch)
   if not return_cache:
     return y, None
   return y, RecurrentBlockCache(rg_lru_state=h, conv1d_state=conv_state)
@@ -170,10 +187,12 @@ class RecurrentBlock(nn.Module):
       else:
         y = self.linear_y(x)
         x = self.linear_x(x)
+      # x * gelu(y) (modules.py:627-628, 644) is part of the core call: inside
+      # the prefill kernel where that runs, one pass after it elsewhere
       x, new_cache = recurrent_core(
           self.conv_1d, self.rg_lru, x, segment_pos, cache, return_cache,
-          in_place=self.decode_in_place and cache is not None and return_cache)
-      x = ops.gelu_mul(x, y)  # x * gelu(y), one pass (modules.py:627-628, 644)
+          in_place=self.decode_in_place and cache is not None and return_cache,
+          gate_branch=y)
       if few_rows and defer_out and ops.PackedLinear.partial_slices(
           x, self.lru_width, self.width):
         x = self._rows_out.partial(x, (self.linear_out.weight,),

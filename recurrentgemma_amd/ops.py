@@ -223,14 +223,16 @@ def recurrent_prefill_chunked(B, T, W, num_heads) -> bool:
 
 def recurrent_prefill(x, segment_pos, conv_w, conv_b, w_x, b_x, w_a, b_a,
                       a_param, h0=None, return_h=True, return_conv_cache=True,
-                      split=True):
+                      split=True, gate_branch=None):
   """conv -> gates -> recurrence of a whole prefill in one launch.
 
   Returns (y, h_last | None, conv_cache | None).  Only for the shapes
   recurrent_prefill_supported() accepts; other shapes go through gates_gemm +
   lru_scan_fused.  split: with few (row, head) pairs the sequences are cut
   into chunks that run side by side (rg_recurrent_prefill_split); False forces
-  one workgroup per pair.
+  one workgroup per pair.  gate_branch: the output of the block's linear_y
+  ([B,T,W], before its activation); y is then y * gelu(gate_branch), the input
+  of linear_out (rg_recurrent_prefill_gelu_mul).
   """
   B, T, W = x.shape
   H = w_x.shape[0]
@@ -258,8 +260,21 @@ def recurrent_prefill(x, segment_pos, conv_w, conv_b, w_x, b_x, w_a, b_a,
   lib = _lib.lib()
   need = (lib.rg_recurrent_prefill_split_workspace_bytes(B, T, W, H)
           if split else 0)
+  if gate_branch is not None:
+    assert split, "the joined form decides about chunks itself"
+    assert gate_branch.shape == x.shape
+    _same(x.dtype, x.device, gate_branch=gate_branch)
+    gate_branch = _dev(gate_branch, "gate_branch")
   with torch.cuda.device(x.device):
-    if need:
+    if gate_branch is not None:
+      ws = (torch.empty(need, dtype=torch.uint8, device=x.device)
+            if need else None)
+      _lib.check(lib.rg_recurrent_prefill_gelu_mul(
+          _p(x), _p(gate_branch), _p(seg), is64, _p(cw), _p(cb), _p(wx_),
+          _p(bx_), _p(wa_), _p(ba_), _p(packed), _p(ap_), _p(h0), _p(y),
+          _p(h_last), _p(cache), _p(ws), need, B, T, W, H, _dtype_code(x),
+          _stream(x)))
+    elif need:
       ws = torch.empty(need, dtype=torch.uint8, device=x.device)
       _lib.check(lib.rg_recurrent_prefill_split(
           _p(x), _p(seg), is64, _p(cw), _p(cb), _p(wx_), _p(bx_), _p(wa_),

@@ -446,6 +446,40 @@ def test_recurrent_block_module():
   assert helpers.max_rel(got1, want[:, :1]) < 1e-4
 
 
+def test_recurrent_block_module_joined_kernel(monkeypatch):
+  """bf16 RecurrentBlock with enough (row, head) pairs for the prefill kernel
+  that also applies the x * gelu(y) join: one core launch, no gelu_mul pass,
+  and the block output bit for bit what the separate pass gives."""
+  B, T, width, H = 80, 70, 512, 2  # 160 pairs
+  torch.manual_seed(6)
+  blk = rg.RecurrentBlock(width=width, num_heads=H,
+                          dtype=torch.bfloat16).to(DEV)
+  with torch.no_grad():
+    blk.linear_y.bias.normal_(0, 0.3)
+    blk.rg_lru.input_gate.b.normal_(0, 0.3)
+  x = _dev(torch.randn(B, T, width).to(torch.bfloat16))
+  seg = _dev(helpers.document_positions(B, T, 25, seed=4))
+  calls = []
+  real_gelu_mul, real_prefill = ops.gelu_mul, ops.recurrent_prefill
+  monkeypatch.setattr(ops, "gelu_mul",
+                      lambda *a, **k: calls.append("gelu_mul") or
+                      real_gelu_mul(*a, **k))
+  monkeypatch.setattr(ops, "recurrent_prefill",
+                      lambda *a, **k: calls.append(
+                          ("prefill", k.get("gate_branch") is not None)) or
+                      real_prefill(*a, **k))
+  got, cache = blk(x, seg)
+  assert calls == [("prefill", True)], calls
+  # the same block with the join as a pass of its own
+  yb = blk.linear_y(x)
+  core, cache2 = rg.recurrent_core(blk.conv_1d, blk.rg_lru, blk.linear_x(x),
+                                   seg)
+  want = blk.linear_out(real_gelu_mul(core, yb))
+  assert torch.equal(got, want)
+  assert torch.equal(cache.rg_lru_state, cache2.rg_lru_state)
+  assert torch.equal(cache.conv1d_state, cache2.conv1d_state)
+
+
 # ------------------------------------------- single-launch prefill kernel --
 
 
@@ -519,6 +553,64 @@ def test_recurrent_prefill_single_launch(B, T, W, H, mean_doc, seg_dtype,
   assert (y1.float() - y.float()).abs().max().item() <= 0.0625
   if not ops.recurrent_prefill_chunked(B, T, W, H):
     assert torch.equal(y1, y) and torch.equal(h1, h)
+
+
+@pytest.mark.parametrize("B,T,W,H,mean_doc", [
+    (2, 200, 512, 2, 37),      # whole rows, ragged last tile, documents
+    (1, 70, 256, 1, None),
+    (1, 1024, 512, 2, 300),    # rows in chunks
+    (3, 640, 768, 3, None),
+    (40, 130, 1024, 4, 50),    # 160 (row, head) pairs
+])
+def test_prefill_joined_with_gate_branch(B, T, W, H, mean_doc):
+  """rg_recurrent_prefill_gelu_mul (the block's x * gelu(y) join applied where
+  the prefill kernel stores its output) against the same kernel followed by
+  rg_gelu_mul: bit for bit, also with the output written over the gate branch;
+  state outputs identical."""
+  _announce("prefill joined", B, T, W, H, mean_doc)
+  seed = 7300 + T
+  p = R.make_params(W, H, torch.bfloat16, seed=seed, gate_bias_std=0.5)
+  g = torch.Generator().manual_seed(seed + 1)
+  x = _dev(torch.randn(B, T, W, generator=g).to(torch.bfloat16))
+  gate = _dev((torch.randn(B, T, W, generator=g) * 2).to(torch.bfloat16))
+  seg = (torch.arange(T).expand(B, T).contiguous() if mean_doc is None
+         else helpers.document_positions(B, T, mean_doc, seed=seed))
+  segd = _dev(seg)
+  P = {k: _dev(v) for k, v in p.items()}
+  args = (x, segd, P["conv_w"], P["conv_b"], P["w_x"], P["b_x"], P["w_a"],
+          P["b_a"], P["a_param"])
+  y, h, cache = ops.recurrent_prefill(*args)
+  want = ops.gelu_mul(y, gate)
+  got, h2, cache2 = ops.recurrent_prefill(*args, gate_branch=gate)
+  assert torch.equal(got, want)
+  assert torch.equal(h2, h) and torch.equal(cache2, cache)
+  # the reference's op sequence on the same values
+  ref = (y.float() * torch.nn.functional.gelu(
+      gate.float(), approximate="tanh").to(torch.bfloat16).float()).to(
+          torch.bfloat16)
+  assert helpers.max_rel(got, ref) < BF16_TOL
+  # through the C ABI with the output over the gate branch
+  from recurrentgemma_amd import _lib
+  lib = _lib.lib()
+  need = lib.rg_recurrent_prefill_split_workspace_bytes(B, T, W, H)
+  ws = torch.empty(max(need, 16), dtype=torch.uint8, device=DEV)
+  over = gate.clone()
+  ptr = lambda t: t.data_ptr()
+  _lib.check(lib.rg_recurrent_prefill_gelu_mul(
+      ptr(x), ptr(over), ptr(segd), 1, ptr(P["conv_w"]), ptr(P["conv_b"]),
+      ptr(P["w_x"]), ptr(P["b_x"]), ptr(P["w_a"]), ptr(P["b_a"]), None,
+      ptr(P["a_param"]), None, ptr(over), None, None,
+      ptr(ws) if need else None, need, B, T, W, H, 1, None))
+  torch.cuda.synchronize()
+  assert torch.equal(over, want)
+  # refused where the plain call is
+  xf = x.float()
+  rc = lib.rg_recurrent_prefill_gelu_mul(
+      ptr(xf), ptr(gate), ptr(segd), 1, ptr(P["conv_w"]), ptr(P["conv_b"]),
+      ptr(P["w_x"]), ptr(P["b_x"]), ptr(P["w_a"]), ptr(P["b_a"]), None,
+      ptr(P["a_param"]), None, ptr(over), None, None, None, 0, B, T, W, H, 0,
+      None)
+  assert rc == -2
 
 
 @pytest.mark.parametrize("B,W,H,in_place", [(1, 256, 1, False),
