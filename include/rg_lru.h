@@ -125,6 +125,22 @@ int rg_linear_scan(const void* x, const void* a, const void* reset,
                    const void* h0, void* y, void* h_last, int B, int T, int W,
                    int dtype, void* stream);
 
+/* Backward pass of rnn_scan (what autograd computes through the loop of
+ * recurrentgemma/torch/layers.py:181-189; the reference's own formulation is
+ * recurrentgemma/jax/pallas.py:792-846: the recurrence on dy from the end of
+ * the sequence, then da = dx * y shifted by one step).  With a' = a zeroed at
+ * resets:
+ *   g_t = dy_t + a'_{t+1} g_{t+1}  (the term behind the last token is dh_last)
+ *   dx_t = g_t,  da_t = g_t * h_{t-1} (0 at resets; h_{-1} = h0),  dh0 = a'_0 g_0
+ * dy, a, y, dx, da [B,T,W] in `dtype` (y: the forward output), reset [B,T]
+ * bytes, h0 / dh_last / dh0 (all nullable) float32 [B,W].  The recurrence runs
+ * in float32; dx is g rounded to `dtype`, da the product of the rounded g and
+ * y rounded again.  dx may alias dy; no other aliasing. */
+int rg_linear_scan_backward(const void* dy, const void* a, const void* reset,
+                            const void* y, const void* h0, const void* dh_last,
+                            void* dx, void* da, void* dh0, int B, int T, int W,
+                            int dtype, void* stream);
+
 /* The two scans above for few rows and channels: one workgroup per (row, slab
  * of 256 or 128 channels) leaves most of the GPU idle when B * W / 256 is
  * small (a single prompt: 10 to 16 workgroups).  These variants cut every

@@ -525,6 +525,42 @@ int rg_linear_scan_split(const void* x, const void* a, const void* reset,
                           workspace_bytes, true, B, T, W, dtype, stream);
 }
 
+int rg_linear_scan_backward(const void* dy, const void* a, const void* reset,
+                            const void* y, const void* h0, const void* dh_last,
+                            void* dx, void* da, void* dh0, int B, int T, int W,
+                            int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(B > 0 && T > 0 && W > 0, "%s: B=%d T=%d W=%d must be positive",
+             __func__, B, T, W);
+  RG_CHECK_PTR(dy);
+  RG_CHECK_PTR(a);
+  RG_CHECK_PTR(reset);
+  RG_CHECK_PTR(y);
+  RG_CHECK_PTR(dx);
+  RG_CHECK_PTR(da);
+  RG_CHECK_OPT_PTR(h0);
+  RG_CHECK_OPT_PTR(dh_last);
+  RG_CHECK_OPT_PTR(dh0);
+  RG_REQUIRE(dx != a && dx != y && da != a && da != y && da != dy && dx != da,
+             "%s: dx and da must not alias a, y or each other (da nor dy)",
+             __func__);
+  rg::ScanBwdArgs s{};
+  s.dy = dy;
+  s.a = a;
+  s.reset = reset;
+  s.y = y;
+  s.h0 = (const float*)h0;
+  s.dh_last = (const float*)dh_last;
+  s.dx = dx;
+  s.da = da;
+  s.dh0 = (float*)dh0;
+  s.B = B;
+  s.T = T;
+  s.W = W;
+  return launch_status(__func__, rg::launch_linear_scan_backward(
+                                     s, dtype, (hipStream_t)stream));
+}
+
 size_t rg_recurrent_step_workspace_bytes(int B, int W, int dtype) {
   if (B <= 0 || W <= 0) return 0;
   // conv output + two gate pre-activations, each [B,W], 256-byte aligned

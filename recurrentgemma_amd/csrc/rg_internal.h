@@ -153,6 +153,22 @@ hipError_t launch_gemm_generic(const GemmArgs& a, int dtype, hipStream_t s);
 hipError_t launch_gemm_mfma_bf16(const GemmArgs& a, hipStream_t s);
 hipError_t launch_gemm_mfma_f32(const GemmArgs& a, hipStream_t s);
 hipError_t launch_lru_scan(const ScanArgs& a, int dtype, hipStream_t s);
+
+// Backward pass of rnn_scan (rg_scan_bwd.hip).
+struct ScanBwdArgs {
+  const void* dy;        // [B, T, W] gradient of y
+  const void* a;         // [B, T, W] the forward coefficients
+  const void* reset;     // [B, T] bytes
+  const void* y;         // [B, T, W] the forward outputs
+  const float* h0;       // [B, W] or null
+  const float* dh_last;  // [B, W] or null: gradient of the final state
+  void* dx;              // [B, T, W]
+  void* da;              // [B, T, W]
+  float* dh0;            // [B, W] or null
+  int B, T, W;
+};
+hipError_t launch_linear_scan_backward(const ScanBwdArgs& a, int dtype,
+                                       hipStream_t s);
 void scan_split_plan(int B, int T, int W, int granule, int* chunks,
                      int* t_chunk);
 // Chunk lengths are multiples of this for the kernel that handles (dtype, W).

@@ -312,6 +312,32 @@ def linear_scan(x, a, reset, h0=None, split=True):
   return y, h_last
 
 
+def linear_scan_backward(dy, a, reset, y, h0=None, dh_last=None):
+  """Gradients of linear_scan: (dx, da, dh0 | None) from the gradient of y
+  (and of the final state); one kernel, no flipped copies."""
+  B, T, W = y.shape
+  y = _dev(y, "y")
+  _same(y.dtype, y.device, dy=dy, a=a)
+  dy, a = _dev(dy, "dy"), _dev(a, "a")
+  assert dy.shape == a.shape == y.shape
+  assert reset.shape == (B, T) and reset.dtype == torch.bool
+  reset = _dev(reset, "reset")
+  if h0 is not None:
+    assert h0.dtype == torch.float32 and h0.shape == (B, W)
+    h0 = _dev(h0, "h0")
+  if dh_last is not None:
+    assert dh_last.dtype == torch.float32 and dh_last.shape == (B, W)
+    dh_last = _dev(dh_last, "dh_last")
+  dx, da = torch.empty_like(y), torch.empty_like(y)
+  dh0 = (torch.empty((B, W), dtype=torch.float32, device=y.device)
+         if h0 is not None else None)
+  with torch.cuda.device(y.device):
+    _lib.check(_lib.lib().rg_linear_scan_backward(
+        _p(dy), _p(a), _p(reset), _p(y), _p(h0), _p(dh_last), _p(dx), _p(da),
+        _p(dh0), B, T, W, _dtype_code(y), _stream(y)))
+  return dx, da, dh0
+
+
 def _workspace(B, W, dtype, device):
   """Scratch of one rg_recurrent_step call, allocated per call: under graph
   capture it then comes from the graph's own pool and stays valid for the

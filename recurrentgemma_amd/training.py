@@ -59,23 +59,9 @@ class _LinearScan(torch.autograd.Function):
   @staticmethod
   def backward(ctx, dy, dh_last):
     a, reset, y, h0 = ctx.saved_tensors
-    B, T, W = y.shape
-    a_eff = a * (~reset)[..., None].to(a.dtype)
-    # time reversed, coefficient of step s = a'_{T-s} (s >= 1); step 0 takes
-    # dh_last in as the initial state with coefficient one
-    a_rev = torch.cat([torch.ones_like(a_eff[:, :1]),
-                       torch.flip(a_eff[:, 1:], dims=[1])], dim=1)
-    dy_rev = torch.flip(dy, dims=[1]).contiguous()
-    carry = (torch.zeros((B, W), dtype=torch.float32, device=y.device)
-             if dh_last is None else dh_last.float().contiguous())
-    no_reset = torch.zeros((B, T), dtype=torch.bool, device=y.device)
-    g_rev, g0 = ops.linear_scan(dy_rev, a_rev.contiguous(), no_reset, carry)
-    g = torch.flip(g_rev, dims=[1])
-    first = (torch.zeros_like(y[:, :1]) if h0 is None
-             else h0.to(y.dtype)[:, None])
-    h_prev = torch.cat([first, y[:, :-1]], dim=1)
-    da = g * h_prev * (~reset)[..., None].to(g.dtype)
-    dh0 = None if h0 is None else a_eff[:, 0].float() * g0
+    dh = None if dh_last is None else dh_last.float().contiguous()
+    dy = torch.zeros_like(y) if dy is None else dy.contiguous()
+    g, da, dh0 = ops.linear_scan_backward(dy, a, reset, y, h0, dh)
     return g, da, None, dh0
 
 

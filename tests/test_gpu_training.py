@@ -87,7 +87,7 @@ def test_rglru_gradients_with_initial_state(golden):
     close(p.grad, golden[f"lru/grad/{name}"], "d" + name)
 
 
-@pytest.mark.parametrize("T", [1, 2, 65, 300])
+@pytest.mark.parametrize("T", [1, 2, 65, 300, 2050])
 def test_scan_gradients_against_sequential_loop(T):
   """The scan Function alone against autograd through a float64 Python loop
   on the CPU, with resets and an initial state, at lengths that span one and
@@ -115,3 +115,48 @@ def test_scan_gradients_against_sequential_loop(T):
   close(xg.grad, xd.grad.float().numpy(), "dx")
   close(ag.grad, ad.grad.float().numpy(), "da")
   close(hg.grad, hd.grad.float().numpy(), "dh0")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,T,W", [(2, 1, 64), (3, 17, 96), (1, 333, 130),
+                                   (2, 1000, 257), (1, 4099, 512)])
+def test_scan_backward_kernel(dtype, B, T, W):
+  """rg_linear_scan_backward against its definition evaluated step by step in
+  float64 on the same (dtype-valued) inputs: g_t = dy_t + a'_{t+1} g_{t+1}
+  with dh_last behind the last token, dx = g, da = g h_{t-1} masked at resets,
+  dh0 = a'_0 g_0; widths that take two channels per lane and one, sequences
+  from one token to several rows per wave, with and without h0 / dh_last."""
+  from recurrentgemma_amd import ops
+  gen = torch.Generator().manual_seed(B * 1000 + T)
+  dy = torch.randn(B, T, W, generator=gen).to(dtype)
+  a = (torch.rand(B, T, W, generator=gen) * 0.6 + 0.4).to(dtype)
+  y = torch.randn(B, T, W, generator=gen).to(dtype)
+  reset = torch.rand(B, T, generator=gen) < 0.05
+  h0 = torch.randn(B, W, generator=gen)
+  dh_last = torch.randn(B, W, generator=gen)
+  tol = 1e-5 if dtype == torch.float32 else 1e-2
+  for with_state in (True, False):
+    got_dx, got_da, got_dh0 = ops.linear_scan_backward(
+        dy.to(DEV), a.to(DEV), reset.to(DEV), y.to(DEV),
+        h0.to(DEV) if with_state else None,
+        dh_last.to(DEV) if with_state else None)
+    ae = a.double() * (~reset)[..., None]
+    g = dh_last.double() if with_state else torch.zeros(B, W, dtype=torch.float64)
+    dx = torch.zeros(B, T, W, dtype=torch.float64)
+    for t in range(T - 1, -1, -1):
+      coef = ae[:, t + 1] if t + 1 < T else 1.0
+      g = dy[:, t].double() + coef * g
+      dx[:, t] = g
+    first = (h0.to(dtype).double() if with_state
+             else torch.zeros(B, W, dtype=torch.float64))
+    h_prev = torch.cat([first[:, None], y[:, :-1].double()], dim=1)
+    da = dx * h_prev * (~reset)[..., None]
+    scale = lambda t: t.abs().max().clamp_min(1e-30)
+    assert ((got_dx.double().cpu() - dx).abs().max() / scale(dx)) < tol
+    assert ((got_da.double().cpu() - da).abs().max() / scale(da)) < tol
+    assert got_dx.dtype == dtype and got_da.dtype == dtype
+    if with_state:
+      dh0 = ae[:, 0] * dx[:, 0]
+      assert ((got_dh0.double().cpu() - dh0).abs().max() / scale(dh0)) < 1e-5
+    else:
+      assert got_dh0 is None
