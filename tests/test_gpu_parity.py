@@ -499,6 +499,8 @@ def test_recurrent_block_module_joined_kernel(monkeypatch):
     (2, 2048, 256, 1, None, torch.int64, False),
     (1, 777, 768, 3, 100, torch.int32, True),
     (3, 1500, 256, 1, 7, torch.int64, False),
+    (1, 8192, 256, 1, 1024, torch.int64, True),  # 64 chunks of two tiles
+    (2, 900, 256, 1, -300, torch.int32, False),  # chunks, left padding
 ])
 def test_recurrent_prefill_single_launch(B, T, W, H, mean_doc, seg_dtype,
                                          with_h0):
