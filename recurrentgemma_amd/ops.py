@@ -65,7 +65,29 @@ def _segpos(segment_pos: torch.Tensor, B: int, T: int):
 
 
 def _stream(t: torch.Tensor) -> int:
-  return torch.cuda.current_stream(t.device).cuda_stream
+  # (the raw handle: current_stream() builds a Stream object per call, which
+  # is a microsecond of a decode step's host time)
+  return torch._C._cuda_getCurrentRawStream(t.device.index)
+
+
+class _NoGuard:
+  def __enter__(self):
+    return None
+
+  def __exit__(self, *exc):
+    return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def _on(device):
+  """Context that makes `device` the current one for a launch; free when it
+  already is (entering torch.cuda.device costs more than the rest of the
+  argument handling of a small call)."""
+  if torch.cuda.current_device() == device.index:
+    return _NO_GUARD
+  return torch.cuda.device(device)
 
 
 def _p(t):
@@ -83,7 +105,7 @@ def conv1d_prefill(x, segment_pos, w, b, return_cache=True):
   seg, is64 = _segpos(segment_pos, B, T)
   out = torch.empty_like(x)
   cache = x.new_empty((B, K - 1, W)) if return_cache else None
-  with torch.cuda.device(x.device):
+  with _on(x.device):
     _lib.check(_lib.lib().rg_conv1d_prefill(
         _p(x), _p(seg), is64, _p(w), _p(b), _p(out), _p(cache), B, T, W, K,
         _dtype_code(x), _stream(x)))
@@ -101,7 +123,7 @@ def conv1d_step(x, cache, w, b, return_cache=True):
   cache_in = _dev(cache.to(x.dtype), "cache")
   out = torch.empty_like(x)
   new_cache = torch.empty_like(cache_in) if return_cache else None
-  with torch.cuda.device(x.device):
+  with _on(x.device):
     _lib.check(_lib.lib().rg_conv1d_step(
         _p(x), _p(cache_in), _p(w), _p(b), _p(out), _p(new_cache), B, W, K,
         _dtype_code(x), _stream(x)))
@@ -122,7 +144,7 @@ def block_diag_linear(x, w, b):
   M = x.numel() // (H * bw)
   if M == 0:
     return y
-  with torch.cuda.device(x.device):
+  with _on(x.device):
     _lib.check(_lib.lib().rg_block_diag_linear(
         _p(x), _p(w), _p(b), _p(y), M, H, bw, _dtype_code(x), _stream(x)))
   return y
@@ -148,7 +170,7 @@ def gates_gemm(x, w_x, b_x, w_a, b_a, conv=None):
     seg, is64 = _segpos(segment_pos, B, T)
   gx = torch.empty_like(x)
   ga = torch.empty_like(x)
-  with torch.cuda.device(x.device):
+  with _on(x.device):
     _lib.check(_lib.lib().rg_gates_gemm(
         _p(x), int(conv is not None), _p(seg), is64, _p(cw), _p(cb), _p(w_x),
         _p(b_x), _p(w_a), _p(b_a), _p(gx), _p(ga), B, T, W, H, _dtype_code(x),
@@ -193,7 +215,7 @@ def lru_scan_fused(x, gx_pre, ga_pre, a_param, segment_pos, h0=None, conv=None,
     assert conv is not None
     cache = x.new_empty((B, 3, W))
   ws = _scan_workspace(B, T, W, x.device, split)
-  with torch.cuda.device(x.device):
+  with _on(x.device):
     if ws is None:
       _lib.check(_lib.lib().rg_lru_scan_fused(
           _p(x), int(conv is not None), _p(cw), _p(cb), _p(gx_pre), _p(ga_pre),
@@ -265,7 +287,7 @@ def recurrent_prefill(x, segment_pos, conv_w, conv_b, w_x, b_x, w_a, b_a,
     assert gate_branch.shape == x.shape
     _same(x.dtype, x.device, gate_branch=gate_branch)
     gate_branch = _dev(gate_branch, "gate_branch")
-  with torch.cuda.device(x.device):
+  with _on(x.device):
     if gate_branch is not None:
       ws = (torch.empty(need, dtype=torch.uint8, device=x.device)
             if need else None)
@@ -300,7 +322,7 @@ def linear_scan(x, a, reset, h0=None, split=True):
   y = torch.empty_like(x)
   h_last = torch.empty((B, W), dtype=torch.float32, device=x.device)
   ws = _scan_workspace(B, T, W, x.device, split)
-  with torch.cuda.device(x.device):
+  with _on(x.device):
     if ws is None:
       _lib.check(_lib.lib().rg_linear_scan(
           _p(x), _p(a), _p(reset), _p(h0), _p(y), _p(h_last), B, T, W,
@@ -331,7 +353,7 @@ def linear_scan_backward(dy, a, reset, y, h0=None, dh_last=None):
   dx, da = torch.empty_like(y), torch.empty_like(y)
   dh0 = (torch.empty((B, W), dtype=torch.float32, device=y.device)
          if h0 is not None else None)
-  with torch.cuda.device(y.device):
+  with _on(y.device):
     _lib.check(_lib.lib().rg_linear_scan_backward(
         _p(dy), _p(a), _p(reset), _p(y), _p(h0), _p(dh_last), _p(dx), _p(da),
         _p(dh0), B, T, W, _dtype_code(y), _stream(y)))
@@ -353,7 +375,7 @@ def gelu_mul(a, g):
   _same(a.dtype, a.device, g=g)
   g = _dev(g, "g")
   out = torch.empty_like(a)
-  with torch.cuda.device(a.device):
+  with _on(a.device):
     _lib.check(_lib.lib().rg_gelu_mul(_p(a), _p(g), _p(out), a.numel(),
                                       _dtype_code(a), _stream(a)))
   return out
@@ -367,7 +389,7 @@ def rms_norm(x, scale, eps=1e-6):
   width = x.shape[-1]
   assert scale.shape == (width,)
   out = torch.empty_like(x)
-  with torch.cuda.device(x.device):
+  with _on(x.device):
     _lib.check(_lib.lib().rg_rms_norm(_p(x), _p(scale), _p(out),
                                       x.numel() // width, width, eps,
                                       _dtype_code(x), _stream(x)))
@@ -386,7 +408,7 @@ def add_rms_norm(x, addend, scale, eps=1e-6):
   width = x.shape[-1]
   assert scale.shape == (width,)
   total, out = torch.empty_like(x), torch.empty_like(x)
-  with torch.cuda.device(x.device):
+  with _on(x.device):
     _lib.check(_lib.lib().rg_add_rms_norm(
         _p(x), _p(addend), _p(scale), _p(total), _p(out), x.numel() // width,
         width, eps, _dtype_code(x), _stream(x)))
@@ -397,7 +419,7 @@ def soft_cap(x, cap):
   """tanh(x / cap) * cap, one pass."""
   x = _dev(x, "x")
   out = torch.empty_like(x)
-  with torch.cuda.device(x.device):
+  with _on(x.device):
     _lib.check(_lib.lib().rg_soft_cap(_p(x), _p(out), x.numel(), float(cap),
                                       _dtype_code(x), _stream(x)))
   return out
@@ -408,7 +430,7 @@ def argmax_last(x):
   x = _dev(x, "x")
   n = x.shape[-1]
   out = torch.empty(x.shape[:-1], dtype=torch.int64, device=x.device)
-  with torch.cuda.device(x.device):
+  with _on(x.device):
     _lib.check(_lib.lib().rg_argmax_rows(_p(x), _p(out), x.numel() // n, n,
                                          _dtype_code(x), _stream(x)))
   return out
@@ -428,7 +450,7 @@ def _add_rms_norm_partial(ps, addend, scale, eps):
     addend = _dev(addend, "addend")
   total = torch.empty(ps.shape, dtype=ps.dtype, device=ps.sums.device)
   out = torch.empty_like(total)
-  with torch.cuda.device(total.device):
+  with _on(total.device):
     _lib.check(_lib.lib().rg_add_rms_norm_partial(
         _p(ps.sums), slices, _p(ps.bias), _p(addend), _p(scale), _p(total),
         _p(out), rows, width, eps, _DTYPES[ps.dtype], _stream(total)))
@@ -444,7 +466,7 @@ def rope(x, positions, inv_freq):
   inv = _dev(inv_freq, "inv_freq")
   assert inv.dtype == torch.float32 and inv.shape == (hd // 4,)
   out = torch.empty_like(x)
-  with torch.cuda.device(x.device):
+  with _on(x.device):
     _lib.check(_lib.lib().rg_rope(_p(x), _p(pos), is64, _p(inv), _p(out),
                                   B * T, n, hd, _dtype_code(x), _stream(x)))
   return out
@@ -461,7 +483,7 @@ def rope_pair(q, k, positions, inv_freq):
   inv = _dev(inv_freq, "inv_freq")
   assert inv.dtype == torch.float32 and inv.shape == (hd // 4,)
   q_out, k_out = torch.empty_like(q), torch.empty_like(k)
-  with torch.cuda.device(q.device):
+  with _on(q.device):
     _lib.check(_lib.lib().rg_rope_pair(
         _p(q), _p(k), _p(pos), is64, _p(inv), _p(q_out), _p(k_out), B * T, n,
         k.shape[2], hd, _dtype_code(q), _stream(q)))
@@ -481,7 +503,7 @@ def attention_decode_probs(scores, q, k_new, num_tokens, scale):
   nt = _dev(num_tokens, "num_tokens")
   probs = torch.empty((B, heads, window + 1), dtype=scores.dtype,
                       device=scores.device)
-  with torch.cuda.device(scores.device):
+  with _on(scores.device):
     _lib.check(_lib.lib().rg_attention_decode_probs(
         _p(scores), _p(q), _p(k_new), _p(nt), _p(probs), B, heads, hd, window,
         scale, _dtype_code(scores), _stream(scores)))
@@ -508,7 +530,7 @@ def attention_decode_finish(from_ring, probs, k_new, v_new, ring_keys,
   assert ring_keys.numel() == B * window * hd == ring_values.numel()
   assert num_tokens.dtype == torch.int32 and num_tokens.shape == (B,)
   out = torch.empty_like(from_ring)
-  with torch.cuda.device(out.device):
+  with _on(out.device):
     _lib.check(_lib.lib().rg_attention_decode_finish(
         _p(from_ring), _p(probs), _p(k_new), _p(v_new), _p(out),
         _p(ring_keys), _p(ring_values), _p(num_tokens), B, heads, hd, window,
@@ -550,7 +572,7 @@ def packed_gate_weights(w_x, w_a):
   if nbytes == 0:
     return None
   packed = torch.empty(nbytes // 2, dtype=w_x.dtype, device=w_x.device)
-  with torch.cuda.device(w_x.device):
+  with _on(w_x.device):
     _lib.check(_lib.lib().rg_pack_gate_weights(
         _p(_dev(w_x, "w_x")), _p(_dev(w_a, "w_a")), _p(packed), W, H,
         _dtype_code(w_x), _stream(w_x)))
@@ -635,7 +657,7 @@ class PackedLinear:
     if nbytes == 0:
       raise ValueError(f"unsupported linear shape N={N} K={K}")
     packed = torch.empty(nbytes // 2, dtype=w0.dtype, device=w0.device)
-    with torch.cuda.device(w0.device):
+    with _on(w0.device):
       if self.layout == 0:
         at = 0
         for w in weights:  # tile blocks of consecutive rows are consecutive
@@ -680,7 +702,7 @@ class PackedLinear:
     assert slices > 0
     M = x.numel() // K
     sums = torch.empty((slices, M, N), dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on(x.device):
       _lib.check(_lib.lib().rg_linear_rows_partial(
           _p(x), _p(self._packed), _p(sums), M, K, N, slices, _stream(x)))
     return PartialSums(sums, self._bias, (*x.shape[:-1], N), x.dtype, addend)
@@ -718,7 +740,7 @@ class PackedLinear:
     need = lib.rg_linear_rows_workspace_bytes(M, K, N)
     ws = (torch.empty(need, dtype=torch.uint8, device=x.device)
           if need and not self.gelu_pair else None)
-    with torch.cuda.device(x.device):
+    with _on(x.device):
       _lib.check(lib.rg_linear_rows(
           _p(x), _p(self._packed), _p(self._bias), _p(residual), _p(out),
           _p(ws), need if ws is not None else 0, M, K, N, g,
@@ -763,7 +785,7 @@ def recurrent_step(x, segment_pos, conv_cache, h, conv_w, conv_b, w_x, b_x, w_a,
     packed = packed_gate_weights(w_x, w_a)
   if packed is not None:
     cw, cb, wx_, bx_, wa_, ba_, ap_ = args
-    with torch.cuda.device(x.device):
+    with _on(x.device):
       _lib.check(_lib.lib().rg_recurrent_step_packed(
           _p(x), _p(seg), is64, _p(cache_in), _p(cache_out), _p(h_in),
           _p(h_out), _p(cw), _p(cb), _p(packed), _p(bx_), _p(ba_), _p(ap_),
@@ -772,7 +794,7 @@ def recurrent_step(x, segment_pos, conv_cache, h, conv_w, conv_b, w_x, b_x, w_a,
       cache_out = cache_out.to(conv_cache.dtype)
     return y, h_out, cache_out
   ws = _workspace(B, W, x.dtype, x.device)
-  with torch.cuda.device(x.device):
+  with _on(x.device):
     _lib.check(_lib.lib().rg_recurrent_step(
         _p(x), _p(seg), is64, _p(cache_in), _p(cache_out), _p(h_in), _p(h_out),
         *[_p(t) for t in args], _p(y), _p(ws), ws.numel(), B, W, H,
