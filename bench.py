@@ -460,7 +460,7 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
   path = args.path
   if path == "auto":
     path = ("single" if ops.recurrent_prefill_supported(x, H)
-            and (B * H >= 144 or chunked) else "split")
+            and (B * H >= 129 or chunked) else "split")
   step = step_single if path == "single" else step_split
 
   def timed(fn, steps, warmup):

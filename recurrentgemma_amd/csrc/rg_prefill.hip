@@ -932,7 +932,11 @@ void prefill_chunk_plan(int B, int H, int T, int* chunks, int* tiles_per_chunk) 
   *chunks = 1;
   *tiles_per_chunk = ntiles;
   const int64_t groups = (int64_t)B * H;
-  if (groups * 2 > 256 || ntiles < 6) return;
+  // (below about 1500 tokens the two prologues and the second launch cost
+  // what the idle CUs would: measured at W2560 H10, 10-120 pairs, chunks
+  // against the gate GEMM + scan pair: T768 +10..25 %, T1024 even, T2048
+  // -5..20 %, T4096 -10..25 %)
+  if (groups * 2 > 256 || ntiles < 24) return;
   int want = (int)(256 / groups) + 1;  // workgroups per launch and row, + 1
   if (want > ntiles / 2) want = ntiles / 2;
   if (want < 3) return;

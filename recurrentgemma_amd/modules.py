@@ -33,11 +33,12 @@ def gelu(x: torch.Tensor) -> torch.Tensor:
 
 # rg_recurrent_prefill runs one workgroup per (sequence row, head), so its time
 # does not shrink below 256 groups, while the two-kernel form scales with the
-# number of tokens.  Measured on MI355X (T = 1024 and 4096, 256-wide heads) the
-# two cross between 128 groups (two kernels 5 % ahead) and 160 (single launch
-# 25 % ahead).  With few groups and long rows the sequences are cut into
-# chunks that run as workgroups of their own (rg_recurrent_prefill_split).
-_MIN_GROUPS_FOR_SINGLE_LAUNCH = 144
+# number of tokens.  Measured on MI355X (W2560 H10, T512 and T4096): from 130
+# groups on the single kernel is 20-25 % ahead (405 against 498 us at T4096);
+# at 120 groups and below the two-kernel form wins for short rows, and long
+# rows are cut into chunks that run as workgroups of their own
+# (rg_recurrent_prefill_split, up to 128 groups).
+_MIN_GROUPS_FOR_SINGLE_LAUNCH = 129
 
 
 def _single_launch_pays(x, num_heads) -> bool:

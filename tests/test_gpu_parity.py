@@ -495,12 +495,12 @@ def test_recurrent_block_module_joined_kernel(monkeypatch):
     (130, 70, 256, 1, 20, torch.int64, False),  # more workgroups than CUs/2
     (2, 100, 256, 1, -7, torch.int32, False),   # left padding: positions < 0
     # few (row, head) pairs, long rows: the sequences run as chunks
-    (1, 1000, 512, 2, 200, torch.int64, True),
+    (1, 1600, 512, 2, 200, torch.int64, True),
     (2, 2048, 256, 1, None, torch.int64, False),
-    (1, 777, 768, 3, 100, torch.int32, True),
-    (3, 1500, 256, 1, 7, torch.int64, False),
+    (1, 1777, 768, 3, 100, torch.int32, True),
+    (3, 1540, 256, 1, 7, torch.int64, False),
     (1, 8192, 256, 1, 1024, torch.int64, True),  # 64 chunks of two tiles
-    (2, 900, 256, 1, -300, torch.int32, False),  # chunks, left padding
+    (2, 1700, 256, 1, -300, torch.int32, False),  # chunks, left padding
 ])
 def test_recurrent_prefill_single_launch(B, T, W, H, mean_doc, seg_dtype,
                                          with_h0):
@@ -560,8 +560,8 @@ def test_recurrent_prefill_single_launch(B, T, W, H, mean_doc, seg_dtype,
 @pytest.mark.parametrize("B,T,W,H,mean_doc", [
     (2, 200, 512, 2, 37),      # whole rows, ragged last tile, documents
     (1, 70, 256, 1, None),
-    (1, 1024, 512, 2, 300),    # rows in chunks
-    (3, 640, 768, 3, None),
+    (1, 2048, 512, 2, 300),    # rows in chunks
+    (3, 1600, 768, 3, None),
     (40, 130, 1024, 4, 50),    # 160 (row, head) pairs
 ])
 def test_prefill_joined_with_gate_branch(B, T, W, H, mean_doc):
