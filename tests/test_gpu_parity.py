@@ -203,6 +203,10 @@ def test_scans_cut_into_chunks(dtype, B, T, W, mean_doc):
          else torch.arange(T)[None].expand(B, T).contiguous())
   seg = _dev(seg)
   tol_y = F32_TOL if dtype == torch.float32 else 2.0 ** -7
+  # element by element: one bf16 unit where the state was combined in another
+  # float32 order
+  elt = (dict(rtol=1e-4, atol_of_max=1e-5) if dtype == torch.float32
+         else dict(rtol=2.0 ** -7, atol_of_max=2e-3))
   for conv in (None, (cw, cb)):
     for start in (None, h0):
       kw = dict(h0=start, conv=conv, return_conv_cache=conv is not None)
@@ -210,6 +214,9 @@ def test_scans_cut_into_chunks(dtype, B, T, W, mean_doc):
       y2, h2, c2 = ops.lru_scan_fused(x, gx, ga, a_param, seg, split=True, **kw)
       assert helpers.max_rel(y2, y1) < tol_y
       assert helpers.max_rel(h2, h1) < F32_TOL
+      helpers.assert_close_elementwise(y2, y1, what="y, chunks", **elt)
+      helpers.assert_close_elementwise(h2, h1, rtol=1e-4, atol_of_max=1e-5,
+                                       what="h, chunks")
       if conv is not None:
         assert torch.equal(c1, c2)
       if dtype == torch.bfloat16:  # almost every output rounds the same way
@@ -222,6 +229,7 @@ def test_scans_cut_into_chunks(dtype, B, T, W, mean_doc):
     y2, h2 = ops.linear_scan(x, a, reset, start, split=True)
     assert helpers.max_rel(y2, y1) < tol_y
     assert helpers.max_rel(h2, h1) < F32_TOL
+    helpers.assert_close_elementwise(y2, y1, what="y, plain chunks", **elt)
     if B * T * W <= 4097 * 256:
       yo, ho = R.rnn_scan(x.cpu(), a.cpu(), reset.cpu(),
                           None if start is None else start.cpu())
@@ -367,6 +375,11 @@ def test_core_vs_oracle(dtype, B, T, W, H, mean_doc):
   eh = helpers.max_rel(cache.rg_lru_state, co.rg_lru_state)
   print("max-rel y", ey, "h", eh)
   assert ey < tol and eh < tol
+  elt = (dict(rtol=1e-4, atol_of_max=1e-5) if dtype == torch.float32
+         else dict(rtol=1e-2, atol_of_max=2e-3))
+  helpers.assert_close_elementwise(y, yo, what="y", **elt)
+  helpers.assert_close_elementwise(cache.rg_lru_state, co.rg_lru_state,
+                                   what="h", **elt)
   assert torch.equal(cache.conv1d_state.cpu(), co.conv1d_state)
   assert cache.rg_lru_state.dtype == torch.float32
   assert cache.conv1d_state.dtype == dtype
@@ -663,6 +676,8 @@ def test_recurrent_step_single_launch(B, W, H, in_place):
                                      p["w_a"], p["b_a"], cache=ho)
     assert helpers.max_rel(y, yo) < BF16_TOL
     assert helpers.max_rel(hd, ho) < BF16_TOL
+    helpers.assert_close_elementwise(y, yo, what=f"y, step {step}")
+    helpers.assert_close_elementwise(hd, ho, what=f"h, step {step}")
     assert torch.equal(ccd.cpu(), cco)
 
 
