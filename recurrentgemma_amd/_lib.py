@@ -102,6 +102,9 @@ def build(force: bool = True) -> str:
   if force:
     cmd.append("-B")
   subprocess.check_call(cmd)
+  # The prefill kernel numbers its weight registers by hand: a build in which
+  # the register allocator wanted one of them for itself must not be used.
+  subprocess.check_call(["make", "-C", CSRC, "check-registers"])
   return LIB_PATH
 
 

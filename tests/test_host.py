@@ -145,6 +145,18 @@ def test_c_side_validation_without_launch():
   assert lib.rg_packed_gate_weights_bytes(4096, 8, 1) == 0  # 512-wide heads
 
 
+def test_prefill_kernel_keeps_its_hand_numbered_registers():
+  """The prefill kernel's gate weights sit in accumulation registers that the
+  source numbers itself; the compiled kernels may touch those registers only
+  in the hand-written instructions, and may not spill."""
+  import shutil
+  import subprocess
+  if shutil.which("make") is None or not os.path.exists("/opt/rocm/bin/hipcc"):
+    pytest.skip("needs make and hipcc")
+  subprocess.check_call(["make", "-C", _lib.CSRC, "check-registers"],
+                        stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+
+
 def test_no_cpu_fallback():
   conv = rg.Conv1D(width=8, temporal_width=4)
   with pytest.raises(RuntimeError, match="GPU only"):
