@@ -454,14 +454,29 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
       events[2].record()
     return out
 
-  # the choice RecurrentBlock makes: the single kernel where its workgroups
+  def step_core(events=None):
+    # what RecurrentBlock calls: one library call that picks the kernels
+    if events:
+      events[0].record()
+    out = ops.recurrent_core(x, seg, conv.w, conv.b, lru.input_gate.w,
+                             lru.input_gate.b, lru.a_gate.w, lru.a_gate.b,
+                             lru.a_param)
+    if events:
+      events[1].record()
+      events[2].record()
+    return out
+
+  # the choice rg_recurrent_core makes: the single kernel where its workgroups
   # (one per row, head and time chunk) fill the GPU
   chunked = esize == 2 and ops.recurrent_prefill_chunked(B, T, W, H)
   path = args.path
   if path == "auto":
     path = ("single" if ops.recurrent_prefill_supported(x, H)
             and (B * H >= 129 or chunked) else "split")
-  step = step_single if path == "single" else step_split
+  if args.path == "auto":
+    step = step_core
+  else:
+    step = step_single if path == "single" else step_split
 
   def timed(fn, steps, warmup):
     for _ in range(warmup):
@@ -516,9 +531,9 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
     traffic, source = measured_traffic(workload, "single")
     roofline = {
         "kernel": ("block_prefill_bf16_kernel (conv + gate GEMMs + gates + scan)"
-                   + (": summary pass over all chunks but the last, carry "
-                      "kernel, replay pass; avg_launch_ms covers the three"
-                      if chunked else "")),
+                   + (": two launches (chunk 0 + summaries of the chunks "
+                      "after it; replay of chunks 1..n-1); avg_launch_ms "
+                      "covers both" if chunked else "")),
         "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
         "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
         "traffic": traffic, "traffic_source": source,
@@ -526,6 +541,10 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
         "mfma_tflops": gemm_flops / (first_ms * 1e-3) / 1e12,
         "frac_of_bf16_mfma_peak": gemm_flops / (first_ms * 1e-3) / 2.5e15}
   else:
+    if args.path == "auto":
+      # per-kernel durations: the same two launches called one by one, with
+      # events between them, after the timed region
+      _, first_ms, second_ms = timed(step_split, steps, warmup)
     figs = split_figures(first_ms, second_ms)
     roofline = figs["scan"]
 
@@ -574,7 +593,8 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
                    "chunks side by side)" if path == "single" and chunked
                    else "rg_recurrent_prefill (single launch)"
                    if path == "single"
-                   else "rg_gates_gemm(conv on load) + "
+                   else ("rg_recurrent_core: " if args.path == "auto" else "")
+                        + "rg_gates_gemm(conv on load) + "
                         + ("rg_lru_scan_fused_split(conv): sequences in chunks "
                            "side by side" if in_chunks
                            else "rg_lru_scan_fused(conv)"))},

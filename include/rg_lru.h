@@ -242,6 +242,32 @@ int rg_recurrent_prefill_gelu_mul(
     void* conv_cache_out, void* workspace, size_t workspace_bytes, int B, int T,
     int W, int H, int dtype, void* stream);
 
+/* conv_1d -> rg_lru of a prefill as RecurrentBlock.forward chains them
+ * (recurrentgemma/torch/modules.py:632-643), for every shape and both dtypes,
+ * with the choice of kernels made here: the single prefill kernel
+ * (rg_recurrent_prefill_split; bf16, 256-wide heads, enough (row, head) pairs
+ * or rows long enough to be cut into chunks), else rg_gates_gemm with the conv
+ * applied on load followed by rg_lru_scan_fused_split, the pre-activations of
+ * both gates living in the workspace.  gate_branch (nullable, [B,T,W]): the
+ * block's linear_y output; `out` is then rglru(conv1d(x)) * gelu_tanh(
+ * gate_branch) (modules.py:627-628, 644: rg_recurrent_prefill_gelu_mul where
+ * whole rows run in the single kernel, otherwise rg_gelu_mul over `out` as a
+ * last launch), else the plain RG-LRU output.  `workspace` (16-byte aligned)
+ * must hold rg_recurrent_core_workspace_bytes(B, T, W, H, dtype) bytes (0 for
+ * whole rows in the single kernel: workspace may then be null).  Same values
+ * as the calls it is made of; h0 / h_last / conv_cache_out / w_packed as in
+ * rg_recurrent_prefill (w_packed is only read by the single kernel). */
+size_t rg_recurrent_core_workspace_bytes(int B, int T, int W, int H, int dtype);
+int rg_recurrent_core(const void* x, const void* gate_branch,
+                      const void* segpos, int segpos_is_i64,
+                      const void* conv_w, const void* conv_b, const void* w_x,
+                      const void* b_x, const void* w_a, const void* b_a,
+                      const void* w_packed, const void* a_param,
+                      const void* h0, void* out, void* h_last,
+                      void* conv_cache_out, void* workspace,
+                      size_t workspace_bytes, int B, int T, int W, int H,
+                      int dtype, void* stream);
+
 /* One decode step of the conv -> RG-LRU core, as RecurrentBlock.forward chains
  * them with a cache (recurrentgemma/torch/modules.py:632-643 with
  * layers.py:469-474 and :170-177): x [B,1,W], segpos [B,1],

@@ -46,6 +46,9 @@ SIGNATURES = {
                                         _sz, _i, _i, _i, _i, _i, _vp]),
     "rg_recurrent_prefill_gelu_mul": (_i, [_vp, _vp, _vp, _i] + [_vp] * 13 +
                                       [_sz, _i, _i, _i, _i, _i, _vp]),
+    "rg_recurrent_core_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
+    "rg_recurrent_core": (_i, [_vp, _vp, _vp, _i] + [_vp] * 13 +
+                          [_sz, _i, _i, _i, _i, _i, _vp]),
     "rg_linear_scan": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "rg_linear_scan_backward": (_i, [_vp] * 9 + [_i, _i, _i, _i, _vp]),
     "rg_scan_split_workspace_bytes": (_sz, [_i, _i, _i]),

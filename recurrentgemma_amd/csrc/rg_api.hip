@@ -470,6 +470,90 @@ int rg_recurrent_prefill_gelu_mul(
                                 dtype, stream);
 }
 
+// Which form serves a shape: the single prefill kernel where its workgroups
+// (one per row, head and time chunk) fill the GPU, else the gate GEMM and the
+// scan kernel with the pre-activations of both gates in the workspace.
+struct CorePlan {
+  bool single;         // block_prefill_bf16_kernel
+  size_t split_bytes;  // chunk summaries of whichever form runs
+  size_t gate_bytes;   // one gate's pre-activations (two-kernel form), padded
+};
+static CorePlan core_plan(int B, int T, int W, int H, int dtype) {
+  CorePlan p{};
+  const bool fits = dtype == RG_DTYPE_BF16 && W / H == 256 &&
+                    (int64_t)T * W * 2 < (int64_t)0x7fffffff;
+  const size_t chunk_bytes =
+      fits ? rg_recurrent_prefill_split_workspace_bytes(B, T, W, H) : 0;
+  p.single = fits && ((int64_t)B * H >= rg::kPrefillMinGroups || chunk_bytes > 0);
+  if (p.single) {
+    p.split_bytes = chunk_bytes;
+  } else {
+    p.split_bytes = rg_scan_split_workspace_bytes(B, T, W);
+    const size_t n = (size_t)B * T * W * (dtype == RG_DTYPE_F32 ? 4 : 2);
+    p.gate_bytes = (n + 255) & ~(size_t)255;
+  }
+  return p;
+}
+
+size_t rg_recurrent_core_workspace_bytes(int B, int T, int W, int H,
+                                         int dtype) {
+  if (B <= 0 || T <= 0 || W <= 0 || H <= 0 || W % H != 0 ||
+      (dtype != RG_DTYPE_F32 && dtype != RG_DTYPE_BF16))
+    return 0;
+  const CorePlan p = core_plan(B, T, W, H, dtype);
+  return p.split_bytes + 2 * p.gate_bytes;
+}
+
+int rg_recurrent_core(const void* x, const void* gate_branch,
+                      const void* segpos, int segpos_is_i64,
+                      const void* conv_w, const void* conv_b, const void* w_x,
+                      const void* b_x, const void* w_a, const void* b_a,
+                      const void* w_packed, const void* a_param,
+                      const void* h0, void* out, void* h_last,
+                      void* conv_cache_out, void* workspace,
+                      size_t workspace_bytes, int B, int T, int W, int H,
+                      int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(B > 0 && T > 0 && W > 0 && H > 0,
+             "%s: B=%d T=%d W=%d H=%d must be positive", __func__, B, T, W, H);
+  RG_REQUIRE(W % H == 0, "%s: W=%d is not a multiple of H=%d", __func__, W, H);
+  RG_CHECK_OPT_PTR(gate_branch);
+  RG_REQUIRE(gate_branch == nullptr || gate_branch != x,
+             "%s: gate_branch must not alias x", __func__);
+  const CorePlan p = core_plan(B, T, W, H, dtype);
+  const size_t need = p.split_bytes + 2 * p.gate_bytes;
+  if (need > 0 && (workspace == nullptr || workspace_bytes < need ||
+                   !aligned16(workspace)))
+    return fail(RG_ERR_WORKSPACE,
+                "%s: workspace of %zu bytes (16-byte aligned) required, got %zu",
+                __func__, need, workspace ? workspace_bytes : (size_t)0);
+  if (p.single) {
+    // rows in chunks write the plain output; the join follows as its own pass
+    const bool join_inside = gate_branch != nullptr && p.split_bytes == 0;
+    const int rc = recurrent_prefill_impl(
+        __func__, x, segpos, segpos_is_i64, conv_w, conv_b, w_x, b_x, w_a, b_a,
+        w_packed, a_param, h0, join_inside ? gate_branch : nullptr, out, h_last,
+        conv_cache_out, workspace, workspace_bytes, true, B, T, W, H, dtype,
+        stream);
+    if (rc != RG_OK || gate_branch == nullptr || join_inside) return rc;
+  } else {
+    char* const ws = (char*)workspace;
+    void* const gx = ws + p.split_bytes;
+    void* const ga = ws + p.split_bytes + p.gate_bytes;
+    int rc = rg_gates_gemm(x, 1, segpos, segpos_is_i64, conv_w, conv_b, w_x,
+                           b_x, w_a, b_a, gx, ga, B, T, W, H, dtype, stream);
+    if (rc != RG_OK) return rc;
+    rc = lru_scan_fused_impl(__func__, x, 1, conv_w, conv_b, gx, ga, a_param,
+                             segpos, segpos_is_i64, h0, out, h_last,
+                             conv_cache_out, workspace, p.split_bytes, true, B,
+                             T, W, dtype, stream);
+    if (rc != RG_OK || gate_branch == nullptr) return rc;
+  }
+  return launch_status(
+      __func__, rg::launch_gelu_mul(out, gate_branch, out, (int64_t)B * T * W,
+                                    dtype, (hipStream_t)stream));
+}
+
 #undef RG_WHO
 #define RG_WHO who
 static int linear_scan_impl(const char* who, const void* x, const void* a,

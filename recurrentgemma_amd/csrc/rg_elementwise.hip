@@ -19,8 +19,8 @@ constexpr float kGeluC1 = 0.044715f;
 // contiguous 4 KB of every operand) moves 6.4 TB/s, a grid-stride loop over
 // 8192 workgroups 4.7 TB/s.
 __global__ void __launch_bounds__(256)
-gelu_mul_bf16_kernel(const u32x4* __restrict__ a, const u32x4* __restrict__ g,
-                     u32x4* __restrict__ out, int64_t n8,
+gelu_mul_bf16_kernel(const u32x4* a, const u32x4* __restrict__ g, u32x4* out,
+                     int64_t n8,
                      const uint16_t* a_tail, const uint16_t* g_tail,
                      uint16_t* out_tail, int tail) {
   auto one = [](float av, float gv) { return gelu_mul_bf16(av, gv); };
@@ -47,8 +47,8 @@ gelu_mul_bf16_kernel(const u32x4* __restrict__ a, const u32x4* __restrict__ g,
 
 // float32: the reference's own formula; four elements per thread.
 __global__ void __launch_bounds__(256)
-gelu_mul_f32_kernel(const f32x4* __restrict__ a, const f32x4* __restrict__ g,
-                    f32x4* __restrict__ out, int64_t n4, const float* a_tail,
+gelu_mul_f32_kernel(const f32x4* a, const f32x4* __restrict__ g, f32x4* out,
+                    int64_t n4, const float* a_tail,
                     const float* g_tail, float* out_tail, int tail) {
   auto one = [](float av, float gv) {
     const float u = kGeluC0 * (gv + kGeluC1 * gv * gv * gv);

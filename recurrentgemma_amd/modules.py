@@ -4,7 +4,8 @@ RecurrentBlock / RecurrentBlockCache mirror
 recurrentgemma/torch/modules.py:32-37 and :496-680 (same constructor,
 parameter names, forward signature and cache tuple).  linear_x / linear_y /
 linear_out stay torch.nn.Linear (hipBLASLt); conv_1d -> rg_lru runs as
-  prefill: rg_gates_gemm (conv on load) + rg_lru_scan_fused (conv fused)
+  prefill: rg_recurrent_core (the single prefill kernel, or rg_gates_gemm with
+           the conv on load + rg_lru_scan_fused: the library picks)
   decode : rg_recurrent_step
 unless the conv width is not 4, where the stand-alone conv kernel is used.
 """
@@ -29,27 +30,6 @@ class RecurrentBlockCache(NamedTuple):
 
 def gelu(x: torch.Tensor) -> torch.Tensor:
   return nn.functional.gelu(x, approximate="tanh")
-
-
-# rg_recurrent_prefill runs one workgroup per (sequence row, head), so its time
-# does not shrink below 256 groups, while the two-kernel form scales with the
-# number of tokens.  Measured on MI355X (W2560 H10, T512 and T4096): from 130
-# groups on the single kernel is 20-25 % ahead (405 against 498 us at T4096);
-# at 120 groups and below the two-kernel form wins for short rows, and long
-# rows are cut into chunks that run as workgroups of their own
-# (rg_recurrent_prefill_split, up to 128 groups).
-_MIN_GROUPS_FOR_SINGLE_LAUNCH = 129
-
-
-def _single_launch_pays(x, num_heads) -> bool:
-  """Whether prefill goes to the single-launch kernel (whole rows or rows cut
-  into chunks) rather than to the gate GEMM + scan kernel pair."""
-  if not ops.recurrent_prefill_supported(x, num_heads):
-    return False
-  bs, l, w = x.shape
-  if bs * num_heads >= _MIN_GROUPS_FOR_SINGLE_LAUNCH:
-    return True
-  return ops.recurrent_prefill_chunked(bs, l, w, num_heads)
 
 
 @torch.no_grad()
@@ -90,31 +70,22 @@ def recurrent_core(conv_1d: layers.Conv1D, rg_lru: layers.RGLRU, x,
                              return_cache)
     y, h = rg_lru(xc, segment_pos,
                   None if cache is None else cache.rg_lru_state, return_cache)
-  elif _single_launch_pays(x, rg_lru.num_heads):
-    # one workgroup per (row, head) -- or per chunk of one -- pays once there
-    # are enough of them to fill the GPU; otherwise the two-kernel form
-    # spreads over more CUs.  The join with the gate branch goes into the
-    # kernel for whole rows (measured at B16 T8192 W4096: 1.15 ms against
-    # 0.91 + 0.40 ms apart); with rows in chunks it would lengthen the one
-    # workgroup per row that produces outputs in the first launch while the
-    # others only summarise, and the separate pass is as fast (0.33 ms both
-    # ways at B8 T4096 W2560).
-    chunked = ops.recurrent_prefill_chunked(bs, l, x.shape[2], rg_lru.num_heads)
-    y, h, conv_state = ops.recurrent_prefill(
+  else:
+    # One call; the library picks the kernels (rg_recurrent_core): one
+    # workgroup per (row, head) -- or per chunk of one -- where there are
+    # enough of them to fill the GPU (from 129 pairs the single kernel is
+    # 20-25 % ahead of the gate GEMM + scan pair, which spreads over more CUs
+    # below that; long rows of few pairs are cut into chunks), and the join
+    # with the gate branch inside that kernel for whole rows (at B16 T8192
+    # W4096: 1.15 ms against 0.91 + 0.40 ms apart; with rows in chunks it would
+    # lengthen the one workgroup per row that produces outputs in the first
+    # launch while the others only summarise, so it stays a pass of its own).
+    y, h, conv_state = ops.recurrent_core(
         x, segment_pos, conv_1d.w, conv_1d.b, rg_lru.input_gate.w,
         rg_lru.input_gate.b, rg_lru.a_gate.w, rg_lru.a_gate.b, rg_lru.a_param,
         h0=None, return_h=return_cache, return_conv_cache=return_cache,
-        gate_branch=None if chunked else gate_branch)
-    if not chunked:
-      gate_branch = None  # joined inside the kernel
-  else:
-    gx_pre, ga_pre = ops.gates_gemm(
-        x, rg_lru.input_gate.w, rg_lru.input_gate.b, rg_lru.a_gate.w,
-        rg_lru.a_gate.b, conv=(segment_pos, conv_1d.w, conv_1d.b))
-    y, h, conv_state = ops.lru_scan_fused(
-        x, gx_pre, ga_pre, rg_lru.a_param, segment_pos, h0=None,
-        conv=(conv_1d.w, conv_1d.b), return_h=return_cache,
-        return_conv_cache=return_cache)
+        gate_branch=gate_branch)
+    gate_branch = None
   if gate_branch is not None:
     y = ops.gelu_mul(y, gate_branch)
   if not return_cache:

@@ -310,6 +310,54 @@ def recurrent_prefill(x, segment_pos, conv_w, conv_b, w_x, b_x, w_a, b_a,
   return y, h_last, cache
 
 
+def recurrent_core(x, segment_pos, conv_w, conv_b, w_x, b_x, w_a, b_a, a_param,
+                   h0=None, return_h=True, return_conv_cache=True,
+                   gate_branch=None):
+  """conv -> RG-LRU of a prefill for any shape and dtype in one call of the
+  library, which picks the kernels (rg_recurrent_core): the single prefill
+  kernel where it pays, else gate GEMM + scan.  gate_branch: the block's
+  linear_y output; the result is then y * gelu(gate_branch).
+  Returns (y, h_last | None, conv_cache | None)."""
+  B, T, W = x.shape
+  H = w_x.shape[0]
+  assert conv_w.shape == (4, W) and conv_b.shape == (W,)
+  assert w_x.shape == w_a.shape == (H, W // H, W // H)
+  assert b_x.shape == b_a.shape == (H, W // H)
+  assert a_param.shape == (W,)
+  x = _dev(x, "x")
+  _same(x.dtype, x.device, conv_w=conv_w, conv_b=conv_b, w_x=w_x, b_x=b_x,
+        w_a=w_a, b_a=b_a, a_param=a_param)
+  cw, cb, wx_, bx_, wa_, ba_, ap_ = [
+      _dev(t, n) for t, n in ((conv_w, "conv_w"), (conv_b, "conv_b"),
+                              (w_x, "w_x"), (b_x, "b_x"), (w_a, "w_a"),
+                              (b_a, "b_a"), (a_param, "a_param"))]
+  seg, is64 = _segpos(segment_pos, B, T)
+  if h0 is not None:
+    assert h0.dtype == torch.float32, "the RG-LRU state is always float32"
+    assert h0.shape == (B, W)
+    h0 = _dev(h0, "h0")
+  if gate_branch is not None:
+    assert gate_branch.shape == x.shape
+    _same(x.dtype, x.device, gate_branch=gate_branch)
+    gate_branch = _dev(gate_branch, "gate_branch")
+  y = torch.empty_like(x)
+  h_last = (torch.empty((B, W), dtype=torch.float32, device=x.device)
+            if return_h else None)
+  cache = x.new_empty((B, 3, W)) if return_conv_cache else None
+  packed = (packed_gate_weights(w_x, w_a)  # cached per weight version
+            if recurrent_prefill_supported(x, H) else None)
+  lib = _lib.lib()
+  code = _dtype_code(x)
+  need = lib.rg_recurrent_core_workspace_bytes(B, T, W, H, code)
+  ws = torch.empty(need, dtype=torch.uint8, device=x.device) if need else None
+  with _on(x.device):
+    _lib.check(lib.rg_recurrent_core(
+        _p(x), _p(gate_branch), _p(seg), is64, _p(cw), _p(cb), _p(wx_),
+        _p(bx_), _p(wa_), _p(ba_), _p(packed), _p(ap_), _p(h0), _p(y),
+        _p(h_last), _p(cache), _p(ws), need, B, T, W, H, code, _stream(x)))
+  return y, h_last, cache
+
+
 def linear_scan(x, a, reset, h0=None, split=True):
   B, T, W = x.shape
   x = _dev(x, "x")

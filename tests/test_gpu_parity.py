@@ -11,6 +11,7 @@ import torch
 
 import recurrentgemma_amd as rg
 from oracle import torch_ref as R
+from recurrentgemma_amd import _lib
 from recurrentgemma_amd import ops
 from tests import helpers
 
@@ -55,7 +56,6 @@ def _block(params, width, heads, dtype, K=4):
 
 
 def test_library_loaded():
-  from recurrentgemma_amd import _lib
   assert _lib.lib().rg_abi_version() == 1
   assert torch.cuda.is_available()
   name = torch.cuda.get_device_name(0)
@@ -188,7 +188,6 @@ def test_scans_cut_into_chunks(dtype, B, T, W, mean_doc):
   conv cache bit for bit.  Against the oracle: the plain recurrence below
   (all but the largest shape), and the long single row of
   test_core_vs_oracle, which runs through the split path."""
-  from recurrentgemma_amd import _lib
   assert _lib.lib().rg_scan_split_workspace_bytes(B, T, W) > 0
   _announce("split scan", dtype, B, T, W, mean_doc)
   g = torch.Generator().manual_seed(T + W)
@@ -461,8 +460,9 @@ def test_recurrent_block_module():
 
 def test_recurrent_block_module_joined_kernel(monkeypatch):
   """bf16 RecurrentBlock with enough (row, head) pairs for the prefill kernel
-  that also applies the x * gelu(y) join: one core launch, no gelu_mul pass,
-  and the block output bit for bit what the separate pass gives."""
+  that also applies the x * gelu(y) join: the block hands its gate branch to
+  the one library call (no gelu_mul call of its own), and the block output is
+  bit for bit what the separate pass gives."""
   B, T, width, H = 80, 70, 512, 2  # 160 pairs
   torch.manual_seed(6)
   blk = rg.RecurrentBlock(width=width, num_heads=H,
@@ -473,16 +473,18 @@ def test_recurrent_block_module_joined_kernel(monkeypatch):
   x = _dev(torch.randn(B, T, width).to(torch.bfloat16))
   seg = _dev(helpers.document_positions(B, T, 25, seed=4))
   calls = []
-  real_gelu_mul, real_prefill = ops.gelu_mul, ops.recurrent_prefill
+  real_gelu_mul, real_core = ops.gelu_mul, ops.recurrent_core
   monkeypatch.setattr(ops, "gelu_mul",
                       lambda *a, **k: calls.append("gelu_mul") or
                       real_gelu_mul(*a, **k))
-  monkeypatch.setattr(ops, "recurrent_prefill",
+  monkeypatch.setattr(ops, "recurrent_core",
                       lambda *a, **k: calls.append(
-                          ("prefill", k.get("gate_branch") is not None)) or
-                      real_prefill(*a, **k))
+                          ("core", k.get("gate_branch") is not None)) or
+                      real_core(*a, **k))
   got, cache = blk(x, seg)
-  assert calls == [("prefill", True)], calls
+  assert calls == [("core", True)], calls
+  # whole rows in the single kernel: no workspace, the join is inside it
+  assert _lib.lib().rg_recurrent_core_workspace_bytes(B, T, width, H, 1) == 0
   # the same block with the join as a pass of its own
   yb = blk.linear_y(x)
   core, cache2 = rg.recurrent_core(blk.conv_1d, blk.rg_lru, blk.linear_x(x),
@@ -605,7 +607,6 @@ def test_prefill_joined_with_gate_branch(B, T, W, H, mean_doc):
           torch.bfloat16)
   assert helpers.max_rel(got, ref) < BF16_TOL
   # through the C ABI with the output over the gate branch
-  from recurrentgemma_amd import _lib
   lib = _lib.lib()
   need = lib.rg_recurrent_prefill_split_workspace_bytes(B, T, W, H)
   ws = torch.empty(max(need, 16), dtype=torch.uint8, device=DEV)
@@ -637,7 +638,6 @@ def test_recurrent_step_single_launch(B, W, H, in_place):
   against rg_recurrent_step (conv step + gate GEMM + scan step, same
   arithmetic: bit for bit) and the oracle, over three chained steps with a
   position 0 (state reset) in some rows."""
-  from recurrentgemma_amd import _lib
   _announce("recurrent_step packed", B, W, H, in_place)
   seed = 8100 + B
   p = R.make_params(W, H, torch.bfloat16, seed=seed, gate_bias_std=0.5)
@@ -684,7 +684,6 @@ def test_recurrent_step_single_launch(B, W, H, in_place):
 def test_recurrent_prefill_without_packed_weights():
   """rg_recurrent_prefill with w_packed == NULL re-lays the gate weights out
   inside the kernel: same result, bit for bit, as with the packed buffer."""
-  from recurrentgemma_amd import _lib
   B, T, W, H = 3, 150, 512, 2
   p = R.make_params(W, H, torch.bfloat16, seed=61, gate_bias_std=0.5)
   P = {k: _dev(v) for k, v in p.items()}
@@ -709,9 +708,9 @@ def test_recurrent_prefill_without_packed_weights():
 def test_recurrent_core_picks_single_launch():
   """With enough (row, head) pairs recurrent_core runs prefill as one launch
   and decode as one launch; both against the oracle, chained."""
-  from recurrentgemma_amd import modules
   B, T, W, H = 75, 90, 512, 2
-  assert B * H >= modules._MIN_GROUPS_FOR_SINGLE_LAUNCH
+  # no workspace = whole rows in the single kernel
+  assert _lib.lib().rg_recurrent_core_workspace_bytes(B, T, W, H, 1) == 0
   p, x, blk, (y, cache), (yo, co) = _core_case(
       torch.bfloat16, B, T, W, H, helpers.document_positions(B, T, 30, seed=5),
       seed=77)
@@ -727,6 +726,79 @@ def test_recurrent_core_picks_single_launch():
   assert helpers.max_rel(y1, yo1) < BF16_TOL
   assert helpers.max_rel(cache1.rg_lru_state, co1.rg_lru_state) < BF16_TOL
   assert torch.equal(cache1.conv1d_state.cpu(), co1.conv1d_state)
+
+
+@pytest.mark.parametrize("dtype,B,T,W,H", [
+    (torch.float32, 1, 512, 2560, 10),    # float32: gate GEMM + scan in chunks
+    (torch.float32, 3, 70, 384, 3),       # 128-wide heads, generic GEMM
+    (torch.bfloat16, 2, 300, 512, 2),     # few pairs, short rows: two kernels
+    (torch.bfloat16, 70, 130, 512, 2),    # 140 pairs: single kernel, whole rows
+    (torch.bfloat16, 1, 2048, 512, 2),    # long rows of few pairs: chunks
+    (torch.bfloat16, 2, 65, 384, 3),      # bf16, 128-wide heads
+])
+@pytest.mark.parametrize("joined", [False, True])
+def test_recurrent_core_entry_equals_its_parts(dtype, B, T, W, H, joined):
+  """rg_recurrent_core picks the kernels itself; whatever it picks, its
+  outputs are those of the separate calls it stands for, bit for bit."""
+  p = R.make_params(W, H, dtype, seed=301, gate_bias_std=0.3)
+  P = {k: _dev(v) for k, v in p.items()}
+  g = torch.Generator().manual_seed(302)
+  x = _dev(torch.randn(B, T, W, generator=g).to(dtype))
+  gate = _dev(torch.randn(B, T, W, generator=g).to(dtype)) if joined else None
+  h0 = _dev(torch.randn(B, W, generator=g))
+  seg = _dev(helpers.document_positions(B, T, max(T // 3, 2), seed=303))
+  code = 0 if dtype == torch.float32 else 1
+  need = _lib.lib().rg_recurrent_core_workspace_bytes(B, T, W, H, code)
+  y, h, c = ops.recurrent_core(x, seg, P["conv_w"], P["conv_b"], P["w_x"],
+                               P["b_x"], P["w_a"], P["b_a"], P["a_param"],
+                               h0=h0, gate_branch=gate)
+  single = (dtype == torch.bfloat16 and W // H == 256 and
+            (B * H >= 129 or ops.recurrent_prefill_chunked(B, T, W, H)))
+  if single:
+    chunked = ops.recurrent_prefill_chunked(B, T, W, H)
+    assert (need > 0) == chunked
+    y2, h2, c2 = ops.recurrent_prefill(
+        x, seg, P["conv_w"], P["conv_b"], P["w_x"], P["b_x"], P["w_a"],
+        P["b_a"], P["a_param"], h0=h0)
+  else:
+    assert need >= 2 * x.numel() * x.element_size()
+    gx, ga = ops.gates_gemm(x, P["w_x"], P["b_x"], P["w_a"], P["b_a"],
+                            conv=(seg, P["conv_w"], P["conv_b"]))
+    y2, h2, c2 = ops.lru_scan_fused(x, gx, ga, P["a_param"], seg, h0=h0,
+                                    conv=(P["conv_w"], P["conv_b"]),
+                                    return_conv_cache=True)
+  if joined:
+    y2 = ops.gelu_mul(y2, gate)
+  assert torch.equal(y, y2) and torch.equal(h, h2) and torch.equal(c, c2)
+  # and against the oracle
+  ref = R.recurrent_core if dtype == torch.float32 else R.widened_recurrent_core
+  # (the oracle's core has no h0 argument on a prefill: compare a run without)
+  y3, h3, c3 = ops.recurrent_core(x, seg, P["conv_w"], P["conv_b"], P["w_x"],
+                                  P["b_x"], P["w_a"], P["b_a"], P["a_param"])
+  yo, co = ref(x.cpu(), seg.cpu(), p, None)
+  tol = F32_TOL if dtype == torch.float32 else BF16_TOL
+  assert helpers.max_rel(y3, yo) < tol
+  assert helpers.max_rel(h3, co.rg_lru_state) < tol
+  assert torch.equal(c3.cpu(), co.conv1d_state)
+
+
+def test_recurrent_core_entry_rejects_a_short_workspace():
+  B, T, W, H = 1, 512, 512, 2
+  x = _dev(torch.zeros(B, T, W))
+  seg = _dev(torch.arange(T).expand(B, T).contiguous())
+  p = {k: _dev(v) for k, v in R.make_params(W, H, torch.float32, seed=1).items()}
+  y = torch.empty_like(x)
+  need = _lib.lib().rg_recurrent_core_workspace_bytes(B, T, W, H, 0)
+  assert need > 0
+  ws = torch.empty(need - 16, dtype=torch.uint8, device=DEV)
+  ptr = lambda t: t.data_ptr()
+  rc = _lib.lib().rg_recurrent_core(
+      ptr(x), None, ptr(seg), 1, ptr(p["conv_w"]), ptr(p["conv_b"]),
+      ptr(p["w_x"]), ptr(p["b_x"]), ptr(p["w_a"]), ptr(p["b_a"]), None,
+      ptr(p["a_param"]), None, ptr(y), None, None, ptr(ws), need - 16, B, T, W,
+      H, 0, torch.cuda.current_stream().cuda_stream)
+  assert rc == -4
+  assert b"workspace" in _lib.lib().rg_last_error()
 
 
 def test_decode_step_under_graph_capture():
@@ -772,7 +844,6 @@ def test_decode_step_under_graph_capture():
 def test_recurrent_prefill_unsupported_shapes():
   """fp32 and heads that are not 256 wide are refused with RG_ERR_UNSUPPORTED
   (callers use the two-kernel form), nothing is launched."""
-  from recurrentgemma_amd import _lib
   for dtype, W, H in ((torch.float32, 256, 1), (torch.bfloat16, 256, 2)):
     p = {k: _dev(v) for k, v in R.make_params(W, H, dtype, seed=3).items()}
     x = _dev(torch.zeros(1, 8, W, dtype=dtype))
@@ -817,7 +888,6 @@ def test_gelu_mul(dtype, n):
     assert (err > 0).float().mean() < 0.02  # neighbouring-bf16 cases are rare
   # in place on either operand
   a_d, g_d = _dev(a), _dev(g)
-  from recurrentgemma_amd import _lib
   code = 0 if dtype == torch.float32 else 1
   a_io, g_io = a_d.clone(), g_d.clone()
   for src_a, src_g, dst in ((a_io, g_d, a_io), (a_d, g_io, g_io)):
@@ -978,7 +1048,6 @@ def test_config4_full_size_decode():
   tiles x 16 heads, the grid of this shape); at the end: the state and the
   last y equal those of one prefill over all 2112 tokens up to the fp32
   association of the recurrence; a few rows against the oracle end to end."""
-  from recurrentgemma_amd import _lib
   B, T, W, H, steps = 256, 2048, 4096, 16, 64
   dtype = torch.bfloat16
   p = R.make_params(W, H, dtype, seed=1104 + 100)

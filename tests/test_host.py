@@ -24,7 +24,7 @@ def _declared_symbols():
 
 def test_library_exports_every_declared_symbol():
   names = _declared_symbols()
-  assert len(names) == 37, names
+  assert len(names) == 39, names
   lib = ctypes.CDLL(_lib.LIB_PATH)
   for n in names:
     assert hasattr(lib, n), n
@@ -109,6 +109,24 @@ def test_c_side_validation_without_launch():
                           None)
   assert rc == -4 and b"workspace" in lib.rg_last_error()
   # scans cut into chunks: only for few rows and long sequences
+  # rg_recurrent_core: nothing for whole rows in the single kernel, the chunk
+  # summaries for rows in chunks, both gates' pre-activations (+ the scan's
+  # chunk summaries) for the two-kernel form
+  assert lib.rg_recurrent_core_workspace_bytes(16, 8192, 4096, 16, 1) == 0
+  assert (lib.rg_recurrent_core_workspace_bytes(1, 8192, 2560, 10, 1) ==
+          lib.rg_recurrent_prefill_split_workspace_bytes(1, 8192, 2560, 10))
+  assert (lib.rg_recurrent_core_workspace_bytes(1, 512, 2560, 10, 0) ==
+          2 * 512 * 2560 * 4 + lib.rg_scan_split_workspace_bytes(1, 512, 2560))
+  assert lib.rg_recurrent_core_workspace_bytes(2, 100, 512, 2, 1) == 2 * 2 * 100 * 512 * 2
+  assert lib.rg_recurrent_core_workspace_bytes(2, 100, 512, 3, 1) == 0  # W % H
+  rc = lib.rg_recurrent_core(ok, None, ok, 1, ok, ok, ok, ok, ok, ok, None, ok,
+                             None, ok, None, None, None, 0, 2, 100, 512, 2, 1,
+                             None)
+  assert rc == -4 and b"rg_recurrent_core: workspace" in lib.rg_last_error()
+  rc = lib.rg_recurrent_core(ok, ok, ok, 1, ok, ok, ok, ok, ok, ok, None, ok,
+                             None, ok, None, None, None, 0, 16, 64, 4096, 16, 1,
+                             None)
+  assert rc == -1 and b"alias" in lib.rg_last_error()
   assert lib.rg_scan_split_workspace_bytes(16, 8192, 4096) == 0
   assert lib.rg_scan_split_workspace_bytes(1, 500, 2560) == 0
   assert lib.rg_scan_split_workspace_bytes(1, 8192, 2560) == 2 * 22 * 2560 * 4
