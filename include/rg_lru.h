@@ -141,6 +141,26 @@ int rg_linear_scan_backward(const void* dy, const void* a, const void* reset,
                             void* dx, void* da, void* dh0, int B, int T, int W,
                             int dtype, void* stream);
 
+/* Backward pass of RGLRU.forward from the gate pre-activations on
+ * (recurrentgemma/torch/layers.py:335-360 under autograd, with
+ * SqrtBoundDerivative.backward :225-230 and the reversed recurrence of
+ * recurrentgemma/jax/pallas.py:792-846) in one kernel.  Inputs as
+ * rg_lru_scan_fused without the conv takes them: x [B,T,W] (the conv output),
+ * gx_pre / ga_pre [B,T,W], a_param [W], all `dtype`; reset [B,T] bytes
+ * (segment_pos == 0); y the forward output; h0 / dh_last nullable float32
+ * [B,W]; dy the gradient of y.  Outputs: dx, dgx_pre, dga_pre [B,T,W] in
+ * `dtype`; d_a_param_rows float32 [B,W], each row's share of a_param's
+ * gradient (the caller sums over B); dh0 (nullable) float32 [B,W].  The gates
+ * and coefficients are recomputed from the pre-activations with the forward
+ * kernels' arithmetic; everything runs in float32 and is rounded once per
+ * output.  No output may alias an input or another output. */
+int rg_rglru_backward(const void* dy, const void* x, const void* gx_pre,
+                      const void* ga_pre, const void* a_param,
+                      const void* reset, const void* y, const void* h0,
+                      const void* dh_last, void* dx, void* dgx_pre,
+                      void* dga_pre, void* d_a_param_rows, void* dh0, int B,
+                      int T, int W, int dtype, void* stream);
+
 /* The two scans above for few rows and channels: one workgroup per (row, slab
  * of 256 or 128 channels) leaves most of the GPU idle when B * W / 256 is
  * small (a single prompt: 10 to 16 workgroups).  These variants cut every

@@ -645,6 +645,58 @@ int rg_linear_scan_backward(const void* dy, const void* a, const void* reset,
                                      s, dtype, (hipStream_t)stream));
 }
 
+int rg_rglru_backward(const void* dy, const void* x, const void* gx_pre,
+                      const void* ga_pre, const void* a_param,
+                      const void* reset, const void* y, const void* h0,
+                      const void* dh_last, void* dx, void* dgx_pre,
+                      void* dga_pre, void* d_a_param_rows, void* dh0, int B,
+                      int T, int W, int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(B > 0 && T > 0 && W > 0, "%s: B=%d T=%d W=%d must be positive",
+             __func__, B, T, W);
+  RG_CHECK_PTR(dy);
+  RG_CHECK_PTR(x);
+  RG_CHECK_PTR(gx_pre);
+  RG_CHECK_PTR(ga_pre);
+  RG_CHECK_PTR(a_param);
+  RG_CHECK_PTR(reset);
+  RG_CHECK_PTR(y);
+  RG_CHECK_PTR(dx);
+  RG_CHECK_PTR(dgx_pre);
+  RG_CHECK_PTR(dga_pre);
+  RG_CHECK_PTR(d_a_param_rows);
+  RG_CHECK_OPT_PTR(h0);
+  RG_CHECK_OPT_PTR(dh_last);
+  RG_CHECK_OPT_PTR(dh0);
+  const void* ins[] = {dy, x, gx_pre, ga_pre, y};
+  void* outs[] = {dx, dgx_pre, dga_pre};
+  for (void* o : outs)
+    for (const void* i : ins)
+      RG_REQUIRE(o != i, "%s: an output aliases an input", __func__);
+  RG_REQUIRE(dx != dgx_pre && dx != dga_pre && dgx_pre != dga_pre,
+             "%s: outputs alias each other", __func__);
+  rg::RglruBwdArgs s{};
+  s.dy = dy;
+  s.x = x;
+  s.gx = gx_pre;
+  s.ga = ga_pre;
+  s.a_param = a_param;
+  s.reset = reset;
+  s.y = y;
+  s.h0 = (const float*)h0;
+  s.dh_last = (const float*)dh_last;
+  s.dx = dx;
+  s.dgx = dgx_pre;
+  s.dga = dga_pre;
+  s.dlam = (float*)d_a_param_rows;
+  s.dh0 = (float*)dh0;
+  s.B = B;
+  s.T = T;
+  s.W = W;
+  return launch_status(
+      __func__, rg::launch_rglru_backward(s, dtype, (hipStream_t)stream));
+}
+
 size_t rg_recurrent_step_workspace_bytes(int B, int W, int dtype) {
   if (B <= 0 || W <= 0) return 0;
   // conv output + two gate pre-activations, each [B,W], 256-byte aligned

@@ -169,6 +169,25 @@ struct ScanBwdArgs {
 };
 hipError_t launch_linear_scan_backward(const ScanBwdArgs& a, int dtype,
                                        hipStream_t s);
+struct RglruBwdArgs {
+  const void* dy;        // [B, T, W] gradient of y
+  const void* x;         // [B, T, W] the RG-LRU's input (the conv output)
+  const void* gx;        // [B, T, W] input gate pre-activations
+  const void* ga;        // [B, T, W] recurrence gate pre-activations
+  const void* a_param;   // [W]
+  const void* reset;     // [B, T] bytes
+  const void* y;         // [B, T, W] the forward outputs
+  const float* h0;       // [B, W] or null
+  const float* dh_last;  // [B, W] or null: gradient of the final state
+  void* dx;              // [B, T, W]
+  void* dgx;             // [B, T, W]
+  void* dga;             // [B, T, W]
+  float* dlam;           // [B, W]: each row's share of a_param's gradient
+  float* dh0;            // [B, W] or null
+  int B, T, W;
+};
+hipError_t launch_rglru_backward(const RglruBwdArgs& a, int dtype,
+                                 hipStream_t s);
 void scan_split_plan(int B, int T, int W, int granule, int* chunks,
                      int* t_chunk);
 // Chunk lengths are multiples of this for the kernel that handles (dtype, W).

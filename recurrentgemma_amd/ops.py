@@ -586,6 +586,39 @@ def attention_decode_finish(from_ring, probs, k_new, v_new, ring_keys,
   return out
 
 
+def rglru_backward(dy, x, gx_pre, ga_pre, a_param, reset, y, h0=None,
+                   dh_last=None):
+  """Gradients of the RG-LRU from its gate pre-activations on (the forward is
+  lru_scan_fused without the conv): (dx, dgx_pre, dga_pre, d_a_param, dh0 |
+  None) from the gradient of y and of the final state; one kernel."""
+  B, T, W = y.shape
+  y = _dev(y, "y")
+  _same(y.dtype, y.device, dy=dy, x=x, gx_pre=gx_pre, ga_pre=ga_pre,
+        a_param=a_param)
+  assert dy.shape == x.shape == gx_pre.shape == ga_pre.shape == y.shape
+  assert a_param.shape == (W,)
+  dy, x, gx_pre, ga_pre, a_param = (
+      _dev(dy, "dy"), _dev(x, "x"), _dev(gx_pre, "gx_pre"),
+      _dev(ga_pre, "ga_pre"), _dev(a_param, "a_param"))
+  assert reset.shape == (B, T) and reset.dtype == torch.bool
+  reset = _dev(reset, "reset")
+  if h0 is not None:
+    assert h0.dtype == torch.float32 and h0.shape == (B, W)
+    h0 = _dev(h0, "h0")
+  if dh_last is not None:
+    assert dh_last.dtype == torch.float32 and dh_last.shape == (B, W)
+    dh_last = _dev(dh_last, "dh_last")
+  dx, dgx, dga = (torch.empty_like(y) for _ in range(3))
+  rows = torch.empty((B, W), dtype=torch.float32, device=y.device)
+  dh0 = torch.empty_like(h0) if h0 is not None else None
+  with _on(y.device):
+    _lib.check(_lib.lib().rg_rglru_backward(
+        _p(dy), _p(x), _p(gx_pre), _p(ga_pre), _p(a_param), _p(reset), _p(y),
+        _p(h0), _p(dh_last), _p(dx), _p(dgx), _p(dga), _p(rows), _p(dh0), B, T,
+        W, _dtype_code(y), _stream(y)))
+  return dx, dgx, dga, rows.sum(0).to(a_param.dtype), dh0
+
+
 _packed_weights = {}  # (id(w_x), id(w_a)) -> (ref_x, ref_a, stamp, packed)
 
 

@@ -6,7 +6,9 @@ backward pass.  Inside `with training.differentiable():` the drop-in modules
 reference's sequence of tensor ops (recurrentgemma/torch/layers.py:127-137,
 313-365, 447-529) on the GPU under autograd, except for the one part that is
 a Python loop over time there: the linear recurrence (layers.py:140-191),
-which is the scan kernel in both directions --
+which is the scan kernel in both directions (and, for the RG-LRU, the gating
+around it: one forward and one backward kernel from the gate pre-activations
+on, rg_rglru_backward) --
 
   forward   h_t = a_t h_{t-1} + x_t
   backward  g_t = dy_t + a_{t+1} g_{t+1}     (the same recurrence, time
@@ -113,8 +115,41 @@ def conv1d(x, segment_pos, w, b):
   return out + b
 
 
+class _GatedScan(torch.autograd.Function):
+  """RGLRU.forward from the gate pre-activations on (layers.py:338-360): the
+  inference kernel forwards, one kernel backwards (the reversed recurrence
+  with the derivatives of both sigmoids, of exp and of the clipped sqrt
+  inside it); only y and the inputs are kept."""
+
+  @staticmethod
+  def forward(ctx, x, gx_pre, ga_pre, a_param, segment_pos, h0):
+    x, gx_pre, ga_pre = x.contiguous(), gx_pre.contiguous(), ga_pre.contiguous()
+    y, h_last, _ = ops.lru_scan_fused(x, gx_pre, ga_pre, a_param, segment_pos,
+                                      h0=h0)
+    ctx.save_for_backward(x, gx_pre, ga_pre, a_param, segment_pos == 0, y, h0)
+    return y, h_last
+
+  @staticmethod
+  def backward(ctx, dy, dh_last):
+    x, gx_pre, ga_pre, a_param, reset, y, h0 = ctx.saved_tensors
+    dh = None if dh_last is None else dh_last.float().contiguous()
+    dy = torch.zeros_like(y) if dy is None else dy.contiguous()
+    dx, dgx, dga, dlam, dh0 = ops.rglru_backward(
+        dy, x, gx_pre, ga_pre, a_param, reset, y, h0, dh)
+    return dx, dgx, dga, dlam, None, dh0
+
+
 def rg_lru(x, segment_pos, a_param, w_x, b_x, w_a, b_a, h0=None):
-  """RGLRU.forward (layers.py:313-365) with the recurrence on the scan kernel.
+  """RGLRU.forward (layers.py:313-365): the two gate projections as tensor
+  ops, everything after them on the kernels.  Returns (y, h_last)."""
+  return _GatedScan.apply(x, block_diag_linear(x, w_x, b_x),
+                          block_diag_linear(x, w_a, b_a), a_param, segment_pos,
+                          h0)
+
+
+def rg_lru_tensor_ops(x, segment_pos, a_param, w_x, b_x, w_a, b_a, h0=None):
+  """The same as the reference's sequence of tensor ops under autograd, with
+  only the recurrence on the scan kernel (the form rg_lru is tested against).
   Returns (y, h_last)."""
   reset = segment_pos == 0
   gate_x = torch.sigmoid(block_diag_linear(x, w_x, b_x))

@@ -160,3 +160,118 @@ def test_scan_backward_kernel(dtype, B, T, W):
       assert ((got_dh0.double().cpu() - dh0).abs().max() / scale(dh0)) < 1e-5
     else:
       assert got_dh0 is None
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,T,W,H", [(2, 1, 64, 2), (3, 19, 96, 3),
+                                     (1, 333, 130, 1), (2, 700, 256, 2)])
+def test_rglru_backward_kernel(dtype, B, T, W, H):
+  """training.rg_lru (forward and backward kernels from the gate
+  pre-activations on) against autograd through the reference's formulas
+  (layers.py:335-360, the sqrt with its clipped derivative :216-230) evaluated
+  in float64 on the CPU with a loop over time, on the same dtype-valued
+  inputs: y, h_last and the gradients of x, both gate matrices and biases,
+  a_param and h0; document starts, one and two channels per lane, sequences of
+  one token up to several rows per wave.  Tolerance relative to the largest
+  magnitude of each tensor: 1e-4 float32 (sums in another order), 2e-2 bf16
+  (the kernels round x, the pre-activations, y and each gradient to bf16)."""
+  from oracle import torch_ref as R
+  gen = torch.Generator().manual_seed(B * 1000 + T)
+  p = R.make_params(W, H, dtype, seed=T + 5, gate_bias_std=0.3)
+  x = torch.randn(B, T, W, generator=gen).to(dtype)
+  h0 = torch.randn(B, W, generator=gen)
+  seg = torch.arange(T).expand(B, T).clone()
+  for b in range(B):
+    for start in torch.nonzero(torch.rand(T, generator=gen) < 0.04).flatten():
+      seg[b, start:] = torch.arange(T - int(start))
+  if T > 1:
+    seg[0, 0] = 7  # a row that continues a document: h0 counts
+  r = torch.randn(B, T, W, generator=gen)
+  rh = torch.randn(B, W, generator=gen)
+  names = ("a_param", "w_x", "b_x", "w_a", "b_a")
+
+  # float64 on the CPU
+  q = {k: p[k].double().requires_grad_(True) for k in names}
+  xd, hd = x.double().requires_grad_(True), h0.double().requires_grad_(True)
+  reset = seg == 0
+
+  class BoundedSqrt(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, v):
+      ctx.save_for_backward(v)
+      return torch.sqrt(v)
+
+    @staticmethod
+    def backward(ctx, grad):
+      (v,) = ctx.saved_tensors
+      return grad / torch.sqrt(torch.clip(4.0 * v, min=1 / 1000.0 ** 2))
+
+  def bdl(v, w, b):
+    vs = v.reshape(B, T, H, W // H)
+    return (torch.einsum("bthi,hij->bthj", vs, w) + b).reshape(B, T, W)
+
+  # the kernels take the pre-activations as tensors of the activation dtype
+  def as_dtype(v):
+    return v + (v.detach().to(dtype).double() - v.detach())
+  gx = torch.sigmoid(as_dtype(bdl(xd, q["w_x"], q["b_x"])))
+  ga = torch.sigmoid(as_dtype(bdl(xd, q["w_a"], q["b_a"])))
+  log_a = -8.0 * ga * torch.nn.functional.softplus(q["a_param"])
+  a = torch.exp(log_a)
+  mult = BoundedSqrt.apply(1 - torch.exp(2 * log_a))
+  mult = reset[..., None] + ~reset[..., None] * mult
+  xn = xd * gx * mult
+  h, ys = hd, []
+  for t in range(T):
+    h = a[:, t] * (~reset[:, t])[:, None] * h + xn[:, t]
+    ys.append(h)
+  yd = torch.stack(ys, 1)
+  ((yd * r).sum() + (h * rh).sum()).backward()
+
+  # the kernels
+  qg = {k: p[k].to(DEV).requires_grad_(True) for k in names}
+  xg, hg = x.to(DEV).requires_grad_(True), h0.to(DEV).requires_grad_(True)
+  with training.differentiable():
+    y, hl = training.rg_lru(xg, seg.to(DEV), qg["a_param"], qg["w_x"],
+                            qg["b_x"], qg["w_a"], qg["b_a"], hg)
+  ((y.float() * r.to(DEV)).sum() + (hl * rh.to(DEV)).sum()).backward()
+
+  tol = 1e-4 if dtype == torch.float32 else 2e-2
+
+  def near(got, want, what):
+    want = want.detach().double()
+    err = (got.detach().double().cpu() - want).abs().max().item()
+    scale = max(want.abs().max().item(), 1e-12)
+    assert err <= tol * scale, (what, err, scale)
+
+  near(y, yd, "y")
+  near(hl, h, "h_last")
+  near(xg.grad, xd.grad, "dx")
+  near(hg.grad, hd.grad, "dh0")
+  for k in names:
+    assert qg[k].grad.dtype == dtype
+    near(qg[k].grad, q[k].grad, "d" + k)
+
+
+def test_rglru_forms_agree():
+  """The fused form against the same layer as tensor ops around the scan
+  kernels, both on the GPU in float32."""
+  from oracle import torch_ref as R
+  B, T, W, H = 2, 500, 512, 2
+  gen = torch.Generator().manual_seed(3)
+  p = R.make_params(W, H, torch.float32, seed=9, gate_bias_std=0.3)
+  x = torch.randn(B, T, W, generator=gen)
+  seg = torch.arange(T).expand(B, T).clone()
+  seg[1, 200:] -= 200
+  r = torch.randn(B, T, W, generator=gen).to(DEV)
+  names = ("a_param", "w_x", "b_x", "w_a", "b_a")
+  grads = []
+  for fn in (training.rg_lru, training.rg_lru_tensor_ops):
+    q = {k: p[k].to(DEV).requires_grad_(True) for k in names}
+    xg = x.to(DEV).requires_grad_(True)
+    with training.differentiable():
+      y, _ = fn(xg, seg.to(DEV), *(q[k] for k in names))
+    (y * r).sum().backward()
+    grads.append([y, xg.grad] + [q[k].grad for k in names])
+  for got, want, what in zip(grads[0], grads[1], ("y", "dx") + names):
+    err = (got - want).abs().max().item()
+    assert err <= 1e-4 * want.abs().max().item(), (what, err)
