@@ -62,6 +62,22 @@ int rg_conv1d_prefill(const void* x, const void* segpos, int segpos_is_i64,
                       void* cache_out, int B, int T, int W, int K, int dtype,
                       void* stream);
 
+/* Backward pass of rg_conv1d_prefill (Conv1D.forward without a cache under
+ * autograd, recurrentgemma/torch/layers.py:477-520): from dout [B,T,W], the
+ * gradient of the conv output, dx [B,T,W] (`dtype`) and, in `partial`
+ * (float32 [chunks][temporal_width + 1][W], chunks =
+ * rg_conv1d_backward_workspace_bytes / ((temporal_width + 1) * W * 4)), per
+ * chunk of rows the sums that add up to the gradient of w (planes 0 ..
+ * temporal_width-1, laid out like w) and of b (last plane); the caller sums
+ * over the chunks.  Taps cut by a document start carry no gradient, as in the
+ * forward pass.  2 <= temporal_width <= RG_MAX_CONV_WIDTH. */
+size_t rg_conv1d_backward_workspace_bytes(int B, int T, int W,
+                                          int temporal_width);
+int rg_conv1d_backward(const void* dout, const void* x, const void* segpos,
+                       int segpos_is_i64, const void* w, void* dx,
+                       void* partial, size_t partial_bytes, int B, int T, int W,
+                       int temporal_width, int dtype, void* stream);
+
 /* Conv1D.forward, decode branch (cache given, exactly one token):
  * recurrentgemma/torch/layers.py:469-474,491-529,531-550.  No document mask.
  *   out[b,c] = bias[c] + sum_k w[k,c] * concat(cache_in, x)[b,k,c]

@@ -51,6 +51,9 @@ SIGNATURES = {
                           [_sz, _i, _i, _i, _i, _i, _vp]),
     "rg_linear_scan": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "rg_linear_scan_backward": (_i, [_vp] * 9 + [_i, _i, _i, _i, _vp]),
+    "rg_conv1d_backward_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "rg_conv1d_backward": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _sz, _i, _i,
+                                _i, _i, _i, _vp]),
     "rg_rglru_backward": (_i, [_vp] * 14 + [_i, _i, _i, _i, _vp]),
     "rg_scan_split_workspace_bytes": (_sz, [_i, _i, _i]),
     "rg_lru_scan_fused_split": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i,

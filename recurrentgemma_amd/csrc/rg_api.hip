@@ -113,6 +113,49 @@ int rg_conv1d_prefill(const void* x, const void* segpos, int segpos_is_i64,
                        rg::launch_conv1d_prefill(a, dtype, (hipStream_t)stream));
 }
 
+size_t rg_conv1d_backward_workspace_bytes(int B, int T, int W, int K) {
+  if (B <= 0 || T <= 0 || W <= 0 || K < 2 || K > RG_MAX_CONV_WIDTH) return 0;
+  return (size_t)rg::conv1d_backward_chunks(B, T) * (K + 1) * W * sizeof(float);
+}
+
+int rg_conv1d_backward(const void* dout, const void* x, const void* segpos,
+                       int segpos_is_i64, const void* w, void* dx,
+                       void* partial, size_t partial_bytes, int B, int T, int W,
+                       int temporal_width, int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(B > 0 && T > 0 && W > 0, "%s: B=%d T=%d W=%d must be positive",
+             __func__, B, T, W);
+  if (temporal_width < 2 || temporal_width > RG_MAX_CONV_WIDTH)
+    return fail(RG_ERR_UNSUPPORTED, "%s: temporal width %d outside [2,%d]",
+                __func__, temporal_width, RG_MAX_CONV_WIDTH);
+  RG_CHECK_PTR(dout);
+  RG_CHECK_PTR(x);
+  RG_CHECK_PTR(segpos);
+  RG_CHECK_PTR(w);
+  RG_CHECK_PTR(dx);
+  RG_REQUIRE(dx != dout && dx != x, "%s: dx must not alias an input", __func__);
+  const size_t need =
+      rg_conv1d_backward_workspace_bytes(B, T, W, temporal_width);
+  if (partial == nullptr || partial_bytes < need || !aligned16(partial))
+    return fail(RG_ERR_WORKSPACE,
+                "%s: partial sums need %zu bytes (16-byte aligned), got %zu",
+                __func__, need, partial ? partial_bytes : (size_t)0);
+  rg::ConvBwdArgs a{};
+  a.dout = dout;
+  a.x = x;
+  a.segpos = segpos;
+  a.seg_kind = segpos_is_i64 ? 1 : 0;
+  a.w = w;
+  a.dx = dx;
+  a.partial = (float*)partial;
+  a.B = B;
+  a.T = T;
+  a.W = W;
+  a.K = temporal_width;
+  return launch_status(
+      __func__, rg::launch_conv1d_backward(a, dtype, (hipStream_t)stream));
+}
+
 int rg_conv1d_step(const void* x, const void* cache_in, const void* w,
                    const void* bias, void* out, void* cache_out, int B, int W,
                    int K, int dtype, void* stream) {
@@ -488,7 +531,9 @@ static CorePlan core_plan(int B, int T, int W, int H, int dtype) {
   if (p.single) {
     p.split_bytes = chunk_bytes;
   } else {
-    p.split_bytes = rg_scan_split_workspace_bytes(B, T, W);
+    // (rounded up: the gate planes behind it must stay 16-byte aligned)
+    p.split_bytes =
+        (rg_scan_split_workspace_bytes(B, T, W) + 255) & ~(size_t)255;
     const size_t n = (size_t)B * T * W * (dtype == RG_DTYPE_F32 ? 4 : 2);
     p.gate_bytes = (n + 255) & ~(size_t)255;
   }

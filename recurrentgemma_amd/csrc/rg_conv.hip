@@ -54,6 +54,65 @@ conv1d_cache_tail_kernel(const T* __restrict__ x,
   }
 }
 
+// Backward pass of the prefill conv.  With keep_s[t] = "no document starts
+// among tokens t-s+1 .. t" (what conv_point applies tap by tap):
+//   out[t] = bias + sum_s w[K-1-s] x[t-s] keep_s[t]
+//   dx[u]      = sum_s w[K-1-s] dout[u+s] keep_s[u+s]        (u + s < T)
+//   dw[K-1-s] += x[t-s] keep_s[t] dout[t],   dbias += dout[t]
+// A thread owns one channel and a run of kConvBwdRows consecutive flattened
+// rows (b, t): it writes dx for them and leaves its sums of dw and dbias in
+// `partial` [row chunks][K + 1][W] (float32), which the caller adds up.  The
+// neighbouring rows it re-reads come from cache.
+constexpr int kConvBwdRows = 32;
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+conv1d_backward_kernel(const T* __restrict__ dout, const T* __restrict__ x,
+                       const void* __restrict__ segpos, int seg_kind,
+                       const T* __restrict__ w, T* __restrict__ dx,
+                       float* __restrict__ partial, int T_len, int W, int K,
+                       int64_t M) {
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= W) return;
+  const int64_t m0 = (int64_t)blockIdx.x * kConvBwdRows;
+  const int64_t m1 = m0 + kConvBwdRows < M ? m0 + kConvBwdRows : M;
+  constexpr int kMaxK = 16;  // widths above are refused by the caller
+  float wk[kMaxK], dw[kMaxK], db = 0.0f;
+#pragma unroll
+  for (int s = 0; s < kMaxK; ++s) {
+    wk[s] = s < K ? load_scalar(w + (int64_t)(K - 1 - s) * W + c) : 0.0f;
+    dw[s] = 0.0f;
+  }
+  for (int64_t m = m0; m < m1; ++m) {
+    const int t = (int)(m % T_len);
+    const float g = load_scalar(dout + m * W + c);
+    db += g;
+    float acc = 0.0f;
+    bool back = true, ahead = true;
+#pragma unroll
+    for (int s = 0; s < kMaxK; ++s) {
+      if (s < K) {
+        // tap s of token t looks back at x[t-s]
+        if (s > 0 && s <= t && is_doc_start(segpos, seg_kind, m - s + 1))
+          back = false;
+        if (s <= t && back)
+          dw[s] = __builtin_fmaf(load_scalar(x + (m - s) * W + c), g, dw[s]);
+        // token t is x[t'-s] of token t' = t + s
+        if (s > 0 && t + s < T_len && is_doc_start(segpos, seg_kind, m + s))
+          ahead = false;
+        if (t + s < T_len && ahead)
+          acc = __builtin_fmaf(wk[s], load_scalar(dout + (m + s) * W + c), acc);
+      }
+    }
+    store_scalar(dx + m * W + c, acc);
+  }
+  float* out = partial + (int64_t)blockIdx.x * (K + 1) * W + c;
+#pragma unroll
+  for (int s = 0; s < kMaxK; ++s)
+    if (s < K) out[(int64_t)(K - 1 - s) * W] = dw[s];
+  out[(int64_t)K * W] = db;
+}
+
 // Decode step: one thread per (batch row, channel).  All state rows are read
 // into registers before anything is written, so cache_out may alias cache_in.
 template <typename T>
@@ -130,6 +189,30 @@ hipError_t launch_conv1d_prefill(const ConvArgs& a, int dtype, hipStream_t s) {
 hipError_t launch_conv1d_step(const ConvStepArgs& a, int dtype,
                               hipStream_t s) {
   return dtype == 0 ? conv_step_t<float>(a, s) : conv_step_t<uint16_t>(a, s);
+}
+
+int conv1d_backward_chunks(int B, int T) {
+  return (int)(((int64_t)B * T + kConvBwdRows - 1) / kConvBwdRows);
+}
+
+hipError_t launch_conv1d_backward(const ConvBwdArgs& a, int dtype,
+                                  hipStream_t s) {
+  const int64_t M = (int64_t)a.B * a.T;
+  const int64_t chunks = conv1d_backward_chunks(a.B, a.T);
+  const int64_t cblocks = ((int64_t)a.W + 255) / 256;
+  if (chunks <= 0 || chunks > 0x7fffffff || cblocks > 65535 || a.K < 2 ||
+      a.K > 16)
+    return hipErrorInvalidValue;
+  const dim3 grid((unsigned)chunks, (unsigned)cblocks);
+  if (dtype == 0)
+    conv1d_backward_kernel<float><<<grid, 256, 0, s>>>(
+        (const float*)a.dout, (const float*)a.x, a.segpos, a.seg_kind,
+        (const float*)a.w, (float*)a.dx, a.partial, a.T, a.W, a.K, M);
+  else
+    conv1d_backward_kernel<uint16_t><<<grid, 256, 0, s>>>(
+        (const uint16_t*)a.dout, (const uint16_t*)a.x, a.segpos, a.seg_kind,
+        (const uint16_t*)a.w, (uint16_t*)a.dx, a.partial, a.T, a.W, a.K, M);
+  return hipGetLastError();
 }
 
 }  // namespace rg

@@ -149,6 +149,19 @@ struct LinearArgs {
 // Each returns hipSuccess or the launch error.  dtype: 0 = f32, 1 = bf16.
 hipError_t launch_conv1d_prefill(const ConvArgs& a, int dtype, hipStream_t s);
 hipError_t launch_conv1d_step(const ConvStepArgs& a, int dtype, hipStream_t s);
+struct ConvBwdArgs {
+  const void* dout;  // [B, T, W] gradient of the conv output
+  const void* x;     // [B, T, W] the conv input
+  const void* segpos;
+  int seg_kind;
+  const void* w;     // [K, W]
+  void* dx;          // [B, T, W]
+  float* partial;    // [conv1d_backward_chunks(B, T)][K + 1][W]
+  int B, T, W, K;
+};
+int conv1d_backward_chunks(int B, int T);
+hipError_t launch_conv1d_backward(const ConvBwdArgs& a, int dtype,
+                                  hipStream_t s);
 hipError_t launch_gemm_generic(const GemmArgs& a, int dtype, hipStream_t s);
 hipError_t launch_gemm_mfma_bf16(const GemmArgs& a, hipStream_t s);
 hipError_t launch_gemm_mfma_f32(const GemmArgs& a, hipStream_t s);

@@ -112,6 +112,28 @@ def conv1d_prefill(x, segment_pos, w, b, return_cache=True):
   return out, cache
 
 
+def conv1d_backward(dout, x, segment_pos, w):
+  """Gradients of conv1d_prefill: (dx, dw, db) from the gradient of its
+  output; one kernel and a sum over its per-chunk partial sums."""
+  B, T, W = x.shape
+  K = w.shape[0]
+  assert w.shape == (K, W) and dout.shape == x.shape
+  x = _dev(x, "x")
+  _same(x.dtype, x.device, dout=dout, w=w)
+  dout, w = _dev(dout, "dout"), _dev(w, "w")
+  seg, is64 = _segpos(segment_pos, B, T)
+  lib = _lib.lib()
+  need = lib.rg_conv1d_backward_workspace_bytes(B, T, W, K)
+  partial = torch.empty(need // 4, dtype=torch.float32, device=x.device)
+  dx = torch.empty_like(x)
+  with _on(x.device):
+    _lib.check(lib.rg_conv1d_backward(
+        _p(dout), _p(x), _p(seg), is64, _p(w), _p(dx), _p(partial), need, B, T,
+        W, K, _dtype_code(x), _stream(x)))
+  sums = partial.view(-1, K + 1, W).sum(0)
+  return dx, sums[:K].to(w.dtype), sums[K].to(w.dtype)
+
+
 def conv1d_step(x, cache, w, b, return_cache=True):
   B, n_tok, W = x.shape
   K = w.shape[0]

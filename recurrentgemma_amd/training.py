@@ -96,9 +96,33 @@ def block_diag_linear(x, w, b):
   return y.reshape(x.shape)
 
 
+class _Conv1d(torch.autograd.Function):
+  """Conv1D.forward without a cache (layers.py:447-529): the conv kernel
+  forwards, rg_conv1d_backward backwards."""
+
+  @staticmethod
+  def forward(ctx, x, segment_pos, w, b):
+    x = x.contiguous()
+    out, _ = ops.conv1d_prefill(x, segment_pos, w, b, return_cache=False)
+    ctx.save_for_backward(x, segment_pos, w)
+    return out
+
+  @staticmethod
+  def backward(ctx, dout):
+    x, segment_pos, w = ctx.saved_tensors
+    dx, dw, db = ops.conv1d_backward(dout.contiguous(), x, segment_pos, w)
+    return dx, None, dw, db
+
+
 def conv1d(x, segment_pos, w, b):
+  """Conv1D.forward without a cache, on the kernels in both directions."""
+  return _Conv1d.apply(x, segment_pos, w, b)
+
+
+def conv1d_tensor_ops(x, segment_pos, w, b):
   """Conv1D.forward without a cache (layers.py:447-529), functional: tap s of
-  token t is x[t - s] unless a document starts at one of t-s+1 .. t."""
+  token t is x[t - s] unless a document starts at one of t-s+1 .. t.  (The
+  form conv1d is tested against.)"""
   K = w.shape[0]
   T = x.shape[1]
   not_start = (segment_pos != 0).to(x.dtype)  # [B, T]

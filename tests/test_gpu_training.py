@@ -275,3 +275,66 @@ def test_rglru_forms_agree():
   for got, want, what in zip(grads[0], grads[1], ("y", "dx") + names):
     err = (got - want).abs().max().item()
     assert err <= 1e-4 * want.abs().max().item(), (what, err)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,T,W,K", [(2, 1, 64, 4), (3, 19, 96, 4),
+                                     (2, 100, 300, 4), (1, 70, 64, 2),
+                                     (2, 45, 130, 7)])
+def test_conv_backward_kernel(dtype, B, T, W, K):
+  """training.conv1d (conv kernel forwards, rg_conv1d_backward backwards)
+  against autograd through the conv's definition written out token by token
+  in float64 on the CPU (tap s of token t is x[t-s] unless a document starts
+  at one of t-s+1 .. t; layers.py:477-520), same dtype-valued inputs: output
+  and the gradients of x, w and b; document starts including in the last and
+  first positions, temporal widths 2, 4 and 7, row counts that fill one
+  32-row chunk of the kernel, several and a part of one.  Tolerance relative
+  to each tensor's largest magnitude: 1e-5 float32, 1e-2 bf16."""
+  gen = torch.Generator().manual_seed(B * 100 + T + K)
+  x = torch.randn(B, T, W, generator=gen).to(dtype)
+  w = (torch.randn(K, W, generator=gen) * 0.5).to(dtype)
+  b = torch.randn(W, generator=gen).to(dtype)
+  r = torch.randn(B, T, W, generator=gen).to(dtype)
+  seg = torch.arange(T).expand(B, T).clone()
+  for row in range(B):
+    for start in torch.nonzero(torch.rand(T, generator=gen) < 0.1).flatten():
+      seg[row, start:] = torch.arange(T - int(start))
+  seg[-1, T - 1] = 0
+  if T > 1:
+    seg[0, 0] = 5
+
+  xd, wd, bd = (t.double().requires_grad_(True) for t in (x, w, b))
+  rows = []
+  for t in range(T):
+    acc = bd.expand(B, W)
+    alive = torch.ones(B, dtype=torch.bool)
+    for s in range(min(K, t + 1)):
+      if s > 0:
+        alive = alive & (seg[:, t - s + 1] != 0)
+      acc = acc + xd[:, t - s] * alive[:, None] * wd[K - 1 - s]
+    rows.append(acc)
+  outd = torch.stack(rows, 1)
+  (outd * r.double()).sum().backward()
+
+  xg, wg, bg = (t.to(DEV).requires_grad_(True) for t in (x, w, b))
+  with training.differentiable():
+    out = training.conv1d(xg, seg.to(DEV), wg, bg)
+  (out.float() * r.to(DEV).float()).sum().backward()
+  tol = 1e-5 if dtype == torch.float32 else 1e-2
+
+  def near(got, want, what):
+    want = want.detach().double()
+    err = (got.detach().double().cpu() - want).abs().max().item()
+    assert err <= tol * max(want.abs().max().item(), 1e-12), (what, err)
+
+  near(out, outd, "out")
+  near(xg.grad, xd.grad, "dx")
+  near(wg.grad, wd.grad, "dw")
+  near(bg.grad, bd.grad, "db")
+  assert xg.grad.dtype == dtype and wg.grad.dtype == dtype
+
+  # and the tensor-op form of the same conv on the GPU
+  x2, w2, b2 = (t.to(DEV).requires_grad_(True) for t in (x, w, b))
+  out2 = training.conv1d_tensor_ops(x2, seg.to(DEV), w2, b2)
+  (out2.float() * r.to(DEV).float()).sum().backward()
+  near(x2.grad, xd.grad, "dx (tensor ops)")
