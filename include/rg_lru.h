@@ -447,6 +447,22 @@ int rg_recurrent_step_packed(const void* x, const void* segpos,
                              const void* a_param, void* y, int B, int W, int H,
                              int dtype, void* stream);
 
+/* rg_recurrent_step_packed with the recurrent block's join applied where y is
+ * stored (RecurrentBlock.forward, recurrentgemma/torch/modules.py:627-628,
+ * 644, on a decode step): out = y * gelu_tanh(gate_branch), gate_branch
+ * [B,1,W] being the block's linear_y output before its activation.  Same
+ * values, bit for bit, as rg_recurrent_step_packed followed by
+ * rg_gelu_mul(y, gate_branch); out may alias gate_branch, not x.  bf16 with
+ * 256-wide heads only (RG_ERR_UNSUPPORTED otherwise: use the separate calls). */
+int rg_recurrent_step_gelu_mul(const void* x, const void* gate_branch,
+                               const void* segpos, int segpos_is_i64,
+                               const void* conv_cache_in, void* conv_cache_out,
+                               const void* h_in, void* h_out,
+                               const void* conv_w, const void* conv_b,
+                               const void* w_packed, const void* b_x,
+                               const void* b_a, const void* a_param, void* out,
+                               int B, int W, int H, int dtype, void* stream);
+
 /* The two steps between the last linear layer and the next token id:
  * rg_soft_cap: out = tanh(x / cap) * cap over n elements (griffin.py:203-206),
  *   one pass with the roundings of torch's three (quotient as x * (1 / cap),

@@ -91,6 +91,8 @@ SIGNATURES = {
     "rg_recurrent_step_packed": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp,
                                       _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i,
                                       _i, _vp]),
+    "rg_recurrent_step_gelu_mul": (_i, [_vp, _vp, _vp, _i] + [_vp] * 11 +
+                                   [_i, _i, _i, _i, _vp]),
     "rg_recurrent_step": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i,
                                _vp]),

@@ -1122,21 +1122,22 @@ int rg_add_rms_norm_partial(const void* partial, int slices, const void* bias,
                                             width, eps, (hipStream_t)stream));
 }
 
-int rg_recurrent_step_packed(const void* x, const void* segpos,
-                             int segpos_is_i64, const void* conv_cache_in,
-                             void* conv_cache_out, const void* h_in,
-                             void* h_out, const void* conv_w,
-                             const void* conv_b, const void* w_packed,
-                             const void* b_x, const void* b_a,
-                             const void* a_param, void* y, int B, int W, int H,
-                             int dtype, void* stream) {
+#undef RG_WHO
+#define RG_WHO who
+static int recurrent_step_packed_impl(
+    const char* who, const void* x, const void* gate_branch,
+    const void* segpos, int segpos_is_i64, const void* conv_cache_in,
+    void* conv_cache_out, const void* h_in, void* h_out, const void* conv_w,
+    const void* conv_b, const void* w_packed, const void* b_x, const void* b_a,
+    const void* a_param, void* y, int B, int W, int H, int dtype,
+    void* stream) {
   RG_CHECK_DTYPE(dtype);
   RG_REQUIRE(B > 0 && W > 0 && H > 0, "%s: B=%d W=%d H=%d must be positive",
-             __func__, B, W, H);
-  RG_REQUIRE(W % H == 0, "%s: W=%d is not a multiple of H=%d", __func__, W, H);
+             who, B, W, H);
+  RG_REQUIRE(W % H == 0, "%s: W=%d is not a multiple of H=%d", who, W, H);
   if (dtype != RG_DTYPE_BF16 || W / H != 256)
     return fail(RG_ERR_UNSUPPORTED,
-                "%s: needs bf16 and W/H == 256 (dtype=%d W=%d H=%d)", __func__,
+                "%s: needs bf16 and W/H == 256 (dtype=%d W=%d H=%d)", who,
                 dtype, W, H);
   RG_CHECK_PTR(x);
   RG_CHECK_PTR(segpos);
@@ -1151,7 +1152,10 @@ int rg_recurrent_step_packed(const void* x, const void* segpos,
   RG_CHECK_PTR(b_a);
   RG_CHECK_PTR(a_param);
   RG_CHECK_PTR(y);
-  RG_REQUIRE(y != x, "%s: y must not alias x", __func__);
+  RG_CHECK_OPT_PTR(gate_branch);
+  RG_REQUIRE(gate_branch == nullptr || gate_branch != x,
+             "%s: gate_branch must not alias x", who);
+  RG_REQUIRE(y != x, "%s: y must not alias x", who);
   rg::StepArgs a{};
   a.x = x;
   a.segpos = segpos;
@@ -1167,11 +1171,44 @@ int rg_recurrent_step_packed(const void* x, const void* segpos,
   a.b[1] = b_a;
   a.a_param = a_param;
   a.y = y;
+  a.gate_branch = gate_branch;
   a.B = B;
   a.W = W;
   a.H = H;
-  return launch_status(__func__,
+  return launch_status(who,
                        rg::launch_block_step_bf16(a, (hipStream_t)stream));
+}
+#undef RG_WHO
+#define RG_WHO __func__
+
+int rg_recurrent_step_packed(const void* x, const void* segpos,
+                             int segpos_is_i64, const void* conv_cache_in,
+                             void* conv_cache_out, const void* h_in,
+                             void* h_out, const void* conv_w,
+                             const void* conv_b, const void* w_packed,
+                             const void* b_x, const void* b_a,
+                             const void* a_param, void* y, int B, int W, int H,
+                             int dtype, void* stream) {
+  return recurrent_step_packed_impl(__func__, x, nullptr, segpos, segpos_is_i64,
+                                    conv_cache_in, conv_cache_out, h_in, h_out,
+                                    conv_w, conv_b, w_packed, b_x, b_a, a_param,
+                                    y, B, W, H, dtype, stream);
+}
+
+int rg_recurrent_step_gelu_mul(const void* x, const void* gate_branch,
+                               const void* segpos, int segpos_is_i64,
+                               const void* conv_cache_in, void* conv_cache_out,
+                               const void* h_in, void* h_out,
+                               const void* conv_w, const void* conv_b,
+                               const void* w_packed, const void* b_x,
+                               const void* b_a, const void* a_param, void* out,
+                               int B, int W, int H, int dtype, void* stream) {
+  RG_CHECK_PTR(gate_branch);
+  return recurrent_step_packed_impl(__func__, x, gate_branch, segpos,
+                                    segpos_is_i64, conv_cache_in,
+                                    conv_cache_out, h_in, h_out, conv_w, conv_b,
+                                    w_packed, b_x, b_a, a_param, out, B, W, H,
+                                    dtype, stream);
 }
 
 }  // extern "C"

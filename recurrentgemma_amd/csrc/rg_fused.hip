@@ -53,6 +53,10 @@ pack_gate_weights_kernel(const uint16_t* __restrict__ w_x,
 constexpr int kStepRows = 32;
 constexpr int kStepRowsPerThread = 4;  // 32 rows x 64 channel quads / 512
 
+// GELU: y leaves as y * gelu(gate_branch), the join of the recurrent block's
+// two branches (recurrentgemma/torch/modules.py:627-628, 644) with the
+// arithmetic and roundings of the stand-alone gelu_mul pass.
+template <bool GELU>
 __global__ void __launch_bounds__(512) block_step_bf16_kernel(StepArgs p) {
   __shared__ __align__(16) uint16_t stage[kStepRows * kLdsStride];
 
@@ -98,6 +102,9 @@ __global__ void __launch_bounds__(512) block_step_bf16_kernel(StepArgs p) {
       p.h_out + (int64_t)b0 * W, (uint32_t)rows_here * 2u * row_bytes);
   const __amdgpu_buffer_rsrc_t ry = make_rsrc(
       (uint16_t*)p.y + (int64_t)b0 * W, (uint32_t)rows_here * row_bytes);
+  const __amdgpu_buffer_rsrc_t rgate =
+      make_rsrc((const uint16_t*)p.gate_branch + (int64_t)b0 * W,
+                GELU ? (uint32_t)rows_here * row_bytes : 0u);
   // ---- loads, in the order they are needed: the conv step's rows (thread =
   //      four channels of four rows: 8-byte accesses, a wave per access covers
   //      the head's 512 bytes of a row), the small per-channel and per-row
@@ -157,6 +164,17 @@ __global__ void __launch_bounds__(512) block_step_bf16_kernel(StepArgs p) {
         __builtin_amdgcn_raw_buffer_load_b32(
             rhin, (uint32_t)ch * 4u + (upper ? 8u * row_bytes : 0u),
             (uint32_t)(8 * (r >> 2) + (r & 3)) * 2u * row_bytes, 0));
+  }
+
+  // GELU: the gate branch where this lane stores y (see the output stage)
+  uint32_t gate2[8];
+  if (GELU) {
+    const uint32_t lane_rows = ((lane & 1) ? 1u : 0u) + (upper ? 4u : 0u);
+#pragma unroll
+    for (int r = 0; r < 16; r += 2)
+      gate2[r >> 1] = __builtin_amdgcn_raw_buffer_load_b32(
+          rgate, (uint32_t)(ch & ~1) * 2u + lane_rows * row_bytes,
+          (uint32_t)(8 * (r >> 2) + (r & 3)) * row_bytes, 0);
   }
 
   Frag bfrag[16][2];
@@ -276,7 +294,15 @@ __global__ void __launch_bounds__(512) block_step_bf16_kernel(StepArgs p) {
     __builtin_amdgcn_raw_buffer_store_b64(
         u32x2{__float_as_uint(lo), __float_as_uint(hi)}, rhout,
         pair_ch * 4u + lane_rows * 2u * row_bytes, tile_row * 2u * row_bytes, 0);
-    __builtin_amdgcn_raw_buffer_store_b32(pack_bf16x2(lo, hi), ry,
+    uint32_t y2 = pack_bf16x2(lo, hi);
+    if (GELU) {
+      const uint32_t g2 = gate2[r >> 1];
+      y2 = pack_bf16x2(gelu_mul_bf16(__uint_as_float(y2 << 16),
+                                     __uint_as_float(g2 << 16)),
+                       gelu_mul_bf16(__uint_as_float(y2 & 0xffff0000u),
+                                     __uint_as_float(g2 & 0xffff0000u)));
+    }
+    __builtin_amdgcn_raw_buffer_store_b32(y2, ry,
                                           pair_ch * 2u + lane_rows * row_bytes,
                                           tile_row * row_bytes, 0);
   }
@@ -297,7 +323,10 @@ hipError_t launch_block_step_bf16(const StepArgs& a, hipStream_t s) {
   const int tiles = (a.B + kStepRows - 1) / kStepRows;
   if (tiles <= 0 || (int64_t)tiles * a.H > 0x7fffffff)
     return hipErrorInvalidValue;
-  block_step_bf16_kernel<<<dim3((unsigned)(tiles * a.H)), 512, 0, s>>>(a);
+  if (a.gate_branch)
+    block_step_bf16_kernel<true><<<dim3((unsigned)(tiles * a.H)), 512, 0, s>>>(a);
+  else
+    block_step_bf16_kernel<false><<<dim3((unsigned)(tiles * a.H)), 512, 0, s>>>(a);
   return hipGetLastError();
 }
 

@@ -132,6 +132,9 @@ struct StepArgs {
   const void* b[2];
   const void* a_param;
   void* y;               // [B, 1, W]
+  // the block's other branch [B, 1, W] or null: y is written as
+  // y * gelu(gate_branch)
+  const void* gate_branch;
   int B, W, H;
 };
 

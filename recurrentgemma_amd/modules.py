@@ -56,9 +56,8 @@ def recurrent_core(conv_1d: layers.Conv1D, rg_lru: layers.RGLRU, x,
       y, h, conv_state = ops.recurrent_step(
           x, segment_pos, cache.conv1d_state, cache.rg_lru_state, conv_1d.w,
           conv_1d.b, rg_lru.input_gate.w, rg_lru.input_gate.b, rg_lru.a_gate.w,
-          rg_lru.a_gate.b, rg_lru.a_param, in_place=in_place)
-      if gate_branch is not None:
-        y = ops.gelu_mul(y, gate_branch)
+          rg_lru.a_gate.b, rg_lru.a_param, in_place=in_place,
+          gate_branch=gate_branch)
       if not return_cache:
         return y, None
       return y, RecurrentBlockCache(rg_lru_state=h, conv1d_state=conv_state)

@@ -854,12 +854,13 @@ class PackedLinear:
 
 
 def recurrent_step(x, segment_pos, conv_cache, h, conv_w, conv_b, w_x, b_x, w_a,
-                   b_a, a_param, in_place=False):
+                   b_a, a_param, in_place=False, gate_branch=None):
   """One decode step of conv -> RG-LRU.  Returns (y, h_new, conv_cache_new).
 
   bf16 with 256-wide heads runs as one launch on re-laid-out gate weights
   (packed once per weight version); other shapes as conv step + gate GEMM +
-  scan step."""
+  scan step.  gate_branch: the block's linear_y output [B,1,W]; y is then
+  y * gelu(gate_branch) (inside the one launch where that runs)."""
   B, n_tok, W = x.shape
   assert n_tok == 1
   assert conv_cache.shape == (B, 3, W)
@@ -886,13 +887,23 @@ def recurrent_step(x, segment_pos, conv_cache, h, conv_w, conv_b, w_x, b_x, w_a,
   packed = None
   if x.dtype == torch.bfloat16 and W // H == 256 and W % H == 0:
     packed = packed_gate_weights(w_x, w_a)
+  if gate_branch is not None:
+    assert gate_branch.shape == x.shape
+    _same(x.dtype, x.device, gate_branch=gate_branch)
+    gate_branch = _dev(gate_branch, "gate_branch")
   if packed is not None:
     cw, cb, wx_, bx_, wa_, ba_, ap_ = args
     with _on(x.device):
-      _lib.check(_lib.lib().rg_recurrent_step_packed(
-          _p(x), _p(seg), is64, _p(cache_in), _p(cache_out), _p(h_in),
-          _p(h_out), _p(cw), _p(cb), _p(packed), _p(bx_), _p(ba_), _p(ap_),
-          _p(y), B, W, H, _dtype_code(x), _stream(x)))
+      if gate_branch is not None:
+        _lib.check(_lib.lib().rg_recurrent_step_gelu_mul(
+            _p(x), _p(gate_branch), _p(seg), is64, _p(cache_in), _p(cache_out),
+            _p(h_in), _p(h_out), _p(cw), _p(cb), _p(packed), _p(bx_), _p(ba_),
+            _p(ap_), _p(y), B, W, H, _dtype_code(x), _stream(x)))
+      else:
+        _lib.check(_lib.lib().rg_recurrent_step_packed(
+            _p(x), _p(seg), is64, _p(cache_in), _p(cache_out), _p(h_in),
+            _p(h_out), _p(cw), _p(cb), _p(packed), _p(bx_), _p(ba_), _p(ap_),
+            _p(y), B, W, H, _dtype_code(x), _stream(x)))
     if cache_out.dtype != conv_cache.dtype:
       cache_out = cache_out.to(conv_cache.dtype)
     return y, h_out, cache_out
@@ -904,4 +915,6 @@ def recurrent_step(x, segment_pos, conv_cache, h, conv_w, conv_b, w_x, b_x, w_a,
         _dtype_code(x), _stream(x)))
   if cache_out.dtype != conv_cache.dtype:
     cache_out = cache_out.to(conv_cache.dtype)
+  if gate_branch is not None:
+    y = gelu_mul(y, gate_branch)
   return y, h_out, cache_out

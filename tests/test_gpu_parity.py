@@ -801,6 +801,56 @@ def test_recurrent_core_entry_rejects_a_short_workspace():
   assert b"workspace" in _lib.lib().rg_last_error()
 
 
+@pytest.mark.parametrize("B,W,H", [(1, 256, 1), (33, 512, 2), (70, 768, 3),
+                                   (256, 1024, 4)])
+def test_recurrent_step_joined_with_gate_branch(B, W, H):
+  """rg_recurrent_step_gelu_mul: the decode step with the block's join in its
+  output stage gives, bit for bit, the step followed by rg_gelu_mul -- new
+  tensors and in place, ragged row tiles, document starts among the rows, and
+  with the output written over the gate branch."""
+  p = R.make_params(W, H, torch.bfloat16, seed=B + 7, gate_bias_std=0.4)
+  P = {k: _dev(v) for k, v in p.items()}
+  g = torch.Generator().manual_seed(B)
+  x = _dev(torch.randn(B, 1, W, generator=g).to(torch.bfloat16))
+  gate = _dev(torch.randn(B, 1, W, generator=g).to(torch.bfloat16))
+  h = _dev(torch.randn(B, W, generator=g))
+  cc = _dev(torch.randn(B, 3, W, generator=g).to(torch.bfloat16))
+  seg = torch.full((B, 1), 9, dtype=torch.int64)
+  seg[B // 2, 0] = 0
+  seg = _dev(seg)
+  args = (P["conv_w"], P["conv_b"], P["w_x"], P["b_x"], P["w_a"], P["b_a"],
+          P["a_param"])
+  y0, h0, c0 = ops.recurrent_step(x, seg, cc, h, *args)
+  want = ops.gelu_mul(y0, gate)
+  y1, h1, c1 = ops.recurrent_step(x, seg, cc, h, *args, gate_branch=gate)
+  assert torch.equal(y1, want) and torch.equal(h1, h0) and torch.equal(c1, c0)
+  h2, c2 = h.clone(), cc.clone()
+  y2, h2b, c2b = ops.recurrent_step(x, seg, c2, h2, *args, in_place=True,
+                                    gate_branch=gate)
+  assert h2b.data_ptr() == h2.data_ptr() and c2b.data_ptr() == c2.data_ptr()
+  assert torch.equal(y2, want) and torch.equal(h2, h0) and torch.equal(c2, c0)
+  # through the C ABI, the output over the gate branch
+  packed = ops.packed_gate_weights(P["w_x"], P["w_a"])
+  over = gate.clone()
+  h3, c3 = torch.empty_like(h), torch.empty_like(cc)
+  ptr = lambda t: t.data_ptr()
+  _lib.check(_lib.lib().rg_recurrent_step_gelu_mul(
+      ptr(x), ptr(over), ptr(seg), 1, ptr(cc), ptr(c3), ptr(h), ptr(h3),
+      ptr(P["conv_w"]), ptr(P["conv_b"]), ptr(packed), ptr(P["b_x"]),
+      ptr(P["b_a"]), ptr(P["a_param"]), ptr(over), B, W, H, 1,
+      torch.cuda.current_stream().cuda_stream))
+  assert torch.equal(over, want) and torch.equal(h3, h0) and torch.equal(c3, c0)
+  # float32 has no joined kernel: the wrapper adds the pass itself
+  pf = {k: _dev(v) for k, v in
+        R.make_params(W, H, torch.float32, seed=3).items()}
+  argsf = (pf["conv_w"], pf["conv_b"], pf["w_x"], pf["b_x"], pf["w_a"],
+           pf["b_a"], pf["a_param"])
+  yf, _, _ = ops.recurrent_step(x.float(), seg, cc.float(), h, *argsf)
+  yj, _, _ = ops.recurrent_step(x.float(), seg, cc.float(), h, *argsf,
+                                gate_branch=gate.float())
+  assert torch.equal(yj, ops.gelu_mul(yf, gate.float()))
+
+
 def test_decode_step_under_graph_capture():
   """The decode step allocates nothing, never synchronises and only uses the
   stream it is given, so a HIP graph can hold it: capture one in-place step,
