@@ -396,6 +396,23 @@ int rg_rope_pair(const void* q, const void* k, const void* positions,
                  void* k_out, int64_t rows, int q_heads, int k_heads,
                  int head_dim, int dtype, void* stream);
 
+/* Prompt-pass attention of LocalAttentionBlock.forward without a cache
+ * (recurrentgemma/torch/modules.py:404-476; mask :86-127): for every query t
+ * the softmax over the keys first_key[t] .. t of scale * q_t . k_j, times the
+ * values -- multi-query (H heads of queries, one head of keys and values),
+ * bf16, head_dim 256, one kernel (RG_ERR_UNSUPPORTED otherwise: callers keep
+ * their batched products).  q, out [B,T,H,256]; k [B,T,256] (both after the
+ * rotary embedding); v_t [B,256,T_pad]: the values transposed, T_pad a
+ * multiple of 32, zeros from column T on; first_key [B,T] int32,
+ * non-decreasing along T: max(first token of the query's document,
+ * t - window), which is the reference's mask for a prompt.  Scores and the
+ * softmax are float32, the probabilities enter the second product as bf16
+ * like the reference's; out is rounded once. */
+int rg_attention_prefill(const void* q, const void* k, const void* v_t,
+                         const void* first_key, void* out, int B, int T,
+                         int T_pad, int H, int head_dim, float scale, int dtype,
+                         void* stream);
+
 /* Masked softmax of one decoded token against the ring cache and itself
  * (modules.py:152-183 `_compute_cache_mask`, :462-470): scores
  * [B, heads, window] = q . k of the ring slots, unscaled, in `dtype`; q

@@ -54,6 +54,8 @@ SIGNATURES = {
     "rg_conv1d_backward_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "rg_conv1d_backward": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _sz, _i, _i,
                                 _i, _i, _i, _vp]),
+    "rg_attention_prefill": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i,
+                                  ctypes.c_float, _i, _vp]),
     "rg_rglru_backward": (_i, [_vp] * 14 + [_i, _i, _i, _i, _vp]),
     "rg_scan_split_workspace_bytes": (_sz, [_i, _i, _i]),
     "rg_lru_scan_fused_split": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i,

@@ -925,6 +925,45 @@ int rg_rope_pair(const void* q, const void* k, const void* positions,
                                 k_out, k_heads, dtype, (hipStream_t)stream));
 }
 
+int rg_attention_prefill(const void* q, const void* k, const void* v_t,
+                         const void* first_key, void* out, int B, int T,
+                         int T_pad, int H, int head_dim, float scale, int dtype,
+                         void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(B > 0 && T > 0 && H > 0, "%s: B=%d T=%d H=%d must be positive",
+             __func__, B, T, H);
+  if (dtype != RG_DTYPE_BF16 || head_dim != 256)
+    return fail(RG_ERR_UNSUPPORTED,
+                "%s: needs bf16 and head_dim == 256 (dtype=%d head_dim=%d)",
+                __func__, dtype, head_dim);
+  RG_REQUIRE(T_pad >= T && T_pad % 32 == 0,
+             "%s: T_pad=%d must be a multiple of 32 and at least T=%d",
+             __func__, T_pad, T);
+  RG_REQUIRE((int64_t)T * H * 512 < ((int64_t)1 << 31) &&
+                 (int64_t)T_pad * 512 < ((int64_t)1 << 31),
+             "%s: T=%d H=%d: a row's queries exceed 2 GiB", __func__, T, H);
+  RG_CHECK_PTR(q);
+  RG_CHECK_PTR(k);
+  RG_CHECK_PTR(v_t);
+  RG_CHECK_PTR(first_key);
+  RG_CHECK_PTR(out);
+  RG_REQUIRE(out != q && out != k && out != v_t,
+             "%s: out must not alias an input", __func__);
+  rg::AttnPrefillArgs a{};
+  a.q = q;
+  a.k = k;
+  a.v_t = v_t;
+  a.lo = first_key;
+  a.out = out;
+  a.B = B;
+  a.T = T;
+  a.T_pad = T_pad;
+  a.H = H;
+  a.scale = scale;
+  return launch_status(
+      __func__, rg::launch_attn_prefill_bf16(a, (hipStream_t)stream));
+}
+
 int rg_attention_decode_probs(const void* scores, const void* q,
                               const void* k_new, const int32_t* num_tokens,
                               void* probs, int B, int heads, int head_dim,

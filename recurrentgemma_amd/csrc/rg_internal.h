@@ -138,6 +138,19 @@ struct StepArgs {
   int B, W, H;
 };
 
+// Prompt-pass attention (rg_attention_prefill.hip).
+struct AttnPrefillArgs {
+  const void* q;    // [B, T, H, 256] bf16, after the rotary embedding
+  const void* k;    // [B, T, 256] bf16, after the rotary embedding
+  const void* v_t;  // [B, 256, T_pad] bf16: the values transposed, zeros
+                    // behind token T - 1
+  const void* lo;   // [B, T] int32: first key each query sees (non-decreasing)
+  void* out;        // [B, T, H, 256] bf16
+  int B, T, T_pad, H;
+  float scale;      // of the scores (head_dim ** -0.5)
+};
+hipError_t launch_attn_prefill_bf16(const AttnPrefillArgs& a, hipStream_t s);
+
 struct LinearArgs {
   const void* x;         // [M, K] bf16
   const void* w_packed;  // see launch_linear_pack

@@ -249,6 +249,29 @@ def _inference_only(forward):
   return wrapper
 
 
+_first_key = [None, None, None, None]  # tensor (weak), version, window, answer
+
+
+def _first_visible_key(segment_pos, window):
+  """[B, T] int32: the first key each query of a prompt sees -- the later of
+  the first token of its document (the latest position with segment_pos == 0,
+  else the start of the row) and `window` tokens back: what the mask of
+  modules.py:86-127 amounts to for a prompt.  Kept for the tensor object it
+  was computed for (the attention blocks of a model all ask for the same)."""
+  ref, version, w, answer = _first_key
+  now = None if segment_pos.is_inference() else segment_pos._version
+  if (ref is not None and ref() is segment_pos and now is not None and
+      version == now and w == window):
+    return answer
+  b, t = segment_pos.shape
+  pos = torch.arange(t, device=segment_pos.device)[None].expand(b, t)
+  start = torch.cummax(
+      torch.where(segment_pos == 0, pos, torch.zeros_like(pos)), dim=-1).values
+  answer = torch.maximum(start, pos - window).to(torch.int32).contiguous()
+  _first_key[:] = [weakref.ref(segment_pos), now, window, answer]
+  return answer
+
+
 _one_document = [None, None, False]  # tensor (weak), its version, answer
 
 
@@ -368,6 +391,16 @@ class LocalAttentionBlock(nn.Module):
       if return_cache:
         new_cache = self._cache_from_prompt(k, v, segment_pos,
                                             self.window_size)
+      if ops.attention_prefill_supported(q):
+        # bf16, head_dim 256: scores, mask, softmax and values in one kernel
+        # (the mask of modules.py:86-127 for a prompt is a band: a query sees
+        # from the start of its document, or the window's width back, up to
+        # itself)
+        out = ops.attention_prefill(
+            q, k, v, _first_visible_key(segment_pos, self.window_size),
+            self.head_dim ** -0.5)
+        return self._project_out(out.reshape(b, t, self.width),
+                                 defer_out), new_cache
       if (x.is_cuda and 1 < t <= self.window_size + 1 and
           _rows_are_one_document(segment_pos)):
         # one document per row, all of it inside the window: the mask of

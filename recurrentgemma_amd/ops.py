@@ -560,6 +560,35 @@ def rope_pair(q, k, positions, inv_freq):
   return q_out, k_out
 
 
+def attention_prefill_supported(q):
+  """Shapes the prompt-pass attention kernel serves (rg_attention_prefill)."""
+  return (q.is_cuda and q.dtype == torch.bfloat16 and q.ndim == 4 and
+          q.shape[-1] == 256 and q.shape[1] * q.shape[2] * 512 < 2**31)
+
+
+def attention_prefill(q, k, v, first_key, scale):
+  """Sliding-window multi-query attention over a prompt in one kernel.
+  q [B,T,H,256], k and v [B,T,1,256] or [B,T,256] (q, k after the rotary
+  embedding), first_key [B,T] int32: query t sees the keys first_key[t] .. t.
+  Returns [B,T,H,256]."""
+  B, T, H, hd = q.shape
+  q = _dev(q, "q")
+  k = _dev(k.reshape(B, T, hd), "k")
+  _same(q.dtype, q.device, k=k, v=v)
+  assert first_key.shape == (B, T) and first_key.dtype == torch.int32
+  first_key = _dev(first_key, "first_key")
+  t_pad = (T + 63) // 64 * 64
+  # the values transposed (keys contiguous), zeros behind the last token
+  v_t = q.new_zeros((B, hd, t_pad))
+  v_t[:, :, :T] = v.reshape(B, T, hd).transpose(1, 2)
+  out = torch.empty_like(q)
+  with _on(q.device):
+    _lib.check(_lib.lib().rg_attention_prefill(
+        _p(q), _p(k), _p(v_t), _p(first_key), _p(out), B, T, t_pad, H, hd,
+        float(scale), _dtype_code(q), _stream(q)))
+  return out
+
+
 def attention_decode_probs(scores, q, k_new, num_tokens, scale):
   """softmax over the written ring slots and the new token: scores
   [B, heads, window] (unscaled), q [B, heads, hd], k_new [B, hd], num_tokens
