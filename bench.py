@@ -23,6 +23,8 @@ Workloads (the benchmark configurations this build is measured on):
   2b_prefill  B8 T4096 W2560 H10 bf16, documents ~ Geometric(mean 1024)
   2b_f32      B1 T512 W2560 H10 fp32 (the reference's own CPU-runnable case;
               21 MB, i.e. cache resident: warm-cache figures)
+  2b_attention_prompt  prompt-pass attention of one local-attention block of
+              the 2B model (B64 T2047, 10 query heads, head_dim 256)
   9b_decode   B256 W4096 H16 bf16, one token per row and step with the caches
               carried in place (rg_recurrent_step); `roofline` then describes
               the whole step (all its launches) against its algorithmic bytes
@@ -65,6 +67,11 @@ WORKLOADS = {
     # token ids, 256 new tokens each (--steps sets the number of new tokens)
     "2b_griffin_decode": dict(B=64, T=2048, new_tokens=256, seed=1005,
                               griffin=True),
+    # prompt-pass attention of one local-attention block of that model: 64
+    # prompts of 2047 tokens (what the sampler's prompt pass sees), 10 query
+    # heads on one key/value head, head_dim 256, window 2048
+    "2b_attention_prompt": dict(B=64, T=2047, H=10, window=2048, seed=1007,
+                                attention=True),
 }
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (scaled
@@ -183,6 +190,62 @@ def decode_algorithmic_bytes(B, W, H, esize):
   both gate weight matrices, the per-channel parameters."""
   return (2 * B * W * esize + 2 * B * W * 4 + 2 * B * 3 * W * esize
           + 2 * H * (W // H) ** 2 * esize + W * esize * 8 + B * 8)
+
+
+def run_attention(args, torch, ops, wl):
+  """rg_attention_prefill on one block's prompt pass (the transposed copy of
+  the values included in a step), with the library attention (torch SDPA,
+  causal) timed after it for comparison.  Flops counted: the visible
+  (query, key) pairs only, 4 * head_dim each."""
+  dev = torch.device("cuda:0")
+  B, T, H, hd, window = wl["B"], wl["T"], wl["H"], 256, wl["window"]
+  g = torch.Generator().manual_seed(wl["seed"])
+  q = torch.randn(B, T, H, hd, generator=g).to(torch.bfloat16).to(dev)
+  k = torch.randn(B, T, 1, hd, generator=g).to(torch.bfloat16).to(dev)
+  v = torch.randn(B, T, 1, hd, generator=g).to(torch.bfloat16).to(dev)
+  pos = torch.arange(T, device=dev)[None].expand(B, T)
+  first = torch.clamp(pos - window, min=0).to(torch.int32).contiguous()
+  pairs = float((pos - first + 1).sum().item()) * H
+  flops = 4.0 * hd * pairs
+
+  def timed(fn, steps, warmup):
+    for _ in range(warmup):
+      fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+      fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps, e0.elapsed_time(e1) / steps
+
+  wall, ms = timed(lambda: ops.attention_prefill(q, k, v, first, hd ** -0.5),
+                   args.steps, args.warmup)
+
+  def library():
+    return torch.nn.functional.scaled_dot_product_attention(
+        q.transpose(1, 2), k.transpose(1, 2).expand(-1, H, -1, -1),
+        v.transpose(1, 2).expand(-1, H, -1, -1), is_causal=True)
+  _, lib_ms = timed(library, max(3, args.steps // 5), 2)
+  achieved = flops / (ms * 1e-3) / 1e12
+  print(json.dumps({
+      "metric": "prompt-pass attention of one local-attention block, tokens/s",
+      "value": B * T / wall, "unit": "tokens/s", "n_gpus": 1,
+      "steps": args.steps, "warmup": args.warmup, "ms_per_step": wall * 1e3,
+      "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+      "dtype": "bf16", "data": "synthetic",
+      "config": {"workload": args.workload, "batch": B, "seq_len": T,
+                 "query_heads": H, "kv_heads": 1, "head_dim": hd,
+                 "window": window,
+                 "path": "rg_attention_prefill (+ the transposed copy of v)"},
+      "roofline": {"kernel": "attn_prefill_bf16_kernel", "bound": "mfma",
+                   "achieved": achieved, "peak": 2500.0, "unit": "TFLOP/s",
+                   "frac": achieved / 2500.0, "traffic": None,
+                   "algorithmic_flops": flops, "avg_launch_ms": ms},
+      "library_attention": {"what": "torch SDPA, is_causal", "ms": lib_ms}}))
 
 
 def run_griffin(args, torch, rg, wl):
@@ -388,6 +451,9 @@ def main():
     return
   if wl.get("decode"):
     run_decode(args, torch, rg, R, ops, wl)
+    return
+  if wl.get("attention"):
+    run_attention(args, torch, ops, wl)
     return
   result = run_prefill(args, torch, rg, R, ops, args.workload, args.steps,
                        args.warmup, extras=True)
