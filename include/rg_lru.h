@@ -403,7 +403,7 @@ int rg_rope_pair(const void* q, const void* k, const void* positions,
  * bf16, head_dim 256, one kernel (RG_ERR_UNSUPPORTED otherwise: callers keep
  * their batched products).  q, out [B,T,H,256]; k [B,T,256] (both after the
  * rotary embedding); v_t [B,256,T_pad]: the values transposed, T_pad a
- * multiple of 32, zeros from column T on; first_key [B,T] int32,
+ * multiple of 64, zeros from column T on; first_key [B,T] int32,
  * non-decreasing along T: max(first token of the query's document,
  * t - window), which is the reference's mask for a prompt.  Scores and the
  * softmax are float32, the probabilities enter the second product as bf16

@@ -936,8 +936,8 @@ int rg_attention_prefill(const void* q, const void* k, const void* v_t,
     return fail(RG_ERR_UNSUPPORTED,
                 "%s: needs bf16 and head_dim == 256 (dtype=%d head_dim=%d)",
                 __func__, dtype, head_dim);
-  RG_REQUIRE(T_pad >= T && T_pad % 32 == 0,
-             "%s: T_pad=%d must be a multiple of 32 and at least T=%d",
+  RG_REQUIRE(T_pad >= T && T_pad % 64 == 0,
+             "%s: T_pad=%d must be a multiple of 64 and at least T=%d",
              __func__, T_pad, T);
   RG_REQUIRE((int64_t)T * H * 512 < ((int64_t)1 << 31) &&
                  (int64_t)T_pad * 512 < ((int64_t)1 << 31),

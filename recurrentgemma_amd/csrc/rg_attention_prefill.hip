@@ -379,7 +379,7 @@ attn_prefill_bf16_kernel(AttnPrefillArgs p) {
 }  // namespace
 
 hipError_t launch_attn_prefill_bf16(const AttnPrefillArgs& a, hipStream_t s) {
-  // needs head dimension 256, T_pad a multiple of 32 >= T, and rows whose byte
+  // needs head dimension 256, T_pad a multiple of 64 >= T, and rows whose byte
   // offsets fit 32 bits (checked by the caller)
   const int64_t qtiles = (a.T + kAttnQ - 1) / kAttnQ;
   const int64_t blocks = qtiles * a.H * a.B;

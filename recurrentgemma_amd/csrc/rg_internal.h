@@ -143,7 +143,7 @@ struct AttnPrefillArgs {
   const void* q;    // [B, T, H, 256] bf16, after the rotary embedding
   const void* k;    // [B, T, 256] bf16, after the rotary embedding
   const void* v_t;  // [B, 256, T_pad] bf16: the values transposed, zeros
-                    // behind token T - 1
+                    // behind token T - 1 (T_pad a multiple of 64)
   const void* lo;   // [B, T] int32: first key each query sees (non-decreasing)
   void* out;        // [B, T, H, 256] bf16
   int B, T, T_pad, H;

@@ -109,6 +109,35 @@ def test_c_side_validation_without_launch():
                           None)
   assert rc == -4 and b"workspace" in lib.rg_last_error()
   # scans cut into chunks: only for few rows and long sequences
+  # the backward entry points and the prompt attention check their arguments
+  # before any launch
+  rc = lib.rg_rglru_backward(ok, ok, ok, ok, ok, ok, ok, None, None, ok, ok, ok,
+                             ok, None, 1, 4, 8, 0, None)
+  assert rc == -1 and b"alias" in lib.rg_last_error()
+  rc = lib.rg_rglru_backward(None, ok, ok, ok, ok, ok, ok, None, None, ok, ok,
+                             ok, ok, None, 1, 4, 8, 0, None)
+  assert rc == -1 and b"dy is null" in lib.rg_last_error()
+  assert lib.rg_conv1d_backward_workspace_bytes(2, 100, 64, 4) == 7 * 5 * 64 * 4
+  assert lib.rg_conv1d_backward_workspace_bytes(2, 100, 64, 1) == 0
+  rc = lib.rg_conv1d_backward(ok, ok, ok, 1, ok, ctypes.c_void_p(512), None, 0,
+                              2, 100, 64, 4, 0, None)
+  assert rc == -4 and b"partial sums" in lib.rg_last_error()
+  rc = lib.rg_conv1d_backward(ok, ok, ok, 1, ok, ctypes.c_void_p(512), ok, 1 << 20,
+                              2, 100, 64, 17, 0, None)
+  assert rc == -2 and b"temporal width" in lib.rg_last_error()
+  two = ctypes.c_void_p(512)
+  rc = lib.rg_attention_prefill(ok, two, two, two, ctypes.c_void_p(768), 1, 100,
+                                128, 2, 128, 1.0, 1, None)
+  assert rc == -2 and b"head_dim == 256" in lib.rg_last_error()
+  rc = lib.rg_attention_prefill(ok, two, two, two, ctypes.c_void_p(768), 1, 100,
+                                96, 2, 256, 1.0, 1, None)
+  assert rc == -1 and b"multiple of 64" in lib.rg_last_error()
+  rc = lib.rg_attention_prefill(ok, two, two, two, ok, 1, 100, 128, 2, 256, 1.0,
+                                1, None)
+  assert rc == -1 and b"alias" in lib.rg_last_error()
+  rc = lib.rg_recurrent_step_gelu_mul(ok, None, ok, 1, ok, ok, ok, ok, ok, ok,
+                                      ok, ok, ok, ok, two, 4, 512, 2, 1, None)
+  assert rc == -1 and b"gate_branch is null" in lib.rg_last_error()
   # rg_recurrent_core: nothing for whole rows in the single kernel, the chunk
   # summaries for rows in chunks, both gates' pre-activations (+ the scan's
   # chunk summaries) for the two-kernel form
