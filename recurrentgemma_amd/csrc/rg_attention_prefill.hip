@@ -258,7 +258,13 @@ attn_prefill_bf16_kernel(AttnPrefillArgs p) {
           }
         }
       }
+      // (tied to the scores: nothing that reads them may be scheduled above
+      // the wait)
+#pragma unroll
+      for (int kb = 0; kb < kAttnKB; ++kb) asm volatile("" : "+v"(s[kb]));
       wait_for_matrix_results();
+#pragma unroll
+      for (int kb = 0; kb < kAttnKB; ++kb) asm volatile("" : "+v"(s[kb]));
       // ---- mask (only where the band's edges cross the tile) ----------------
       const bool interior = key0 + kAttnK - 1 <= qw0 && key0 >= lo_last_wave;
       if (!interior) {

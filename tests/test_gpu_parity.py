@@ -328,6 +328,62 @@ def _core_case(dtype, B, T, W, H, seg, seed, bias_std=0.2):
   return p, x, blk, (y, cache), (yo, co)
 
 
+def test_recurrent_core_shape_sweep():
+  """Forty shapes drawn from a fixed seed -- head widths 64 to 256, one to four
+  heads, one to 150 rows, one to 1700 tokens, both dtypes, int32 and int64
+  positions, rows that start at position -1 (left padding), 0 or inside a
+  document -- through rg_recurrent_core (whatever kernels it picks) against
+  the oracle, with and without the join of the gate branch."""
+  import random
+  rnd = random.Random(20240607)
+  for case in range(40):
+    dtype = rnd.choice([torch.float32, torch.bfloat16])
+    bw = rnd.choice([64, 128, 256, 256, 256])
+    H = rnd.choice([1, 2, 3, 4])
+    W = bw * H
+    B = rnd.choice([1, 2, 5, 33, 70, 150]) if bw == 256 else rnd.choice([1, 3, 9])
+    T = rnd.choice([1, 2, 3, 5, 63, 64, 65, 200, 513, 1700])
+    if B * T * W > 40e6:
+      T = 65
+    p = R.make_params(W, H, dtype, seed=500 + case, gate_bias_std=0.3)
+    g = torch.Generator().manual_seed(900 + case)
+    x = torch.randn(B, T, W, generator=g).to(dtype)
+    seg = helpers.document_positions(B, T, rnd.choice([4, 50, 4000]),
+                                     seed=case)
+    first = rnd.choice(["zero", "pad", "inside"])
+    if first == "pad" and T > 3:
+      seg[:, 2:] = seg[:, :-2].clone()
+      seg[:, :2] = -1
+    elif first == "inside":
+      seg[0, 0] = 11
+    if rnd.random() < 0.5:
+      seg = seg.to(torch.int32)
+    P = {k: _dev(v) for k, v in p.items()}
+    joined = rnd.random() < 0.5
+    gate = torch.randn(B, T, W, generator=g).to(dtype) if joined else None
+    _announce(f"sweep {case}: {dtype} B{B} T{T} W{W} H{H} {first} "
+              f"{seg.dtype} joined={joined}")
+    y, h, c = ops.recurrent_core(
+        _dev(x), _dev(seg), P["conv_w"], P["conv_b"], P["w_x"], P["b_x"],
+        P["w_a"], P["b_a"], P["a_param"],
+        gate_branch=None if gate is None else _dev(gate))
+    ref = (R.recurrent_core if dtype == torch.float32
+           else R.widened_recurrent_core)
+    yo, co = ref(x, seg.to(torch.int64), p)
+    if joined:
+      gelu = torch.nn.functional.gelu(gate.float(), approximate="tanh")
+      yo = (yo.float() * gelu.to(dtype).float()).to(dtype)
+    tol = F32_TOL if dtype == torch.float32 else BF16_TOL
+    what = f"case {case}"
+    assert helpers.max_rel(h, co.rg_lru_state) < tol, what
+    assert torch.equal(c.cpu(), co.conv1d_state), what
+    if dtype == torch.float32:
+      assert helpers.max_rel(y, yo) < (2e-5 if joined else tol), what
+    else:
+      helpers.assert_close_elementwise(y, yo, rtol=2e-2, atol_of_max=4e-3,
+                                       what=what)
+
+
 def test_config1_fp32_parity():
   """Benchmark configuration 1: B1 T512 W2560 H10 fp32, segment_pos = arange."""
   B, T, W, H = 1, 512, 2560, 10
