@@ -18,6 +18,7 @@ from typing import NamedTuple
 import torch
 from torch import nn
 
+from recurrentgemma_amd import compiled
 from recurrentgemma_amd import layers
 from recurrentgemma_amd import ops
 from recurrentgemma_amd import training
@@ -53,11 +54,18 @@ def recurrent_core(conv_1d: layers.Conv1D, rg_lru: layers.RGLRU, x,
     assert cache.conv1d_state.shape == (b, conv_1d.temporal_width - 1, d)
     assert num_tokens == 1
     if fused:
-      y, h, conv_state = ops.recurrent_step(
-          x, segment_pos, cache.conv1d_state, cache.rg_lru_state, conv_1d.w,
-          conv_1d.b, rg_lru.input_gate.w, rg_lru.input_gate.b, rg_lru.a_gate.w,
-          rg_lru.a_gate.b, rg_lru.a_param, in_place=in_place,
-          gate_branch=gate_branch)
+      if compiled.tracing() and not in_place:
+        # (a traced program holds the step as one operator node)
+        y, h, conv_state = torch.ops.recurrentgemma_amd.recurrent_step(
+            x, segment_pos, cache.conv1d_state, cache.rg_lru_state, conv_1d.w,
+            conv_1d.b, rg_lru.input_gate.w, rg_lru.input_gate.b,
+            rg_lru.a_gate.w, rg_lru.a_gate.b, rg_lru.a_param, gate_branch)
+      else:
+        y, h, conv_state = ops.recurrent_step(
+            x, segment_pos, cache.conv1d_state, cache.rg_lru_state, conv_1d.w,
+            conv_1d.b, rg_lru.input_gate.w, rg_lru.input_gate.b,
+            rg_lru.a_gate.w, rg_lru.a_gate.b, rg_lru.a_param,
+            in_place=in_place, gate_branch=gate_branch)
       if not return_cache:
         return y, None
       return y, RecurrentBlockCache(rg_lru_state=h, conv1d_state=conv_state)
@@ -79,11 +87,17 @@ def recurrent_core(conv_1d: layers.Conv1D, rg_lru: layers.RGLRU, x,
     # W4096: 1.15 ms against 0.91 + 0.40 ms apart; with rows in chunks it would
     # lengthen the one workgroup per row that produces outputs in the first
     # launch while the others only summarise, so it stays a pass of its own).
-    y, h, conv_state = ops.recurrent_core(
-        x, segment_pos, conv_1d.w, conv_1d.b, rg_lru.input_gate.w,
-        rg_lru.input_gate.b, rg_lru.a_gate.w, rg_lru.a_gate.b, rg_lru.a_param,
-        h0=None, return_h=return_cache, return_conv_cache=return_cache,
-        gate_branch=gate_branch)
+    if compiled.tracing():
+      y, h, conv_state = torch.ops.recurrentgemma_amd.recurrent_core(
+          x, segment_pos, conv_1d.w, conv_1d.b, rg_lru.input_gate.w,
+          rg_lru.input_gate.b, rg_lru.a_gate.w, rg_lru.a_gate.b,
+          rg_lru.a_param, None, gate_branch)
+    else:
+      y, h, conv_state = ops.recurrent_core(
+          x, segment_pos, conv_1d.w, conv_1d.b, rg_lru.input_gate.w,
+          rg_lru.input_gate.b, rg_lru.a_gate.w, rg_lru.a_gate.b,
+          rg_lru.a_param, h0=None, return_h=return_cache,
+          return_conv_cache=return_cache, gate_branch=gate_branch)
     gate_branch = None
   if gate_branch is not None:
     y = ops.gelu_mul(y, gate_branch)
@@ -149,7 +163,10 @@ class RecurrentBlock(nn.Module):
     if training.is_enabled():
       return self._forward_differentiable(x, segment_pos, cache, return_cache)
     with torch.no_grad():
+      # (a traced program keeps torch's own linear layers: the few-row
+      # kernels are reached through ctypes, which a tracer cannot follow)
       few_rows = (
+          not compiled.tracing() and
           ops.PackedLinear.usable(x, self.width, self.lru_width) and
           ops.PackedLinear.usable(x, self.lru_width, self.width))
       if few_rows:

@@ -907,6 +907,33 @@ def test_recurrent_step_joined_with_gate_branch(B, W, H):
   assert torch.equal(yj, ops.gelu_mul(yf, gate.float()))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_recurrent_block_traces_as_one_graph(dtype):
+  """torch.compile follows RecurrentBlock without a graph break (fullgraph):
+  the conv -> RG-LRU core is one custom operator node each for a prefill and
+  for a decode step (recurrentgemma_amd/compiled.py).  Backend aot_eager: the
+  traced, functionalised graph is run by torch's own kernels plus ours, and
+  must give what the eager module gives, bit for bit."""
+  B, T, width, H = 3, 40, 512, 2
+  torch.manual_seed(12)
+  blk = rg.RecurrentBlock(width=width, num_heads=H, dtype=dtype).to(DEV)
+  x = _dev(torch.randn(B, T, width).to(dtype))
+  seg = _dev(helpers.document_positions(B, T, 15, seed=8))
+  want, cache = blk(x, seg)
+  traced = torch.compile(blk, backend="aot_eager", fullgraph=True)
+  got, cache_t = traced(x, seg)
+  assert torch.equal(got, want)
+  assert torch.equal(cache_t.rg_lru_state, cache.rg_lru_state)
+  assert torch.equal(cache_t.conv1d_state, cache.conv1d_state)
+  x1 = _dev(torch.randn(B, 1, width).to(dtype))
+  pos = _dev(torch.full((B, 1), T, dtype=torch.int64))
+  want1, cache1 = blk(x1, pos, cache)
+  got1, cache1_t = traced(x1, pos, cache)
+  assert torch.equal(got1, want1)
+  assert torch.equal(cache1_t.rg_lru_state, cache1.rg_lru_state)
+  assert torch.equal(cache1_t.conv1d_state, cache1.conv1d_state)
+
+
 def test_decode_step_under_graph_capture():
   """The decode step allocates nothing, never synchronises and only uses the
   stream it is given, so a HIP graph can hold it: capture one in-place step,

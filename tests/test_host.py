@@ -271,3 +271,28 @@ def test_param_init_same_draws_as_oracle():
   b = torch.empty(100)
   R.rnn_param_init(b, 0.9, 0.999)
   assert torch.equal(a, b)
+
+
+def test_custom_operators_have_shape_functions():
+  """The traced form of the hot path (recurrentgemma_amd/compiled.py): both
+  operators are registered and infer their outputs' shapes and dtypes from
+  fake tensors, without touching a GPU."""
+  from torch._subclasses.fake_tensor import FakeTensorMode
+  from recurrentgemma_amd import compiled  # noqa: F401 (registers the ops)
+  with FakeTensorMode():
+    B, T, W, H = 3, 7, 512, 2
+    x = torch.empty(B, T, W, dtype=torch.bfloat16)
+    seg = torch.empty(B, T, dtype=torch.int64)
+    cw = torch.empty(4, W, dtype=torch.bfloat16)
+    cb = torch.empty(W, dtype=torch.bfloat16)
+    w = torch.empty(H, W // H, W // H, dtype=torch.bfloat16)
+    b = torch.empty(H, W // H, dtype=torch.bfloat16)
+    y, h, c = torch.ops.recurrentgemma_amd.recurrent_core(
+        x, seg, cw, cb, w, b, w, b, cb, None, x)
+    assert y.shape == (B, T, W) and y.dtype == torch.bfloat16
+    assert h.shape == (B, W) and h.dtype == torch.float32
+    assert c.shape == (B, 3, W) and c.dtype == torch.bfloat16
+    x1 = torch.empty(B, 1, W, dtype=torch.bfloat16)
+    y1, h1, c1 = torch.ops.recurrentgemma_amd.recurrent_step(
+        x1, seg[:, :1], c, h, cw, cb, w, b, w, b, cb, None)
+    assert y1.shape == (B, 1, W) and h1.shape == (B, W) and c1.shape == (B, 3, W)
