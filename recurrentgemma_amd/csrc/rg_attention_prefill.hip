@@ -107,10 +107,19 @@ attn_prefill_bf16_kernel(AttnPrefillArgs p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, half = lane >> 5;
   const int qtiles = (p.T + kAttnQ - 1) / kAttnQ;
+  // Workgroups go to the eight XCDs in turn (linear id modulo 8), each with an
+  // L2 of its own: the ids are dealt out so that one XCD gets a contiguous run
+  // of (row, head, query tile) triples, i.e. a row's keys and values are
+  // pulled through one L2 instead of all eight.
+  unsigned id = blockIdx.x;
+  {
+    const unsigned per_xcd = gridDim.x / 8;
+    if (id < 8 * per_xcd) id = (id & 7) * per_xcd + (id >> 3);
+  }
   // the longest workgroups (last query tiles) first
-  const int qt = qtiles - 1 - (int)(blockIdx.x % qtiles);
-  const int head = (int)(blockIdx.x / qtiles) % p.H;
-  const int b = (int)(blockIdx.x / qtiles) / p.H;
+  const int qt = qtiles - 1 - (int)(id % qtiles);
+  const int head = (int)(id / qtiles) % p.H;
+  const int b = (int)(id / qtiles) / p.H;
   const int T = p.T;
   const int q0 = qt * kAttnQ;
   const int qw0 = q0 + 32 * wave;  // this wave's first query
