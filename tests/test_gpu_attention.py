@@ -66,6 +66,26 @@ def test_attention_prefill_kernel(B, T, H, window, mean_doc):
                                    what="attention")
 
 
+def test_attention_prefill_left_padded_rows():
+  """Rows padded on the left with position -1, as the sampler lays out
+  prompts of different lengths (sampler.py:234-238): the first real token
+  starts the document, the pads before it only see each other."""
+  B, T, H, hd, window = 3, 200, 2, 256, 2048
+  g = torch.Generator().manual_seed(5)
+  q = torch.randn(B, T, H, hd, generator=g).to(torch.bfloat16).to(DEV)
+  k = torch.randn(B, T, 1, hd, generator=g).to(torch.bfloat16).to(DEV)
+  v = torch.randn(B, T, 1, hd, generator=g).to(torch.bfloat16).to(DEV)
+  seg = torch.arange(T).expand(B, T).clone()
+  for b, pad in enumerate((0, 37, 150)):
+    seg[b] = torch.cat([torch.full((pad,), -1), torch.arange(T - pad)])
+  seg = seg.to(DEV)
+  got = ops.attention_prefill(q, k, v, band(seg, window), hd ** -0.5)
+  want = reference(q, k, v, seg, window, hd ** -0.5)
+  for b, pad in enumerate((0, 37, 150)):  # the real tokens
+    helpers.assert_close_elementwise(got[b, pad:], want[b, pad:], rtol=2e-2,
+                                     atol_of_max=2e-2, what=f"row {b}")
+
+
 def test_attention_prefill_refuses_other_shapes():
   q = torch.zeros(1, 8, 2, 128, dtype=torch.bfloat16, device=DEV)
   assert not ops.attention_prefill_supported(q)
