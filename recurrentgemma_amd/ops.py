@@ -94,6 +94,19 @@ def _p(t):
   return None if t is None else t.data_ptr()
 
 
+def _empty_prefill(x, h0, return_h, return_conv_cache, taps=3):
+  """What the reference returns for no tokens (or no rows): nothing to
+  compute, the state stays what it was (layers.py:181-189 with an empty loop,
+  :526-527 a conv state padded with zeros)."""
+  B, _, W = x.shape
+  h = None
+  if return_h:
+    h = (h0.clone() if h0 is not None else
+         torch.zeros((B, W), dtype=torch.float32, device=x.device))
+  cache = x.new_zeros((B, taps, W)) if return_conv_cache else None
+  return torch.empty_like(x), h, cache
+
+
 def conv1d_prefill(x, segment_pos, w, b, return_cache=True):
   assert x.ndim == 3, f"x must be [B,T,W], got {tuple(x.shape)}"
   B, T, W = x.shape
@@ -101,6 +114,9 @@ def conv1d_prefill(x, segment_pos, w, b, return_cache=True):
   assert w.shape == (K, W) and b.shape == (W,)
   x = _dev(x, "x")
   _same(x.dtype, x.device, w=w, b=b)
+  if x.numel() == 0:
+    out, _, cache = _empty_prefill(x, None, False, return_cache, K - 1)
+    return out, cache
   w, b = _dev(w, "w"), _dev(b, "b")
   seg, is64 = _segpos(segment_pos, B, T)
   out = torch.empty_like(x)
@@ -192,6 +208,8 @@ def gates_gemm(x, w_x, b_x, w_a, b_a, conv=None):
     seg, is64 = _segpos(segment_pos, B, T)
   gx = torch.empty_like(x)
   ga = torch.empty_like(x)
+  if x.numel() == 0:
+    return gx, ga
   with _on(x.device):
     _lib.check(_lib.lib().rg_gates_gemm(
         _p(x), int(conv is not None), _p(seg), is64, _p(cw), _p(cb), _p(w_x),
@@ -229,6 +247,8 @@ def lru_scan_fused(x, gx_pre, ga_pre, a_param, segment_pos, h0=None, conv=None,
     assert cw.shape == (4, W) and cb.shape == (W,)
     _same(x.dtype, x.device, conv_w=cw, conv_b=cb)
     cw, cb = _dev(cw, "conv_w"), _dev(cb, "conv_b")
+  if x.numel() == 0:
+    return _empty_prefill(x, h0, return_h, return_conv_cache)
   y = torch.empty_like(x)
   h_last = (torch.empty((B, W), dtype=torch.float32, device=x.device)
             if return_h else None)
@@ -295,6 +315,8 @@ def recurrent_prefill(x, segment_pos, conv_w, conv_b, w_x, b_x, w_a, b_a,
     assert h0.dtype == torch.float32, "the RG-LRU state is always float32"
     assert h0.shape == (B, W)
     h0 = _dev(h0, "h0")
+  if x.numel() == 0:
+    return _empty_prefill(x, h0, return_h, return_conv_cache)
   y = torch.empty_like(x)
   h_last = (torch.empty((B, W), dtype=torch.float32, device=x.device)
             if return_h else None)
@@ -362,6 +384,8 @@ def recurrent_core(x, segment_pos, conv_w, conv_b, w_x, b_x, w_a, b_a, a_param,
     assert gate_branch.shape == x.shape
     _same(x.dtype, x.device, gate_branch=gate_branch)
     gate_branch = _dev(gate_branch, "gate_branch")
+  if x.numel() == 0:
+    return _empty_prefill(x, h0, return_h, return_conv_cache)
   y = torch.empty_like(x)
   h_last = (torch.empty((B, W), dtype=torch.float32, device=x.device)
             if return_h else None)
@@ -389,6 +413,9 @@ def linear_scan(x, a, reset, h0=None, split=True):
   reset = _dev(reset, "reset")
   if h0 is not None:
     h0 = _dev(h0, "h0")
+  if x.numel() == 0:
+    y, h_last, _ = _empty_prefill(x, h0, True, False)
+    return y, h_last
   y = torch.empty_like(x)
   h_last = torch.empty((B, W), dtype=torch.float32, device=x.device)
   ws = _scan_workspace(B, T, W, x.device, split)

@@ -384,6 +384,32 @@ def test_recurrent_core_shape_sweep():
                                        what=what)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,T", [(2, 0), (0, 5)])
+def test_empty_inputs(dtype, B, T):
+  """No tokens or no rows: nothing is launched, outputs are empty tensors of
+  the right shape, and the state is what the reference's empty loop leaves
+  (layers.py:181-189: h0 or zeros; :526-527: a conv state of zeros)."""
+  W, H = 512, 2
+  p = R.make_params(W, H, dtype, seed=4)
+  blk = _block(p, W, H, dtype)
+  x = _dev(torch.zeros(B, T, W, dtype=dtype))
+  seg = _dev(torch.zeros(B, T, dtype=torch.int64))
+  y, cache = rg.recurrent_core(blk.conv_1d, blk.rg_lru, x, seg)
+  assert y.shape == (B, T, W) and y.dtype == dtype
+  assert cache.rg_lru_state.shape == (B, W)
+  assert cache.rg_lru_state.dtype == torch.float32
+  assert cache.conv1d_state.shape == (B, 3, W)
+  assert not cache.rg_lru_state.any() and not cache.conv1d_state.any()
+  out, cstate = blk.conv_1d(x, seg)
+  assert out.shape == (B, T, W) and cstate.shape == (B, 3, W)
+  h0 = _dev(torch.randn(B, W))
+  y2, h2 = blk.rg_lru(x, seg, h0)
+  assert y2.shape == (B, T, W) and torch.equal(h2, h0)
+  y3, h3 = rg.rnn_scan(x, x, seg == 0, h0)
+  assert y3.shape == (B, T, W) and torch.equal(h3, h0)
+
+
 def test_config1_fp32_parity():
   """Benchmark configuration 1: B1 T512 W2560 H10 fp32, segment_pos = arange."""
   B, T, W, H = 1, 512, 2560, 10
