@@ -159,6 +159,38 @@ attn_decode_probs_kernel(const T* __restrict__ scores, const T* __restrict__ q,
   dot = block_reduce(dot, scratch, false);
   const float self = round_act<T>(round_act<T>(dot) * scale);
   const bool wrapped = nt >= window;
+  if (window <= 8 * 256) {
+    // the usual window (2048): every thread keeps its eight scores, read once
+    float sv[8];
+    float mx = self;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int j = threadIdx.x + 256 * i;
+      const bool visible = j < window && (wrapped || j < nt);
+      sv[i] = visible ? round_act<T>(load_scalar<T>(srow + (j < window ? j : 0)) *
+                                     scale)
+                      : -__builtin_inff();
+      mx = fmaxf(mx, sv[i]);
+    }
+    mx = block_reduce(mx, scratch, true);
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      sv[i] = expf(sv[i] - mx);  // (exp(-inf) = 0 for the slots not visible)
+      sum += sv[i];
+    }
+    const float self_e = expf(self - mx);
+    if (threadIdx.x == 0) sum += self_e;
+    sum = block_reduce(sum, scratch, false);
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int j = threadIdx.x + 256 * i;
+      if (j < window) store_scalar<T>(prow + j, sv[i] * inv);
+    }
+    if (threadIdx.x == 0) store_scalar<T>(prow + window, self_e * inv);
+    return;
+  }
   float mx = self;
   for (int j = threadIdx.x; j < window; j += 256)
     if (wrapped || j < nt)
