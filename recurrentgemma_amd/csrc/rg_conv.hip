@@ -63,7 +63,7 @@ conv1d_cache_tail_kernel(const T* __restrict__ x,
 // rows (b, t): it writes dx for them and leaves its sums of dw and dbias in
 // `partial` [row chunks][K + 1][W] (float32), which the caller adds up.  The
 // neighbouring rows it re-reads come from cache.
-constexpr int kConvBwdRows = 32;
+constexpr int kConvBwdRows = 32;  // (the 16-byte kernels below share it)
 
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -113,6 +113,251 @@ conv1d_backward_kernel(const T* __restrict__ dout, const T* __restrict__ x,
   out[(int64_t)K * W] = db;
 }
 
+// ---- temporal width 4, 16 bytes per lane: the usual case, streaming ---------
+// A wave takes 32 consecutive flattened rows (b, t) of 64 x 16 bytes of
+// channels; a lane walks its rows in time order with the three rows before the
+// current one in registers (loaded once as a halo), so every row of x is read
+// once (plus 3 in 32 for the halo) and every output row written once, as
+// 16-byte accesses.  A document start -- or the first token of a sequence row --
+// zeroes the history registers: later tokens then see zeros exactly where the
+// definition drops a tap.  Rows are requested eight at a time before the first
+// is used.
+constexpr int kConvRun = 32;    // rows per wave (= kConvBwdRows: the partial planes)
+constexpr int kConvBatch = 8;   // rows requested together
+
+template <typename T>
+struct Vec16;
+template <>
+struct Vec16<float> {
+  static constexpr int N = 4;
+  __device__ static void unpack(u32x4 r, float (&v)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = __uint_as_float(r[i]);
+  }
+  __device__ static u32x4 pack(const float (&v)[4]) {
+    return u32x4{__float_as_uint(v[0]), __float_as_uint(v[1]),
+                 __float_as_uint(v[2]), __float_as_uint(v[3])};
+  }
+};
+template <>
+struct Vec16<uint16_t> {
+  static constexpr int N = 8;
+  __device__ static void unpack(u32x4 r, float (&v)[8]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = __uint_as_float(r[i] << 16);
+      v[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
+    }
+  }
+  __device__ static u32x4 pack(const float (&v)[8]) {
+    return u32x4{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]),
+                 pack_bf16x2(v[4], v[5]), pack_bf16x2(v[6], v[7])};
+  }
+};
+
+// row m starts a history: first token of a sequence row, or of a document
+__device__ __forceinline__ bool conv_row_starts(const void* segpos, int seg_kind,
+                                                int T_len, int64_t m) {
+  return m % T_len == 0 || is_doc_start(segpos, seg_kind, m);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(64)
+conv1d_prefill_k4_kernel(const T* __restrict__ x, const void* __restrict__ segpos,
+                         int seg_kind, const T* __restrict__ w,
+                         const T* __restrict__ bias, T* __restrict__ out,
+                         int T_len, int W, int64_t M) {
+  using V = Vec16<T>;
+  constexpr int N = V::N;
+  const int c = ((int)blockIdx.y * 64 + (int)threadIdx.x) * N;
+  if (c >= W) return;  // W % N == 0 (launcher): a lane is inside or outside
+  const int64_t m0 = (int64_t)blockIdx.x * kConvRun;
+  const int64_t m1 = m0 + kConvRun < M ? m0 + kConvRun : M;
+  auto row = [&](const T* base, int64_t m) {
+    return *reinterpret_cast<const u32x4*>(base + m * W + c);
+  };
+  float w0[N], w1[N], w2[N], w3[N], bb[N];
+  V::unpack(row(w, 0), w0);
+  V::unpack(row(w, 1), w1);
+  V::unpack(row(w, 2), w2);
+  V::unpack(row(w, 3), w3);
+  V::unpack(*reinterpret_cast<const u32x4*>(bias + c), bb);
+  // history: h1 = x[m-1], h2 = x[m-2], h3 = x[m-3], zero where a start cuts
+  float h1[N], h2[N], h3[N];
+#pragma unroll
+  for (int e = 0; e < N; ++e) h1[e] = h2[e] = h3[e] = 0.0f;
+  for (int64_t j = m0 - 3; j < m0; ++j) {
+    if (j < 0) continue;
+    if (conv_row_starts(segpos, seg_kind, T_len, j)) {
+#pragma unroll
+      for (int e = 0; e < N; ++e) h1[e] = h2[e] = 0.0f;
+    }
+#pragma unroll
+    for (int e = 0; e < N; ++e) {
+      h3[e] = h2[e];
+      h2[e] = h1[e];
+    }
+    V::unpack(row(x, j), h1);
+  }
+  for (int64_t mb = m0; mb < m1; mb += kConvBatch) {
+    u32x4 raw[kConvBatch];
+    bool st[kConvBatch];
+#pragma unroll
+    for (int u = 0; u < kConvBatch; ++u) {
+      const int64_t m = mb + u < m1 ? mb + u : m1 - 1;
+      raw[u] = row(x, m);
+      st[u] = conv_row_starts(segpos, seg_kind, T_len, m);
+    }
+#pragma unroll
+    for (int u = 0; u < kConvBatch; ++u) {
+      if (mb + u < m1) {
+        if (st[u]) {
+#pragma unroll
+          for (int e = 0; e < N; ++e) h1[e] = h2[e] = h3[e] = 0.0f;
+        }
+        float cur[N], o[N];
+        V::unpack(raw[u], cur);
+#pragma unroll
+        for (int e = 0; e < N; ++e) {
+          o[e] = conv4(cur[e], h1[e], h2[e], h3[e], w0[e], w1[e], w2[e], w3[e],
+                       bb[e]);
+          h3[e] = h2[e];
+          h2[e] = h1[e];
+          h1[e] = cur[e];
+        }
+        *reinterpret_cast<u32x4*>(out + (mb + u) * W + c) = V::pack(o);
+      }
+    }
+  }
+}
+
+// The backward pass in the same shape: the window of x slides as above (for
+// dw), a window of dout[m .. m+3] slides ahead of it (for dx), with the starts
+// of rows m+1 .. m+3 deciding which of them a tap may use.  Sums for dw and
+// dbias go to the chunk's plane of `partial` like the general kernel's.
+template <typename T>
+__global__ void __launch_bounds__(64)
+conv1d_backward_k4_kernel(const T* __restrict__ dout, const T* __restrict__ x,
+                          const void* __restrict__ segpos, int seg_kind,
+                          const T* __restrict__ w, T* __restrict__ dx,
+                          float* __restrict__ partial, int T_len, int W,
+                          int64_t M) {
+  using V = Vec16<T>;
+  constexpr int N = V::N;
+  const int c = ((int)blockIdx.y * 64 + (int)threadIdx.x) * N;
+  if (c >= W) return;
+  const int64_t m0 = (int64_t)blockIdx.x * kConvRun;
+  const int64_t m1 = m0 + kConvRun < M ? m0 + kConvRun : M;
+  auto row = [&](const T* base, int64_t m) {
+    return *reinterpret_cast<const u32x4*>(base + m * W + c);
+  };
+  // a row behind the last one counts as a start (nothing beyond it is used)
+  auto starts = [&](int64_t m) {
+    return m >= M || conv_row_starts(segpos, seg_kind, T_len, m);
+  };
+  float w0[N], w1[N], w2[N], w3[N];
+  V::unpack(row(w, 0), w0);
+  V::unpack(row(w, 1), w1);
+  V::unpack(row(w, 2), w2);
+  V::unpack(row(w, 3), w3);
+  float h1[N], h2[N], h3[N], d0[N], d1[N], d2[N], d3[N], db[N];
+#pragma unroll
+  for (int e = 0; e < N; ++e)
+    h1[e] = h2[e] = h3[e] = d0[e] = d1[e] = d2[e] = d3[e] = db[e] = 0.0f;
+  for (int64_t j = m0 - 3; j < m0; ++j) {
+    if (j < 0) continue;
+    if (conv_row_starts(segpos, seg_kind, T_len, j)) {
+#pragma unroll
+      for (int e = 0; e < N; ++e) h1[e] = h2[e] = 0.0f;
+    }
+#pragma unroll
+    for (int e = 0; e < N; ++e) {
+      h3[e] = h2[e];
+      h2[e] = h1[e];
+    }
+    V::unpack(row(x, j), h1);
+  }
+  // g0 = dout[m], g1 .. g3 the rows after it; f1 .. f3: those rows start
+  float g0[N], g1[N], g2[N], g3[N];
+  bool f1, f2, f3;
+  auto dout_row = [&](int64_t m, float (&v)[N]) {
+    if (m < M) {
+      V::unpack(row(dout, m), v);
+    } else {
+#pragma unroll
+      for (int e = 0; e < N; ++e) v[e] = 0.0f;
+    }
+  };
+  dout_row(m0, g0);
+  dout_row(m0 + 1, g1);
+  dout_row(m0 + 2, g2);
+  f1 = starts(m0 + 1);
+  f2 = starts(m0 + 2);
+  for (int64_t mb = m0; mb < m1; mb += kConvBatch) {
+    u32x4 xr[kConvBatch], gr[kConvBatch];
+    bool st[kConvBatch], fa[kConvBatch];
+#pragma unroll
+    for (int u = 0; u < kConvBatch; ++u) {
+      const int64_t m = mb + u < m1 ? mb + u : m1 - 1;
+      xr[u] = row(x, m);
+      gr[u] = row(dout, m + 3 < M ? m + 3 : M - 1);
+      st[u] = conv_row_starts(segpos, seg_kind, T_len, m);
+      fa[u] = starts(m + 3);
+    }
+#pragma unroll
+    for (int u = 0; u < kConvBatch; ++u) {
+      const int64_t m = mb + u;
+      if (m < m1) {
+        if (m + 3 < M) {
+          V::unpack(gr[u], g3);
+        } else {
+#pragma unroll
+          for (int e = 0; e < N; ++e) g3[e] = 0.0f;
+        }
+        f3 = fa[u];
+        if (st[u]) {
+#pragma unroll
+          for (int e = 0; e < N; ++e) h1[e] = h2[e] = h3[e] = 0.0f;
+        }
+        float cur[N], o[N];
+        V::unpack(xr[u], cur);
+        const bool ok1 = !f1, ok2 = ok1 && !f2, ok3 = ok2 && !f3;
+#pragma unroll
+        for (int e = 0; e < N; ++e) {
+          float acc = w3[e] * g0[e];
+          acc = __builtin_fmaf(w2[e], ok1 ? g1[e] : 0.0f, acc);
+          acc = __builtin_fmaf(w1[e], ok2 ? g2[e] : 0.0f, acc);
+          acc = __builtin_fmaf(w0[e], ok3 ? g3[e] : 0.0f, acc);
+          o[e] = acc;
+          d3[e] = __builtin_fmaf(cur[e], g0[e], d3[e]);  // w[3] meets x[t]
+          d2[e] = __builtin_fmaf(h1[e], g0[e], d2[e]);
+          d1[e] = __builtin_fmaf(h2[e], g0[e], d1[e]);
+          d0[e] = __builtin_fmaf(h3[e], g0[e], d0[e]);
+          db[e] += g0[e];
+          h3[e] = h2[e];
+          h2[e] = h1[e];
+          h1[e] = cur[e];
+          g0[e] = g1[e];
+          g1[e] = g2[e];
+          g2[e] = g3[e];
+        }
+        f1 = f2;
+        f2 = f3;
+        *reinterpret_cast<u32x4*>(dx + m * W + c) = V::pack(o);
+      }
+    }
+  }
+  float* outp = partial + (int64_t)blockIdx.x * 5 * W + c;
+#pragma unroll
+  for (int e = 0; e < N; ++e) {
+    outp[e] = d0[e];
+    outp[(int64_t)W + e] = d1[e];
+    outp[2 * (int64_t)W + e] = d2[e];
+    outp[3 * (int64_t)W + e] = d3[e];
+    outp[4 * (int64_t)W + e] = db[e];
+  }
+}
+
 // Decode step: one thread per (batch row, channel).  All state rows are read
 // into registers before anything is written, so cache_out may alias cache_in.
 template <typename T>
@@ -155,12 +400,30 @@ inline int grid_for(int64_t total, int block) {
   return (int)(g < 1 ? 1 : (g > cap ? cap : g));
 }
 
+// whether the 16-byte kernels serve this shape
+template <typename T>
+bool conv_k4_fits(int K, int W, int64_t M) {
+  constexpr int N = 16 / (int)sizeof(T);
+  return K == 4 && W % N == 0 && (M + kConvRun - 1) / kConvRun <= 0x7fffffff &&
+         (W / N + 63) / 64 <= 65535;
+}
+
 template <typename T>
 hipError_t conv_prefill_t(const ConvArgs& a, hipStream_t s) {
   const int64_t total = (int64_t)a.B * a.T * a.W;
-  conv1d_prefill_kernel<T><<<grid_for(total, 256), 256, 0, s>>>(
-      (const T*)a.x, a.segpos, a.seg_kind, (const T*)a.w,
-      (const T*)a.bias, (T*)a.out, a.T, a.W, a.K, total);
+  const int64_t M = (int64_t)a.B * a.T;
+  if (conv_k4_fits<T>(a.K, a.W, M)) {
+    constexpr int N = 16 / (int)sizeof(T);
+    const dim3 grid((unsigned)((M + kConvRun - 1) / kConvRun),
+                    (unsigned)((a.W / N + 63) / 64));
+    conv1d_prefill_k4_kernel<T><<<grid, 64, 0, s>>>(
+        (const T*)a.x, a.segpos, a.seg_kind, (const T*)a.w, (const T*)a.bias,
+        (T*)a.out, a.T, a.W, M);
+  } else {
+    conv1d_prefill_kernel<T><<<grid_for(total, 256), 256, 0, s>>>(
+        (const T*)a.x, a.segpos, a.seg_kind, (const T*)a.w,
+        (const T*)a.bias, (T*)a.out, a.T, a.W, a.K, total);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || !a.cache_out) return e;
   const int64_t ctotal = (int64_t)a.B * (a.K - 1) * a.W;
@@ -203,6 +466,21 @@ hipError_t launch_conv1d_backward(const ConvBwdArgs& a, int dtype,
   if (chunks <= 0 || chunks > 0x7fffffff || cblocks > 65535 || a.K < 2 ||
       a.K > 16)
     return hipErrorInvalidValue;
+  if (dtype == 0 ? conv_k4_fits<float>(a.K, a.W, M)
+                 : conv_k4_fits<uint16_t>(a.K, a.W, M)) {
+    if (dtype == 0)
+      conv1d_backward_k4_kernel<float>
+          <<<dim3((unsigned)chunks, (unsigned)((a.W / 4 + 63) / 64)), 64, 0, s>>>(
+              (const float*)a.dout, (const float*)a.x, a.segpos, a.seg_kind,
+              (const float*)a.w, (float*)a.dx, a.partial, a.T, a.W, M);
+    else
+      conv1d_backward_k4_kernel<uint16_t>
+          <<<dim3((unsigned)chunks, (unsigned)((a.W / 8 + 63) / 64)), 64, 0, s>>>(
+              (const uint16_t*)a.dout, (const uint16_t*)a.x, a.segpos,
+              a.seg_kind, (const uint16_t*)a.w, (uint16_t*)a.dx, a.partial, a.T,
+              a.W, M);
+    return hipGetLastError();
+  }
   const dim3 grid((unsigned)chunks, (unsigned)cblocks);
   if (dtype == 0)
     conv1d_backward_kernel<float><<<grid, 256, 0, s>>>(
