@@ -201,6 +201,12 @@ int rg_block_diag_linear(const void* x, const void* w, const void* b, void* y,
   if (dtype == RG_DTYPE_F32 && bw == 256)
     return launch_status(__func__,
                          rg::launch_gemm_mfma_f32(a, (hipStream_t)stream));
+  // (the bf16 matrix kernel addresses rows of x and y with 32-bit offsets
+  // inside one 64-row tile only)
+  if (dtype == RG_DTYPE_BF16 && bw == 256 && aligned16(x) && aligned16(w) &&
+      aligned16(y))
+    return launch_status(__func__,
+                         rg::launch_gemm_mfma_bf16(a, (hipStream_t)stream));
   return launch_status(__func__,
                        rg::launch_gemm_generic(a, dtype, (hipStream_t)stream));
 }

@@ -119,7 +119,11 @@ union Frag {
   f32x4 q;
 };
 
-template <bool CONV>
+// ONE: a single matrix (p.w[0], p.b[0], p.out[0]).  Waves 0-3 then do all of
+// the matrix work; waves 4-7 only take their share of the x staging (the
+// staging loops are laid out for 512 threads), issue no matrix instruction
+// and store through an empty descriptor.
+template <bool CONV, bool ONE = false>
 __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   uint16_t* lds = reinterpret_cast<uint16_t*>(lds_raw);
@@ -134,14 +138,15 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
   const int64_t ntiles = (M + kTM - 1) / kTM;
 
   // ---- this wave's weight slice, resident in registers -----------------
-  const int gate = wave >> 2;         // waves 0-3: input gate, 4-7: a gate
+  const int gate = ONE ? 0 : wave >> 2;  // waves 0-3: input gate, 4-7: a gate
+  const bool active = !ONE || wave < 4;  // wave-uniform
   const int n0 = (wave & 3) * 64;     // first output column inside the gate
   // The weights are [k][n] with n contiguous, the MFMA B operand wants 8
   // consecutive k per lane: transpose through LDS, 128 k-rows of one gate at
   // a time (coalesced 16-byte global reads, 2-byte LDS reads).
   Frag bfrag[16][2];
 #pragma unroll
-  for (int g = 0; g < 2; ++g) {
+  for (int g = 0; g < (ONE ? 1 : 2); ++g) {
 #pragma unroll
     for (int kh = 0; kh < 2; ++kh) {
       const uint16_t* src =
@@ -379,8 +384,8 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
     char* const tilep = outbase + row_first * W * 2;            // uniform
     const int rows_left =
         (int)((M - row_first) < kTM ? (M - row_first) : kTM);   // uniform, > 0
-    const __amdgpu_buffer_rsrc_t ro =
-        make_rsrc(tilep, (uint32_t)rows_left * out_row_bytes);
+    const __amdgpu_buffer_rsrc_t ro = make_rsrc(
+        tilep, active ? (uint32_t)rows_left * out_row_bytes : 0u);
 
     // The block goes through this wave's LDS patch (row-major, bf16) so that
     // each lane stores 16 contiguous bytes (8 rows x 128 bytes per
@@ -440,10 +445,12 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
 #pragma unroll
         for (int ks = 0; ks < 16; ++ks) {
           if (ks < 14) a[(ks + 2) % 3] = a_read(0, ks + 2);
-          acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              bfrag[ks][0].v, a[ks % 3].v, acc0, 0, 0, 0);
-          acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              bfrag[ks][1].v, a[ks % 3].v, acc1, 0, 0, 0);
+          if (active) {
+            acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                bfrag[ks][0].v, a[ks % 3].v, acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                bfrag[ks][1].v, a[ks % 3].v, acc1, 0, 0, 0);
+          }
           stage_row(kHalo + ks, buf ^ 1, NoCuts{});
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -457,10 +464,12 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
 #pragma unroll
         for (int ks = 0; ks < 16; ++ks) {
           if (ks < 15) a[(ks + 1) % 3] = a_read(0, ks + 1);
-          acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              bfrag[ks][0].v, a[ks % 3].v, acc0, 0, 0, 0);
-          acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              bfrag[ks][1].v, a[ks % 3].v, acc1, 0, 0, 0);
+          if (active) {
+            acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                bfrag[ks][0].v, a[ks % 3].v, acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                bfrag[ks][1].v, a[ks % 3].v, acc1, 0, 0, 0);
+          }
         }
       }
       result_to_lds(acc0, acc1);
@@ -478,10 +487,12 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
 #pragma unroll
       for (int ks = 0; ks < 16; ++ks) {
         if (ks < 14) a[(ks + 2) % 3] = a_read(1, ks + 2);
-        acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            bfrag[ks][0].v, a[ks % 3].v, acc0, 0, 0, 0);
-        acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            bfrag[ks][1].v, a[ks % 3].v, acc1, 0, 0, 0);
+        if (active) {
+          acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              bfrag[ks][0].v, a[ks % 3].v, acc0, 0, 0, 0);
+          acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              bfrag[ks][1].v, a[ks % 3].v, acc1, 0, 0, 0);
+        }
         if (ks < 4) {
           patch_store(0, ks, pv);
           if (ks < 3) pv = patch_read(ks + 1);
@@ -704,7 +715,7 @@ hipError_t launch_gemm_mfma_f32(const GemmArgs& a, hipStream_t s) {
 }
 
 hipError_t launch_gemm_mfma_bf16(const GemmArgs& a, hipStream_t s) {
-  // needs both gates, bw == 256 (checked by the caller)
+  // needs bw == 256 (checked by the caller); one matrix or both gates
   const int64_t ntiles = (a.M + kTM - 1) / kTM;
   int per_head = 256 / a.H;  // about one resident workgroup per CU
   if (per_head < 1) per_head = 1;
@@ -712,7 +723,14 @@ hipError_t launch_gemm_mfma_bf16(const GemmArgs& a, hipStream_t s) {
   if (a.H > 65535) return hipErrorInvalidValue;
   dim3 grid((unsigned)per_head, (unsigned)a.H);
   hipError_t e;
-  if (a.apply_conv) {
+  if (a.ngates == 1) {
+    if (a.apply_conv) return hipErrorInvalidValue;
+    static OncePerDevice once;
+    e = set_max_dynamic_lds(
+        once, (const void*)gates_mfma_bf16_kernel<false, true>, kMfmaLdsBytes);
+    if (e != hipSuccess) return e;
+    gates_mfma_bf16_kernel<false, true><<<grid, 512, kMfmaLdsBytes, s>>>(a);
+  } else if (a.apply_conv) {
     static OncePerDevice once;
     e = set_max_dynamic_lds(once, (const void*)gates_mfma_bf16_kernel<true>,
                             kMfmaLdsBytes);

@@ -134,7 +134,8 @@ def test_conv1d_vs_oracle(dtype, K):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("width,blocks", [(128, 1), (128, 16), (1024, 1),
-                                          (1024, 16), (512, 2), (60, 3)])
+                                          (1024, 16), (512, 2), (60, 3),
+                                          (2560, 10)])
 def test_block_diagonal_linear(dtype, width, blocks):
   g = torch.Generator().manual_seed(width + blocks)
   bw = width // blocks
@@ -146,7 +147,10 @@ def test_block_diagonal_linear(dtype, width, blocks):
   m.load_state_dict({"w": w, "b": b})
   m = m.to(DEV)
   tol = F32_TOL if dtype == torch.float32 else BF16_TOL
-  for xi in (x, x2):
+  cases = [x, x2]
+  if bw == 256:  # the matrix-core kernels: many row tiles, a ragged last one
+    cases.append(torch.randn(5, 1231, width, generator=g).to(dtype))
+  for xi in cases:
     _announce("bdl", dtype, width, blocks, tuple(xi.shape))
     want = R.block_diagonal_linear(xi.float(), w.float(), b.float())
     assert helpers.max_rel(m(_dev(xi)), want) < tol
