@@ -292,7 +292,11 @@ int rg_recurrent_prefill_gelu_mul(
  * must hold rg_recurrent_core_workspace_bytes(B, T, W, H, dtype) bytes (0 for
  * whole rows in the single kernel: workspace may then be null).  Same values
  * as the calls it is made of; h0 / h_last / conv_cache_out / w_packed as in
- * rg_recurrent_prefill (w_packed is only read by the single kernel). */
+ * rg_recurrent_prefill (w_packed is only read by the single kernel).
+ * conv_w == conv_b == NULL (conv_cache_out then NULL too): x is the conv
+ * output already, and the call is RGLRU.forward on its own
+ * (recurrentgemma/torch/layers.py:313-365); rg_recurrent_prefill and its
+ * variants take the same. */
 size_t rg_recurrent_core_workspace_bytes(int B, int T, int W, int H, int dtype);
 int rg_recurrent_core(const void* x, const void* gate_branch,
                       const void* segpos, int segpos_is_i64,

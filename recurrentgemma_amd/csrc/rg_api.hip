@@ -407,8 +407,13 @@ static int recurrent_prefill_impl(const char* who, const void* x,
   RG_REQUIRE(W % H == 0, "%s: W=%d is not a multiple of H=%d", who, W, H);
   RG_CHECK_PTR(x);
   RG_CHECK_PTR(segpos);
-  RG_CHECK_PTR(conv_w);
-  RG_CHECK_PTR(conv_b);
+  RG_CHECK_OPT_PTR(conv_w);
+  RG_CHECK_OPT_PTR(conv_b);
+  // no conv weights: x is the conv output already (a stand-alone RG-LRU)
+  RG_REQUIRE((conv_w == nullptr) == (conv_b == nullptr),
+             "%s: conv_w and conv_b go together", who);
+  RG_REQUIRE(conv_w != nullptr || conv_cache_out == nullptr,
+             "%s: no conv state without a conv", who);
   RG_CHECK_PTR(w_x);
   RG_CHECK_PTR(b_x);
   RG_CHECK_PTR(w_a);
@@ -571,6 +576,11 @@ int rg_recurrent_core(const void* x, const void* gate_branch,
   RG_CHECK_OPT_PTR(gate_branch);
   RG_REQUIRE(gate_branch == nullptr || gate_branch != x,
              "%s: gate_branch must not alias x", __func__);
+  RG_REQUIRE((conv_w == nullptr) == (conv_b == nullptr),
+             "%s: conv_w and conv_b go together", __func__);
+  RG_REQUIRE(conv_w != nullptr || conv_cache_out == nullptr,
+             "%s: no conv state without a conv", __func__);
+  const int conv = conv_w != nullptr;
   const CorePlan p = core_plan(B, T, W, H, dtype);
   const size_t need = p.split_bytes + 2 * p.gate_bytes;
   if (need > 0 && (workspace == nullptr || workspace_bytes < need ||
@@ -591,10 +601,10 @@ int rg_recurrent_core(const void* x, const void* gate_branch,
     char* const ws = (char*)workspace;
     void* const gx = ws + p.split_bytes;
     void* const ga = ws + p.split_bytes + p.gate_bytes;
-    int rc = rg_gates_gemm(x, 1, segpos, segpos_is_i64, conv_w, conv_b, w_x,
+    int rc = rg_gates_gemm(x, conv, segpos, segpos_is_i64, conv_w, conv_b, w_x,
                            b_x, w_a, b_a, gx, ga, B, T, W, H, dtype, stream);
     if (rc != RG_OK) return rc;
-    rc = lru_scan_fused_impl(__func__, x, 1, conv_w, conv_b, gx, ga, a_param,
+    rc = lru_scan_fused_impl(__func__, x, conv, conv_w, conv_b, gx, ga, a_param,
                              segpos, segpos_is_i64, h0, out, h_last,
                              conv_cache_out, workspace, p.split_bytes, true, B,
                              T, W, dtype, stream);

@@ -276,13 +276,19 @@ __device__ __forceinline__ void prefill_body(const FusedArgs& p,
 
   // ---- conv table -------------------------------------------------------------
   if (tid < 128) {
-    const uint16_t* cw = (const uint16_t*)p.conv_w + h * kBW + tid * 2;
-    const uint32_t u0 = *reinterpret_cast<const uint32_t*>(cw);
-    const uint32_t u1 = *reinterpret_cast<const uint32_t*>(cw + W);
-    const uint32_t u2 = *reinterpret_cast<const uint32_t*>(cw + 2 * W);
-    const uint32_t u3 = *reinterpret_cast<const uint32_t*>(cw + 3 * W);
-    const uint32_t ub = *reinterpret_cast<const uint32_t*>(
-        (const uint16_t*)p.conv_b + h * kBW + tid * 2);
+    // Without conv weights x is the conv output already (a stand-alone
+    // RG-LRU): the table then holds the identity, w3 = 1 and nothing else,
+    // which hands every finite x[t] through exactly.
+    uint32_t u0 = 0, u1 = 0, u2 = 0, u3 = 0x3f803f80u, ub = 0;
+    if (p.conv_w != nullptr) {
+      const uint16_t* cw = (const uint16_t*)p.conv_w + h * kBW + tid * 2;
+      u0 = *reinterpret_cast<const uint32_t*>(cw);
+      u1 = *reinterpret_cast<const uint32_t*>(cw + W);
+      u2 = *reinterpret_cast<const uint32_t*>(cw + 2 * W);
+      u3 = *reinterpret_cast<const uint32_t*>(cw + 3 * W);
+      ub = *reinterpret_cast<const uint32_t*>(
+          (const uint16_t*)p.conv_b + h * kBW + tid * 2);
+    }
     // w0 multiplies x[t-3], w3 multiplies x[t] (layers.py:514)
     const u32x4 t0 = {(u0 & 0xffffu) | (u1 << 16), (u2 & 0xffffu) | (u3 << 16),
                       (u0 >> 16) | (u1 & 0xffff0000u),

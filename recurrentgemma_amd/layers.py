@@ -139,11 +139,12 @@ class RGLRU(nn.Module):
       return self._forward_kernels(x, segment_pos, cache, return_cache)
 
   def _forward_kernels(self, x, segment_pos, cache, return_cache):
-    gx_pre, ga_pre = ops.gates_gemm(x, self.input_gate.w, self.input_gate.b,
-                                    self.a_gate.w, self.a_gate.b)
-    y, last_h, _ = ops.lru_scan_fused(x, gx_pre, ga_pre, self.a_param,
-                                      segment_pos, h0=cache,
-                                      return_h=return_cache)
+    # one call without conv weights: the library picks the single prefill
+    # kernel or gate GEMM + scan as it does for the whole block
+    y, last_h, _ = ops.recurrent_core(
+        x, segment_pos, None, None, self.input_gate.w, self.input_gate.b,
+        self.a_gate.w, self.a_gate.b, self.a_param, h0=cache,
+        return_h=return_cache, return_conv_cache=False)
     if not return_cache:
       return y, None
     return y, last_h

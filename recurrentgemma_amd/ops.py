@@ -361,19 +361,28 @@ def recurrent_core(x, segment_pos, conv_w, conv_b, w_x, b_x, w_a, b_a, a_param,
   library, which picks the kernels (rg_recurrent_core): the single prefill
   kernel where it pays, else gate GEMM + scan.  gate_branch: the block's
   linear_y output; the result is then y * gelu(gate_branch).
+  conv_w = conv_b = None: x is the conv output already (RGLRU.forward on its
+  own, layers.py:313-365); there is then no conv cache to return.
   Returns (y, h_last | None, conv_cache | None)."""
   B, T, W = x.shape
   H = w_x.shape[0]
-  assert conv_w.shape == (4, W) and conv_b.shape == (W,)
+  if conv_w is None:
+    assert conv_b is None
+    return_conv_cache = False
+  else:
+    assert conv_w.shape == (4, W) and conv_b.shape == (W,)
   assert w_x.shape == w_a.shape == (H, W // H, W // H)
   assert b_x.shape == b_a.shape == (H, W // H)
   assert a_param.shape == (W,)
   x = _dev(x, "x")
-  _same(x.dtype, x.device, conv_w=conv_w, conv_b=conv_b, w_x=w_x, b_x=b_x,
-        w_a=w_a, b_a=b_a, a_param=a_param)
-  cw, cb, wx_, bx_, wa_, ba_, ap_ = [
-      _dev(t, n) for t, n in ((conv_w, "conv_w"), (conv_b, "conv_b"),
-                              (w_x, "w_x"), (b_x, "b_x"), (w_a, "w_a"),
+  _same(x.dtype, x.device, w_x=w_x, b_x=b_x, w_a=w_a, b_a=b_a,
+        a_param=a_param)
+  cw = cb = None
+  if conv_w is not None:
+    _same(x.dtype, x.device, conv_w=conv_w, conv_b=conv_b)
+    cw, cb = _dev(conv_w, "conv_w"), _dev(conv_b, "conv_b")
+  wx_, bx_, wa_, ba_, ap_ = [
+      _dev(t, n) for t, n in ((w_x, "w_x"), (b_x, "b_x"), (w_a, "w_a"),
                               (b_a, "b_a"), (a_param, "a_param"))]
   seg, is64 = _segpos(segment_pos, B, T)
   if h0 is not None:
