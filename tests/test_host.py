@@ -156,6 +156,16 @@ def test_c_side_validation_without_launch():
                              None, ok, None, None, None, 0, 16, 64, 4096, 16, 1,
                              None)
   assert rc == -1 and b"alias" in lib.rg_last_error()
+  # without conv weights (the RG-LRU on its own): both or neither, and no
+  # conv state to return
+  rc = lib.rg_recurrent_core(ok, None, ok, 1, ok, None, ok, ok, ok, ok, None, ok,
+                             None, y, None, None, None, 0, 16, 64, 4096, 16, 1,
+                             None)
+  assert rc == -1 and b"go together" in lib.rg_last_error()
+  rc = lib.rg_recurrent_core(ok, None, ok, 1, None, None, ok, ok, ok, ok, None,
+                             ok, None, y, None, y, None, 0, 16, 64, 4096, 16, 1,
+                             None)
+  assert rc == -1 and b"no conv state" in lib.rg_last_error()
   assert lib.rg_scan_split_workspace_bytes(16, 8192, 4096) == 0
   assert lib.rg_scan_split_workspace_bytes(1, 500, 2560) == 0
   assert lib.rg_scan_split_workspace_bytes(1, 8192, 2560) == 2 * 22 * 2560 * 4
