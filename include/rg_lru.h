@@ -443,6 +443,33 @@ int rg_attention_decode_finish(const void* from_ring, const void* probs,
                                int head_dim, int window, int update_cache,
                                int dtype, void* stream);
 
+/* One decoded token per row of the local-attention block against its ring
+ * cache, from the projections to the block's output before proj_final
+ * (recurrentgemma/torch/modules.py:431-476; cache :152-216): rotary embedding
+ * of the queries and the new key (:52-83), scores against the ring, mask (slot
+ * j is visible iff it was ever written), softmax with the new token's own
+ * score, weighted sum of the values, the new token's share; with update_cache
+ * the rotated key and the value go into slot num_tokens % window and
+ * num_tokens is incremented, in place.  Two launches that read the ring once
+ * (rg_rope + two batched products + rg_attention_decode_probs + _finish
+ * otherwise).  bf16, head_dim 256, heads <= 16, window <= 16384.
+ * q [B, heads*256] rows ldq elements apart, k_new / v_new [B, 256] rows ldk /
+ * ldv apart, all three as the projections left them (slices of one wider
+ * output qualify: strides are multiples of 8); positions [B] int32/int64;
+ * inv_freq [64] float32; ring_* [B, window, 256]; out [B, heads, 256];
+ * workspace: rg_attention_decode_fused_workspace_bytes(B, heads, window) bytes
+ * (0: unsupported shape).  Roundings as the separate calls, except that the
+ * probabilities enter the second product unnormalised (streaming softmax). */
+size_t rg_attention_decode_fused_workspace_bytes(int B, int heads, int window);
+int rg_attention_decode_fused(const void* q, int64_t ldq, const void* k_new,
+                              int64_t ldk, const void* v_new, int64_t ldv,
+                              const void* positions, int positions_are_i64,
+                              const float* inv_freq, void* ring_keys,
+                              void* ring_values, int32_t* num_tokens, void* out,
+                              void* workspace, size_t workspace_bytes, int B,
+                              int heads, int head_dim, int window, float scale,
+                              int update_cache, int dtype, void* stream);
+
 /* The same decode step in ONE launch, for bf16 with 256-wide heads (no
  * counterpart call in the reference: it is RecurrentBlock.forward with a
  * cache, modules.py:632-643, after a one-time re-layout of the two gate

@@ -88,6 +88,11 @@ SIGNATURES = {
     "rg_attention_decode_probs": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i,
                                        ctypes.c_float, _i, _vp]),
     "rg_attention_decode_finish": (_i, [_vp] * 8 + [_i] * 6 + [_vp]),
+    "rg_attention_decode_fused_workspace_bytes": (_sz, [_i, _i, _i]),
+    "rg_attention_decode_fused": (_i, [_vp, ctypes.c_int64, _vp, ctypes.c_int64,
+                                       _vp, ctypes.c_int64, _vp, _i, _vp, _vp,
+                                       _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i,
+                                       ctypes.c_float, _i, _i, _vp]),
     "rg_packed_gate_weights_bytes": (_sz, [_i, _i, _i]),
     "rg_pack_gate_weights": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "rg_recurrent_step_packed": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp,

@@ -1030,6 +1030,80 @@ int rg_attention_decode_finish(const void* from_ring, const void* probs,
                                     (hipStream_t)stream));
 }
 
+size_t rg_attention_decode_fused_workspace_bytes(int B, int heads, int window) {
+  if (B <= 0 || heads <= 0 || heads > 16 || window <= 0) return 0;
+  const size_t chunks =
+      ((size_t)window + rg::kAttnDecodeChunk - 1) / rg::kAttnDecodeChunk;
+  if (chunks > (size_t)rg::kAttnDecodeMaxChunks) return 0;
+  return (size_t)B * chunks * heads * (256 + 2) * sizeof(float);
+}
+
+int rg_attention_decode_fused(const void* q, int64_t ldq, const void* k_new,
+                              int64_t ldk, const void* v_new, int64_t ldv,
+                              const void* positions, int positions_are_i64,
+                              const float* inv_freq, void* ring_keys,
+                              void* ring_values, int32_t* num_tokens, void* out,
+                              void* workspace, size_t workspace_bytes, int B,
+                              int heads, int head_dim, int window, float scale,
+                              int update_cache, int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(B > 0 && heads > 0 && head_dim > 0 && window > 0,
+             "%s: B=%d heads=%d head_dim=%d window=%d must be positive",
+             __func__, B, heads, head_dim, window);
+  const size_t need = rg_attention_decode_fused_workspace_bytes(B, heads, window);
+  if (dtype != RG_DTYPE_BF16 || head_dim != 256 || need == 0 || B > 65535)
+    return fail(RG_ERR_UNSUPPORTED,
+                "%s: needs bf16, head_dim 256, at most 16 heads, window <= %d, "
+                "B <= 65535 (dtype=%d head_dim=%d heads=%d window=%d B=%d)",
+                __func__, rg::kAttnDecodeChunk * rg::kAttnDecodeMaxChunks, dtype,
+                head_dim, heads, window, B);
+  RG_CHECK_PTR(q);
+  RG_CHECK_PTR(k_new);
+  RG_CHECK_PTR(v_new);
+  RG_CHECK_PTR(positions);
+  RG_CHECK_PTR(inv_freq);
+  RG_CHECK_PTR(ring_keys);
+  RG_CHECK_PTR(ring_values);
+  RG_CHECK_PTR(num_tokens);
+  RG_CHECK_PTR(out);
+  RG_REQUIRE(ldq >= (int64_t)heads * 256 && ldk >= 256 && ldv >= 256 &&
+                 ldq % 8 == 0 && ldk % 8 == 0 && ldv % 8 == 0,
+             "%s: row strides ldq=%lld ldk=%lld ldv=%lld must cover a row and "
+             "be multiples of 8 elements", __func__, (long long)ldq,
+             (long long)ldk, (long long)ldv);
+  RG_REQUIRE(aligned16(q) && aligned16(k_new) && aligned16(v_new) &&
+                 aligned16(ring_keys) && aligned16(ring_values) && aligned16(out),
+             "%s: tensors must be 16-byte aligned", __func__);
+  if (workspace == nullptr || workspace_bytes < need || !aligned16(workspace))
+    return fail(RG_ERR_WORKSPACE,
+                "%s: workspace of %zu bytes (16-byte aligned) required, got %zu",
+                __func__, need, workspace ? workspace_bytes : (size_t)0);
+  rg::AttnDecodeArgs a{};
+  a.q = (const uint16_t*)q;
+  a.k_new = (const uint16_t*)k_new;
+  a.v_new = (const uint16_t*)v_new;
+  a.ldq = ldq;
+  a.ldk = ldk;
+  a.ldv = ldv;
+  a.pos = positions;
+  a.pos_kind = positions_are_i64 ? 1 : 0;
+  a.inv_freq = inv_freq;
+  a.ring_k = (uint16_t*)ring_keys;
+  a.ring_v = (uint16_t*)ring_values;
+  a.num_tokens = num_tokens;
+  a.out = (uint16_t*)out;
+  a.B = B;
+  a.heads = heads;
+  a.window = window;
+  a.chunks = (window + rg::kAttnDecodeChunk - 1) / rg::kAttnDecodeChunk;
+  a.part_o = (float*)workspace;
+  a.part_ml = a.part_o + (size_t)B * a.chunks * heads * 256;
+  a.scale = scale;
+  a.update = update_cache ? 1 : 0;
+  return launch_status(__func__,
+                       rg::launch_attn_decode_fused(a, (hipStream_t)stream));
+}
+
 size_t rg_packed_gate_weights_bytes(int W, int H, int dtype) {
   if (W <= 0 || H <= 0 || W % H != 0 || dtype != RG_DTYPE_BF16 || W / H != 256)
     return 0;

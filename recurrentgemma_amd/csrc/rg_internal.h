@@ -151,6 +151,29 @@ struct AttnPrefillArgs {
 };
 hipError_t launch_attn_prefill_bf16(const AttnPrefillArgs& a, hipStream_t s);
 
+// One decoded token against the ring cache (rg_attention_decode.hip).
+constexpr int kAttnDecodeChunk = 256;     // ring slots per workgroup
+constexpr int kAttnDecodeMaxChunks = 64;  // window <= 16384
+struct AttnDecodeArgs {
+  const uint16_t* q;      // [B, heads, 256] rows ldq apart, before the rotary
+  const uint16_t* k_new;  // [B, 256] rows ldk apart, before the rotary
+  const uint16_t* v_new;  // [B, 256] rows ldv apart
+  int64_t ldq, ldk, ldv;  // in elements
+  const void* pos;        // [B] positions of the new tokens
+  int pos_kind;           // 0: int32, 1: int64
+  const float* inv_freq;  // [64]
+  uint16_t* ring_k;       // [B, window, 256]
+  uint16_t* ring_v;
+  int32_t* num_tokens;    // [B] tokens seen before this one
+  uint16_t* out;          // [B, heads, 256]
+  float* part_o;          // [B, chunks, heads, 256]
+  float* part_ml;         // [B, chunks, heads, 2]: maximum, denominator
+  int B, heads, window, chunks;
+  float scale;
+  int update;             // write the ring slot and count the token
+};
+hipError_t launch_attn_decode_fused(const AttnDecodeArgs& a, hipStream_t s);
+
 struct LinearArgs {
   const void* x;         // [M, K] bf16
   const void* w_packed;  // see launch_linear_pack

@@ -310,6 +310,7 @@ class LocalAttentionBlock(nn.Module):
     # the projections for at most 64 rows (a decode step)
     self._rows_q = ops.PackedLinear()
     self._rows_kv = ops.PackedLinear()
+    self._rows_qkv = ops.PackedLinear()  # a decode step: one launch for all
     self._rows_final = ops.PackedLinear()
     self._inv_freq = None
     self.reset_parameters()
@@ -355,6 +356,15 @@ class LocalAttentionBlock(nn.Module):
     """defer_out: as for RecurrentBlock.forward."""
     b, t, _ = x.shape
     assert segment_pos.shape == (b, t), segment_pos.shape
+    if self._inv_freq is None or self._inv_freq.device != x.device:
+      self._inv_freq = _inv_frequencies(self.head_dim, x.device)
+    if (cache is not None and t == 1 and
+        ops.PackedLinear.usable(x, self.width,
+                                self.width + 2 * self.head_dim) and
+        ops.attention_decode_fused_supported(
+            x, self.num_heads, self.head_dim, self.window_size)):
+      return self._decode_step_fused(x, segment_pos, cache, return_cache,
+                                     defer_out)
     few_rows = (ops.PackedLinear.usable(x, self.width, self.width) and
                 ops.PackedLinear.usable(x, self.width, 2 * self.head_dim))
     if few_rows:
@@ -365,8 +375,6 @@ class LocalAttentionBlock(nn.Module):
     q = q.reshape(b, t, self.num_heads, self.head_dim)
     k = k.reshape(b, t, 1, self.head_dim)
     v = v.reshape(b, t, 1, self.head_dim)
-    if self._inv_freq is None or self._inv_freq.device != x.device:
-      self._inv_freq = _inv_frequencies(self.head_dim, x.device)
     # rotary embedding of queries and keys (modules.py:431-432), one kernel
     q, k = ops.rope_pair(q, k, segment_pos, self._inv_freq)
 
@@ -445,6 +453,29 @@ class LocalAttentionBlock(nn.Module):
     k_pos = torch.where(now < n, now, now - w)
     q_pos = torch.arange(t, device=n.device)[None] + n
     return k_pos, q_pos
+
+  def _decode_step_fused(self, x, segment_pos, cache, return_cache,
+                         defer_out=False):
+    """One new token (bf16, head_dim 256) in three launches: the three
+    projections as one pass over their weights, then rotary embedding, scores
+    against the ring as it lies, mask, softmax, values, the new token's own
+    share, ring update and token count as one call that reads the ring once
+    (rg_attention_decode_fused), then proj_final.  Roundings as in
+    _decode_step, except that the probabilities enter the second product
+    unnormalised."""
+    b = x.shape[0]
+    if cache.num_tokens.dtype != torch.int32:
+      raise TypeError("AttentionBlockCache.num_tokens must be int32")
+    qkv = self._rows_qkv(
+        x, (self.proj_q.weight, self.proj_k.weight, self.proj_v.weight))
+    qkv = qkv.reshape(b, self.width + 2 * self.head_dim)
+    out = ops.attention_decode_fused(
+        qkv[:, :self.width], qkv[:, self.width:self.width + self.head_dim],
+        qkv[:, self.width + self.head_dim:], segment_pos, self._inv_freq,
+        cache.keys, cache.values, cache.num_tokens, self.head_dim ** -0.5,
+        update_cache=return_cache)
+    out = self._project_out(out.reshape(b, 1, self.width), defer_out)
+    return out, (cache if return_cache else None)
 
   def _decode_step(self, x, q, k, v, cache, return_cache, defer_out=False):
     """One new token against the ring and itself, without concatenating or

@@ -673,6 +673,76 @@ def attention_decode_finish(from_ring, probs, k_new, v_new, ring_keys,
   return out
 
 
+def attention_decode_fused_supported(x, heads, head_dim, window) -> bool:
+  """Whether attention_decode_fused takes this shape: bf16 on the GPU,
+  head_dim 256, at most 16 heads, a window the chunk table covers."""
+  return (x.is_cuda and x.dtype == torch.bfloat16 and head_dim == 256 and
+          x.shape[0] <= 65535 and
+          _lib.lib().rg_attention_decode_fused_workspace_bytes(
+              x.shape[0], heads, window) > 0)
+
+
+def _rows_view(t, name, width):
+  """[B, width] with unit stride inside a row (rows may lie apart: a slice of
+  a wider projection output): (tensor, row stride in elements)."""
+  if t.dim() != 2 or t.shape[1] != width:
+    raise ValueError(f"{name} must be [B, {width}], got {tuple(t.shape)}")
+  if not t.is_cuda:
+    raise ValueError(f"{name} must live on the GPU")
+  if (t.shape[0] > 1 and t.stride(0) % 8) or t.stride(1) != 1 or (
+      t.data_ptr() % 16):
+    t = t.contiguous()
+  return t, (t.stride(0) if t.shape[0] > 1 else width)
+
+
+def attention_decode_fused(q, k_new, v_new, positions, inv_freq, ring_keys,
+                           ring_values, num_tokens, scale, update_cache=True):
+  """One new token per row against the ring cache and itself
+  (modules.py:431-476): rotary embedding of q and k_new, scores, mask,
+  softmax, values, the new token's share; with update_cache the rotated key
+  and the value go into slot num_tokens % window (in place) and num_tokens is
+  incremented (in place).  q [B, heads * 256], k_new, v_new [B, 256] as the
+  projections left them (slices of one wider output are taken as they lie);
+  positions [B]; ring_* [B, window, 256].  Returns [B, heads, 256]."""
+  B = q.shape[0]
+  hd = 256
+  heads = q.shape[1] // hd
+  window = ring_keys.numel() // (B * hd)
+  q, ldq = _rows_view(q, "q", heads * hd)
+  k_new, ldk = _rows_view(k_new, "k_new", hd)
+  v_new, ldv = _rows_view(v_new, "v_new", hd)
+  _same(q.dtype, q.device, k_new=k_new, v_new=v_new, ring_keys=ring_keys,
+        ring_values=ring_values)
+  for t, name in ((ring_keys, "ring_keys"), (ring_values, "ring_values"),
+                  (num_tokens, "num_tokens")):
+    # updated in place: no silent copies
+    if not (t.is_cuda and t.is_contiguous() and t.data_ptr() % 16 == 0):
+      raise ValueError(f"{name} must be a contiguous, 16-byte aligned GPU "
+                       "tensor (it is updated in place)")
+  assert ring_keys.numel() == B * window * hd == ring_values.numel()
+  assert num_tokens.dtype == torch.int32 and num_tokens.shape == (B,)
+  positions = _dev(positions.reshape(-1), "positions")
+  assert positions.shape == (B,)
+  if positions.dtype not in (torch.int32, torch.int64):
+    raise TypeError("positions must be int32 or int64")
+  inv_freq = _dev(inv_freq, "inv_freq")
+  assert inv_freq.dtype == torch.float32 and inv_freq.numel() == hd // 4
+  lib = _lib.lib()
+  need = lib.rg_attention_decode_fused_workspace_bytes(B, heads, window)
+  if need == 0:
+    raise ValueError(f"unsupported shape heads={heads} window={window}")
+  ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+  out = torch.empty((B, heads, hd), dtype=q.dtype, device=q.device)
+  with _on(q.device):
+    _lib.check(lib.rg_attention_decode_fused(
+        _p(q), ldq, _p(k_new), ldk, _p(v_new), ldv, _p(positions),
+        int(positions.dtype == torch.int64), _p(inv_freq), _p(ring_keys),
+        _p(ring_values), _p(num_tokens), _p(out), _p(ws), need, B, heads, hd,
+        window, float(scale), int(bool(update_cache)), _dtype_code(q),
+        _stream(q)))
+  return out
+
+
 def rglru_backward(dy, x, gx_pre, ga_pre, a_param, reset, y, h0=None,
                    dh_last=None):
   """Gradients of the RG-LRU from its gate pre-activations on (the forward is
@@ -776,8 +846,9 @@ class PackedLinear:
   to or re-pointed; the parameters themselves are passed with every call.
 
   layout 0: `weights` are torch.nn.Linear weights [N_i, K] applied to the same
-    input; several of them (equal N_i) run as one launch and come back as a
-    tuple of outputs.
+    input; several of them run as one launch and come back as a tuple of
+    outputs (equal N_i) or as one output [..., sum N_i] for the caller to
+    slice (unequal N_i, multiples of 32).
   layout 1: one stacked Einsum weight [G, K, E] (layers.py:76-101) with bias
     [G, 1, 1, E]; outputs as a tuple of G tensors, or, with gelu_pair (G = 2),
     gelu(out[0]) * out[1] as one tensor (modules.py:752-757).
@@ -812,9 +883,17 @@ class PackedLinear:
     if self.layout == 0:
       K = w0.shape[1]
       rows = [w.shape[0] for w in weights]
-      if len(set(rows)) != 1 or any(w.shape[1] != K for w in weights):
-        raise ValueError("layers packed together must have equal shapes")
-      groups, N = len(weights), sum(rows)
+      if any(w.shape[1] != K for w in weights):
+        raise ValueError("layers packed together must read the same input")
+      if len(set(rows)) == 1:
+        groups, N = len(weights), sum(rows)
+      else:
+        # unequal layers: one output [..., sum of rows], which the caller
+        # slices (whole 32-row tiles each, so that the tiles stay apart)
+        if any(r % 32 for r in rows):
+          raise ValueError("unequal layers packed together need row counts "
+                           "that are multiples of 32")
+        groups, N = 1, sum(rows)
     else:
       assert len(weights) == 1
       groups, K, E = w0.shape

@@ -94,3 +94,106 @@ def test_attention_prefill_refuses_other_shapes():
   with pytest.raises(Exception):
     ops.attention_prefill(q, q[:, :, :1], q[:, :, :1],
                           torch.zeros(1, 8, dtype=torch.int32, device=DEV), 1.0)
+
+
+# ------------------------------------------------ one decoded token --------
+
+
+def _decode_case(B, heads, window, tokens_seen, seed, ld=None):
+  hd = 256
+  g = torch.Generator().manual_seed(seed)
+  width = (heads + 2) * hd if ld is None else ld
+  qkv = (torch.randn(B, width, generator=g) * 1.2).to(torch.bfloat16).to(DEV)
+  ring_k = (torch.randn(B, window, hd, generator=g) * 1.2).to(torch.bfloat16)
+  ring_v = torch.randn(B, window, hd, generator=g).to(torch.bfloat16)
+  nt = torch.tensor(tokens_seen, dtype=torch.int32)
+  assert nt.shape == (B,)
+  pos = (nt + 3).to(torch.int64)
+  return qkv, ring_k.to(DEV), ring_v.to(DEV), nt.to(DEV), pos.to(DEV)
+
+
+def _decode_separate_calls(qkv, heads, ring_k, ring_v, nt, pos, inv_freq, scale):
+  """The same step as the block ran it before: rotary embedding, a batched
+  product, the softmax kernel, a second product, the finishing kernel."""
+  B, hd = qkv.shape[0], 256
+  window = ring_k.shape[1]
+  q = qkv[:, :heads * hd].reshape(B, 1, heads, hd).contiguous()
+  k = qkv[:, heads * hd:(heads + 1) * hd].reshape(B, 1, 1, hd).contiguous()
+  v = qkv[:, (heads + 1) * hd:(heads + 2) * hd].contiguous()
+  q, k = ops.rope_pair(q, k, pos.reshape(B, 1), inv_freq)
+  qh = q[:, 0]
+  scores = torch.bmm(qh, ring_k.transpose(1, 2))
+  probs = ops.attention_decode_probs(scores, qh, k[:, 0, 0], nt, scale)
+  from_ring = torch.bmm(probs[..., :window], ring_v)
+  return ops.attention_decode_finish(from_ring, probs, k[:, 0, 0], v, ring_k,
+                                     ring_v, nt, update_cache=True)
+
+
+@pytest.mark.parametrize("B,heads,window,tokens_seen", [
+    (4, 10, 2048, [2048, 5000, 2047, 300]),  # the usual window: wrapped or not
+    (5, 10, 512, [0, 1, 15, 16, 17]),        # an empty ring, first passes
+    (3, 16, 256, [255, 256, 257]),           # one chunk, sixteen heads
+    (2, 1, 300, [299, 301]),                 # a window that is no multiple
+    (3, 3, 1024, [64, 65, 700]),             # waves and chunks without a slot
+    (2, 2, 16, [3, 40]),                     # a window shorter than a pass
+])
+def test_attention_decode_fused(B, heads, window, tokens_seen):
+  """rg_attention_decode_fused against the separate calls (same roundings up
+  to the unnormalised probabilities of a streaming softmax) and against the
+  reference's op sequence in float32 tensor ops."""
+  hd = 256
+  scale = hd ** -0.5
+  qkv, ring_k, ring_v, nt, pos = _decode_case(B, heads, window, tokens_seen,
+                                              seed=B * 100 + window)
+  freq = torch.arange(hd // 4, device=DEV)
+  inv_freq = 1.0 / (10000 ** (2 * freq / (hd // 2)))
+  assert ops.attention_decode_fused_supported(qkv, heads, hd, window)
+  rk1, rv1, nt1 = ring_k.clone(), ring_v.clone(), nt.clone()
+  want = _decode_separate_calls(qkv, heads, rk1, rv1, nt1, pos, inv_freq, scale)
+  rk2, rv2, nt2 = ring_k.clone(), ring_v.clone(), nt.clone()
+  print("[case] decode attention", B, heads, window, tokens_seen, flush=True)
+  got = ops.attention_decode_fused(
+      qkv[:, :heads * hd], qkv[:, heads * hd:(heads + 1) * hd],
+      qkv[:, (heads + 1) * hd:], pos, inv_freq, rk2, rv2, nt2, scale)
+  torch.cuda.synchronize()
+  assert got.shape == (B, heads, hd) and got.dtype == torch.bfloat16
+  # the ring and the count: bit for bit
+  assert torch.equal(nt2, nt1) and torch.equal(nt2, nt + 1)
+  assert torch.equal(rk2, rk1) and torch.equal(rv2, rv1)
+  helpers.assert_close_elementwise(got, want, what="out", rtol=2e-2,
+                                   atol_of_max=1e-2)
+  # float32 tensor ops on the same values (the rotated q and k of the
+  # separate calls; scores rounded as the reference's bf16 product is)
+  q = qkv[:, :heads * hd].reshape(B, 1, heads, hd).contiguous()
+  k = qkv[:, heads * hd:(heads + 1) * hd].reshape(B, 1, 1, hd).contiguous()
+  v = qkv[:, (heads + 1) * hd:].float()
+  q, k = ops.rope_pair(q, k, pos.reshape(B, 1), inv_freq)
+  keys = torch.cat([ring_k.float(), k[:, 0].float()], dim=1)     # [B, w+1, hd]
+  vals = torch.cat([ring_v.float(), v[:, None]], dim=1)
+  logits = torch.einsum("bhd,bsd->bhs", q[:, 0].float(), keys)
+  logits = (logits.bfloat16().float() * scale).bfloat16().float()
+  slot = torch.arange(window, device=DEV)[None]
+  seen = (nt[:, None] >= window) | (slot < nt[:, None])
+  seen = torch.cat([seen, torch.ones_like(seen[:, :1])], dim=1)
+  logits = torch.where(seen[:, None], logits, float("-inf"))
+  ref = torch.einsum("bhs,bsd->bhd", torch.softmax(logits, dim=-1), vals)
+  helpers.assert_close_elementwise(got, ref, what="out vs float32", rtol=2e-2,
+                                   atol_of_max=1e-2)
+  # without the update nothing but the output is written
+  rk3, rv3, nt3 = ring_k.clone(), ring_v.clone(), nt.clone()
+  again = ops.attention_decode_fused(
+      qkv[:, :heads * hd].contiguous(),
+      qkv[:, heads * hd:(heads + 1) * hd].contiguous(),
+      qkv[:, (heads + 1) * hd:].contiguous(), pos.to(torch.int32), inv_freq,
+      rk3, rv3, nt3, scale, update_cache=False)
+  assert torch.equal(again, got)
+  assert torch.equal(rk3, ring_k) and torch.equal(rv3, ring_v)
+  assert torch.equal(nt3, nt)
+
+
+def test_attention_decode_fused_refuses_what_it_cannot_run():
+  x = torch.zeros(2, 12 * 256, dtype=torch.bfloat16, device=DEV)
+  assert not ops.attention_decode_fused_supported(x, 17, 256, 2048)
+  assert not ops.attention_decode_fused_supported(x, 10, 128, 2048)
+  assert not ops.attention_decode_fused_supported(x, 10, 256, 16385)
+  assert not ops.attention_decode_fused_supported(x.float(), 10, 256, 2048)

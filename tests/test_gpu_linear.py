@@ -106,8 +106,14 @@ def test_layers_packed_together():
   assert len(both) == 2
   assert torch.equal(both[0], ops.PackedLinear()(x, (w1,), (b1,)))
   assert torch.equal(both[1], ops.PackedLinear()(x, (w2,), (b2,)))
+  # unequal layers: one output, each slice the layer run alone
+  joined = ops.PackedLinear()(x, (w1, w2[:64], w2[64:320]),
+                              (b1, b2[:64], b2[64:320]))
+  assert joined.shape == (M, N + 320)
+  assert torch.equal(joined[:, :N], both[0])
+  assert torch.equal(joined[:, N:], both[1][:, :320])
   with pytest.raises(ValueError):
-    ops.PackedLinear()(x, (w1, w2[:64]), (b1, b2[:64]))
+    ops.PackedLinear()(x, (w1, w2[:40]), (b1, b2[:40]))
 
 
 @pytest.mark.parametrize("M,K,E", [(64, 2560, 7680), (3, 128, 96)])
