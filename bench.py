@@ -300,7 +300,9 @@ def run_griffin(args, torch, rg, wl):
                             "as a captured HIP graph")
                          + "), recurrent blocks: "
                          "rg_recurrent_prefill_gelu_mul (prompt) + "
-                         "rg_recurrent_step_gelu_mul (step); linear "
+                         "rg_recurrent_step_gelu_mul (step); attention "
+                         "blocks: rg_attention_prefill (prompt) + "
+                         "rg_attention_decode_fused (step); linear "
                          "layers of a decode step: rg_linear_rows"},
       "prompt_pass": {"ms": t_prompt * 1e3,
                       "tokens_per_s": B * T / t_prompt},
