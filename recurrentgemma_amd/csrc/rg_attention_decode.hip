@@ -111,6 +111,44 @@ attn_decode_chunks_kernel(AttnDecodeArgs p) {
     return;
   }
 
+  unsigned char* const ktile = lds + kQBytes + wave * kWaveBytes;
+  unsigned char* const vtile = ktile + kTileBytes;
+  const int wave_first = slot_first + wave * kWaveSlots;
+  // passes with a visible slot (wave-uniform)
+  int npass = (visible_end - wave_first + kPass - 1) / kPass;
+  npass = npass < 0 ? 0 : (npass > kPasses ? kPasses : npass);
+
+  // rows of the ring beyond the window read as zero (and are masked)
+  const uint32_t ring_bytes = (uint32_t)p.window * (kHd * 2);
+  const __amdgpu_buffer_rsrc_t rk =
+      make_rsrc(p.ring_k + (int64_t)b * p.window * kHd, ring_bytes);
+  const __amdgpu_buffer_rsrc_t rv =
+      make_rsrc(p.ring_v + (int64_t)b * p.window * kHd, ring_bytes);
+  // a load instruction covers two rows: lane -> row lane / 32, 16-byte piece
+  // lane % 32
+  const uint32_t lane_bytes = (uint32_t)(lane >> 5) * (kHd * 2) + 16u * (lane & 31);
+  const uint32_t lane_lds = (uint32_t)(lane >> 5) * kRowBytes + 16u * (lane & 31);
+  u32x4 kreg[8], vreg[8];
+  auto request = [&](const __amdgpu_buffer_rsrc_t& r, u32x4 (&dst)[8], int pass) {
+    const uint32_t row0 = (uint32_t)(wave_first + pass * kPass);
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      dst[i] = __builtin_amdgcn_raw_buffer_load_b128(
+          r, lane_bytes, (row0 + 2 * i) * (kHd * 2), 0);
+  };
+  auto to_tile = [&](unsigned char* tile, const u32x4 (&src)[8]) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      *reinterpret_cast<u32x4*>(tile + lane_lds + 2 * i * kRowBytes) = src[i];
+  };
+
+  // the first pass's keys and values are on their way while the queries are
+  // rotated
+  if (npass > 0) {
+    request(rk, kreg, 0);
+    request(rv, vreg, 0);
+  }
+
   // ---- queries after the rotary embedding, 16 head rows (zeros past heads)
   {
     const uint16_t* qrow = p.q + (int64_t)b * p.ldq;
@@ -152,46 +190,11 @@ attn_decode_chunks_kernel(AttnDecodeArgs p) {
     qf[ks].u = *reinterpret_cast<const u32x4*>(lds + head * kRowBytes +
                                                2 * (32 * ks + 8 * quad));
 
-  unsigned char* const ktile = lds + kQBytes + wave * kWaveBytes;
-  unsigned char* const vtile = ktile + kTileBytes;
-  const int wave_first = slot_first + wave * kWaveSlots;
-  // passes with a visible slot (wave-uniform)
-  int npass = (visible_end - wave_first + kPass - 1) / kPass;
-  npass = npass < 0 ? 0 : (npass > kPasses ? kPasses : npass);
-
-  // rows of the ring beyond the window read as zero (and are masked)
-  const uint32_t ring_bytes = (uint32_t)p.window * (kHd * 2);
-  const __amdgpu_buffer_rsrc_t rk =
-      make_rsrc(p.ring_k + (int64_t)b * p.window * kHd, ring_bytes);
-  const __amdgpu_buffer_rsrc_t rv =
-      make_rsrc(p.ring_v + (int64_t)b * p.window * kHd, ring_bytes);
-  // a load instruction covers two rows: lane -> row lane / 32, 16-byte piece
-  // lane % 32
-  const uint32_t lane_bytes = (uint32_t)(lane >> 5) * (kHd * 2) + 16u * (lane & 31);
-  const uint32_t lane_lds = (uint32_t)(lane >> 5) * kRowBytes + 16u * (lane & 31);
-  u32x4 kreg[8], vreg[8];
-  auto request = [&](const __amdgpu_buffer_rsrc_t& r, u32x4 (&dst)[8], int pass) {
-    const uint32_t row0 = (uint32_t)(wave_first + pass * kPass);
-#pragma unroll
-    for (int i = 0; i < 8; ++i)
-      dst[i] = __builtin_amdgcn_raw_buffer_load_b128(
-          r, lane_bytes, (row0 + 2 * i) * (kHd * 2), 0);
-  };
-  auto to_tile = [&](unsigned char* tile, const u32x4 (&src)[8]) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i)
-      *reinterpret_cast<u32x4*>(tile + lane_lds + 2 * i * kRowBytes) = src[i];
-  };
-
   f32x4 o[16];  // O^T: rows 16 blk + 4 quad + r (head dimension), column head
 #pragma unroll
   for (int blk = 0; blk < 16; ++blk) o[blk] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
   float m_run = kNegInf, l_run = 0.0f;
 
-  if (npass > 0) {
-    request(rk, kreg, 0);
-    request(rv, vreg, 0);
-  }
   for (int pass = 0; pass < npass; ++pass) {
     wave_lds_sync();  // the previous pass has read both tiles
     to_tile(ktile, kreg);
