@@ -611,10 +611,16 @@ __device__ __forceinline__ void prefill_body(const FusedArgs& p,
       if (general) {
         // (kept a branch: as selects it would cost the common case 3.5 vector
         // instructions per element)
-        asm volatile("");
-        const int row = blk * 32 + 8 * g + (upper ? 4 : 0);
+        // (the lane's row offset passes through an empty statement here so
+        // that what is computed from it -- the shifted mask, four token
+        // numbers -- stays inside the branch: hoisted above it, as the
+        // compiler does otherwise, it is five vector instructions per run on
+        // the path that needs none of them)
+        int half_rows = upper ? 4 : 0;
+        asm volatile("" : "+v"(half_rows));
+        const int row = blk * 32 + 8 * g + half_rows;
         const uint32_t starts = (uint32_t)(m_tile >> row) & 0xfu;
-        const int t_run = t_blk + 8 * g + (upper ? 4 : 0);
+        const int t_run = t_blk + 8 * g + half_rows;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           av[q] = ((starts >> q) & 1u) ? 0.0f : av[q];

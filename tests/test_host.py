@@ -138,6 +138,26 @@ def test_c_side_validation_without_launch():
   rc = lib.rg_recurrent_step_gelu_mul(ok, None, ok, 1, ok, ok, ok, ok, ok, ok,
                                       ok, ok, ok, ok, two, 4, 512, 2, 1, None)
   assert rc == -1 and b"gate_branch is null" in lib.rg_last_error()
+  # one decoded token of the attention block: shapes, strides, workspace
+  assert lib.rg_attention_decode_fused_workspace_bytes(64, 10, 2048) == (
+      64 * 8 * 10 * 258 * 4)
+  assert lib.rg_attention_decode_fused_workspace_bytes(2, 17, 2048) == 0
+  assert lib.rg_attention_decode_fused_workspace_bytes(2, 10, 16385) == 0
+  assert lib.rg_attention_decode_fused_workspace_bytes(2, 1, 300) == (
+      2 * 2 * 1 * 258 * 4)
+
+  def decode(ldq=3072, hd=256, dtype=1, ws=ok, ws_bytes=1 << 30, heads=10):
+    return lib.rg_attention_decode_fused(
+        ok, ldq, ok, 3072, ok, 3072, ok, 1, ok, ok, ok, ok, ok, ws, ws_bytes, 4,
+        heads, hd, 2048, 0.0625, 1, dtype, None)
+
+  assert decode(hd=128) == -2 and b"head_dim 256" in lib.rg_last_error()
+  assert decode(dtype=0) == -2
+  assert decode(heads=17) == -2
+  assert decode(ldq=2559) == -1 and b"row strides" in lib.rg_last_error()
+  assert decode(ldq=2564) == -1
+  assert decode(ws=None) == -4 and b"workspace" in lib.rg_last_error()
+  assert decode(ws_bytes=1000) == -4
   # rg_recurrent_core: nothing for whole rows in the single kernel, the chunk
   # summaries for rows in chunks, both gates' pre-activations (+ the scan's
   # chunk summaries) for the two-kernel form
