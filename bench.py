@@ -25,6 +25,9 @@ Workloads (the benchmark configurations this build is measured on):
               21 MB, i.e. cache resident: warm-cache figures)
   2b_attention_prompt  prompt-pass attention of one local-attention block of
               the 2B model (B64 T2047, 10 query heads, head_dim 256)
+  2b_attention_decode  one decoded token of that block against a full ring
+              cache (B64, window 2048): rg_attention_decode_fused, with the
+              separate calls it replaces timed after it
   9b_decode   B256 W4096 H16 bf16, one token per row and step with the caches
               carried in place (rg_recurrent_step); `roofline` then describes
               the whole step (all its launches) against its algorithmic bytes
@@ -72,6 +75,9 @@ WORKLOADS = {
     # heads on one key/value head, head_dim 256, window 2048
     "2b_attention_prompt": dict(B=64, T=2047, H=10, window=2048, seed=1007,
                                 attention=True),
+    # ... and one decoded token of it: every ring slot written
+    "2b_attention_decode": dict(B=64, H=10, window=2048, seed=1008,
+                                attention_step=True),
 }
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (scaled
@@ -246,6 +252,81 @@ def run_attention(args, torch, ops, wl):
                    "frac": achieved / 2500.0, "traffic": None,
                    "algorithmic_flops": flops, "avg_launch_ms": ms},
       "library_attention": {"what": "torch SDPA, is_causal", "ms": lib_ms}}))
+
+
+def run_attention_step(args, torch, ops, wl):
+  """rg_attention_decode_fused on one block's decode step (projections in,
+  block output before proj_final out; ring and count updated in place), then
+  the separate calls it replaces.  Algorithmic bytes: both rings once, the
+  projections, the output, the written slot."""
+  dev = torch.device("cuda:0")
+  B, H, hd, window = wl["B"], wl["H"], 256, wl["window"]
+  g = torch.Generator().manual_seed(wl["seed"])
+  qkv = torch.randn(B, (H + 2) * hd, generator=g).to(torch.bfloat16).to(dev)
+  ring_k = torch.randn(B, window, hd, generator=g).to(torch.bfloat16).to(dev)
+  ring_v = torch.randn(B, window, hd, generator=g).to(torch.bfloat16).to(dev)
+  nt = torch.full((B,), window + 17, dtype=torch.int32, device=dev)
+  pos = nt.to(torch.int64)
+  freq = torch.arange(hd // 4, device=dev)
+  inv_freq = 1.0 / (10000 ** (2 * freq / (hd // 2)))
+  scale = hd ** -0.5
+  q, k, v = (qkv[:, :H * hd], qkv[:, H * hd:(H + 1) * hd],
+             qkv[:, (H + 1) * hd:])
+
+  def timed(fn, steps, warmup):
+    for _ in range(warmup):
+      fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+      fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps, e0.elapsed_time(e1) / steps
+
+  def fused():
+    return ops.attention_decode_fused(q, k, v, pos, inv_freq, ring_k, ring_v,
+                                      nt, scale)
+
+  def separate():
+    q4 = q.reshape(B, 1, H, hd).contiguous()
+    k4 = k.reshape(B, 1, 1, hd).contiguous()
+    qr, kr = ops.rope_pair(q4, k4, pos.reshape(B, 1), inv_freq)
+    qh = qr[:, 0]
+    scores = torch.bmm(qh, ring_k.transpose(1, 2))
+    probs = ops.attention_decode_probs(scores, qh, kr[:, 0, 0], nt, scale)
+    from_ring = torch.bmm(probs[..., :window], ring_v)
+    return ops.attention_decode_finish(from_ring, probs, kr[:, 0, 0],
+                                       v.contiguous(), ring_k, ring_v, nt,
+                                       update_cache=True)
+
+  wall, ms = timed(fused, args.steps, args.warmup)
+  _, sep_ms = timed(separate, max(3, args.steps // 2), 2)
+  nbytes = (2 * B * window * hd * 2 + B * (H + 2) * hd * 2 + B * H * hd * 2 +
+            2 * B * hd * 2)
+  achieved = nbytes / (ms * 1e-3) / 1e9
+  print(json.dumps({
+      "metric": "decode-step attention of one local-attention block, tokens/s",
+      "value": B / wall, "unit": "tokens/s", "n_gpus": 1,
+      "steps": args.steps, "warmup": args.warmup, "ms_per_step": wall * 1e3,
+      "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+      "dtype": "bf16", "data": "synthetic",
+      "config": {"workload": args.workload, "batch": B, "query_heads": H,
+                 "kv_heads": 1, "head_dim": hd, "window": window,
+                 "path": "rg_attention_decode_fused, launched from Python "
+                         "(two kernels per step)"},
+      "roofline": {"kernel": "attn_decode_chunks_kernel + "
+                             "attn_decode_combine_kernel (avg_launch_ms covers "
+                             "both)",
+                   "bound": "hbm", "achieved": achieved, "peak": 8000.0,
+                   "unit": "GB/s", "frac": achieved / 8000.0, "traffic": None,
+                   "algorithmic_bytes": nbytes, "avg_launch_ms": ms},
+      "separate_calls": {"what": "rg_rope_pair, torch.bmm, "
+                                 "rg_attention_decode_probs, torch.bmm, "
+                                 "rg_attention_decode_finish", "ms": sep_ms}}))
 
 
 def run_griffin(args, torch, rg, wl):
@@ -456,6 +537,9 @@ def main():
     return
   if wl.get("attention"):
     run_attention(args, torch, ops, wl)
+    return
+  if wl.get("attention_step"):
+    run_attention_step(args, torch, ops, wl)
     return
   result = run_prefill(args, torch, rg, R, ops, args.workload, args.steps,
                        args.warmup, extras=True)

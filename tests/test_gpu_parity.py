@@ -354,6 +354,14 @@ def test_rglru_alone_every_route(dtype, B, T, W, H, mean_doc, with_h0):
   assert helpers.max_rel(y, y2) < tol and helpers.max_rel(h, h2) < tol
   y_nc, none = lru(_dev(x), _dev(seg), _dev(h0), return_cache=False)
   assert none is None and torch.equal(y_nc, y)
+  # the join with a gate branch works without conv weights too: the same
+  # values as the separate pass, bit for bit
+  gb = torch.randn(B, T, W, generator=g).to(dtype)
+  yj, hj, none = ops.recurrent_core(
+      _dev(x), _dev(seg), None, None, *[_dev(t) for t in prm[1:]],
+      _dev(prm[0]), h0=_dev(h0), gate_branch=_dev(gb))
+  assert none is None and torch.equal(hj, h)
+  assert torch.equal(yj, ops.gelu_mul(y, _dev(gb)))
 
 
 # ------------------------------------------------- fused conv -> rg_lru ----
