@@ -135,6 +135,7 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
   const int64_t M = p.M;
   const int64_t W = p.W;
   const int T_len = p.T;
+  const int bw = p.bw;  // 8 .. 256, a multiple of 8 (the launcher checks)
   const int64_t ntiles = (M + kTM - 1) / kTM;
 
   // ---- this wave's weight slice, resident in registers -----------------
@@ -149,12 +150,16 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
   for (int g = 0; g < (ONE ? 1 : 2); ++g) {
 #pragma unroll
     for (int kh = 0; kh < 2; ++kh) {
+      // (a head narrower than the 256 x 256 tile -- bw a multiple of 8 --
+      // is padded with zeros: rows and columns from bw on)
       const uint16_t* src =
-          (const uint16_t*)p.w[g] + ((int64_t)h * kBW + kh * 128) * kBW;
+          (const uint16_t*)p.w[g] + ((int64_t)h * bw + kh * 128) * bw;
       for (int e = tid; e < 128 * 32; e += 512) {
         const int r = e >> 5, q = e & 31;
-        *reinterpret_cast<f32x4*>(lds + (size_t)r * kLdsStride + q * 8) =
-            *reinterpret_cast<const f32x4*>(src + (size_t)r * kBW + q * 8);
+        f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (kh * 128 + r < bw && q * 8 < bw)
+          v = *reinterpret_cast<const f32x4*>(src + (size_t)r * bw + q * 8);
+        *reinterpret_cast<f32x4*>(lds + (size_t)r * kLdsStride + q * 8) = v;
       }
       __syncthreads();
       if (gate == g) {
@@ -179,16 +184,21 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
   // as 64 floats (one 16-byte read per quad).
   float* const bias_lds =
       reinterpret_cast<float*>(lds_raw + kBiasLdsOffset) + wave * 64;
-  bias_lds[lane] = bf16_bits_to_f32(
-      ((const uint16_t*)p.b[gate])[h * kBW + n0 + lane]);
+  bias_lds[lane] =
+      n0 + lane < bw
+          ? bf16_bits_to_f32(((const uint16_t*)p.b[gate])[h * bw + n0 + lane])
+          : 0.0f;
   const float* const bias_r = bias_lds + 4 * (lane >> 5);
   // Output addressing: a wave-uniform tile pointer plus this 32-bit lane
   // offset.  Lane l stores the 16-byte chunk l%8 of rows l/8, l/8+8, ... of
   // the wave's 32 x 64 block.
   const uint32_t out_row_bytes = 2u * (uint32_t)p.W;
+  // (a chunk of columns from bw on belongs to the next head: never stored)
   const uint32_t out_lane_bytes =
-      (uint32_t)(lane >> 3) * out_row_bytes + 2u * (h * kBW + n0) +
-      16u * (lane & 7);
+      n0 + 8 * (lane & 7) < bw
+          ? (uint32_t)(lane >> 3) * out_row_bytes + 2u * (h * bw + n0) +
+                16u * (lane & 7)
+          : kBufferOutOfRange;
   unsigned char* const epi =
       lds_raw + kStageLdsBytes + (size_t)wave * kEpiBytesPerWave;
   // write side: x row lane%32, channels 4*(lane/32) + 8*g (+ 32)
@@ -200,14 +210,17 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
   // ---- x staging: thread -> (channel pair, group of 16 rows) -----------
   const int cp = tid & 127;
   const int rg = __builtin_amdgcn_readfirstlane(tid >> 7);
-  const uint32_t c = h * kBW + cp * 2;  // lane offset inside a row of x
-  const uint32_t c_bytes = 2u * c;
+  const uint32_t c = h * bw + cp * 2;  // lane offset inside a row of x
+  const bool c_valid = cp * 2 < bw;    // else: the tile's zero padding
+  // (out of range by itself and together with an out-of-range scalar offset:
+  // the sum of two kBufferOutOfRange would wrap around to a valid address)
+  const uint32_t c_bytes = c_valid ? 2u * c : kBufferOutOfRange / 2;
   const uint16_t* const xbase = (const uint16_t*)p.x;
   const uint32_t x_row_bytes = 2u * (uint32_t)p.W;
   constexpr int kHalo = CONV ? 3 : 0;
   constexpr int kRaw = kRowsPerGroup + kHalo;
   uint32_t cwp[5] = {0, 0, 0, 0, 0};  // conv w[0..3] and bias, two bf16 each
-  if (CONV) {
+  if (CONV && c_valid) {
     const uint16_t* cw = (const uint16_t*)p.conv_w + c;
     cwp[0] = *reinterpret_cast<const uint32_t*>(cw);
     cwp[1] = *reinterpret_cast<const uint32_t*>(cw + W);
@@ -715,7 +728,10 @@ hipError_t launch_gemm_mfma_f32(const GemmArgs& a, hipStream_t s) {
 }
 
 hipError_t launch_gemm_mfma_bf16(const GemmArgs& a, hipStream_t s) {
-  // needs bw == 256 (checked by the caller); one matrix or both gates
+  // bw <= 256 and a multiple of 8 (narrower heads are padded with zeros
+  // inside the kernel: the caller picks it where that still pays); one matrix
+  // or both gates
+  if (a.bw < 8 || a.bw > kBW || a.bw % 8 != 0) return hipErrorInvalidValue;
   const int64_t ntiles = (a.M + kTM - 1) / kTM;
   int per_head = 256 / a.H;  // about one resident workgroup per CU
   if (per_head < 1) per_head = 1;

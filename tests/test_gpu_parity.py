@@ -135,7 +135,8 @@ def test_conv1d_vs_oracle(dtype, K):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("width,blocks", [(128, 1), (128, 16), (1024, 1),
                                           (1024, 16), (512, 2), (60, 3),
-                                          (2560, 10)])
+                                          (2560, 10), (352, 2), (600, 3),
+                                          (5632, 32)])
 def test_block_diagonal_linear(dtype, width, blocks):
   g = torch.Generator().manual_seed(width + blocks)
   bw = width // blocks
@@ -148,7 +149,8 @@ def test_block_diagonal_linear(dtype, width, blocks):
   m = m.to(DEV)
   tol = F32_TOL if dtype == torch.float32 else BF16_TOL
   cases = [x, x2]
-  if bw == 256:  # the matrix-core kernels: many row tiles, a ragged last one
+  if 128 <= bw <= 256:  # the matrix-core kernels (bf16: narrower heads
+    # padded inside the tile): many row tiles, a ragged last one
     cases.append(torch.randn(5, 1231, width, generator=g).to(dtype))
   for xi in cases:
     _announce("bdl", dtype, width, blocks, tuple(xi.shape))
@@ -491,6 +493,8 @@ def test_config1_fp32_parity():
     (3, 129, 768, 3, 7),      # dense document starts
     (1, 2050, 256, 1, 500),   # long row, many steps
     (2, 33, 384, 6, 5),       # bw 64: generic GEMM
+    (2, 300, 704, 4, 50),     # bw 176 (the paper models' heads): padded MFMA
+    (1, 130, 5632, 32, 40),   # ... at their width
     (2, 3, 256, 1, 2),        # shorter than the conv
     (5, 1, 256, 1, 1),        # single token, every row starts a document
     (2, 64, 130, 1, 16),      # width not a multiple of the slab
