@@ -185,7 +185,13 @@ linear_scan_backward_kernel(ScanBwdArgs p) {
 // nothing but y is kept from the forward pass.  The coefficient of step t is
 // a' of token t+1, which pass 2 has just computed for that token's own gate
 // gradients: it is carried in registers, not loaded again.
-constexpr int kGateBwdRows = 4;
+// Rows of the five streams requested before the first is used: eight where
+// the registers allow (128 per wave at 16 waves), four for float32 with two
+// channels per lane.
+template <typename T, int CH>
+constexpr int gate_bwd_rows() {
+  return sizeof(T) == 4 && CH == 2 ? 4 : 8;
+}
 
 template <typename T, int CH, bool FAST>
 __global__ void __launch_bounds__(kBwdWaves * 64)
@@ -307,6 +313,7 @@ rglru_backward_kernel(RglruBwdArgs p) {
     for (int ch = 0; ch < CH; ++ch)
       a_next[ch] = r ? 0.0f : a_from_gate(sigmoid_of(pav[ch]), ch);
   }
+  constexpr int kGateBwdRows = gate_bwd_rows<T, CH>();
   for (int tb = t1; tb > t0; tb -= kGateBwdRows) {
     float dyv[kGateBwdRows][CH], hp[kGateBwdRows][CH], xv[kGateBwdRows][CH];
     float pxv[kGateBwdRows][CH], pav[kGateBwdRows][CH];
