@@ -191,6 +191,41 @@ def test_attention_decode_fused(B, heads, window, tokens_seen):
   assert torch.equal(nt3, nt)
 
 
+def test_attention_decode_fused_shape_sweep():
+  """Seeded random shapes (heads, window, batch, fill of the ring, row
+  strides) against the separate calls: output within the bf16 bar, ring and
+  count bit for bit."""
+  import random
+  rnd = random.Random(20240917)
+  hd, scale = 256, 256 ** -0.5
+  freq = torch.arange(hd // 4, device=DEV)
+  inv_freq = 1.0 / (10000 ** (2 * freq / (hd // 2)))
+  for case in range(24):
+    heads = rnd.choice([1, 2, 4, 7, 10, 16])
+    window = rnd.choice([8, 40, 256, 257, 600, 1024, 2048, 4096])
+    B = rnd.randint(1, 9)
+    seen = [rnd.choice([0, 1, rnd.randint(0, window), window,
+                        window + rnd.randint(1, 3 * window)]) for _ in range(B)]
+    ld = (heads + 2) * hd + 8 * rnd.randint(0, 5)
+    print("[case] decode attention sweep", case, heads, window, B, seen, ld,
+          flush=True)
+    qkv, ring_k, ring_v, nt, pos = _decode_case(B, heads, window, seen,
+                                                seed=1000 + case, ld=ld)
+    rk1, rv1, nt1 = ring_k.clone(), ring_v.clone(), nt.clone()
+    want = _decode_separate_calls(qkv, heads, rk1, rv1, nt1, pos, inv_freq,
+                                  scale)
+    rk2, rv2, nt2 = ring_k.clone(), ring_v.clone(), nt.clone()
+    got = ops.attention_decode_fused(
+        qkv[:, :heads * hd], qkv[:, heads * hd:(heads + 1) * hd],
+        qkv[:, (heads + 1) * hd:(heads + 2) * hd], pos, inv_freq, rk2, rv2, nt2,
+        scale)
+    torch.cuda.synchronize()
+    assert torch.equal(nt2, nt1) and torch.equal(rk2, rk1)
+    assert torch.equal(rv2, rv1)
+    helpers.assert_close_elementwise(got, want, what=f"out, case {case}",
+                                     rtol=2e-2, atol_of_max=1e-2)
+
+
 def test_attention_decode_fused_refuses_what_it_cannot_run():
   x = torch.zeros(2, 12 * 256, dtype=torch.bfloat16, device=DEV)
   assert not ops.attention_decode_fused_supported(x, 17, 256, 2048)
