@@ -28,6 +28,9 @@ Workloads (the benchmark configurations this build is measured on):
   2b_attention_decode  one decoded token of that block against a full ring
               cache (B64, window 2048): rg_attention_decode_fused, with the
               separate calls it replaces timed after it
+  9b_modules  the drop-in modules called one by one at the 9b_prefill shape:
+              Conv1D, BlockDiagonalLinear (one gate), RGLRU, each with its own
+              algorithmic bytes and HBM fraction
   9b_decode   B256 W4096 H16 bf16, one token per row and step with the caches
               carried in place (rg_recurrent_step); `roofline` then describes
               the whole step (all its launches) against its algorithmic bytes
@@ -75,6 +78,9 @@ WORKLOADS = {
     # heads on one key/value head, head_dim 256, window 2048
     "2b_attention_prompt": dict(B=64, T=2047, H=10, window=2048, seed=1007,
                                 attention=True),
+    # the modules of the path called stand-alone, one after the other
+    "9b_modules": dict(B=16, T=8192, W=4096, H=16, mean_doc=None, seed=1009,
+                       modules=True),
     # ... and one decoded token of it: every ring slot written
     "2b_attention_decode": dict(B=64, H=10, window=2048, seed=1008,
                                 attention_step=True),
@@ -252,6 +258,90 @@ def run_attention(args, torch, ops, wl):
                    "frac": achieved / 2500.0, "traffic": None,
                    "algorithmic_flops": flops, "avg_launch_ms": ms},
       "library_attention": {"what": "torch SDPA, is_causal", "ms": lib_ms}}))
+
+
+def run_modules(args, torch, rg, R, wl):
+  """Conv1D.forward, BlockDiagonalLinear.forward and RGLRU.forward as a caller
+  of the stand-alone modules runs them (recurrentgemma/torch/layers.py:
+  447-529, 127-137, 313-365), one after the other on the same input shape.  A
+  step = the three calls; each module is also timed by itself with HIP
+  events."""
+  dev = torch.device("cuda:0")
+  B, T, W, H = wl["B"], wl["T"], wl["W"], wl["H"]
+  dtype = torch.bfloat16
+  params = R.make_params(W, H, dtype, seed=wl["seed"] + 100)
+  conv = rg.Conv1D(W, 4, dtype=dtype)
+  conv.load_state_dict({"w": params["conv_w"], "b": params["conv_b"]})
+  lru = rg.RGLRU(W, H, dtype=dtype)
+  lru.load_state_dict({"a_param": params["a_param"],
+                       "input_gate.w": params["w_x"],
+                       "input_gate.b": params["b_x"],
+                       "a_gate.w": params["w_a"], "a_gate.b": params["b_a"]})
+  conv, lru = conv.to(dev), lru.to(dev)
+  g = torch.Generator().manual_seed(wl["seed"])
+  x = torch.randn(B, T, W, generator=g).to(dtype).to(dev)
+  seg = make_segment_pos(torch, B, T, wl["mean_doc"], wl["seed"]).to(dev)
+  n = B * T * W
+  calls = [
+      ("Conv1D.forward", "conv1d_prefill_k4_kernel (rg_conv1d_prefill)",
+       lambda: conv(x, seg), 2 * n * 2),
+      ("BlockDiagonalLinear.forward",
+       "gates_mfma_bf16_kernel, one matrix (rg_block_diag_linear)",
+       lambda: lru.input_gate(x), 2 * n * 2),
+      ("RGLRU.forward",
+       "block_prefill_bf16_kernel without conv weights (rg_recurrent_core)",
+       lambda: lru(x, seg), 2 * n * 2),
+  ]
+
+  def events(fn, steps, warmup):
+    for _ in range(warmup):
+      fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+      fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+  def step():
+    for _, _, fn, _ in calls:
+      fn()
+
+  for _ in range(args.warmup):
+    step()
+  torch.cuda.synchronize()
+  t0 = time.perf_counter()
+  for _ in range(args.steps):
+    step()
+  torch.cuda.synchronize()
+  wall = (time.perf_counter() - t0) / args.steps
+  modules = []
+  for name, kernel, fn, nbytes in calls:
+    ms = events(fn, max(5, args.steps // 2), 3)
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    modules.append({"module": name, "kernel": kernel, "ms": ms,
+                    "algorithmic_bytes": nbytes, "achieved_gbs": gbs,
+                    "frac_of_hbm_peak": gbs / 8000.0})
+  worst = max(modules, key=lambda m: m["ms"])
+  print(json.dumps({
+      "metric": "stand-alone Conv1D + BlockDiagonalLinear + RGLRU, tokens/s",
+      "value": B * T / wall, "unit": "tokens/s", "n_gpus": 1,
+      "steps": args.steps, "warmup": args.warmup, "ms_per_step": wall * 1e3,
+      "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+      "dtype": "bf16", "data": "synthetic",
+      "config": {"workload": args.workload, "batch": B, "seq_len": T,
+                 "lru_width": W, "heads": H,
+                 "path": "the drop-in modules called one by one"},
+      "roofline": {"kernel": worst["kernel"], "bound": "hbm",
+                   "achieved": worst["achieved_gbs"], "peak": 8000.0,
+                   "unit": "GB/s", "frac": worst["frac_of_hbm_peak"],
+                   "traffic": None,
+                   "algorithmic_bytes": worst["algorithmic_bytes"],
+                   "avg_launch_ms": worst["ms"]},
+      "modules": modules}))
 
 
 def run_attention_step(args, torch, ops, wl):
@@ -540,6 +630,9 @@ def main():
     return
   if wl.get("attention_step"):
     run_attention_step(args, torch, ops, wl)
+    return
+  if wl.get("modules"):
+    run_modules(args, torch, rg, R, wl)
     return
   result = run_prefill(args, torch, rg, R, ops, args.workload, args.steps,
                        args.warmup, extras=True)

@@ -155,13 +155,32 @@ struct Vec16<uint16_t> {
   }
 };
 
+// Which of the rows around a run (fewer than `span` of them, from `base` on)
+// is the first token of a sequence row: at most one when the sequences are at
+// least `span` tokens long, found once per wave instead of a 64-bit remainder
+// per row.
+struct SeqStarts {
+  int64_t first;  // first row >= base that begins a sequence row
+  int T_len;
+  bool one;       // the sequences are long enough for `first` to be the only one
+  __device__ SeqStarts(int64_t base, int T, int span) : T_len(T), one(T >= span) {
+    const int64_t r = base % T;
+    first = r == 0 ? base : base + (T - r);
+  }
+  __device__ bool at(int64_t m) const {
+    return one ? m == first : m % T_len == 0;
+  }
+};
+
 // row m starts a history: first token of a sequence row, or of a document
 __device__ __forceinline__ bool conv_row_starts(const void* segpos, int seg_kind,
-                                                int T_len, int64_t m) {
-  return m % T_len == 0 || is_doc_start(segpos, seg_kind, m);
+                                                const SeqStarts& seq, int64_t m) {
+  return seq.at(m) || is_doc_start(segpos, seg_kind, m);
 }
 
-template <typename T>
+// RUN rows per wave: the longer, the fewer halo rows are read twice (3 per
+// run) and the fewer workgroups are dispatched.
+template <typename T, int RUN>
 __global__ void __launch_bounds__(64)
 conv1d_prefill_k4_kernel(const T* __restrict__ x, const void* __restrict__ segpos,
                          int seg_kind, const T* __restrict__ w,
@@ -171,8 +190,9 @@ conv1d_prefill_k4_kernel(const T* __restrict__ x, const void* __restrict__ segpo
   constexpr int N = V::N;
   const int c = ((int)blockIdx.y * 64 + (int)threadIdx.x) * N;
   if (c >= W) return;  // W % N == 0 (launcher): a lane is inside or outside
-  const int64_t m0 = (int64_t)blockIdx.x * kConvRun;
-  const int64_t m1 = m0 + kConvRun < M ? m0 + kConvRun : M;
+  const int64_t m0 = (int64_t)blockIdx.x * RUN;
+  const int64_t m1 = m0 + RUN < M ? m0 + RUN : M;
+  const SeqStarts seq(m0 >= 3 ? m0 - 3 : 0, T_len, RUN + 3);
   auto row = [&](const T* base, int64_t m) {
     return *reinterpret_cast<const u32x4*>(base + m * W + c);
   };
@@ -188,7 +208,7 @@ conv1d_prefill_k4_kernel(const T* __restrict__ x, const void* __restrict__ segpo
   for (int e = 0; e < N; ++e) h1[e] = h2[e] = h3[e] = 0.0f;
   for (int64_t j = m0 - 3; j < m0; ++j) {
     if (j < 0) continue;
-    if (conv_row_starts(segpos, seg_kind, T_len, j)) {
+    if (conv_row_starts(segpos, seg_kind, seq, j)) {
 #pragma unroll
       for (int e = 0; e < N; ++e) h1[e] = h2[e] = 0.0f;
     }
@@ -206,7 +226,7 @@ conv1d_prefill_k4_kernel(const T* __restrict__ x, const void* __restrict__ segpo
     for (int u = 0; u < kConvBatch; ++u) {
       const int64_t m = mb + u < m1 ? mb + u : m1 - 1;
       raw[u] = row(x, m);
-      st[u] = conv_row_starts(segpos, seg_kind, T_len, m);
+      st[u] = conv_row_starts(segpos, seg_kind, seq, m);
     }
 #pragma unroll
     for (int u = 0; u < kConvBatch; ++u) {
@@ -248,12 +268,13 @@ conv1d_backward_k4_kernel(const T* __restrict__ dout, const T* __restrict__ x,
   if (c >= W) return;
   const int64_t m0 = (int64_t)blockIdx.x * kConvRun;
   const int64_t m1 = m0 + kConvRun < M ? m0 + kConvRun : M;
+  const SeqStarts seq(m0 >= 3 ? m0 - 3 : 0, T_len, kConvRun + 6);
   auto row = [&](const T* base, int64_t m) {
     return *reinterpret_cast<const u32x4*>(base + m * W + c);
   };
   // a row behind the last one counts as a start (nothing beyond it is used)
   auto starts = [&](int64_t m) {
-    return m >= M || conv_row_starts(segpos, seg_kind, T_len, m);
+    return m >= M || conv_row_starts(segpos, seg_kind, seq, m);
   };
   float w0[N], w1[N], w2[N], w3[N];
   V::unpack(row(w, 0), w0);
@@ -266,7 +287,7 @@ conv1d_backward_k4_kernel(const T* __restrict__ dout, const T* __restrict__ x,
     h1[e] = h2[e] = h3[e] = d0[e] = d1[e] = d2[e] = d3[e] = db[e] = 0.0f;
   for (int64_t j = m0 - 3; j < m0; ++j) {
     if (j < 0) continue;
-    if (conv_row_starts(segpos, seg_kind, T_len, j)) {
+    if (conv_row_starts(segpos, seg_kind, seq, j)) {
 #pragma unroll
       for (int e = 0; e < N; ++e) h1[e] = h2[e] = 0.0f;
     }
@@ -301,7 +322,7 @@ conv1d_backward_k4_kernel(const T* __restrict__ dout, const T* __restrict__ x,
       const int64_t m = mb + u < m1 ? mb + u : m1 - 1;
       xr[u] = row(x, m);
       gr[u] = row(dout, m + 3 < M ? m + 3 : M - 1);
-      st[u] = conv_row_starts(segpos, seg_kind, T_len, m);
+      st[u] = conv_row_starts(segpos, seg_kind, seq, m);
       fa[u] = starts(m + 3);
     }
 #pragma unroll
@@ -414,11 +435,20 @@ hipError_t conv_prefill_t(const ConvArgs& a, hipStream_t s) {
   const int64_t M = (int64_t)a.B * a.T;
   if (conv_k4_fits<T>(a.K, a.W, M)) {
     constexpr int N = 16 / (int)sizeof(T);
-    const dim3 grid((unsigned)((M + kConvRun - 1) / kConvRun),
-                    (unsigned)((a.W / N + 63) / 64));
-    conv1d_prefill_k4_kernel<T><<<grid, 64, 0, s>>>(
-        (const T*)a.x, a.segpos, a.seg_kind, (const T*)a.w, (const T*)a.bias,
-        (T*)a.out, a.T, a.W, M);
+    const unsigned slabs = (unsigned)((a.W / N + 63) / 64);
+    // long runs where that still leaves eight waves for every SIMD
+    constexpr int kLongRun = 128;
+    if ((M / kLongRun) * slabs >= 8192) {
+      const dim3 grid((unsigned)((M + kLongRun - 1) / kLongRun), slabs);
+      conv1d_prefill_k4_kernel<T, kLongRun><<<grid, 64, 0, s>>>(
+          (const T*)a.x, a.segpos, a.seg_kind, (const T*)a.w,
+          (const T*)a.bias, (T*)a.out, a.T, a.W, M);
+    } else {
+      const dim3 grid((unsigned)((M + kConvRun - 1) / kConvRun), slabs);
+      conv1d_prefill_k4_kernel<T, kConvRun><<<grid, 64, 0, s>>>(
+          (const T*)a.x, a.segpos, a.seg_kind, (const T*)a.w,
+          (const T*)a.bias, (T*)a.out, a.T, a.W, M);
+    }
   } else {
     conv1d_prefill_kernel<T><<<grid_for(total, 256), 256, 0, s>>>(
         (const T*)a.x, a.segpos, a.seg_kind, (const T*)a.w,
