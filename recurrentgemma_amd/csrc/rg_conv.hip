@@ -181,14 +181,16 @@ __device__ __forceinline__ bool conv_row_starts(const void* segpos, int seg_kind
 // RUN rows per wave: the longer, the fewer halo rows are read twice (3 per
 // run) and the fewer workgroups are dispatched.
 template <typename T, int RUN>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(1024)
 conv1d_prefill_k4_kernel(const T* __restrict__ x, const void* __restrict__ segpos,
                          int seg_kind, const T* __restrict__ w,
                          const T* __restrict__ bias, T* __restrict__ out,
                          int T_len, int W, int64_t M) {
   using V = Vec16<T>;
   constexpr int N = V::N;
-  const int c = ((int)blockIdx.y * 64 + (int)threadIdx.x) * N;
+  // the waves of a workgroup lie side by side along a row (up to 16 of them:
+  // 16 KB of a row), so that what they request together is contiguous
+  const int c = ((int)blockIdx.y * (int)blockDim.x + (int)threadIdx.x) * N;
   if (c >= W) return;  // W % N == 0 (launcher): a lane is inside or outside
   const int64_t m0 = (int64_t)blockIdx.x * RUN;
   const int64_t m1 = m0 + RUN < M ? m0 + RUN : M;
@@ -436,16 +438,18 @@ hipError_t conv_prefill_t(const ConvArgs& a, hipStream_t s) {
   if (conv_k4_fits<T>(a.K, a.W, M)) {
     constexpr int N = 16 / (int)sizeof(T);
     const unsigned slabs = (unsigned)((a.W / N + 63) / 64);
+    const unsigned waves = slabs < 16 ? slabs : 16;  // per workgroup
+    const unsigned across = (slabs + waves - 1) / waves;
     // long runs where that still leaves eight waves for every SIMD
     constexpr int kLongRun = 128;
     if ((M / kLongRun) * slabs >= 8192) {
-      const dim3 grid((unsigned)((M + kLongRun - 1) / kLongRun), slabs);
-      conv1d_prefill_k4_kernel<T, kLongRun><<<grid, 64, 0, s>>>(
+      const dim3 grid((unsigned)((M + kLongRun - 1) / kLongRun), across);
+      conv1d_prefill_k4_kernel<T, kLongRun><<<grid, waves * 64, 0, s>>>(
           (const T*)a.x, a.segpos, a.seg_kind, (const T*)a.w,
           (const T*)a.bias, (T*)a.out, a.T, a.W, M);
     } else {
-      const dim3 grid((unsigned)((M + kConvRun - 1) / kConvRun), slabs);
-      conv1d_prefill_k4_kernel<T, kConvRun><<<grid, 64, 0, s>>>(
+      const dim3 grid((unsigned)((M + kConvRun - 1) / kConvRun), across);
+      conv1d_prefill_k4_kernel<T, kConvRun><<<grid, waves * 64, 0, s>>>(
           (const T*)a.x, a.segpos, a.seg_kind, (const T*)a.w,
           (const T*)a.bias, (T*)a.out, a.T, a.W, M);
     }
