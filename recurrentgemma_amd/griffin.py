@@ -193,7 +193,8 @@ class MLPBlock(nn.Module):
   def forward(self, x, residual=None, defer_out=False):
     """residual: added to the result (the block's skip connection,
     modules.py:897-898).  defer_out: the caller normalises the result next and
-    accepts it as ops.PartialSums (returned where that saves a pass)."""
+    accepts it as ops.PartialSums or ops.PendingSum (returned where that saves
+    a pass)."""
     if (ops.PackedLinear.usable(x, self.width, 2 * self.expanded_width, True)
         and ops.PackedLinear.usable(x, self.expanded_width, self.width)):
       hidden = self._rows_up(x, (self.ffw_up.w,), (self.ffw_up.b,))
@@ -205,7 +206,10 @@ class MLPBlock(nn.Module):
                              (self.ffw_down.bias,), residual=residual)
     gate, up = self.ffw_up(x)
     out = self.ffw_down(ops.gelu_mul(up, gate))  # gelu(gate) * up, one pass
-    return out if residual is None else out + residual
+    if residual is None:
+      return out
+    # (many rows: the norm that reads the sum next adds the two in its pass)
+    return ops.PendingSum(out, residual) if defer_out else out + residual
 
 
 def _inv_frequencies(head_dim, device, max_wavelength=_MAX_WAVELENGTH):
@@ -561,9 +565,12 @@ class ResidualBlock(nn.Module):
     """x and, with defer_out, the result may be ops.PartialSums: the output of
     the previous block's last layer before its slices of K are added, which
     the norm kernel that reads it next does (Griffin.forward chains the blocks
-    that way for a decode step)."""
+    that way for a decode step) -- or, with many rows, ops.PendingSum: that
+    output and the skip connection before they are added."""
     if isinstance(x, ops.PartialSums):
       x, normed = self.temporal_pre_norm.add_then_norm(x, None)
+    elif isinstance(x, ops.PendingSum):
+      x, normed = self.temporal_pre_norm.add_then_norm(x.a, x.b)
     else:
       normed = self.temporal_pre_norm(x)
     mixed, new_cache = self.temporal_block(normed, segment_pos, cache,
@@ -664,6 +671,8 @@ class Griffin(nn.Module):
       return None, new_cache
     if isinstance(x, ops.PartialSums):
       x = self.final_norm.add_then_norm(x, None)[1]
+    elif isinstance(x, ops.PendingSum):
+      x = self.final_norm.add_then_norm(x.a, x.b)[1]
     else:
       x = self.final_norm(x)
     logits = self.embedder.decode(x)

@@ -839,6 +839,18 @@ class PartialSums:
     return out if self.addend is None else out + self.addend
 
 
+class PendingSum:
+  """a + b, not added yet: the norm kernel that reads the sum next forms it
+  in the same pass (add_rms_norm), which saves the pass of the add."""
+
+  def __init__(self, a, b):
+    assert a.shape == b.shape
+    self.a, self.b = a, b
+
+  def materialize(self):
+    return self.a + self.b
+
+
 class PackedLinear:
   """Linear layers that read the same few rows (a decode step), on the
   weight-streaming kernel (rg_linear_rows).  Holds the weights in the kernel's
