@@ -31,6 +31,9 @@ Workloads (the benchmark configurations this build is measured on):
   9b_modules  the drop-in modules called one by one at the 9b_prefill shape:
               Conv1D, BlockDiagonalLinear (one gate), RGLRU, each with its own
               algorithmic bytes and HBM fraction
+  2b_block_training  RecurrentBlock forward + backward under
+              training.differentiable() (B4 T2048 W2560 H10 bf16), with the
+              backward kernels of the recurrent path timed by themselves
   9b_decode   B256 W4096 H16 bf16, one token per row and step with the caches
               carried in place (rg_recurrent_step); `roofline` then describes
               the whole step (all its launches) against its algorithmic bytes
@@ -78,6 +81,9 @@ WORKLOADS = {
     # heads on one key/value head, head_dim 256, window 2048
     "2b_attention_prompt": dict(B=64, T=2047, H=10, window=2048, seed=1007,
                                 attention=True),
+    # the differentiable path: one block, forward and backward
+    "2b_block_training": dict(B=4, T=2048, W=2560, H=10, mean_doc=512,
+                              seed=1010, training=True),
     # the modules of the path called stand-alone, one after the other
     "9b_modules": dict(B=16, T=8192, W=4096, H=16, mean_doc=None, seed=1009,
                        modules=True),
@@ -258,6 +264,112 @@ def run_attention(args, torch, ops, wl):
                    "frac": achieved / 2500.0, "traffic": None,
                    "algorithmic_flops": flops, "avg_launch_ms": ms},
       "library_attention": {"what": "torch SDPA, is_causal", "ms": lib_ms}}))
+
+
+def run_training(args, torch, rg, ops, wl):
+  """RecurrentBlock.forward and the backward pass through it inside
+  training.differentiable(): conv, gate projections (bf16), RG-LRU gating and
+  recurrence on kernels in both directions, the block's three linear layers
+  as torch autograd.  A step = forward + loss + backward.  The backward
+  kernels of the recurrent path are then timed alone on the same shapes."""
+  from recurrentgemma_amd import training
+  dev = torch.device("cuda:0")
+  B, T, W, H = wl["B"], wl["T"], wl["W"], wl["H"]
+  dtype = torch.bfloat16
+  torch.manual_seed(wl["seed"])
+  blk = rg.RecurrentBlock(width=W, num_heads=H, dtype=dtype).to(dev)
+  g = torch.Generator().manual_seed(wl["seed"])
+  x = torch.randn(B, T, W, generator=g).to(dtype).to(dev).requires_grad_(True)
+  seg = make_segment_pos(torch, B, T, wl["mean_doc"], wl["seed"]).to(dev)
+
+  def step():
+    for p in blk.parameters():
+      p.grad = None
+    x.grad = None
+    with training.differentiable():
+      y, _ = blk(x, seg, return_cache=False)
+      y.float().square().mean().backward()
+
+  for _ in range(args.warmup):
+    step()
+  torch.cuda.synchronize()
+  t0 = time.perf_counter()
+  for _ in range(args.steps):
+    step()
+  torch.cuda.synchronize()
+  wall = (time.perf_counter() - t0) / args.steps
+  with torch.no_grad():
+    for _ in range(3):
+      blk(x, seg, return_cache=False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+      blk(x, seg, return_cache=False)
+    torch.cuda.synchronize()
+    forward_only = (time.perf_counter() - t0) / args.steps
+
+  def events(fn, steps=20, warmup=3):
+    for _ in range(warmup):
+      fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+      fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+  n = B * T * W
+  xc = torch.randn(B, T, W, generator=g).to(dtype).to(dev)
+  gx = torch.randn(B, T, W, generator=g).to(dtype).to(dev)
+  ga = torch.randn(B, T, W, generator=g).to(dtype).to(dev)
+  dy = torch.randn(B, T, W, generator=g).to(dtype).to(dev)
+  lru, conv = blk.rg_lru, blk.conv_1d
+  with torch.no_grad():
+    y, _, _ = ops.lru_scan_fused(xc, gx, ga, lru.a_param, seg)
+    reset = seg == 0
+    a = torch.rand(B, T, W, generator=g).to(dtype).to(dev)
+    kernels = []
+    for name, fn, per_element in (
+        ("rg_rglru_backward", lambda: ops.rglru_backward(
+            dy, xc, gx, ga, lru.a_param, reset, y, None, None), 8),
+        ("rg_linear_scan_backward", lambda: ops.linear_scan_backward(
+            dy, a, reset, y, None, None), 5),
+        ("rg_conv1d_backward (+ the sum of its per-chunk planes)",
+         lambda: ops.conv1d_backward(dy, xc, seg, conv.w), 3),
+        ("rg_gates_gemm (forward of both gate projections)",
+         lambda: ops.gates_gemm(xc, lru.input_gate.w, lru.input_gate.b,
+                                lru.a_gate.w, lru.a_gate.b), 3),
+        ("rg_lru_scan_fused (forward of gating and recurrence)",
+         lambda: ops.lru_scan_fused(xc, gx, ga, lru.a_param, seg), 4)):
+      ms = events(fn)
+      nbytes = per_element * n * 2
+      gbs = nbytes / (ms * 1e-3) / 1e9
+      kernels.append({"call": name, "ms": ms, "algorithmic_bytes": nbytes,
+                      "achieved_gbs": gbs, "frac_of_hbm_peak": gbs / 8000.0})
+  main = kernels[0]
+  print(json.dumps({
+      "metric": "RecurrentBlock forward + backward, tokens/s",
+      "value": B * T / wall, "unit": "tokens/s", "n_gpus": 1,
+      "steps": args.steps, "warmup": args.warmup, "ms_per_step": wall * 1e3,
+      "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+      "dtype": "bf16", "data": "synthetic",
+      "config": {"workload": args.workload, "batch": B, "seq_len": T,
+                 "width": W, "lru_width": W, "heads": H,
+                 "documents": "geometric mean %d" % wl["mean_doc"],
+                 "path": "training.differentiable(): kernels for conv, gate "
+                         "projections, RG-LRU in both directions; linear "
+                         "layers torch autograd"},
+      "forward_only_ms": forward_only * 1e3,
+      "roofline": {"kernel": "rglru_backward_kernel (rg_rglru_backward)",
+                   "bound": "hbm", "achieved": main["achieved_gbs"],
+                   "peak": 8000.0, "unit": "GB/s",
+                   "frac": main["frac_of_hbm_peak"], "traffic": None,
+                   "algorithmic_bytes": main["algorithmic_bytes"],
+                   "avg_launch_ms": main["ms"]},
+      "kernels": kernels}))
 
 
 def run_modules(args, torch, rg, R, wl):
@@ -633,6 +745,9 @@ def main():
     return
   if wl.get("modules"):
     run_modules(args, torch, rg, R, wl)
+    return
+  if wl.get("training"):
+    run_training(args, torch, rg, ops, wl)
     return
   result = run_prefill(args, torch, rg, R, ops, args.workload, args.steps,
                        args.warmup, extras=True)
