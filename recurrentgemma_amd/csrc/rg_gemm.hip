@@ -123,7 +123,9 @@ union Frag {
 // the matrix work; waves 4-7 only take their share of the x staging (the
 // staging loops are laid out for 512 threads), issue no matrix instruction
 // and store through an empty descriptor.
-template <bool CONV, bool ONE = false>
+// NARROW: heads narrower than the tile (bw < 256); the waves whose columns
+// and the k-steps whose rows are all padding issue no matrix instruction.
+template <bool CONV, bool ONE = false, bool NARROW = false>
 __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   uint16_t* lds = reinterpret_cast<uint16_t*>(lds_raw);
@@ -140,7 +142,10 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
 
   // ---- this wave's weight slice, resident in registers -----------------
   const int gate = ONE ? 0 : wave >> 2;  // waves 0-3: input gate, 4-7: a gate
-  const bool active = !ONE || wave < 4;  // wave-uniform
+  // (wave-uniform; n0 and bw come further down)
+  const bool active = (!ONE || wave < 4) &&
+                      (!NARROW || (wave & 3) * 64 < p.bw);
+  const int ksteps = NARROW ? (p.bw + 15) / 16 : 16;  // k-steps with a row < bw
   const int n0 = (wave & 3) * 64;     // first output column inside the gate
   // The weights are [k][n] with n contiguous, the MFMA B operand wants 8
   // consecutive k per lane: transpose through LDS, 128 k-rows of one gate at
@@ -458,7 +463,7 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
 #pragma unroll
         for (int ks = 0; ks < 16; ++ks) {
           if (ks < 14) a[(ks + 2) % 3] = a_read(0, ks + 2);
-          if (active) {
+          if (active && (!NARROW || ks < ksteps)) {
             acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
                 bfrag[ks][0].v, a[ks % 3].v, acc0, 0, 0, 0);
             acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
@@ -477,7 +482,7 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
 #pragma unroll
         for (int ks = 0; ks < 16; ++ks) {
           if (ks < 15) a[(ks + 1) % 3] = a_read(0, ks + 1);
-          if (active) {
+          if (active && (!NARROW || ks < ksteps)) {
             acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
                 bfrag[ks][0].v, a[ks % 3].v, acc0, 0, 0, 0);
             acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
@@ -500,7 +505,7 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
 #pragma unroll
       for (int ks = 0; ks < 16; ++ks) {
         if (ks < 14) a[(ks + 2) % 3] = a_read(1, ks + 2);
-        if (active) {
+        if (active && (!NARROW || ks < ksteps)) {
           acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
               bfrag[ks][0].v, a[ks % 3].v, acc0, 0, 0, 0);
           acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
@@ -738,28 +743,24 @@ hipError_t launch_gemm_mfma_bf16(const GemmArgs& a, hipStream_t s) {
   if (per_head > ntiles) per_head = (int)ntiles;
   if (a.H > 65535) return hipErrorInvalidValue;
   dim3 grid((unsigned)per_head, (unsigned)a.H);
-  hipError_t e;
-  if (a.ngates == 1) {
-    if (a.apply_conv) return hipErrorInvalidValue;
-    static OncePerDevice once;
-    e = set_max_dynamic_lds(
-        once, (const void*)gates_mfma_bf16_kernel<false, true>, kMfmaLdsBytes);
+  if (a.ngates == 1 && a.apply_conv) return hipErrorInvalidValue;
+  auto launch = [&](auto kernel, OncePerDevice& once) {
+    const hipError_t e =
+        set_max_dynamic_lds(once, (const void*)kernel, kMfmaLdsBytes);
     if (e != hipSuccess) return e;
-    gates_mfma_bf16_kernel<false, true><<<grid, 512, kMfmaLdsBytes, s>>>(a);
-  } else if (a.apply_conv) {
-    static OncePerDevice once;
-    e = set_max_dynamic_lds(once, (const void*)gates_mfma_bf16_kernel<true>,
-                            kMfmaLdsBytes);
-    if (e != hipSuccess) return e;
-    gates_mfma_bf16_kernel<true><<<grid, 512, kMfmaLdsBytes, s>>>(a);
-  } else {
-    static OncePerDevice once;
-    e = set_max_dynamic_lds(once, (const void*)gates_mfma_bf16_kernel<false>,
-                            kMfmaLdsBytes);
-    if (e != hipSuccess) return e;
-    gates_mfma_bf16_kernel<false><<<grid, 512, kMfmaLdsBytes, s>>>(a);
-  }
-  return hipGetLastError();
+    kernel<<<grid, 512, kMfmaLdsBytes, s>>>(a);
+    return hipGetLastError();
+  };
+  static OncePerDevice once[6];
+  const bool narrow = a.bw < kBW;
+  if (a.ngates == 1)
+    return narrow ? launch(gates_mfma_bf16_kernel<false, true, true>, once[0])
+                  : launch(gates_mfma_bf16_kernel<false, true, false>, once[1]);
+  if (a.apply_conv)
+    return narrow ? launch(gates_mfma_bf16_kernel<true, false, true>, once[2])
+                  : launch(gates_mfma_bf16_kernel<true, false, false>, once[3]);
+  return narrow ? launch(gates_mfma_bf16_kernel<false, false, true>, once[4])
+                : launch(gates_mfma_bf16_kernel<false, false, false>, once[5]);
 }
 
 }  // namespace rg
