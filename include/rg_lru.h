@@ -282,7 +282,8 @@ int rg_recurrent_prefill_gelu_mul(
  * (recurrentgemma/torch/modules.py:632-643), for every shape and both dtypes,
  * with the choice of kernels made here: the single prefill kernel
  * (rg_recurrent_prefill_split; bf16, 256-wide heads, enough (row, head) pairs
- * or rows long enough to be cut into chunks), else rg_gates_gemm with the conv
+ * or rows long enough to be cut into chunks, but not more than 256 pairs of
+ * fewer than 64 tokens), else rg_gates_gemm with the conv
  * applied on load followed by rg_lru_scan_fused_split, the pre-activations of
  * both gates living in the workspace.  gate_branch (nullable, [B,T,W]): the
  * block's linear_y output; `out` is then rglru(conv1d(x)) * gelu_tanh(

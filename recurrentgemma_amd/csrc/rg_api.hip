@@ -548,7 +548,14 @@ static CorePlan core_plan(int B, int T, int W, int H, int dtype) {
                     (int64_t)T * W * 2 < (int64_t)0x7fffffff;
   const size_t chunk_bytes =
       fits ? rg_recurrent_prefill_split_workspace_bytes(B, T, W, H) : 0;
-  p.single = fits && ((int64_t)B * H >= rg::kPrefillMinGroups || chunk_bytes > 0);
+  // Many short rows are the exception: with more workgroups than CUs each CU
+  // loads a head's 256 KB of gate weights again for every pair it runs, and
+  // below one 64-token tile per row that outweighs the rest (measured, W2560
+  // H10, 640 pairs: T32 54 us against 47 us for gate GEMM + scan, T64 57
+  // against 61; 2560 pairs, T1: 160 against 29).
+  const bool many_short_rows = (int64_t)B * H > 256 && T < 64;
+  p.single = fits && !many_short_rows &&
+             ((int64_t)B * H >= rg::kPrefillMinGroups || chunk_bytes > 0);
   if (p.single) {
     p.split_bytes = chunk_bytes;
   } else {

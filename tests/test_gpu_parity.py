@@ -873,6 +873,8 @@ def test_recurrent_core_picks_single_launch():
     (torch.bfloat16, 70, 130, 512, 2),    # 140 pairs: single kernel, whole rows
     (torch.bfloat16, 1, 2048, 512, 2),    # long rows of few pairs: chunks
     (torch.bfloat16, 2, 65, 384, 3),      # bf16, 128-wide heads
+    (torch.bfloat16, 140, 5, 512, 2),     # 280 pairs of 5 tokens: two kernels
+    (torch.bfloat16, 140, 64, 512, 2),    # ... of 64: single kernel
 ])
 @pytest.mark.parametrize("joined", [False, True])
 def test_recurrent_core_entry_equals_its_parts(dtype, B, T, W, H, joined):
@@ -891,6 +893,7 @@ def test_recurrent_core_entry_equals_its_parts(dtype, B, T, W, H, joined):
                                P["b_x"], P["w_a"], P["b_a"], P["a_param"],
                                h0=h0, gate_branch=gate)
   single = (dtype == torch.bfloat16 and W // H == 256 and
+            not (B * H > 256 and T < 64) and
             (B * H >= 129 or ops.recurrent_prefill_chunked(B, T, W, H)))
   if single:
     chunked = ops.recurrent_prefill_chunked(B, T, W, H)

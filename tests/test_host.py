@@ -168,6 +168,11 @@ def test_c_side_validation_without_launch():
           2 * 512 * 2560 * 4 + lib.rg_scan_split_workspace_bytes(1, 512, 2560))
   assert lib.rg_recurrent_core_workspace_bytes(2, 100, 512, 2, 1) == 2 * 2 * 100 * 512 * 2
   assert lib.rg_recurrent_core_workspace_bytes(2, 100, 512, 3, 1) == 0  # W % H
+  # many short rows: more (row, head) pairs than CUs and less than a tile each
+  # take the two-kernel form (both gates' pre-activations in the workspace)
+  assert lib.rg_recurrent_core_workspace_bytes(256, 1, 4096, 16, 1) == (
+      2 * 256 * 4096 * 2)
+  assert lib.rg_recurrent_core_workspace_bytes(256, 64, 4096, 16, 1) == 0
   rc = lib.rg_recurrent_core(ok, None, ok, 1, ok, ok, ok, ok, ok, ok, None, ok,
                              None, ok, None, None, None, 0, 2, 100, 512, 2, 1,
                              None)
