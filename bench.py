@@ -203,6 +203,54 @@ def cpu_baseline(torch, R, wl, params, seconds_target=20.0):
   }
 
 
+def shader_clock_ghz(torch, iters=2000):
+  """Shader clock right now, from rg_clock_probe: one light wave per compute
+  unit for about 0.2 ms, shader-clock cycles over the constant 100 MHz
+  counter.  A light probe: under the matrix-instruction load of the prefill
+  kernel the clock sits lower than what this reads."""
+  import ctypes
+  from recurrentgemma_amd import _lib
+  out = torch.zeros(3, dtype=torch.int64, device="cuda:0")
+  rc = _lib.lib().rg_clock_probe(
+      ctypes.c_void_p(out.data_ptr()), iters,
+      ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+  if rc != 0:
+    return None
+  torch.cuda.synchronize()
+  cycles, ticks = (int(v) for v in out[:2].cpu())
+  return cycles / (ticks * 10.0) if ticks > 0 else None
+
+
+def settle(torch, fn, cap_s=0.5, window=10, rel=0.01, min_launches=30):
+  """Untimed launches of fn() until the GPU has left its idle clocks: stops
+  when the median duration of the last `window` launches is within `rel` of
+  the median of the `window` before them (at least `min_launches`), or after
+  cap_s seconds.  A launch right after start-up runs up to 20 % longer than
+  the sustained ones (clock ramp), for some tens of launches.  Returns the
+  number of launches made."""
+  e0 = torch.cuda.Event(enable_timing=True)
+  e1 = torch.cuda.Event(enable_timing=True)
+  ms = []
+  t0 = time.perf_counter()
+  med = lambda v: sorted(v)[len(v) // 2]
+  while time.perf_counter() - t0 < cap_s:
+    e0.record()
+    fn()
+    e1.record()
+    e1.synchronize()
+    ms.append(e0.elapsed_time(e1))
+    if len(ms) >= max(min_launches, 2 * window) and len(ms) % window == 0:
+      a, b = med(ms[-2 * window:-window]), med(ms[-window:])
+      if abs(a - b) <= rel * b:
+        break
+  return len(ms)
+
+
+def launch_stats(ms_list):
+  v = sorted(ms_list)
+  return {"min": v[0], "median": v[len(v) // 2], "max": v[-1]}
+
+
 def decode_algorithmic_bytes(B, W, H, esize):
   """One decode step: x in, y out, fp32 state and conv state read and written,
   both gate weight matrices, the per-channel parameters."""
@@ -602,9 +650,10 @@ def run_griffin(args, torch, rg, wl):
   print(json.dumps(result))
 
 
-def run_decode(args, torch, rg, R, ops, wl):
+def run_decode(args, torch, rg, R, ops, wl, cpu_leg=True, name=None):
   """Times rg_recurrent_step (conv step, both gate projections, gate
-  activations, state update) on B rows with the caches updated in place."""
+  activations, state update) on B rows with the caches updated in place.
+  Returns the result line as a dict."""
   B, W, H = wl["B"], wl["W"], wl["H"]
   dev = torch.device("cuda:0")
   dtype = torch.bfloat16
@@ -621,6 +670,7 @@ def run_decode(args, torch, rg, R, ops, wl):
                               P["w_x"], P["b_x"], P["w_a"], P["b_a"],
                               P["a_param"], in_place=True)
 
+  settle_launches = 0 if args.no_settle else settle(torch, step, cap_s=0.2)
   for _ in range(args.warmup):
     step()
   torch.cuda.synchronize()
@@ -649,13 +699,17 @@ def run_decode(args, torch, rg, R, ops, wl):
         step()
     graph.replay()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    e0.record()
-    graph.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    dev_ms = e0.elapsed_time(e1) / args.steps
+    # the graph of K steps replayed a few times: the median replay counts
+    reps = []
+    for _ in range(5):
+      t0 = time.perf_counter()
+      e0.record()
+      graph.replay()
+      e1.record()
+      torch.cuda.synchronize()
+      reps.append((e0.elapsed_time(e1) / args.steps, time.perf_counter() - t0))
+    reps.sort()
+    dev_ms, elapsed = reps[len(reps) // 2]
   algo = decode_algorithmic_bytes(B, W, H, 2)
   achieved = algo / (dev_ms * 1e-3) / 1e9
   result = {
@@ -665,7 +719,7 @@ def run_decode(args, torch, rg, R, ops, wl):
       "ms_per_step": elapsed * 1e3 / args.steps, "higher_is_better": True,
       "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
       "data": "synthetic",
-      "config": {"workload": args.workload, "batch": B, "seq_len": 1,
+      "config": {"workload": name or args.workload, "batch": B, "seq_len": 1,
                  "lru_width": W, "heads": H, "activations": "bf16",
                  "state": "f32",
                  "path": "rg_recurrent_step, caches in place, "
@@ -677,9 +731,11 @@ def run_decode(args, torch, rg, R, ops, wl):
                    "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
                    "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                    "traffic": None, "algorithmic_bytes": algo,
-                   "avg_launch_ms": dev_ms},
+                   "avg_launch_ms": dev_ms,
+                   "settle_launches": settle_launches,
+                   "shader_clock_ghz_after": shader_clock_ghz(torch)},
   }
-  if not args.no_cpu_baseline:
+  if cpu_leg and not args.no_cpu_baseline:
     cores = host_cores()
     torch.set_num_threads(cores)
     xc, cc, hc = x.cpu(), conv_cache.cpu(), h.cpu()
@@ -697,7 +753,7 @@ def run_decode(args, torch, rg, R, ops, wl):
         "sample": (f"oracle/torch_ref.recurrent_core with caches, bf16, {n} "
                    f"decode steps of {B} rows (W={W}, H={H}), mean, torch "
                    f"threads={torch.get_num_threads()}")}
-  print(json.dumps(result))
+  return result
 
 
 def main():
@@ -710,6 +766,10 @@ def main():
   ap.add_argument("--no-cpu-baseline", action="store_true",
                   help="lean run for the profiler: no CPU leg and no "
                        "additional 2B-width measurement")
+  ap.add_argument("--no-settle", action="store_true",
+                  help="skip the untimed settle phase before the warm-up steps "
+                       "(launches until their durations stop moving, at most "
+                       "0.5 s)")
   ap.add_argument("--eager", action="store_true",
                   help="2b_griffin_decode, 9b_decode: launch every kernel of a "
                        "decode step from Python instead of replaying a "
@@ -735,7 +795,7 @@ def main():
     run_griffin(args, torch, rg, wl)
     return
   if wl.get("decode"):
-    run_decode(args, torch, rg, R, ops, wl)
+    print(json.dumps(run_decode(args, torch, rg, R, ops, wl)))
     return
   if wl.get("attention"):
     run_attention(args, torch, ops, wl)
@@ -761,14 +821,33 @@ def main():
         k: r2[k] for k in ("value", "unit", "steps", "warmup", "ms_per_step",
                            "config", "roofline", "gate_gemm",
                            "two_kernel_path") if k in r2}
+    # ... and the other single-block configurations, each a few seconds: the
+    # decode step (steps as one captured graph) and the float32 case, whose
+    # 21 MB stay in the caches (warm and cold figures)
+    saved = args.steps, args.warmup
+    args.steps, args.warmup = 64, 10
+    rd = run_decode(args, torch, rg, R, ops, WORKLOADS["9b_decode"],
+                    cpu_leg=False, name="9b_decode")
+    args.steps, args.warmup = saved
+    result["at_decode"] = {
+        k: rd[k] for k in ("value", "unit", "steps", "warmup", "ms_per_step",
+                           "config", "eager_loop", "roofline") if k in rd}
+    rf = run_prefill(args, torch, rg, R, ops, "2b_f32", 50, 10, extras=False,
+                     cold_too=True)
+    result["at_f32"] = {
+        k: rf[k] for k in ("value", "unit", "steps", "warmup", "ms_per_step",
+                           "dtype", "config", "roofline", "gate_gemm",
+                           "cold_caches") if k in rf}
   print(json.dumps(result))
 
 
-def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
+def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras,
+                cold_too=False):
   """One prefill workload: `warmup` untimed steps, `steps` timed ones; returns
   the result line as a dict; with the default path also the two-kernel form
   of a single-kernel workload, after the timed region.  extras: the
-  calibration copy and the CPU baseline too."""
+  calibration copy and the CPU baseline too; cold_too: for a working set that
+  fits the caches, also the figure with the caches flushed between steps."""
   wl = WORKLOADS[workload]
   B, T, W, H = wl["B"], wl["T"], wl["W"], wl["H"]
   dev = torch.device("cuda:0")
@@ -838,7 +917,9 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
   else:
     step = step_single if path == "single" else step_split
 
-  def timed(fn, steps, warmup):
+  per_launch = {}
+
+  def timed(fn, steps, warmup, key=None):
     for _ in range(warmup):
       fn()
     torch.cuda.synchronize()
@@ -850,11 +931,17 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
       fn(evs[i])
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    first = sum(e[0].elapsed_time(e[1]) for e in evs) / steps
-    second = sum(e[1].elapsed_time(e[2]) for e in evs) / steps
-    return elapsed, first, second
+    a = [e[0].elapsed_time(e[1]) for e in evs]
+    b = [e[1].elapsed_time(e[2]) for e in evs]
+    if key:
+      per_launch[key] = (launch_stats(a), launch_stats(b))
+    return elapsed, sum(a) / steps, sum(b) / steps
 
-  elapsed, first_ms, second_ms = timed(step, steps, warmup)
+  # untimed: until the launch durations stop moving (the clock ramp after
+  # start-up), before the --warmup steps
+  settle_launches = 0 if args.no_settle else settle(torch, step)
+  elapsed, first_ms, second_ms = timed(step, steps, warmup, key="main")
+  clock_ghz = shader_clock_ghz(torch)
 
   tokens = B * T
   from recurrentgemma_amd import _lib
@@ -898,18 +985,23 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
         "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
         "traffic": traffic, "traffic_source": source,
         "algorithmic_bytes": algo, "avg_launch_ms": first_ms,
+        "launch_ms": per_launch["main"][0],
         "mfma_tflops": gemm_flops / (first_ms * 1e-3) / 1e12,
         "frac_of_bf16_mfma_peak": gemm_flops / (first_ms * 1e-3) / 2.5e15}
   else:
     if args.path == "auto":
       # per-kernel durations: the same two launches called one by one, with
       # events between them, after the timed region
-      _, first_ms, second_ms = timed(step_split, steps, warmup)
+      _, first_ms, second_ms = timed(step_split, steps, warmup, key="main")
     figs = split_figures(first_ms, second_ms)
+    figs["gate_gemm"]["launch_ms"] = per_launch["main"][0]
+    figs["scan"]["launch_ms"] = per_launch["main"][1]
     roofline = figs["scan"]
+  roofline["settle_launches"] = settle_launches
+  roofline["shader_clock_ghz_after"] = clock_ghz
 
   cold = None
-  if extras and x.numel() * esize * 4 < (256 << 20):
+  if (extras or cold_too) and x.numel() * esize * 4 < (256 << 20):
     # The whole working set fits the caches (4 MB of L2 per XCD, 256 MB behind
     # them): the timed loop above is a warm-cache figure.  Cold: 1 GiB is
     # written between the steps and each step is timed on its own.
@@ -966,9 +1058,13 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras):
     result["gate_gemm"] = figs["gate_gemm"]
   elif args.path == "auto":
     # the two-kernel form of the same step, measured after the timed region
-    n2 = max(5, steps // 2)
-    e2, g_ms, s_ms = timed(step_split, n2, 3)
+    n2 = max(20, steps // 2)
+    if not args.no_settle:
+      settle(torch, step_split, cap_s=0.25)
+    e2, g_ms, s_ms = timed(step_split, n2, 3, key="split")
     figs = split_figures(g_ms, s_ms)
+    figs["gate_gemm"]["launch_ms"] = per_launch["split"][0]
+    figs["scan"]["launch_ms"] = per_launch["split"][1]
     result["two_kernel_path"] = {
         "value": tokens / (e2 / n2), "unit": "tokens/s", "steps": n2,
         "scan": figs["scan"], "gate_gemm": figs["gate_gemm"]}

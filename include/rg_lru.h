@@ -524,6 +524,15 @@ int rg_soft_cap(const void* x, void* out, int64_t n, float cap, int dtype,
 int rg_argmax_rows(const void* x, int64_t* out, int rows, int n, int dtype,
                    void* stream);
 
+/* Measurement aid, no counterpart in the reference: one wave per compute unit
+ * runs `iters` (1 .. 2^20) rounds of 64 dependent multiply-adds (about 260
+ * cycles a round) and leaves in out[0] the shader-clock cycles and in out[1]
+ * the ticks of the constant 100 MHz counter that took; out[0] / out[1] / 10 is
+ * the shader clock in GHz at that moment.  out: 3 x uint64 of device memory
+ * (out[2] is scratch).  bench.py reports it next to its timings, which scale
+ * with that clock. */
+int rg_clock_probe(uint64_t* out, int iters, void* stream);
+
 /* The linear layers around the recurrent and attention blocks for a decode
  * step (at most 64 rows), bf16: torch.nn.Linear (modules.py:579-601 linear_y /
  * linear_x / linear_out, :717-721 ffw_down, :334-352 the attention projections)

@@ -871,6 +871,14 @@ int rg_soft_cap(const void* x, void* out, int64_t n, float cap, int dtype,
       __func__, rg::launch_soft_cap(x, out, n, cap, dtype, (hipStream_t)stream));
 }
 
+int rg_clock_probe(uint64_t* out, int iters, void* stream) {
+  RG_REQUIRE(out != nullptr, "%s: out is null", __func__);
+  RG_REQUIRE(iters > 0 && iters <= (1 << 20), "%s: iters=%d out of range",
+             __func__, iters);
+  return launch_status(
+      __func__, rg::launch_clock_probe(out, iters, (hipStream_t)stream));
+}
+
 int rg_argmax_rows(const void* x, int64_t* out, int rows, int n, int dtype,
                    void* stream) {
   RG_CHECK_DTYPE(dtype);

@@ -413,4 +413,37 @@ hipError_t launch_rms_norm_partial(const float* sums, int slices,
   return hipGetLastError();
 }
 
+
+// ------------------------------------------------------------ clock probe ----
+// One wave per CU spins through `iters` rounds of 64 dependent fused
+// multiply-adds and notes the shader-clock counter (s_memtime) and the
+// constant 100 MHz counter (s_memrealtime) before and after: their ratio is
+// the shader clock the GPU runs at right now.  out[0] = shader cycles, out[1] =
+// 10 ns ticks (workgroup 0's).
+namespace {
+__global__ void __launch_bounds__(64) clock_probe_kernel(uint64_t* out,
+                                                         int iters) {
+  float v = (float)threadIdx.x;
+  const uint64_t c0 = __builtin_readcyclecounter();
+  const uint64_t r0 = __builtin_amdgcn_s_memrealtime();
+  for (int i = 0; i < iters; ++i) {
+#pragma unroll
+    for (int j = 0; j < 64; ++j) v = __builtin_fmaf(v, 0.999f, 0.5f);
+    asm volatile("" : "+v"(v));
+  }
+  const uint64_t c1 = __builtin_readcyclecounter();
+  const uint64_t r1 = __builtin_amdgcn_s_memrealtime();
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    out[0] = c1 - c0;
+    out[1] = r1 - r0;
+    out[2] = (uint64_t)__float_as_uint(v);  // keeps the loop
+  }
+}
+}  // namespace
+
+hipError_t launch_clock_probe(uint64_t* out, int iters, hipStream_t s) {
+  clock_probe_kernel<<<256, 64, 0, s>>>(out, iters);
+  return hipGetLastError();
+}
+
 }  // namespace rg

@@ -298,6 +298,9 @@ hipError_t launch_rms_norm_partial(const float* sums, int slices,
                                    const void* scale, void* sum_out, void* out,
                                    int rows, int width, float eps,
                                    hipStream_t s);
+// out[0] = shader cycles, out[1] = 10 ns ticks that `iters` rounds of a short
+// dependent instruction chain took (rg_elementwise.hip)
+hipError_t launch_clock_probe(uint64_t* out, int iters, hipStream_t s);
 hipError_t launch_pack_gate_weights(const void* w_x, const void* w_a,
                                     void* packed, int H, hipStream_t s);
 

@@ -38,8 +38,13 @@ constexpr int kXcTileBytes = kTM * kXcRowBytes;
 constexpr int kRawHalo = 4;
 constexpr int kRawRows = kTM + kRawHalo;
 constexpr int kRawRowBytes = kBW * 2;
-constexpr int kRawTileBytes = kRawRows * kRawRowBytes;
 constexpr int kRawLoads = kRawRows / 2;  // wave-wide 16-byte loads per tile
+// ... shared out evenly: every wave issues the same number of loads without
+// looking at its wave number (a branch per load costs a lone wave more than
+// the load); the loads beyond kRawLoads are sent out of range and fill rows
+// of padding behind the tile with zeros
+constexpr int kRawLoadsPerWave = (kRawLoads + kWaves - 1) / kWaves;
+constexpr int kRawTileBytes = kRawLoadsPerWave * kWaves * 2 * kRawRowBytes;
 // Per-wave output patch: 16 tokens x 64 channels in bf16, rows padded to 144
 // bytes (16-byte aligned row reads, spread over the banks).
 constexpr int kPatchStride = 144;
@@ -346,14 +351,13 @@ __device__ __forceinline__ void prefill_body(const FusedArgs& p,
     lds_byte* const dst = lds3 + kRawOff + buf * kRawTileBytes;
     const int t0 = tile * kTM - kRawHalo + (lane >> 5);
 #pragma unroll
-    for (int j = 0; j < (kRawLoads + kWaves - 1) / kWaves; ++j) {
+    for (int j = 0; j < kRawLoadsPerWave; ++j) {
       const int i = wave + kWaves * j;
-      if (i < kRawLoads) {
-        const uint32_t voff =
-            (uint32_t)((t0 + 2 * i) * (int)row_bytes) + dma_lane_off;
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, dst + i * 1024, 16, voff,
-                                                 0, 0, 0);
-      }
+      uint32_t voff = (uint32_t)((t0 + 2 * i) * (int)row_bytes) + dma_lane_off;
+      if (kWaves * j + kWaves > kRawLoads)  // the last round only
+        voff = i < kRawLoads ? voff : kBufferOutOfRange;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, dst + i * 1024, 16, voff, 0,
+                                               0, 0);
     }
   };
 
@@ -460,9 +464,12 @@ __device__ __forceinline__ void prefill_body(const FusedArgs& p,
   // half `half` of a tile with start mask m_tile, m_before being the mask of
   // the tile before it.
   auto conv_cuts = [&](int half, uint64_t m_tile, uint64_t m_before) -> uint32_t {
-    const int base = half * 32 + rgp * kConvRows;
-    const uint64_t bits = base == 0 ? ((m_tile << 3) | (m_before >> 61))
-                                    : (m_tile >> (base - 3));
+    // first row of the group: 32 half + kConvRows rgp; bit i <- row first - 3 + i
+    // (written without a choice between the two forms at run time: a branch
+    // costs a lone wave tens of cycles)
+    const uint64_t bits =
+        half == 0 ? ((m_tile << 3) | (m_before >> 61)) >> (rgp * kConvRows)
+                  : m_tile >> (29 + rgp * kConvRows);
     return (uint32_t)bits & ((1u << (kConvRows + 3)) - 1u);
   };
 
@@ -522,27 +529,27 @@ __device__ __forceinline__ void prefill_body(const FusedArgs& p,
   u32x4 y_pending[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
   u32x4 g_pending[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};  // GELU: same positions
   uint32_t y_pending_row = kBufferOutOfRange;  // byte offset of its first row
-  auto flush_y = [&]() {
+  auto flush_y_half = [&](int j) {
     if (GELU) {
       // y * gelu(gate branch), each factor a bf16 tensor as in the reference
       // (recurrentgemma/torch/modules.py:627-628, 644): the arithmetic and
       // roundings of the stand-alone gelu_mul pass
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const float lo =
-              gelu_mul_bf16(__uint_as_float(y_pending[j][k] << 16),
-                            __uint_as_float(g_pending[j][k] << 16));
-          const float hi =
-              gelu_mul_bf16(__uint_as_float(y_pending[j][k] & 0xffff0000u),
-                            __uint_as_float(g_pending[j][k] & 0xffff0000u));
-          y_pending[j][k] = pack_bf16x2(lo, hi);
-        }
+      for (int k = 0; k < 4; ++k) {
+        const float lo = gelu_mul_bf16(__uint_as_float(y_pending[j][k] << 16),
+                                       __uint_as_float(g_pending[j][k] << 16));
+        const float hi =
+            gelu_mul_bf16(__uint_as_float(y_pending[j][k] & 0xffff0000u),
+                          __uint_as_float(g_pending[j][k] & 0xffff0000u));
+        y_pending[j][k] = pack_bf16x2(lo, hi);
+      }
     }
-    buffer_store_16(y_pending[0], ry, y_lane_bytes, y_pending_row);
-    buffer_store_16(y_pending[1], ry, y_lane_bytes,
-                    y_pending_row + 8u * row_bytes);
+    buffer_store_16(y_pending[j], ry, y_lane_bytes,
+                    y_pending_row + (uint32_t)(8 * j) * row_bytes);
+  };
+  auto flush_y = [&]() {
+    flush_y_half(0);
+    flush_y_half(1);
   };
   auto gate_block = [&](int it, int blk, auto BI, const BlockAcc& acc,
                         uint64_t m_tile, auto&& hook) {
@@ -608,7 +615,7 @@ __device__ __forceinline__ void prefill_body(const FusedArgs& p,
       pinned(8 * r + 3);
       // piece 4: document start: a = 0; past the end of the sequence: a = 1,
       // no input.  The input scale sqrt(1 - a^2) comes out as 1 at a start.
-      if (general) {
+      if (__builtin_expect(general, 0)) {
         // (kept a branch: as selects it would cost the common case 3.5 vector
         // instructions per element)
         // (the lane's row offset passes through an empty statement here so
@@ -796,6 +803,7 @@ __device__ __forceinline__ void prefill_body(const FusedArgs& p,
           mfma_step(i, bi, 1, a, acc1);
         else
           mfma_step(i, bn, 0, a, acc0);
+
         // row pair j of this thread's kConvRows / 2: its two raw rows were
         // requested a run earlier, the pair after it is requested now
         const int j = i >> 3;
@@ -817,7 +825,7 @@ __device__ __forceinline__ void prefill_body(const FusedArgs& p,
         gate_block(it, 0, BI, acc0, m_cur, hook);
       else
         gate_block(it, 1, BI, acc1, m_cur, hook);
-      if (cuts != 0) conv_rows_with_cuts(bn, half, cuts);
+      if (__builtin_expect(cuts != 0, 0)) conv_rows_with_cuts(bn, half, cuts);
       wait_for_matrix_results();
       if (half == 0) lds_barrier();
     }
