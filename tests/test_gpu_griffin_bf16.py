@@ -152,3 +152,42 @@ def test_sampler_against_reference_bf16(model, golden, use_graph):
     within_reference_error(got_l[:same], ref_bf16[:same], ref_f32[:same],
                            f"c2/logits{i}[:{same}]")
     assert same >= n_prompt + 1, (i, same)
+
+
+def test_config5_full_shape_graph_equals_eager():
+  """Benchmark configuration 5 at its full shape: the 2B preset (26 blocks,
+  width 2560, 10 heads of 256, window 2048, vocabulary 256000), random-init
+  bf16, batch 64.  A short left-padded prompt, then a few greedy steps: the
+  decode step replayed as a captured graph gives the tokens and logits of the
+  eager loop bit for bit, every logit is finite and inside the soft cap, and
+  a row's tokens do not depend on its neighbours.  (Reference-written vectors
+  pin the same kernels at width 512: test_sampler_against_reference_bf16.)"""
+  cfg = G.GriffinConfig.from_preset(G.Preset.RECURRENT_GEMMA_2B_V1)
+  torch.manual_seed(1005)
+  print("config5 full shape: model", flush=True)
+  m = G.Griffin(cfg, device=DEV, dtype=torch.bfloat16).eval()
+  B, L, steps = 64, 40, 6
+  g = torch.Generator().manual_seed(1005)
+  toks = torch.randint(3, cfg.vocab_size, (B, L), generator=g).to(
+      DEV, torch.int32)
+  lens = torch.full((B,), L, device=DEV, dtype=torch.int32)
+  lens[1::2] = L - 7  # every second row left-padded
+  for b in range(1, B, 2):
+    toks[b, :7] = 0
+  print("config5 full shape: eager", flush=True)
+  want_t, want_l = S.Sampler(m).sample_tokens(toks, lens, steps,
+                                              return_logits=True)
+  print("config5 full shape: graph", flush=True)
+  got_t, got_l = S.Sampler(m, use_graph=True).sample_tokens(
+      toks, lens, steps, return_logits=True)
+  torch.cuda.synchronize()
+  assert torch.equal(got_t, want_t)
+  assert torch.equal(got_l, want_l)
+  assert torch.isfinite(got_l.float()).all()
+  assert got_l.float().abs().max().item() <= cfg.logits_soft_cap
+  print("config5 full shape: four rows alone", flush=True)
+  alone_t, _ = S.Sampler(m).sample_tokens(toks[:4].contiguous(),
+                                          lens[:4].contiguous(), steps)
+  # (other batch sizes take other kernels for the linear layers: the logits
+  # agree to rounding, the greedy tokens almost always)
+  assert (alone_t == want_t[:4]).float().mean().item() >= 0.75

@@ -1247,11 +1247,23 @@ def _full_size_properties(B, T, W, H, seg, seed):
   assert (y_row.float() - y[:1].float()).abs().max().item() <= 0.125
   assert helpers.max_rel(c_row.rg_lru_state, cache.rg_lru_state[:1]) < BF16_TOL
   assert torch.equal(c_row.conv1d_state, cache.conv1d_state[:1])
-  # (6) spot parity against the oracle on one row's first tokens
-  n = 300
-  yo, _ = R.widened_recurrent_core(x[:1, :n].cpu(), seg[:1, :n], p)
-  assert helpers.max_rel(y[:1, :n], yo) < BF16_TOL
-  assert helpers.max_rel(y_core[:1, :n], yo) < BF16_TOL
+  # (6) parity against the oracle over the WHOLE sequence on two sampled rows
+  #     (not row 0): y element by element, the final state and the conv state,
+  #     for what recurrent_core ran at this grid (every chunk boundary of a
+  #     chunked launch and the tail of the row included) and for the
+  #     two-kernel form
+  for row in sorted({B // 2, B - 1}):
+    _announce("full size: oracle on row", row)
+    yo, co = R.widened_recurrent_core(x[row:row + 1].cpu(), seg[row:row + 1], p)
+    for name, yy, hh, cc in (
+        ("recurrent_core", y_core, cache_core.rg_lru_state,
+         cache_core.conv1d_state),
+        ("two kernels", y, cache.rg_lru_state, cache.conv1d_state)):
+      helpers.assert_close_elementwise(yy[row:row + 1], yo,
+                                       what=f"{name} row {row} y")
+      assert helpers.max_rel(yy[row:row + 1], yo) < BF16_TOL
+      assert helpers.max_rel(hh[row:row + 1], co.rg_lru_state) < 2e-3, name
+      assert torch.equal(cc[row:row + 1].cpu(), co.conv1d_state), name
 
 
 def test_config2_full_size_properties():
