@@ -101,9 +101,11 @@ int rg_block_diag_linear(const void* x, const void* w, const void* b, void* y,
  *   conv_w [4,W], conv_b [W] and the segpos mask (prefill semantics of
  *   rg_conv1d_prefill, rounded to `dtype` like the reference's module output);
  *   segpos must then be given.
- * bw = W / H.  bf16 with bw == 256 runs on the MFMA kernel (weights held in
- * registers, x tiles staged through LDS); any other combination runs on a
- * plain FMA kernel with fp32 accumulation. */
+ * bw = W / H.  On the matrix cores: bf16 with 128 <= bw <= 256 (bw a multiple
+ * of 8; weights held in registers, x tiles staged through LDS, narrower heads
+ * padded to the 256-wide tile inside the kernel) and float32 with bw == 256
+ * (true float32 products, v_mfma_f32_32x32x2_f32).  Any other combination runs
+ * on a plain FMA kernel with fp32 accumulation. */
 int rg_gates_gemm(const void* x, int apply_conv, const void* segpos,
                   int segpos_is_i64, const void* conv_w, const void* conv_b,
                   const void* w_x, const void* b_x, const void* w_a,

@@ -5,9 +5,14 @@ block :294-493, MLP block :683-760, residual block :763-932, embedder
 :935-1003), recurrentgemma/torch/griffin.py:27-209 (model, cache dictionary
 keyed "blocks.{i}") and the config types of recurrentgemma/common.py:22-190:
 same constructor arguments, parameter names (reference state dicts load
-unchanged), forward signatures and cache tuples.  Only the recurrent block
-runs on this package's kernels; everything else here is plain torch on the GPU
-(hipBLASLt GEMMs, scaled_dot_product_attention) and exists so that the
+unchanged), forward signatures and cache tuples.  On this package's kernels:
+the recurrent block, RMSNorm (with the residual sums in front of it), the two
+gelu(a) * b joins, the rotary embedding, the prompt attention and the decode
+step of the attention block (bf16, head_dim 256), the linear layers of a
+decode step of at most 64 rows, the logits' soft cap and the greedy pick.
+Library calls: linear layers with more rows and the logits projection
+(hipBLASLt), attention in other dtypes and head sizes
+(scaled_dot_product_attention / batched products).  It exists so that the
 recurrent path can be exercised and measured inside the model it belongs to.
 Inference only (no autograd through the kernels).
 """
@@ -235,18 +240,25 @@ def _visible(q_pos, k_pos, window, q_doc=None, k_doc=None):
 def _inference_only(forward):
   """The residual stack around the recurrent block runs without an autograd
   graph (its few-row linear layers, attention and normalisation kernels have
-  no backward pass).  A caller that would expect gradients -- inside
-  training.differentiable(), or with gradients enabled on a module in
-  training mode -- gets an error instead of silently detached tensors."""
+  no backward pass).  Called the way the reference's own tests call it --
+  constructed, not switched to eval(), gradients enabled
+  (recurrentgemma/torch/griffin_test.py, modules_test.py) -- it simply
+  computes, under no_grad.  A caller that asks for gradients through it --
+  inside training.differentiable(), or with an input tensor that requires
+  grad -- gets an error instead of silently detached tensors."""
 
   @functools.wraps(forward)
   def wrapper(self, *args, **kwargs):
     from recurrentgemma_amd import training
-    if training.is_enabled() or (torch.is_grad_enabled() and self.training):
+    wants_grad = training.is_enabled() or (
+        torch.is_grad_enabled() and any(
+            isinstance(a, torch.Tensor) and a.requires_grad
+            for a in itertools.chain(args, kwargs.values())))
+    if wants_grad:
       raise NotImplementedError(
-          f"{type(self).__name__} is forward only: call .eval() or run it "
-          "under torch.no_grad() (only RecurrentBlock, Conv1D and RGLRU have "
-          "a differentiable path, inside training.differentiable())")
+          f"{type(self).__name__} is forward only: no gradient flows through "
+          "it (only RecurrentBlock, Conv1D and RGLRU have a differentiable "
+          "path, inside training.differentiable())")
     with torch.no_grad():
       return forward(self, *args, **kwargs)
 

@@ -229,12 +229,22 @@ def test_stack_refuses_to_run_where_gradients_are_expected():
   m = _bf16_model()
   toks = torch.randint(3, 512, (1, 4)).to(DEV, torch.int32)
   pos = torch.arange(4, device=DEV)[None]
+  # the way the reference's own tests call a model: not switched to eval(),
+  # gradients enabled -- computes, like under no_grad
   m.train()
-  with pytest.raises(NotImplementedError, match="forward only"):
-    m(toks, pos)
+  logits, _ = m(toks, pos)
+  assert not logits.requires_grad
   with torch.no_grad():
-    m(toks, pos)  # fine without gradients
+    again, _ = m(toks, pos)
+  assert torch.equal(logits, again)
   m.eval()
+  # asked for gradients: an input that requires grad, or the differentiable
+  # path switched on
+  blk = m.blocks[0]
+  x = torch.randn(1, 4, m.config.width, device=DEV,
+                  dtype=torch.bfloat16).requires_grad_(True)
+  with pytest.raises(NotImplementedError, match="forward only"):
+    blk(x, pos)
   from recurrentgemma_amd import training
   with training.differentiable():
     with pytest.raises(NotImplementedError, match="forward only"):

@@ -318,6 +318,50 @@ def test_rglru_golden(golden):
   assert worst_ref_form[0] <= 0.0, worst_ref_form[0]
 
 
+def test_rglru_golden_256_wide_heads_in_both_forms(golden):
+  """The reference-written bf16 RG-LRU vectors with a 256-wide head, through
+  BOTH forms the library may pick for such a layer (the choice depends on the
+  batch size, and the two forms round the gate pre-activations differently:
+  the gate GEMM + scan pair to bf16 like the reference's modules, the single
+  kernel keeps them in float32): each against the reference's own outputs in
+  the reference's tolerance form (layers_test.py:131) and against the widened
+  oracle; the two forms against each other to a bf16 ulp or two."""
+  keys = [k for k in golden.cases("rglru/") if "/bfloat16/W256H1/" in k]
+  assert len(keys) >= 10
+  for key in keys:
+    _announce(key)
+    pkey = "/".join(key.split("/")[:3])
+    a_param, w_x, b_x, w_a, b_a = (
+        golden.get(pkey + "/" + n)
+        for n in ("a_param", "w_x", "b_x", "w_a", "b_a"))
+    x, seg = golden.get(key + "/x"), golden.get(key + "/seg")
+    h0 = golden.get(key + "/h0") if golden.has(key + "/h0") else None
+    W = x.shape[-1]
+    P = [_dev(t) for t in (w_x, b_x, w_a, b_a, a_param)]
+    # the single kernel with a conv that hands x through (w3 = 1)
+    ident = torch.zeros(4, W, dtype=x.dtype)
+    ident[3] = 1.0
+    y1, h1, _ = ops.recurrent_prefill(
+        _dev(x), _dev(seg), _dev(ident), _dev(torch.zeros(W, dtype=x.dtype)),
+        P[0], P[1], P[2], P[3], P[4], h0=_dev(h0), split=False)
+    gx, ga = ops.gates_gemm(_dev(x), P[0], P[1], P[2], P[3])
+    y2, h2, _ = ops.lru_scan_fused(_dev(x), gx, ga, P[4], _dev(seg),
+                                   h0=_dev(h0))
+    gold_y = golden.get(key + "/y").float()
+    gold_h = golden.get(key + "/h").float()
+    yo, ho = R.widened_rglru_forward(x, seg, a_param, w_x, b_x, w_a, b_a,
+                                     cache=h0)
+    for name, y, h in (("single kernel", y1, h1), ("two kernels", y2, h2)):
+      d = (y.cpu().float() - gold_y).abs()
+      assert (d <= 3e-2 + 1e-2 * gold_y.abs()).all(), (key, name)
+      dh = (h.cpu() - gold_h).abs()
+      assert (dh <= 3e-2 + 1e-2 * gold_h.abs()).all(), (key, name)
+      assert helpers.max_rel(y, yo) < BF16_TOL, (key, name)
+      assert helpers.max_rel(h, ho) < BF16_TOL, (key, name)
+    assert (y1.float() - y2.float()).abs().max().item() <= 0.0625, key
+    assert helpers.max_rel(h1, h2) < 2e-3, key
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("B,T,W,H,mean_doc,with_h0", [
     (13, 200, 2560, 10, 40, False),  # 130 (row, head) pairs: the single kernel
