@@ -154,9 +154,8 @@ __device__ __forceinline__ bool is_doc_start(const void* segpos, int kind,
 }
 
 // ------------------------------------------------------------- conv ----
-// Width-4 tap chain in the one fixed order every kernel uses, so that the gate
-// GEMM (conv on load) and the scan kernel see bit-identical conv outputs:
-// newest tap first, bias as the starting value, fused multiply-adds.
+// Width-4 tap chain of the float32 kernels, in one fixed order: newest tap
+// first, bias as the starting value, fused multiply-adds.
 // x0 = x[t], x1 = x[t-1], ... ; w3 multiplies x[t] (layers.py:514).
 __device__ __forceinline__ float conv4(float x0, float x1, float x2, float x3,
                                        float w0, float w1, float w2, float w3,
@@ -168,6 +167,89 @@ __device__ __forceinline__ float conv4(float x0, float x1, float x2, float x3,
   return acc;
 }
 
+// The bf16 kernels' width-4 conv, one arithmetic everywhere (gate GEMM with
+// the conv on load, scan kernel, single prefill kernel, stand-alone conv,
+// decode step), so that all of them see bit-identical conv outputs: per
+// channel the rows are paired in time, P_t = (x[t-1], x[t]) as two bf16 in one
+// register, the taps as w10 = (w0, w1) and w32 = (w2, w3), and
+//   out[t] = (bias + P_{t-2} . w10) + P_t . w32
+// is two v_dot2_f32_bf16 (float32 products and sums), rounded to bf16 by the
+// caller.  Nothing is unpacked: 3.5 vector instructions per output where the
+// chain of fused multiply-adds on floats takes 5.75.
+constexpr uint32_t kPairSelLo = 0x05040100u;  // (lo16(earlier), lo16(later))
+constexpr uint32_t kPairSelHi = 0x07060302u;  // (hi16(earlier), hi16(later))
+// Two rows of a channel pair (two bf16 per register) -> the time pairs of the
+// low and the high channel.
+__device__ __forceinline__ void pair_up(uint32_t earlier, uint32_t later,
+                                        uint32_t& lo, uint32_t& hi) {
+  lo = __builtin_amdgcn_perm(later, earlier, kPairSelLo);
+  hi = __builtin_amdgcn_perm(later, earlier, kPairSelHi);
+}
+// The result of a dot instruction may be read by an instruction of another
+// kind only three issue slots later, and the compiler does not count them for
+// inline assembly: each group ends with the wait itself.
+__device__ __forceinline__ float conv4_dot(uint32_t p_old, uint32_t p_new,
+                                           uint32_t w10, uint32_t w32,
+                                           float bias) {
+  float out;
+  asm("v_dot2_f32_bf16 %0, %1, %3, %5\n\t"
+      "v_dot2_f32_bf16 %0, %2, %4, %0\n\t"
+      "s_nop 2"
+      : "=&v"(out)
+      : "v"(p_old), "v"(p_new), "v"(w10), "v"(w32), "v"(bias));
+  return out;
+}
+__device__ __forceinline__ void conv4_dot_x2(
+    const uint32_t (&p_old)[2], const uint32_t (&p_new)[2],
+    const uint32_t (&w10)[2], const uint32_t (&w32)[2], const float (&bias)[2],
+    float (&out)[2]) {
+  asm("v_dot2_f32_bf16 %0, %2, %6, %10\n\t"
+      "v_dot2_f32_bf16 %1, %3, %7, %11\n\t"
+      "v_dot2_f32_bf16 %0, %4, %8, %0\n\t"
+      "v_dot2_f32_bf16 %1, %5, %9, %1\n\t"
+      "s_nop 2"
+      : "=&v"(out[0]), "=&v"(out[1])
+      : "v"(p_old[0]), "v"(p_old[1]), "v"(p_new[0]), "v"(p_new[1]),
+        "v"(w10[0]), "v"(w10[1]), "v"(w32[0]), "v"(w32[1]), "v"(bias[0]),
+        "v"(bias[1]));
+}
+__device__ __forceinline__ void conv4_dot_x4(
+    const uint32_t (&p_old)[4], const uint32_t (&p_new)[4],
+    const uint32_t (&w10)[4], const uint32_t (&w32)[4], const float (&bias)[4],
+    float (&out)[4]) {
+  asm("v_dot2_f32_bf16 %0, %4, %12, %20\n\t"
+      "v_dot2_f32_bf16 %1, %5, %13, %21\n\t"
+      "v_dot2_f32_bf16 %2, %6, %14, %22\n\t"
+      "v_dot2_f32_bf16 %3, %7, %15, %23\n\t"
+      "v_dot2_f32_bf16 %0, %8, %16, %0\n\t"
+      "v_dot2_f32_bf16 %1, %9, %17, %1\n\t"
+      "v_dot2_f32_bf16 %2, %10, %18, %2\n\t"
+      "v_dot2_f32_bf16 %3, %11, %19, %3\n\t"
+      "s_nop 2"
+      : "=&v"(out[0]), "=&v"(out[1]), "=&v"(out[2]), "=&v"(out[3])
+      : "v"(p_old[0]), "v"(p_old[1]), "v"(p_old[2]), "v"(p_old[3]),
+        "v"(p_new[0]), "v"(p_new[1]), "v"(p_new[2]), "v"(p_new[3]),
+        "v"(w10[0]), "v"(w10[1]), "v"(w10[2]), "v"(w10[3]), "v"(w32[0]),
+        "v"(w32[1]), "v"(w32[2]), "v"(w32[3]), "v"(bias[0]), "v"(bias[1]),
+        "v"(bias[2]), "v"(bias[3]));
+}
+// The same output from bf16 values held as floats (the element-per-thread
+// kernels): packing them back is exact.  x0 = x[t], x1 = x[t-1], ...
+__device__ __forceinline__ float conv4_bf16(float x0, float x1, float x2,
+                                            float x3, float w0, float w1,
+                                            float w2, float w3, float bias) {
+  return conv4_dot(pack_bf16x2(x3, x2), pack_bf16x2(x1, x0),
+                   pack_bf16x2(w0, w1), pack_bf16x2(w2, w3), bias);
+}
+// conv4 for the element type: float32 the multiply-add chain, bf16 the dots.
+template <typename T>
+__device__ __forceinline__ float conv4_as(float x0, float x1, float x2,
+                                          float x3, float w0, float w1,
+                                          float w2, float w3, float bias) {
+  if (sizeof(T) == 2) return conv4_bf16(x0, x1, x2, x3, w0, w1, w2, w3, bias);
+  return conv4(x0, x1, x2, x3, w0, w1, w2, w3, bias);
+}
+
 // Generic-width conv output at flattened row m = b*T + t, channel c, straight
 // from the definition (same accumulation order as conv4 for K == 4).
 template <typename T>
@@ -176,6 +258,21 @@ __device__ __forceinline__ float conv_point(const T* x, const void* segpos,
                                             const T* bias, int T_len, int W,
                                             int K, int64_t m, int c) {
   int t = (int)(m % T_len);
+  if (sizeof(T) == 2 && K == 4) {
+    // the bf16 kernels' width-4 arithmetic (conv4_dot)
+    float xs[4];
+    bool alive = true;
+    for (int s = 0; s < 4; ++s) {
+      if (s > t) alive = false;
+      if (s > 0 && s <= t && is_doc_start(segpos, seg_kind, m - s + 1))
+        alive = false;
+      xs[s] = alive ? load_scalar(x + (m - s) * W + c) : 0.0f;
+    }
+    return round_act<T>(conv4_bf16(
+        xs[0], xs[1], xs[2], xs[3], load_scalar(w + c),
+        load_scalar(w + (int64_t)W + c), load_scalar(w + 2 * (int64_t)W + c),
+        load_scalar(w + 3 * (int64_t)W + c), load_scalar(bias + c)));
+  }
   float acc = load_scalar(bias + c);
   bool alive = true;
   for (int s = 0; s < K && s <= t; ++s) {

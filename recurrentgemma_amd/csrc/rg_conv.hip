@@ -198,6 +198,88 @@ conv1d_prefill_k4_kernel(const T* __restrict__ x, const void* __restrict__ segpo
   auto row = [&](const T* base, int64_t m) {
     return *reinterpret_cast<const u32x4*>(base + m * W + c);
   };
+  if constexpr (sizeof(T) == 2) {
+    // bf16: the kernels' one width-4 arithmetic (conv4_dot of rg_common.h) on
+    // rows that stay packed: per channel the time pairs (x[t-1], x[t]), two
+    // dot products per output
+    float bb[N];
+    V::unpack(*reinterpret_cast<const u32x4*>(bias + c), bb);
+    uint32_t w10[N], w32[N];
+    {
+      const u32x4 t0 = row(w, 0), t1 = row(w, 1), t2 = row(w, 2), t3 = row(w, 3);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        pair_up(t0[q], t1[q], w10[2 * q], w10[2 * q + 1]);
+        pair_up(t2[q], t3[q], w32[2 * q], w32[2 * q + 1]);
+      }
+    }
+    // history: the row before (packed) and the pairs that ended one and two
+    // rows back; zero where a start cuts
+    u32x4 r1 = {0, 0, 0, 0};
+    uint32_t pn1[N], pn2[N];
+#pragma unroll
+    for (int e = 0; e < N; ++e) pn1[e] = pn2[e] = 0u;
+    auto cut = [&]() {
+      r1 = u32x4{0, 0, 0, 0};
+#pragma unroll
+      for (int e = 0; e < N; ++e) pn1[e] = pn2[e] = 0u;
+    };
+    auto push = [&](const u32x4& cur, uint32_t (&pn0)[N]) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        pair_up(r1[q], cur[q], pn0[2 * q], pn0[2 * q + 1]);
+    };
+    auto shift = [&](const u32x4& cur, const uint32_t (&pn0)[N]) {
+#pragma unroll
+      for (int e = 0; e < N; ++e) {
+        pn2[e] = pn1[e];
+        pn1[e] = pn0[e];
+      }
+      r1 = cur;
+    };
+    for (int64_t j = m0 - 3; j < m0; ++j) {
+      if (j < 0) continue;
+      if (conv_row_starts(segpos, seg_kind, seq, j)) cut();
+      const u32x4 cur = row(x, j);
+      uint32_t pn0[N];
+      push(cur, pn0);
+      shift(cur, pn0);
+    }
+    for (int64_t mb = m0; mb < m1; mb += kConvBatch) {
+      u32x4 raw[kConvBatch];
+      bool st[kConvBatch];
+#pragma unroll
+      for (int u = 0; u < kConvBatch; ++u) {
+        const int64_t m = mb + u < m1 ? mb + u : m1 - 1;
+        raw[u] = row(x, m);
+        st[u] = conv_row_starts(segpos, seg_kind, seq, m);
+      }
+#pragma unroll
+      for (int u = 0; u < kConvBatch; ++u) {
+        if (mb + u < m1) {
+          if (st[u]) cut();
+          uint32_t pn0[N];
+          push(raw[u], pn0);
+          float o[N];
+#pragma unroll
+          for (int q = 0; q < N; q += 4) {
+            const uint32_t po[4] = {pn2[q], pn2[q + 1], pn2[q + 2], pn2[q + 3]};
+            const uint32_t pw[4] = {pn0[q], pn0[q + 1], pn0[q + 2], pn0[q + 3]};
+            const uint32_t wa[4] = {w10[q], w10[q + 1], w10[q + 2], w10[q + 3]};
+            const uint32_t wb[4] = {w32[q], w32[q + 1], w32[q + 2], w32[q + 3]};
+            const float bq[4] = {bb[q], bb[q + 1], bb[q + 2], bb[q + 3]};
+            float oq[4];
+            conv4_dot_x4(po, pw, wa, wb, bq, oq);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[q + e] = oq[e];
+          }
+          shift(raw[u], pn0);
+          *reinterpret_cast<u32x4*>(out + (mb + u) * W + c) = V::pack(o);
+        }
+      }
+    }
+    return;
+  }
   float w0[N], w1[N], w2[N], w3[N], bb[N];
   V::unpack(row(w, 0), w0);
   V::unpack(row(w, 1), w1);
@@ -400,12 +482,22 @@ conv1d_step_kernel(const T* __restrict__ x, const T* cache_in,
       st[k] = (k < K - 1) ? load_scalar(cache_in + (b * (K - 1) + k) * W + c)
                           : 0.0f;
     const float xv = load_scalar(x + idx);
-    float acc = load_scalar(bias + c);
-    acc = __builtin_fmaf(xv, load_scalar(w + (int64_t)(K - 1) * W + c), acc);
+    float acc;
+    if (sizeof(T) == 2 && K == 4) {
+      // the bf16 kernels' width-4 arithmetic (conv4_dot of rg_common.h)
+      acc = conv4_bf16(xv, st[2], st[1], st[0], load_scalar(w + c),
+                       load_scalar(w + (int64_t)W + c),
+                       load_scalar(w + 2 * (int64_t)W + c),
+                       load_scalar(w + 3 * (int64_t)W + c),
+                       load_scalar(bias + c));
+    } else {
+      acc = load_scalar(bias + c);
+      acc = __builtin_fmaf(xv, load_scalar(w + (int64_t)(K - 1) * W + c), acc);
 #pragma unroll
-    for (int k = 14; k >= 0; --k)  // newest state row first
-      if (k < K - 1)
-        acc = __builtin_fmaf(st[k], load_scalar(w + (int64_t)k * W + c), acc);
+      for (int k = 14; k >= 0; --k)  // newest state row first
+        if (k < K - 1)
+          acc = __builtin_fmaf(st[k], load_scalar(w + (int64_t)k * W + c), acc);
+    }
     store_scalar(out + idx, acc);
     if (cache_out) {
 #pragma unroll

@@ -199,17 +199,17 @@ __global__ void __launch_bounds__(512) block_step_bf16_kernel(StepArgs p) {
       u32x2 packed;
 #pragma unroll
       for (int w2 = 0; w2 < 2; ++w2) {
+        // the bf16 kernels' width-4 arithmetic (conv4_dot of rg_common.h):
+        // s0, s1, s2 are the state rows x[t-3], x[t-2], x[t-1], xr is x[t]
+        uint32_t p_old[2], p_new[2], w10[2], w32[2];
+        pair_up(s0[j][w2], s1[j][w2], p_old[0], p_old[1]);
+        pair_up(s2[j][w2], xr[j][w2], p_new[0], p_new[1]);
+        pair_up(u0[w2], u1[w2], w10[0], w10[1]);
+        pair_up(u2[w2], u3[w2], w32[0], w32[1]);
+        const float bias2[2] = {__uint_as_float(ub[w2] << 16),
+                                __uint_as_float(ub[w2] & 0xffff0000u)};
         float o[2];
-#pragma unroll
-        for (int k = 0; k < 2; ++k) {
-          auto unpack = [&](const u32x2& v) {
-            return k == 0 ? __uint_as_float(v[w2] << 16)
-                          : __uint_as_float(v[w2] & 0xffff0000u);
-          };
-          o[k] = conv4(unpack(xr[j]), unpack(s2[j]), unpack(s1[j]),
-                       unpack(s0[j]), unpack(u0), unpack(u1), unpack(u2),
-                       unpack(u3), unpack(ub));
-        }
+        conv4_dot_x2(p_old, p_new, w10, w32, bias2, o);
         packed[w2] = pack_bf16x2(o[0], o[1]);
       }
       *reinterpret_cast<u32x2*>(stage + (size_t)row * kLdsStride + cq * 4) =

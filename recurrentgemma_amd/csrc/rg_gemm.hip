@@ -296,17 +296,22 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
   //   stage_begin: document-start mask of the tile's rows, history cleared
   //   stage_row(j): j < kHalo feeds the history; j >= kHalo writes LDS row
   //                 j - kHalo of this thread's group
-  float cw0[2], cw1[2], cw2[2], cw3[2], cb[2];
+  // The conv in the bf16 kernels' one arithmetic (conv4_dot of rg_common.h):
+  // per channel the taps paired as (w0, w1), (w2, w3), the rows paired in
+  // time, two dot products per output; nothing is unpacked between the MFMAs.
+  uint32_t cw10[2] = {0, 0}, cw32[2] = {0, 0};
+  float cb[2] = {0.0f, 0.0f};
   if (CONV) {
-    // unpacked once: ten registers, but no unpacking between the MFMAs
-    cw0[0] = __uint_as_float(cwp[0] << 16); cw0[1] = __uint_as_float(cwp[0] & 0xffff0000u);
-    cw1[0] = __uint_as_float(cwp[1] << 16); cw1[1] = __uint_as_float(cwp[1] & 0xffff0000u);
-    cw2[0] = __uint_as_float(cwp[2] << 16); cw2[1] = __uint_as_float(cwp[2] & 0xffff0000u);
-    cw3[0] = __uint_as_float(cwp[3] << 16); cw3[1] = __uint_as_float(cwp[3] & 0xffff0000u);
-    cb[0] = __uint_as_float(cwp[4] << 16);  cb[1] = __uint_as_float(cwp[4] & 0xffff0000u);
+    pair_up(cwp[0], cwp[1], cw10[0], cw10[1]);
+    pair_up(cwp[2], cwp[3], cw32[0], cw32[1]);
+    cb[0] = __uint_as_float(cwp[4] << 16);
+    cb[1] = __uint_as_float(cwp[4] & 0xffff0000u);
   }
   uint32_t cut = 0;
-  float h0[2], h1[2], h2[2];
+  // history of this thread's channel pair: the row before (still packed) and
+  // the time pairs (x[t-1], x[t]) that ended one and two rows back, zero where
+  // a start cuts
+  uint32_t r1 = 0, pn1[2] = {0, 0}, pn2[2] = {0, 0};
   uint16_t* const stage_dst0 =
       lds + (size_t)(rg * kRowsPerGroup) * kLdsStride + cp * 2;
 
@@ -335,7 +340,7 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
       if (lane < kRaw && m >= 0 && m < M) st = seq_start || ((lo | hi) == 0u);
     }
     cut = (uint32_t)__ballot(st);
-    h0[0] = h0[1] = h1[0] = h1[1] = h2[0] = h2[1] = 0.0f;
+    r1 = pn1[0] = pn1[1] = pn2[0] = pn2[1] = 0u;
   };
   // CUTS = false is the straight-line form for a tile without any sequence or
   // document start among its rows (cut == 0).
@@ -346,26 +351,23 @@ __global__ void __launch_bounds__(512) gates_mfma_bf16_kernel(GemmArgs p) {
       *reinterpret_cast<uint32_t*>(dst + (size_t)j * kLdsStride) = raw[j];
       return;
     }
-    float xv[2];
-    xv[0] = __uint_as_float(raw[j] << 16);
-    xv[1] = __uint_as_float(raw[j] & 0xffff0000u);
     if (CUTS && ((cut >> j) & 1u)) {
-      h0[0] = h0[1] = h1[0] = h1[1] = h2[0] = h2[1] = 0.0f;
+      r1 = pn1[0] = pn1[1] = pn2[0] = pn2[1] = 0u;
     }
+    uint32_t pn0[2];
+    pair_up(r1, raw[j], pn0[0], pn0[1]);
     if (j >= kHalo) {
-      const float o0 = conv4(xv[0], h0[0], h1[0], h2[0], cw0[0], cw1[0],
-                             cw2[0], cw3[0], cb[0]);
-      const float o1 = conv4(xv[1], h0[1], h1[1], h2[1], cw0[1], cw1[1],
-                             cw2[1], cw3[1], cb[1]);
+      float o[2];
+      conv4_dot_x2(pn2, pn0, cw10, cw32, cb, o);
       *reinterpret_cast<uint32_t*>(dst + (size_t)(j - kHalo) * kLdsStride) =
-          pack_bf16x2(o0, o1);
+          pack_bf16x2(o[0], o[1]);
     }
 #pragma unroll
     for (int ch = 0; ch < 2; ++ch) {
-      h2[ch] = h1[ch];
-      h1[ch] = h0[ch];
-      h0[ch] = xv[ch];
+      pn2[ch] = pn1[ch];
+      pn1[ch] = pn0[ch];
     }
+    r1 = raw[j];
   };
   using WithCuts = std::integral_constant<bool, true>;
   using NoCuts = std::integral_constant<bool, false>;

@@ -161,9 +161,49 @@ struct Buf<float, 1> {
 
 template <int CH>
 struct ChanConst {
+  // float32: the four taps as floats.  bf16: the taps stay packed in pairs,
+  // w10 = (w0, w1) and w32 = (w2, w3), the operands of the two-element dot
+  // product (w0..w3 unused and optimised away)
   float w0[CH], w1[CH], w2[CH], w3[CH], bias[CH];
+  uint32_t w10[CH], w32[CH];
   float decay[CH];  // FAST: -8 softplus(L) log2(e);  precise: softplus(L)
 };
+
+// ---- width-4 conv on packed bf16 rows (conv4_dot of rg_common.h) ----------
+// A row of a lane is CH bf16 channels in CH/2 registers; per channel the rows
+// are paired in time, P_t = (x[t-1], x[t]).
+template <int CH>
+struct PairRow {
+  uint32_t p[CH];  // per channel: (x[t-1], x[t])
+};
+__device__ __forceinline__ PairRow<4> pair_rows(u32x2 earlier, u32x2 later) {
+  PairRow<4> r;
+  pair_up(earlier.x, later.x, r.p[0], r.p[1]);
+  pair_up(earlier.y, later.y, r.p[2], r.p[3]);
+  return r;
+}
+__device__ __forceinline__ PairRow<2> pair_rows(uint32_t earlier,
+                                                uint32_t later) {
+  PairRow<2> r;
+  pair_up(earlier, later, r.p[0], r.p[1]);
+  return r;
+}
+__device__ __forceinline__ void conv_dot(const PairRow<2>& older,
+                                         const PairRow<2>& newer,
+                                         const ChanConst<2>& k,
+                                         float (&out)[2]) {
+  conv4_dot_x2(older.p, newer.p, k.w10, k.w32, k.bias, out);
+}
+__device__ __forceinline__ void conv_dot(const PairRow<4>& older,
+                                         const PairRow<4>& newer,
+                                         const ChanConst<4>& k,
+                                         float (&out)[4]) {
+  conv4_dot_x4(older.p, newer.p, k.w10, k.w32, k.bias, out);
+}
+// Whether this instantiation convolves packed rows with dot products.
+template <typename T, int CH, bool CONV>
+constexpr bool kPackedConv = CONV && sizeof(T) == 2 && (CH == 2 || CH == 4);
+
 
 // Where a wave's rows for one step live: descriptors based at the wave's first
 // token (clamped into the sequence) and the scalar row offset of each token,
@@ -326,9 +366,18 @@ __device__ __forceinline__ void phase1(
     const ChanConst<CH>& k, float (&a_)[KL][CH], float (&xn_)[KL][CH],
     float (&P)[CH], float (&H)[CH]) {
   using B = Buf<T, CH>;
+  constexpr bool PACKED = kPackedConv<T, CH, CONV>;
   float hist[3][CH];
+  PairRow<CH> pp2, pp1;  // PACKED: the pairs ending one and two rows back
+  typename B::Raw prev_row{};
+  if constexpr (PACKED) {
+    pp2 = pair_rows(tl.halo[2], tl.halo[1]);
+    pp1 = pair_rows(tl.halo[1], tl.halo[0]);
+    prev_row = tl.halo[0];
+  } else {
 #pragma unroll
-  for (int s = 0; s < 3; ++s) B::unpack(tl.halo[s], hist[s]);
+    for (int s = 0; s < 3; ++s) B::unpack(tl.halo[s], hist[s]);
+  }
   // The reload must follow the last read of the registers it overwrites;
   // without these fences the scheduler hoists it, old and new values overlap,
   // and the new tile needs register copies (and full waits) every step.
@@ -342,17 +391,28 @@ __device__ __forceinline__ void phase1(
 #pragma unroll
   for (int i = 0; i < KL; ++i) {
     float xv[CH], gxv[CH], gav[CH], xc[CH];
-    B::unpack(tl.x[i], xv);
+    PairRow<CH> pp0;
+    if constexpr (PACKED) {
+      pp0 = pair_rows(prev_row, tl.x[i]);
+      prev_row = tl.x[i];
+    } else {
+      B::unpack(tl.x[i], xv);
+    }
     if (!PLAIN) B::unpack(tl.gx[i], gxv);
     B::unpack(tl.ga[i], gav);
     __builtin_amdgcn_sched_barrier(0);
     load_token<T, CH, KL, PLAIN>(tl, i, next, voff);
     __builtin_amdgcn_sched_barrier(0);
-    if (CONV) {
+    if constexpr (PACKED) {
+      conv_dot(pp2, pp0, k, xc);
+      pp2 = pp1;
+      pp1 = pp0;
+      B::round(xc);  // the conv output is a module output: activation dtype
+    } else if (CONV) {
 #pragma unroll
       for (int ch = 0; ch < CH; ++ch) {
-        xc[ch] = conv4(xv[ch], hist[0][ch], hist[1][ch], hist[2][ch], k.w0[ch],
-                       k.w1[ch], k.w2[ch], k.w3[ch], k.bias[ch]);
+        xc[ch] = conv4_as<T>(xv[ch], hist[0][ch], hist[1][ch], hist[2][ch],
+                             k.w0[ch], k.w1[ch], k.w2[ch], k.w3[ch], k.bias[ch]);
         hist[2][ch] = hist[1][ch];
         hist[1][ch] = hist[0][ch];
         hist[0][ch] = xv[ch];
@@ -381,24 +441,29 @@ __device__ __forceinline__ void phase1_with_starts(
     const ChanConst<CH>& k, float (&a_)[KL][CH], float (&xn_)[KL][CH],
     float (&P)[CH], float (&H)[CH]) {
   using B = Buf<T, CH>;
+  constexpr bool PACKED = kPackedConv<T, CH, CONV>;
   float hist[3][CH];
+  typename B::Raw rows[3] = {};  // PACKED: rows[s] = x[t-1-s], still packed
 #pragma unroll
   for (int s = 0; s < 3; ++s)
 #pragma unroll
     for (int ch = 0; ch < CH; ++ch) hist[s][ch] = 0.0f;
   if (CONV && at.has_halo) {
 #pragma unroll
-    for (int s = 0; s < 3; ++s)  // hist[s] = x[first-1-s]
-      B::unpack(B::template load<0>(at.rhalo, voff,
-                                    (uint32_t)(2 - s) * at.row_bytes),
-                hist[s]);
+    for (int s = 0; s < 3; ++s) {  // hist[s] = x[first-1-s]
+      rows[s] =
+          B::template load<0>(at.rhalo, voff, (uint32_t)(2 - s) * at.row_bytes);
+      B::unpack(rows[s], hist[s]);
+    }
     // a document start at first-1 hides x[first-2], x[first-3]; one at
     // first-2 hides x[first-3]
     if (starts & 4u) {
+      rows[1] = rows[2] = typename B::Raw{};
 #pragma unroll
       for (int ch = 0; ch < CH; ++ch) hist[1][ch] = hist[2][ch] = 0.0f;
     }
     if (starts & 2u) {
+      rows[2] = typename B::Raw{};
 #pragma unroll
       for (int ch = 0; ch < CH; ++ch) hist[2][ch] = 0.0f;
     }
@@ -413,15 +478,24 @@ __device__ __forceinline__ void phase1_with_starts(
     const bool start = (starts >> (i + 3)) & 1u;
     const uint32_t so = at.soff(i);
     float xv[CH], gxv[CH], gav[CH], xc[CH];
-    B::unpack(B::template load<0>(at.rx, voff, so), xv);
+    const typename B::Raw xraw = B::template load<0>(at.rx, voff, so);
+    B::unpack(xraw, xv);
     if (!PLAIN) B::unpack(B::template load<0>(at.rgx, voff, so), gxv);
     B::unpack(B::template load<0>(at.rga, voff, so), gav);
-    if (CONV) {
+    if constexpr (PACKED) {
+      // the same two dot products per output as on the hot path
+      if (start) rows[0] = rows[1] = rows[2] = typename B::Raw{};
+      conv_dot(pair_rows(rows[2], rows[1]), pair_rows(rows[0], xraw), k, xc);
+      rows[2] = rows[1];
+      rows[1] = rows[0];
+      rows[0] = xraw;
+      B::round(xc);
+    } else if (CONV) {
 #pragma unroll
       for (int ch = 0; ch < CH; ++ch) {
         if (start) hist[0][ch] = hist[1][ch] = hist[2][ch] = 0.0f;
-        xc[ch] = conv4(xv[ch], hist[0][ch], hist[1][ch], hist[2][ch], k.w0[ch],
-                       k.w1[ch], k.w2[ch], k.w3[ch], k.bias[ch]);
+        xc[ch] = conv4_as<T>(xv[ch], hist[0][ch], hist[1][ch], hist[2][ch],
+                             k.w0[ch], k.w1[ch], k.w2[ch], k.w3[ch], k.bias[ch]);
         hist[2][ch] = hist[1][ch];
         hist[1][ch] = hist[0][ch];
         hist[0][ch] = xv[ch];
@@ -520,8 +594,17 @@ lru_scan_kernel(ScanArgs p) {
       k.w2[ch] = load_scalar(cw + 2 * W + c + ch);
       k.w3[ch] = load_scalar(cw + 3 * W + c + ch);
       k.bias[ch] = load_scalar((const T*)p.conv_b + c + ch);
+      if (sizeof(T) == 2) {
+        const uint16_t* cb = (const uint16_t*)p.conv_w;
+        k.w10[ch] = (uint32_t)cb[c + ch] | ((uint32_t)cb[W + c + ch] << 16);
+        k.w32[ch] = (uint32_t)cb[2 * W + c + ch] |
+                    ((uint32_t)cb[3 * W + c + ch] << 16);
+      } else {
+        k.w10[ch] = k.w32[ch] = 0u;
+      }
     } else {
       k.w0[ch] = k.w1[ch] = k.w2[ch] = k.w3[ch] = k.bias[ch] = 0.0f;
+      k.w10[ch] = k.w32[ch] = 0u;
     }
     if (PLAIN) {
       k.decay[ch] = 0.0f;
