@@ -691,10 +691,18 @@ lru_scan_kernel(ScanArgs p) {
 
     // exchange
     AggRow* const agg = agg0 + buf * nw;
+    if (!any) {  // past the end of the sequence: the identity pair
+      RG_RARE_BLOCK();
+#pragma unroll
+      for (int ch = 0; ch < CH; ++ch) {
+        P[ch] = 1.0f;
+        H[ch] = 0.0f;
+      }
+    }
 #pragma unroll
     for (int ch = 0; ch < CH; ++ch) {
-      agg[wave][lane][ch] = any ? P[ch] : 1.0f;
-      agg[wave][lane][CH + ch] = any ? H[ch] : 0.0f;
+      agg[wave][lane][ch] = P[ch];
+      agg[wave][lane][CH + ch] = H[ch];
     }
     lds_barrier();  // LDS only: prefetched rows and earlier stores stay in flight
     if (step > 0) {
@@ -710,7 +718,7 @@ lru_scan_kernel(ScanArgs p) {
     }
     if (SPLIT == kChunkSummary) {  // complete in the last wave only
 #pragma unroll
-      for (int ch = 0; ch < CH; ++ch) chunk_p[ch] *= any ? P[ch] : 1.0f;
+      for (int ch = 0; ch < CH; ++ch) chunk_p[ch] *= P[ch];
     }
 
     {
@@ -724,26 +732,23 @@ lru_scan_kernel(ScanArgs p) {
       if (SPLIT == kChunkReplay && !last_chunk) h_end = nullptr;
       float* const h_last_lane =
           (h_end && active && any && t0 + n_valid == T_len) ? h_end : nullptr;
-      float hw[CH];  // replay on a copy: a wave without tokens must hand the
-#pragma unroll       // carry on unchanged
-      for (int ch = 0; ch < CH; ++ch) hw[ch] = h[ch];
       if (SPLIT == kChunkSummary) {
         // no outputs to replay for: the wave's pair applied to its incoming
         // state is its final state (summaries are taken of whole steps only:
-        // the last chunk of a row, which may end inside a step, has none)
+        // the last chunk of a row, which may end inside a step, has none; a
+        // wave without tokens holds the identity pair)
 #pragma unroll
         for (int ch = 0; ch < CH; ++ch)
-          hw[ch] = __builtin_fmaf(P[ch], h[ch], H[ch]);
+          h[ch] = __builtin_fmaf(P[ch], h[ch], H[ch]);
         if (h_last_lane) {
 #pragma unroll
-          for (int ch = 0; ch < CH; ++ch) h_last_lane[ch] = hw[ch];
+          for (int ch = 0; ch < CH; ++ch) h_last_lane[ch] = h[ch];
         }
-      } else {
+      } else if (any) {
+        // (a wave without tokens hands the carry on unchanged)
         phase2<T, CH, KL>(ry, voff, row_bytes, n_valid, h_last_lane, a_, xn_,
-                          hw);
+                          h);
       }
-#pragma unroll
-      for (int ch = 0; ch < CH; ++ch) h[ch] = any ? hw[ch] : h[ch];
     }
     if (wave == nw - 1) {
 #pragma unroll
