@@ -221,6 +221,26 @@ def shader_clock_ghz(torch, iters=2000):
   return cycles / (ticks * 10.0) if ticks > 0 else None
 
 
+def prefill_clock_under_load(torch, fn):
+  """Shader clock while the single prefill kernel runs, from the counters its
+  workgroup (0, 0) keeps around its tile loop (rg_prefill_clock_probe): one
+  extra launch of fn() after the timed region.  None if fn() did not take that
+  kernel."""
+  import ctypes
+  from recurrentgemma_amd import _lib
+  lib = _lib.lib()
+  out = torch.zeros(2, dtype=torch.int64, device="cuda:0")
+  torch.cuda.synchronize()
+  lib.rg_prefill_clock_probe(ctypes.c_void_p(out.data_ptr()))
+  try:
+    fn()
+    torch.cuda.synchronize()
+  finally:
+    lib.rg_prefill_clock_probe(None)
+  cycles, ticks = (int(v) for v in out.cpu())
+  return cycles / (ticks * 10.0) if ticks > 0 else None
+
+
 def settle(torch, fn, cap_s=0.5, window=10, rel=0.01, min_launches=30):
   """Untimed launches of fn() until the GPU has left its idle clocks: stops
   when the median duration of the last `window` launches is within `rel` of
@@ -942,6 +962,7 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras,
   settle_launches = 0 if args.no_settle else settle(torch, step)
   elapsed, first_ms, second_ms = timed(step, steps, warmup, key="main")
   clock_ghz = shader_clock_ghz(torch)
+  clock_loaded = prefill_clock_under_load(torch, step) if esize == 2 else None
 
   tokens = B * T
   from recurrentgemma_amd import _lib
@@ -999,6 +1020,8 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras,
     roofline = figs["scan"]
   roofline["settle_launches"] = settle_launches
   roofline["shader_clock_ghz_after"] = clock_ghz
+  if path == "single":
+    roofline["shader_clock_ghz_under_load"] = clock_loaded
 
   cold = None
   if (extras or cold_too) and x.numel() * esize * 4 < (256 << 20):

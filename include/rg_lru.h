@@ -534,6 +534,14 @@ int rg_argmax_rows(const void* x, int64_t* out, int rows, int n, int dtype,
  * (out[2] is scratch).  bench.py reports it next to its timings, which scale
  * with that clock. */
 int rg_clock_probe(uint64_t* out, int iters, void* stream);
+/* The same for the clock UNDER the load of the single prefill kernel (its
+ * matrix instructions pull the clock below what a light probe reads): while
+ * `out` (2 x uint64 of device memory) is set, every rg_recurrent_prefill*
+ * / rg_recurrent_core launch that takes that kernel has its workgroup (0, 0)
+ * leave in out[0] the shader-clock cycles and in out[1] the 100 MHz ticks of
+ * its tile loop.  Process-wide; pass NULL to switch it off again (the state
+ * it starts in).  Measurement aid, no counterpart in the reference. */
+int rg_prefill_clock_probe(uint64_t* out);
 
 /* The linear layers around the recurrent and attention blocks for a decode
  * step (at most 64 rows), bf16: torch.nn.Linear (modules.py:579-601 linear_y /

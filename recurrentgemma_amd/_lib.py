@@ -29,6 +29,7 @@ _sz = ctypes.c_size_t
 SIGNATURES = {
     "rg_abi_version": (_i, []),
     "rg_clock_probe": (_i, [_vp, _i, _vp]),
+    "rg_prefill_clock_probe": (_i, [_vp]),
     "rg_last_error": (ctypes.c_char_p, []),
     "rg_conv1d_prefill": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i,
                                _i, _vp]),

@@ -84,6 +84,10 @@ size_t esize(int dtype) { return dtype == RG_DTYPE_F32 ? 4 : 2; }
 
 }  // namespace
 
+// rg_prefill_clock_probe: where the single prefill kernel leaves its cycle and
+// tick counts (null: nowhere)
+static std::atomic<uint64_t*> g_prefill_timing{nullptr};
+
 extern "C" {
 
 int rg_abi_version(void) { return RG_ABI_VERSION; }
@@ -447,6 +451,7 @@ static int recurrent_prefill_impl(const char* who, const void* x,
                 who, dtype, W, H, T);
   }
   rg::FusedArgs a{};
+  a.timing = g_prefill_timing.load(std::memory_order_relaxed);
   a.x = x;
   a.segpos = segpos;
   a.seg_kind = segpos_is_i64 ? 1 : 0;
@@ -869,6 +874,11 @@ int rg_soft_cap(const void* x, void* out, int64_t n, float cap, int dtype,
   RG_CHECK_PTR(out);
   return launch_status(
       __func__, rg::launch_soft_cap(x, out, n, cap, dtype, (hipStream_t)stream));
+}
+
+int rg_prefill_clock_probe(uint64_t* out) {
+  g_prefill_timing.store(out, std::memory_order_relaxed);
+  return RG_OK;
 }
 
 int rg_clock_probe(uint64_t* out, int iters, void* stream) {

@@ -116,6 +116,9 @@ struct FusedArgs {
   int chunks, tiles_per_chunk;
   float* ws_p;
   float* ws_h;
+  // or null: workgroup (0, 0) leaves here the shader-clock cycles and the
+  // 100 MHz ticks its tile loop took (rg_prefill_clock_probe)
+  uint64_t* timing;
 };
 
 struct StepArgs {

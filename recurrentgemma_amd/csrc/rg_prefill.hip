@@ -827,19 +827,43 @@ __device__ __forceinline__ void prefill_body(const FusedArgs& p,
         gate_block(it, 1, BI, acc1, m_cur, hook);
       if (__builtin_expect(cuts != 0, 0)) conv_rows_with_cuts(bn, half, cuts);
       wait_for_matrix_results();
-      if (half == 0) lds_barrier();
+      // Between the phases the waves hand each other conv outputs, written by
+      // ordinary LDS stores: the barrier waits for those alone.  (The
+      // compiler's workgroup fence on LDS also waits for the memory pipe's
+      // own LDS writes -- the raw rows of tile it+2 requested at the top of
+      // this tile -- which nobody reads before the end of the tile: half a
+      // tile is not always enough for them to arrive.)
+      if (half == 0)
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }
-    // the loads of tile it+2 were issued before this tile's y stores
+    // the loads of tile it+2 were issued before this tile's eight y stores
     if (MODE == kChunkSummary)
       wait_vmcnt<0>();
     else
-      wait_vmcnt<6>();
+      wait_vmcnt<8>();
     lds_barrier();
     m_cur = m_next;
   };
+  // (measurement aid: one workgroup notes how long its tile loop takes on the
+  // shader clock and on the constant 100 MHz counter -- their ratio is the
+  // clock the GPU runs this kernel at)
+  const bool timed = p.timing != nullptr && blockIdx.x == 0 && blockIdx.y == 0;
+  uint64_t clk0 = 0, tick0 = 0;
+  if (timed) {
+    clk0 = __builtin_readcyclecounter();
+    tick0 = __builtin_amdgcn_s_memrealtime();
+  }
   for (int it = tile_begin; it < tile_end; it += 2) {
     tile_body(std::integral_constant<int, 0>{}, it);
     if (it + 1 < tile_end) tile_body(std::integral_constant<int, 1>{}, it + 1);
+  }
+  if (timed) {
+    const uint64_t clk1 = __builtin_readcyclecounter();
+    const uint64_t tick1 = __builtin_amdgcn_s_memrealtime();
+    if (tid == 0) {
+      p.timing[0] = clk1 - clk0;
+      p.timing[1] = tick1 - tick0;
+    }
   }
   if (MODE != kChunkSummary) flush_y();  // the last sixteen tokens
 
