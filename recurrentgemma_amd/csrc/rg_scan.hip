@@ -364,7 +364,7 @@ template <typename T, int CH, int KL, bool CONV, bool FAST, bool PLAIN>
 __device__ __forceinline__ void phase1(
     Tile<T, CH, KL>& tl, const StepAddr<KL>& next, uint32_t voff,
     const ChanConst<CH>& k, float (&a_)[KL][CH], float (&xn_)[KL][CH],
-    float (&P)[CH], float (&H)[CH]) {
+    float (&P)[CH], float (&H)[CH], bool halo_from_memory) {
   using B = Buf<T, CH>;
   constexpr bool PACKED = kPackedConv<T, CH, CONV>;
   float hist[3][CH];
@@ -382,7 +382,9 @@ __device__ __forceinline__ void phase1(
   // without these fences the scheduler hoists it, old and new values overlap,
   // and the new tile needs register copies (and full waits) every step.
   __builtin_amdgcn_sched_barrier(0);
-  load_halo<T, CH, KL, CONV>(tl, next, voff);
+  // (the other waves get the next step's look-back rows from the wave before
+  // them, through LDS: see the exchange)
+  if (halo_from_memory) load_halo<T, CH, KL, CONV>(tl, next, voff);
 #pragma unroll
   for (int ch = 0; ch < CH; ++ch) {
     P[ch] = 1.0f;
@@ -569,6 +571,16 @@ lru_scan_kernel(ScanArgs p) {
   AggRow* const agg0 = reinterpret_cast<AggRow*>(lds_f);   // [2][nw]
   CarryRow* const carry_s =
       reinterpret_cast<CarryRow*>(lds_f + 2 * nw * kWave * 2 * CH);  // [2]
+  // The three look-back rows of a wave's conv are the last three rows of the
+  // wave before it: instead of reading them from memory a second time, every
+  // wave leaves the last three of the rows it has prefetched for the next
+  // step in LDS before the step's barrier and takes its neighbour's behind
+  // it, [2][nw][3][64].  Wave 0, whose look-back rows belong to the step
+  // before, keeps loading them.
+  typedef typename Buf<T, CH>::Raw RawRow;
+  RawRow* const halo_s = reinterpret_cast<RawRow*>(
+      lds_f + 2 * nw * kWave * 2 * CH + 2 * kWave * CH);
+  const bool share_halo = CONV && KL >= 3 && nw > 1;
   // tokens [t_lo, T_len) of the row are this workgroup's; everything below
   // treats T_len as the end of the sequence
   const int chunk = SPLIT == kWholeRow ? 0 : (int)blockIdx.y;
@@ -680,7 +692,8 @@ lru_scan_kernel(ScanArgs p) {
         step_addr<KL>(xrow, gxrow, garow, t0 + span, T_len, row_bytes);
     // next step's document starts: loaded now, looked at after this step
     const SegRaw seg_next = load_seg<KL, CONV>(p, row0, t0 + span, T_len, lane);
-    phase1<T, CH, KL, CONV, FAST, PLAIN>(tl, next, voff, k, a_, xn_, P, H);
+    phase1<T, CH, KL, CONV, FAST, PLAIN>(tl, next, voff, k, a_, xn_, P, H,
+                                         !share_halo || wave == 0);
     if (starts != 0u) {
       RG_RARE_BLOCK();
       const StepAddr<KL> cur =
@@ -704,7 +717,18 @@ lru_scan_kernel(ScanArgs p) {
       agg[wave][lane][ch] = P[ch];
       agg[wave][lane][CH + ch] = H[ch];
     }
+    if (share_halo) {  // tl.x holds the next step's rows by now
+      RawRow* const dst = halo_s + ((buf * nw + wave) * 3) * kWave + lane;
+#pragma unroll
+      for (int s = 0; s < 3; ++s) dst[s * kWave] = tl.x[KL - 1 - s];
+    }
     lds_barrier();  // LDS only: prefetched rows and earlier stores stay in flight
+    if (share_halo && wave > 0) {
+      const RawRow* const src =
+          halo_s + ((buf * nw + wave - 1) * 3) * kWave + lane;
+#pragma unroll
+      for (int s = 0; s < 3; ++s) tl.halo[s] = src[s * kWave];  // x[first-1-s]
+    }
     if (step > 0) {
 #pragma unroll
       for (int ch = 0; ch < CH; ++ch) h[ch] = carry_s[buf ^ 1][lane][ch];
@@ -807,12 +831,18 @@ hipError_t launch_t(const ScanArgs& a, hipStream_t s) {
   if (blocks > 0x7fffffff ||
       (int64_t)a.W * sizeof(T) * (KL + 3) >= (int64_t)kOutOfRange)
     return hipErrorInvalidValue;
-  const size_t lds = sizeof(float) * (2 * nw * kWave * 2 * CH + 2 * kWave * CH);
+  const size_t halo_rows =
+      CONV && KL >= 3 && nw > 1
+          ? (size_t)2 * nw * 3 * kWave * sizeof(typename Buf<T, CH>::Raw)
+          : 0;
+  const size_t lds =
+      sizeof(float) * (2 * nw * kWave * 2 * CH + 2 * kWave * CH) + halo_rows;
   auto kern = lru_scan_kernel<T, CH, KL, CONV, FAST, PLAIN, SPLIT>;
   // the limit is raised once, to what the largest workgroup of this
   // instantiation needs
   constexpr size_t lds_max =
-      sizeof(float) * (2 * kMaxNW * kWave * 2 * CH + 2 * kWave * CH);
+      sizeof(float) * (2 * kMaxNW * kWave * 2 * CH + 2 * kWave * CH) +
+      (size_t)2 * kMaxNW * 3 * kWave * sizeof(typename Buf<T, CH>::Raw);
   if (lds_max > 48 * 1024) {
     static OncePerDevice once;  // one per instantiation of this launcher
     hipError_t e = set_max_dynamic_lds(once, (const void*)kern, lds_max);
