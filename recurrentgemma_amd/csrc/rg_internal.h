@@ -248,6 +248,7 @@ void scan_split_plan(int B, int T, int W, int granule, int* chunks,
 // Chunk lengths are multiples of this for the kernel that handles (dtype, W).
 int scan_split_granule(int dtype, int W);
 hipError_t launch_block_prefill_bf16(const FusedArgs& a, hipStream_t s);
+hipError_t launch_block_prefill_teams_bf16(const FusedArgs& a, hipStream_t s);
 void prefill_chunk_plan(int B, int H, int T, int* chunks, int* tiles_per_chunk);
 // (row, head) pairs from which one workgroup per pair beats the gate GEMM +
 // scan pair (measured at W2560 and W4096, T512-8192: the two forms cross

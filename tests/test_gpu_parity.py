@@ -863,18 +863,25 @@ def test_recurrent_step_single_launch(B, W, H, in_place):
     assert torch.equal(ccd.cpu(), cco)
 
 
-def test_recurrent_prefill_without_packed_weights():
+@pytest.mark.parametrize("B,T,W,H,mean_doc,with_h0", [
+    (3, 150, 512, 2, 40, False), (2, 1000, 768, 3, 100, True),
+    (1, 31, 256, 1, 5, False), (2, 4096, 1024, 4, 500, True)])
+def test_recurrent_prefill_without_packed_weights(B, T, W, H, mean_doc, with_h0):
   """rg_recurrent_prefill with w_packed == NULL re-lays the gate weights out
-  inside the kernel: same result, bit for bit, as with the packed buffer."""
-  B, T, W, H = 3, 150, 512, 2
+  inside the kernel: same result, bit for bit, as with the packed buffer.
+
+  The two calls also run two different kernels -- with packed weights whole
+  rows go to the form with two waves per SIMD, without them to the form with
+  one -- so this is the check that the two forms compute the same thing."""
   p = R.make_params(W, H, torch.bfloat16, seed=61, gate_bias_std=0.5)
   P = {k: _dev(v) for k, v in p.items()}
   g = torch.Generator().manual_seed(62)
   x = _dev(torch.randn(B, T, W, generator=g).to(torch.bfloat16))
-  seg = _dev(helpers.document_positions(B, T, 40, seed=63))
+  seg = _dev(helpers.document_positions(B, T, mean_doc, seed=63))
+  h0 = _dev(torch.randn(B, W, generator=g)) if with_h0 else None
   y1, h1, c1 = ops.recurrent_prefill(x, seg, P["conv_w"], P["conv_b"],
                                      P["w_x"], P["b_x"], P["w_a"], P["b_a"],
-                                     P["a_param"])
+                                     P["a_param"], h0=h0, split=False)
   y2 = torch.empty_like(x)
   h2 = torch.empty(B, W, dtype=torch.float32, device=DEV)
   c2 = x.new_empty(B, 3, W)
@@ -882,7 +889,7 @@ def test_recurrent_prefill_without_packed_weights():
   _lib.check(_lib.lib().rg_recurrent_prefill(
       ptr(x), ptr(seg), 1, ptr(P["conv_w"]), ptr(P["conv_b"]), ptr(P["w_x"]),
       ptr(P["b_x"]), ptr(P["w_a"]), ptr(P["b_a"]), None, ptr(P["a_param"]),
-      None, ptr(y2), ptr(h2), ptr(c2), B, T, W, H, 1,
+      ptr(h0) if with_h0 else None, ptr(y2), ptr(h2), ptr(c2), B, T, W, H, 1,
       torch.cuda.current_stream().cuda_stream))
   assert torch.equal(y1, y2) and torch.equal(h1, h2) and torch.equal(c1, c2)
 
