@@ -469,7 +469,7 @@ def run_modules(args, torch, rg, R, wl):
        "gates_mfma_bf16_kernel, one matrix (rg_block_diag_linear)",
        lambda: lru.input_gate(x), 2 * n * 2),
       ("RGLRU.forward",
-       "block_prefill_bf16_kernel without conv weights (rg_recurrent_core)",
+       "block_prefill_teams_bf16_kernel without conv weights (rg_recurrent_core)",
        lambda: lru(x, seg), 2 * n * 2),
   ]
 
@@ -998,10 +998,12 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras,
     achieved = algo / (first_ms * 1e-3) / 1e9
     traffic, source = measured_traffic(workload, "single")
     roofline = {
-        "kernel": ("block_prefill_bf16_kernel (conv + gate GEMMs + gates + scan)"
-                   + (": two launches (chunk 0 + summaries of the chunks "
-                      "after it; replay of chunks 1..n-1); avg_launch_ms "
-                      "covers both" if chunked else "")),
+        "kernel": ("block_prefill_bf16_kernel (conv + gate GEMMs + gates + "
+                   "scan): two launches (chunk 0 + summaries of the chunks "
+                   "after it; replay of chunks 1..n-1); avg_launch_ms covers "
+                   "both" if chunked else
+                   "block_prefill_teams_bf16_kernel (conv + gate GEMMs + gates "
+                   "+ scan, two waves per SIMD)"),
         "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
         "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
         "traffic": traffic, "traffic_source": source,
