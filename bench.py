@@ -930,8 +930,9 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras,
   chunked = esize == 2 and ops.recurrent_prefill_chunked(B, T, W, H)
   path = args.path
   if path == "auto":
+    many_short = (B * H > 512 and T <= 16) or (B * H > 1024 and T <= 32)
     path = ("single" if ops.recurrent_prefill_supported(x, H)
-            and (B * H >= 129 or chunked) else "split")
+            and not many_short else "split")
   if args.path == "auto":
     step = step_core
   else:
@@ -998,12 +999,11 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras,
     achieved = algo / (first_ms * 1e-3) / 1e9
     traffic, source = measured_traffic(workload, "single")
     roofline = {
-        "kernel": ("block_prefill_bf16_kernel (conv + gate GEMMs + gates + "
-                   "scan): two launches (chunk 0 + summaries of the chunks "
-                   "after it; replay of chunks 1..n-1); avg_launch_ms covers "
-                   "both" if chunked else
-                   "block_prefill_teams_bf16_kernel (conv + gate GEMMs + gates "
-                   "+ scan, two waves per SIMD)"),
+        "kernel": ("block_prefill_teams_bf16_kernel (conv + gate GEMMs + gates "
+                   "+ scan, two waves per SIMD)"
+                   + (": two launches (chunk 0 + summaries of the chunks "
+                      "after it; replay of chunks 1..n-1); avg_launch_ms "
+                      "covers both" if chunked else "")),
         "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS,
         "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
         "traffic": traffic, "traffic_source": source,

@@ -553,14 +553,18 @@ static CorePlan core_plan(int B, int T, int W, int H, int dtype) {
                     (int64_t)T * W * 2 < (int64_t)0x7fffffff;
   const size_t chunk_bytes =
       fits ? rg_recurrent_prefill_split_workspace_bytes(B, T, W, H) : 0;
-  // Many short rows are the exception: with more workgroups than CUs each CU
-  // loads a head's 256 KB of gate weights again for every pair it runs, and
-  // below one 64-token tile per row that outweighs the rest (measured, W2560
-  // H10, 640 pairs: T32 54 us against 47 us for gate GEMM + scan, T64 57
-  // against 61; 2560 pairs, T1: 160 against 29).
-  const bool many_short_rows = (int64_t)B * H > 256 && T < 64;
-  p.single = fits && !many_short_rows &&
-             ((int64_t)B * H >= rg::kPrefillMinGroups || chunk_bytes > 0);
+  // The single kernel serves every such shape (measured against the gate GEMM
+  // + scan pair at W2560 H10, 10-640 (row, head) pairs, T32-4096: 10-50 %
+  // ahead everywhere, whole rows or chunks) but many very short rows: with
+  // more workgroups than CUs each CU loads a head's 256 KB of gate weights
+  // again for every pair it runs, and with a few tokens per row that
+  // outweighs the rest (us, single / pair: 640 pairs T1 37/28, T16 40/36, T32
+  // 42/48; 1280 pairs T16 68/47, T32 70/66, T48 72/85; 2560 pairs T1 122/28,
+  // T32 136/112, T48 138/146).
+  const int64_t pairs = (int64_t)B * H;
+  const bool many_short_rows =
+      (pairs > 512 && T <= 16) || (pairs > 1024 && T <= 32);
+  p.single = fits && !many_short_rows;
   if (p.single) {
     p.split_bytes = chunk_bytes;
   } else {
@@ -612,7 +616,10 @@ int rg_recurrent_core(const void* x, const void* gate_branch,
                 __func__, need, workspace ? workspace_bytes : (size_t)0);
   if (p.single) {
     // rows in chunks write the plain output; the join follows as its own pass
-    const bool join_inside = gate_branch != nullptr && p.split_bytes == 0;
+    // (and so do whole rows of few (row, head) pairs: the kernel form that
+    // has the join is the slower one, worth it only with all CUs at work)
+    const bool join_inside = gate_branch != nullptr && p.split_bytes == 0 &&
+                             (int64_t)B * H >= rg::kPrefillJoinMinGroups;
     const int rc = recurrent_prefill_impl(
         __func__, x, segpos, segpos_is_i64, conv_w, conv_b, w_x, b_x, w_a, b_a,
         w_packed, a_param, h0, join_inside ? gate_branch : nullptr, out, h_last,

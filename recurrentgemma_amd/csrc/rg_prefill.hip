@@ -976,11 +976,11 @@ void prefill_chunk_plan(int B, int H, int T, int* chunks, int* tiles_per_chunk) 
   *chunks = 1;
   *tiles_per_chunk = ntiles;
   const int64_t groups = (int64_t)B * H;
-  // (below about 1500 tokens the two prologues and the second launch cost
-  // what the idle CUs would: measured at W2560 H10, 10-120 pairs, chunks
-  // against the gate GEMM + scan pair: T768 +10..25 %, T1024 even, T2048
-  // -5..20 %, T4096 -10..25 %)
-  if (groups * 2 > 256 || ntiles < 24) return;
+  // (measured at W2560 H10 with the two-wave kernel, us, chunks / whole rows:
+  // T384 10-120 pairs even; T512 10 pairs 35/43, 80 pairs 45/49, 120 pairs
+  // 54/51; T768 10 pairs 37/61, 120 pairs 69/73; T1024 10 pairs 38/78, 120
+  // pairs 89/92; T4096 10 pairs 58/288, 80 pairs 231/298, 120 pairs 307/314)
+  if (groups > 128 || ntiles < 8 || (ntiles < 12 && groups > 96)) return;
   int want = (int)(256 / groups) + 1;  // workgroups per launch and row, + 1
   if (want > ntiles / 2) want = ntiles / 2;
   if (want < 3) return;
@@ -996,10 +996,9 @@ hipError_t launch_block_prefill_bf16(const FusedArgs& a, hipStream_t s) {
   // (checked by the caller)
   const int64_t blocks = (int64_t)a.B * a.H;
   if (blocks <= 0 || blocks > 0x7fffffff) return hipErrorInvalidValue;
-  // whole rows with re-laid-out weights and a plain y: the form with two
-  // waves per SIMD (rg_prefill_teams.hip), about a tenth faster
-  if (a.chunks <= 1 && !a.gate_branch && a.w_packed)
-    return launch_block_prefill_teams_bf16(a, s);
+  // with re-laid-out weights and a plain y: the form with two waves per SIMD
+  // (rg_prefill_teams.hip), about a tenth faster
+  if (!a.gate_branch && a.w_packed) return launch_block_prefill_teams_bf16(a, s);
   if (a.chunks <= 1) return launch_pass<kPassWholeRows>(a, 1, s);
   if (a.chunks < 3 || a.chunks > 65535) return hipErrorInvalidValue;
   hipError_t e = launch_pass<kPassFirst>(a, a.chunks - 1, s);

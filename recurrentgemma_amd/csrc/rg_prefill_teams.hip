@@ -180,8 +180,20 @@ __device__ __forceinline__ void phase_barrier() {
   __builtin_amdgcn_sched_barrier(0);
 }
 
-__global__ void __launch_bounds__(kThreads) block_prefill_teams_bf16_kernel(
-    FusedArgs p) {
+// What one workgroup does with its tiles.  A row cut into chunks takes two
+// launches: the first runs chunk 0 as kChunkHead and chunks 1 .. n-2 as
+// kChunkSummary side by side, the second chunks 1 .. n-1 as kChunkReplay,
+// each starting from the summaries of the chunks before it.
+enum PrefillMode {
+  kWholeRow = 0,      // a whole row of one head: y, h_last, conv state
+  kChunkSummary = 1,  // a chunk from a zero state: (prod a, h_end), no y
+  kChunkReplay = 2,   // a chunk from its incoming state: y, ...
+  kChunkHead = 3      // chunk 0 from h0: y, and its end state as a summary
+};
+
+template <int MODE>
+__device__ __forceinline__ void prefill_teams_body(const FusedArgs& p,
+                                                   const int chunk) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   lds_byte* const lds3 = (lds_byte*)lds_raw;
 
@@ -194,7 +206,11 @@ __global__ void __launch_bounds__(kThreads) block_prefill_teams_bf16_kernel(
   const int h = blockIdx.x % p.H;
   const int T_len = p.T;
   const int64_t W = p.W;
-  const int ntiles = (T_len + kTM - 1) / kTM;
+  const int ntiles = (T_len + kTM - 1) / kTM;  // of the whole row
+  const int tile_begin = MODE == kWholeRow ? 0 : chunk * p.tiles_per_chunk;
+  int tile_end = MODE == kWholeRow ? ntiles : tile_begin + p.tiles_per_chunk;
+  if (tile_end > ntiles) tile_end = ntiles;
+  const bool last_chunk = tile_end == ntiles;
   const bool upper = lane >= 32;
   const int n0 = wave * 32;  // first channel of this wave in the head
 
@@ -242,8 +258,8 @@ __global__ void __launch_bounds__(kThreads) block_prefill_teams_bf16_kernel(
   const uint32_t seq_bytes = (uint32_t)T_len * row_bytes;  // < 2^31 (launcher)
   const __amdgpu_buffer_rsrc_t rx =
       make_rsrc((const char*)p.x + (int64_t)b * seq_bytes, seq_bytes);
-  const __amdgpu_buffer_rsrc_t ry =
-      make_rsrc((char*)p.y + (int64_t)b * seq_bytes, seq_bytes);
+  const __amdgpu_buffer_rsrc_t ry = make_rsrc(
+      (char*)p.y + (int64_t)b * seq_bytes, MODE == kChunkSummary ? 0 : seq_bytes);
   const bool seg_is64 = p.seg_kind == kSegI64;
   const uint32_t seg_esize = seg_is64 ? 8u : 4u;
   const __amdgpu_buffer_rsrc_t rseg =
@@ -408,7 +424,20 @@ __global__ void __launch_bounds__(kThreads) block_prefill_teams_bf16_kernel(
   const float decay =
       (-8.0f * kLog2e) *
       softplus_precise(bf16_bits_to_f32(((const uint16_t*)p.a_param)[ch]));
-  float hc = p.h0 ? p.h0[(int64_t)b * W + ch] : 0.0f;
+  float hc = 0.0f;    // carried state of this lane's channel
+  float prod = 1.0f;  // kChunkSummary: product of a over this lane's tokens
+  if (MODE == kChunkReplay) {
+    // state at the start of this chunk from the summaries of the chunks
+    // before it: h <- P[k] h + H[k] (the scan operator of
+    // recurrentgemma/jax/scan.py:161-187 over chunks); chunk 0 has P = 0 and
+    // H = its end state
+    const float* sp = p.ws_p + (int64_t)b * p.chunks * W + ch;
+    const float* sh = p.ws_h + (int64_t)b * p.chunks * W + ch;
+    for (int k = 0; k < chunk; ++k)
+      hc = __builtin_fmaf(sp[(int64_t)k * W], hc, sh[(int64_t)k * W]);
+  } else if ((MODE == kWholeRow || MODE == kChunkHead) && p.h0) {
+    hc = p.h0[(int64_t)b * W + ch];
+  }
   f32x16 acc_x, acc_a;
   // conv outputs of the block in phase G, this lane's tokens, as floats
   uint32_t xr[16];
@@ -416,7 +445,7 @@ __global__ void __launch_bounds__(kThreads) block_prefill_teams_bf16_kernel(
   uint32_t y_pending_row = kBufferOutOfRange;
   // start masks of the tile before the current G block's, of its own, and of
   // the next
-  uint64_t m_prev = 0, m_cur, m_next;
+  uint64_t m_prev, m_cur, m_next;
 
   // gate arithmetic on accumulator elements [i0, i1), in place: the input
   // gate's sigmoid; a = exp2(sigmoid(recurrence gate) * decay)
@@ -560,13 +589,18 @@ __global__ void __launch_bounds__(kThreads) block_prefill_teams_bf16_kernel(
         hh = __builtin_fmaf(av[q], hh, xn[q]);
         hv[q] = hh;
       }
-      const uint32_t y01 = pack_bf16x2(hv[0], hv[1]);
-      const uint32_t y23 = pack_bf16x2(hv[2], hv[3]);
       {
         const auto sw = __builtin_amdgcn_permlane32_swap(
             __float_as_uint(hh), __float_as_uint(hh), false, false);
         hc = __uint_as_float(sw[1]);  // all lanes: end value of 32-63
       }
+      if (MODE == kChunkSummary) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) prod *= av[q];
+        continue;
+      }
+      const uint32_t y01 = pack_bf16x2(hv[0], hv[1]);
+      const uint32_t y23 = pack_bf16x2(hv[2], hv[3]);
       // the four tokens into the wave's patch: the low halves of the packed
       // pairs, and the high halves as they are
       const uint32_t pw = patch_w_lane + (8 * (g & 1)) * kPatchStride;
@@ -603,14 +637,16 @@ __global__ void __launch_bounds__(kThreads) block_prefill_teams_bf16_kernel(
   };
 
   // ---- prologue -------------------------------------------------------------
-  fetch_seg(0);
-  m_cur = start_mask(0);
-  fetch_seg(1);
-  m_next = start_mask(1);
+  fetch_seg(tile_begin - 1);
+  m_prev = start_mask(tile_begin - 1);
+  fetch_seg(tile_begin);
+  m_cur = start_mask(tile_begin);
+  fetch_seg(tile_begin + 1);
+  m_next = start_mask(tile_begin + 1);
 #pragma unroll
   for (int j = 0; j < kRawLoadsPerWave; ++j) {
-    dma_tile(0, j);
-    dma_tile(1, j);
+    dma_tile(tile_begin, j);
+    dma_tile(tile_begin + 1, j);
   }
   wait_vmcnt<0>();
   __syncthreads();  // conv table, raw tiles
@@ -625,12 +661,12 @@ __global__ void __launch_bounds__(kThreads) block_prefill_teams_bf16_kernel(
   }
   {
     ConvRows cr;
-    conv_load(0, cr);
-    conv_with_cuts(cr, conv_cuts(0, m_cur, m_prev));
+    conv_load(2 * tile_begin, cr);
+    conv_with_cuts(cr, conv_cuts(2 * tile_begin, m_cur, m_prev));
   }
   phase_barrier();
 
-  const bool timed = p.timing != nullptr && blockIdx.x == 0;
+  const bool timed = p.timing != nullptr && blockIdx.x == 0 && blockIdx.y == 0;
   uint64_t clk0 = 0, tick0 = 0;
   if (timed) {
     clk0 = __builtin_readcyclecounter();
@@ -640,7 +676,7 @@ __global__ void __launch_bounds__(kThreads) block_prefill_teams_bf16_kernel(
   if (team == 1) phase_barrier();
   // (whole tiles: a block past the end of the sequence is all identity, and
   // its stores fall outside the descriptor)
-  for (int kb = 0; kb < 2 * ntiles; kb += 2) {
+  for (int kb = 2 * tile_begin; kb < 2 * tile_end; kb += 2) {
     phase_m(kb, std::false_type{});
     phase_barrier();
     phase_g(kb, std::false_type{});
@@ -654,7 +690,7 @@ __global__ void __launch_bounds__(kThreads) block_prefill_teams_bf16_kernel(
   if (timed) {
     const uint64_t clk1 = __builtin_readcyclecounter();
     const uint64_t tick1 = __builtin_amdgcn_s_memrealtime();
-    if (tid == 0 && blockIdx.x == 0) {
+    if (tid == 0) {
       p.timing[0] = clk1 - clk0;
       p.timing[1] = tick1 - tick0;
     }
@@ -662,6 +698,29 @@ __global__ void __launch_bounds__(kThreads) block_prefill_teams_bf16_kernel(
   buffer_store_16(y_pending[0], ry, y_lane_bytes, y_pending_row);
   buffer_store_16(y_pending[1], ry, y_lane_bytes, y_pending_row + 16u * row_bytes);
 
+  if (MODE == kChunkSummary) {
+    // this chunk from a zero state: h_end = prod(a) * h_in + hc
+    const auto sw = __builtin_amdgcn_permlane32_swap(
+        __float_as_uint(prod), __float_as_uint(prod), false, false);
+    const float total = __uint_as_float(sw[0]) * __uint_as_float(sw[1]);
+    if (!upper) {
+      const int64_t at = ((int64_t)b * p.chunks + chunk) * W + ch;
+      p.ws_p[at] = total;
+      p.ws_h[at] = hc;
+    }
+    return;
+  }
+  if (MODE == kChunkHead) {
+    // whatever came before the row is in hc already: a summary with a zero
+    // product makes the replay take hc as the next chunk's start
+    if (!upper) {
+      const int64_t at = (int64_t)b * p.chunks * W + ch;
+      p.ws_p[at] = 0.0f;
+      p.ws_h[at] = hc;
+    }
+    return;
+  }
+  if (!last_chunk) return;
   if (p.h_last && !upper) p.h_last[(int64_t)b * W + ch] = hc;
 
   // Masked conv state: rows T-3..T-1 of x, each zeroed if a document starts in
@@ -684,19 +743,48 @@ __global__ void __launch_bounds__(kThreads) block_prefill_teams_bf16_kernel(
   }
 }
 
+enum PrefillPass { kPassWholeRows = 0, kPassFirst = 1, kPassReplay = 2 };
+
+// blockIdx.x: (row, head); blockIdx.y: which chunk (kPassFirst: chunk 0 with
+// its outputs beside the summaries of chunks 1 .. n-2; kPassReplay: chunks
+// 1 .. n-1).
+template <int PASS>
+__global__ void __launch_bounds__(kThreads) block_prefill_teams_bf16_kernel(
+    FusedArgs p) {
+  if (PASS == kPassWholeRows) {
+    prefill_teams_body<kWholeRow>(p, 0);
+  } else if (PASS == kPassReplay) {
+    prefill_teams_body<kChunkReplay>(p, (int)blockIdx.y + 1);
+  } else if (blockIdx.y == 0) {
+    prefill_teams_body<kChunkHead>(p, 0);
+  } else {
+    prefill_teams_body<kChunkSummary>(p, (int)blockIdx.y);
+  }
+}
+
+template <int PASS>
+hipError_t launch_teams_pass(const FusedArgs& a, int grid_y, hipStream_t s) {
+  static OncePerDevice once;
+  hipError_t e = set_max_dynamic_lds(
+      once, (const void*)block_prefill_teams_bf16_kernel<PASS>, kTeamsLdsBytes);
+  if (e != hipSuccess) return e;
+  block_prefill_teams_bf16_kernel<PASS>
+      <<<dim3((unsigned)(a.B * a.H), (unsigned)grid_y), kThreads, kTeamsLdsBytes,
+         s>>>(a);
+  return hipGetLastError();
+}
+
 }  // namespace
 
 hipError_t launch_block_prefill_teams_bf16(const FusedArgs& a, hipStream_t s) {
   const int64_t blocks = (int64_t)a.B * a.H;
   if (blocks <= 0 || blocks > 0x7fffffff) return hipErrorInvalidValue;
-  if (a.chunks > 1 || a.gate_branch || !a.w_packed) return hipErrorInvalidValue;
-  static OncePerDevice once;
-  hipError_t e = set_max_dynamic_lds(
-      once, (const void*)block_prefill_teams_bf16_kernel, kTeamsLdsBytes);
+  if (a.gate_branch || !a.w_packed) return hipErrorInvalidValue;
+  if (a.chunks <= 1) return launch_teams_pass<kPassWholeRows>(a, 1, s);
+  if (a.chunks < 3 || a.chunks > 65535) return hipErrorInvalidValue;
+  hipError_t e = launch_teams_pass<kPassFirst>(a, a.chunks - 1, s);
   if (e != hipSuccess) return e;
-  block_prefill_teams_bf16_kernel<<<dim3((unsigned)blocks), kThreads,
-                                    kTeamsLdsBytes, s>>>(a);
-  return hipGetLastError();
+  return launch_teams_pass<kPassReplay>(a, a.chunks - 1, s);
 }
 
 }  // namespace rg

@@ -78,15 +78,14 @@ def recurrent_core(conv_1d: layers.Conv1D, rg_lru: layers.RGLRU, x,
     y, h = rg_lru(xc, segment_pos,
                   None if cache is None else cache.rg_lru_state, return_cache)
   else:
-    # One call; the library picks the kernels (rg_recurrent_core): one
-    # workgroup per (row, head) -- or per chunk of one -- where there are
-    # enough of them to fill the GPU (from 129 pairs the single kernel is
-    # 20-25 % ahead of the gate GEMM + scan pair, which spreads over more CUs
-    # below that; long rows of few pairs are cut into chunks), and the join
-    # with the gate branch inside that kernel for whole rows (at B16 T8192
-    # W4096: 1.15 ms against 0.91 + 0.40 ms apart; with rows in chunks it would
-    # lengthen the one workgroup per row that produces outputs in the first
-    # launch while the others only summarise, so it stays a pass of its own).
+    # One call; the library picks the kernels (rg_recurrent_core): for bf16
+    # and 256-wide heads the single-launch kernel, one workgroup per (row,
+    # head) or -- rows of few pairs -- per chunk of one (many rows of a few
+    # tokens and every other dtype or head width: gate GEMM + scan), and the
+    # join with the gate branch inside that kernel for whole rows of at least
+    # 129 pairs (with rows in chunks it would lengthen the one workgroup per
+    # row that produces outputs in the first launch while the others only
+    # summarise, so there it stays a pass of its own).
     if compiled.tracing():
       y, h, conv_state = torch.ops.recurrentgemma_amd.recurrent_core(
           x, segment_pos, conv_1d.w, conv_1d.b, rg_lru.input_gate.w,

@@ -894,6 +894,42 @@ def test_recurrent_prefill_without_packed_weights(B, T, W, H, mean_doc, with_h0)
   assert torch.equal(y1, y2) and torch.equal(h1, h2) and torch.equal(c1, c2)
 
 
+@pytest.mark.parametrize("B,T,W,H,mean_doc,with_h0", [
+    (1, 8192, 2560, 10, 0, False), (4, 4096, 512, 2, 300, True),
+    (2, 3000, 768, 3, 50, True)])
+def test_recurrent_prefill_in_chunks_without_packed_weights(B, T, W, H,
+                                                            mean_doc, with_h0):
+  """Rows cut into chunks (rg_recurrent_prefill_split): with and without the
+  packed weights, i.e. through the kernel form with two waves per SIMD and
+  the form with one -- same chunk plan, same arithmetic, same bits."""
+  lib = _lib.lib()
+  need = lib.rg_recurrent_prefill_split_workspace_bytes(B, T, W, H)
+  assert need > 0, "this shape is meant to be cut into chunks"
+  p = R.make_params(W, H, torch.bfloat16, seed=71, gate_bias_std=0.5)
+  P = {k: _dev(v) for k, v in p.items()}
+  g = torch.Generator().manual_seed(72)
+  x = _dev(torch.randn(B, T, W, generator=g).to(torch.bfloat16))
+  if mean_doc:
+    seg = _dev(helpers.document_positions(B, T, mean_doc, seed=73))
+  else:
+    seg = _dev(torch.arange(T, dtype=torch.int64).repeat(B, 1))
+  h0 = _dev(torch.randn(B, W, generator=g)) if with_h0 else None
+  y1, h1, c1 = ops.recurrent_prefill(x, seg, P["conv_w"], P["conv_b"],
+                                     P["w_x"], P["b_x"], P["w_a"], P["b_a"],
+                                     P["a_param"], h0=h0, split=True)
+  y2 = torch.empty_like(x)
+  h2 = torch.empty(B, W, dtype=torch.float32, device=DEV)
+  c2 = x.new_empty(B, 3, W)
+  ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+  ptr = lambda t: t.data_ptr()
+  _lib.check(lib.rg_recurrent_prefill_split(
+      ptr(x), ptr(seg), 1, ptr(P["conv_w"]), ptr(P["conv_b"]), ptr(P["w_x"]),
+      ptr(P["b_x"]), ptr(P["w_a"]), ptr(P["b_a"]), None, ptr(P["a_param"]),
+      ptr(h0) if with_h0 else None, ptr(y2), ptr(h2), ptr(c2), ptr(ws), need,
+      B, T, W, H, 1, torch.cuda.current_stream().cuda_stream))
+  assert torch.equal(y1, y2) and torch.equal(h1, h2) and torch.equal(c1, c2)
+
+
 def test_recurrent_core_picks_single_launch():
   """With enough (row, head) pairs recurrent_core runs prefill as one launch
   and decode as one launch; both against the oracle, chained."""
@@ -920,11 +956,15 @@ def test_recurrent_core_picks_single_launch():
 @pytest.mark.parametrize("dtype,B,T,W,H", [
     (torch.float32, 1, 512, 2560, 10),    # float32: gate GEMM + scan in chunks
     (torch.float32, 3, 70, 384, 3),       # 128-wide heads, generic GEMM
-    (torch.bfloat16, 2, 300, 512, 2),     # few pairs, short rows: two kernels
-    (torch.bfloat16, 70, 130, 512, 2),    # 140 pairs: single kernel, whole rows
+    (torch.bfloat16, 2, 300, 512, 2),     # few pairs, short rows: single
+                                          # kernel, whole rows, join apart
+    (torch.bfloat16, 70, 130, 512, 2),    # 140 pairs: single kernel, whole
+                                          # rows, join inside
     (torch.bfloat16, 1, 2048, 512, 2),    # long rows of few pairs: chunks
+    (torch.bfloat16, 2, 600, 512, 2),     # ... from 512 tokens on
     (torch.bfloat16, 2, 65, 384, 3),      # bf16, 128-wide heads
-    (torch.bfloat16, 140, 5, 512, 2),     # 280 pairs of 5 tokens: two kernels
+    (torch.bfloat16, 300, 5, 512, 2),     # 600 pairs of 5 tokens: two kernels
+    (torch.bfloat16, 140, 5, 512, 2),     # 280 pairs of 5: single kernel
     (torch.bfloat16, 140, 64, 512, 2),    # ... of 64: single kernel
 ])
 @pytest.mark.parametrize("joined", [False, True])
@@ -943,12 +983,12 @@ def test_recurrent_core_entry_equals_its_parts(dtype, B, T, W, H, joined):
   y, h, c = ops.recurrent_core(x, seg, P["conv_w"], P["conv_b"], P["w_x"],
                                P["b_x"], P["w_a"], P["b_a"], P["a_param"],
                                h0=h0, gate_branch=gate)
-  single = (dtype == torch.bfloat16 and W // H == 256 and
-            not (B * H > 256 and T < 64) and
-            (B * H >= 129 or ops.recurrent_prefill_chunked(B, T, W, H)))
+  many_short = (B * H > 512 and T <= 16) or (B * H > 1024 and T <= 32)
+  single = dtype == torch.bfloat16 and W // H == 256 and not many_short
   if single:
     chunked = ops.recurrent_prefill_chunked(B, T, W, H)
     assert (need > 0) == chunked
+    assert chunked == (B * H <= 128 and T > 448)
     y2, h2, c2 = ops.recurrent_prefill(
         x, seg, P["conv_w"], P["conv_b"], P["w_x"], P["b_x"], P["w_a"],
         P["b_a"], P["a_param"], h0=h0)

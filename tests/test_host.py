@@ -166,15 +166,31 @@ def test_c_side_validation_without_launch():
           lib.rg_recurrent_prefill_split_workspace_bytes(1, 8192, 2560, 10))
   assert (lib.rg_recurrent_core_workspace_bytes(1, 512, 2560, 10, 0) ==
           2 * 512 * 2560 * 4 + lib.rg_scan_split_workspace_bytes(1, 512, 2560))
-  assert lib.rg_recurrent_core_workspace_bytes(2, 100, 512, 2, 1) == 2 * 2 * 100 * 512 * 2
+  # bf16 with 256-wide heads: the single kernel whatever the number of rows ...
+  assert lib.rg_recurrent_core_workspace_bytes(2, 100, 512, 2, 1) == 0
+  # ... other head widths: the two-kernel form
+  assert lib.rg_recurrent_core_workspace_bytes(2, 100, 512, 4, 1) == 2 * 2 * 100 * 512 * 2
   assert lib.rg_recurrent_core_workspace_bytes(2, 100, 512, 3, 1) == 0  # W % H
-  # many short rows: more (row, head) pairs than CUs and less than a tile each
-  # take the two-kernel form (both gates' pre-activations in the workspace)
+  # many very short rows: twice as many (row, head) pairs as CUs and a few
+  # tokens each take the two-kernel form (both gates' pre-activations in the
+  # workspace)
   assert lib.rg_recurrent_core_workspace_bytes(256, 1, 4096, 16, 1) == (
       2 * 256 * 4096 * 2)
+  assert lib.rg_recurrent_core_workspace_bytes(256, 32, 4096, 16, 1) == (
+      2 * 256 * 32 * 4096 * 2)
+  assert lib.rg_recurrent_core_workspace_bytes(256, 33, 4096, 16, 1) == 0
+  assert lib.rg_recurrent_core_workspace_bytes(32, 16, 4096, 16, 1) == 0
+  assert lib.rg_recurrent_core_workspace_bytes(33, 16, 4096, 16, 1) == (
+      2 * 33 * 16 * 4096 * 2)
   assert lib.rg_recurrent_core_workspace_bytes(256, 64, 4096, 16, 1) == 0
+  # rows in chunks: from 512 tokens on for at most 128 pairs
+  assert lib.rg_recurrent_prefill_split_workspace_bytes(1, 512, 2560, 10) > 0
+  assert lib.rg_recurrent_prefill_split_workspace_bytes(1, 448, 2560, 10) == 0
+  assert lib.rg_recurrent_prefill_split_workspace_bytes(12, 512, 2560, 10) == 0
+  assert lib.rg_recurrent_prefill_split_workspace_bytes(12, 768, 2560, 10) > 0
+  assert lib.rg_recurrent_prefill_split_workspace_bytes(13, 4096, 2560, 10) == 0
   rc = lib.rg_recurrent_core(ok, None, ok, 1, ok, ok, ok, ok, ok, ok, None, ok,
-                             None, ok, None, None, None, 0, 2, 100, 512, 2, 1,
+                             None, ok, None, None, None, 0, 2, 100, 512, 4, 1,
                              None)
   assert rc == -4 and b"rg_recurrent_core: workspace" in lib.rg_last_error()
   rc = lib.rg_recurrent_core(ok, ok, ok, 1, ok, ok, ok, ok, ok, ok, None, ok,
