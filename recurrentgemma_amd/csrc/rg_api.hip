@@ -616,10 +616,7 @@ int rg_recurrent_core(const void* x, const void* gate_branch,
                 __func__, need, workspace ? workspace_bytes : (size_t)0);
   if (p.single) {
     // rows in chunks write the plain output; the join follows as its own pass
-    // (and so do whole rows of few (row, head) pairs: the kernel form that
-    // has the join is the slower one, worth it only with all CUs at work)
-    const bool join_inside = gate_branch != nullptr && p.split_bytes == 0 &&
-                             (int64_t)B * H >= rg::kPrefillJoinMinGroups;
+    const bool join_inside = gate_branch != nullptr && p.split_bytes == 0;
     const int rc = recurrent_prefill_impl(
         __func__, x, segpos, segpos_is_i64, conv_w, conv_b, w_x, b_x, w_a, b_a,
         w_packed, a_param, h0, join_inside ? gate_branch : nullptr, out, h_last,

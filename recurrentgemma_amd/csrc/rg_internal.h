@@ -250,10 +250,6 @@ int scan_split_granule(int dtype, int W);
 hipError_t launch_block_prefill_bf16(const FusedArgs& a, hipStream_t s);
 hipError_t launch_block_prefill_teams_bf16(const FusedArgs& a, hipStream_t s);
 void prefill_chunk_plan(int B, int H, int T, int* chunks, int* tiles_per_chunk);
-// (row, head) pairs from which the block's GELU join runs inside the
-// single-launch kernel (its form with one wave per SIMD); below, the plain
-// kernel (two waves per SIMD) is followed by the join as a pass of its own
-constexpr int kPrefillJoinMinGroups = 129;
 hipError_t launch_block_step_bf16(const StepArgs& a, hipStream_t s);
 // bf16 [H,256,256] x 2 -> one buffer of the same total size in MFMA operand
 // order (head, wave, k-step, gate, lane, 8 values).

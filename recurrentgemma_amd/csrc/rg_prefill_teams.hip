@@ -22,8 +22,9 @@
 // arithmetic in the same order as the one-wave-per-SIMD form in rg_prefill.hip:
 // the two give bit-identical results.
 //
-// Whole rows only, packed weights, no GELU join: the launcher in
-// rg_prefill.hip sends everything else to the other form.
+// Whole rows and rows in chunks, with or without the block's GELU join; needs
+// the weights re-laid-out (rg_pack_gate_weights): the launcher in
+// rg_prefill.hip sends callers without them to the other form.
 //
 // Replaces the chain Conv1D.forward -> RGLRU.forward of
 // recurrentgemma/torch/modules.py:632-643 (layers.py:447-529, 313-365,
@@ -73,8 +74,12 @@ constexpr int kARing = 4;
 // at the end of phase M, the rest at the top of phase G (measured at B16 T8192
 // W4096: 0 -> 778 us, 8 -> 764 us, 12 -> 779 us a launch), and the same for the
 // recurrence gate (any part of it there was slower).
-constexpr int kTailX = 8;
-constexpr int kTailA = 0;
+constexpr int kTailXPlain = 8;
+constexpr int kTailAPlain = 0;
+// ... and with the GELU join in phase G (B16 T8192 W4096: 1057-1062 us a launch
+// for 8-16 input-gate and 0-8 recurrence-gate sigmoids here: no difference)
+constexpr int kTailXJoined = 16;
+constexpr int kTailAJoined = 4;
 // Priority of a wave while it issues its matrix instructions (the wave in
 // phase G stays at 0 and fills the gaps).
 constexpr int kMatrixPriority = 1;
@@ -191,9 +196,16 @@ enum PrefillMode {
   kChunkHead = 3      // chunk 0 from h0: y, and its end state as a summary
 };
 
-template <int MODE>
+// GELU: y is written as y * gelu(gate_branch), the join of the recurrent
+// block's two branches (recurrentgemma/torch/modules.py:627-628, 644),
+// instead of the plain RG-LRU output.
+template <int MODE, bool GELU>
 __device__ __forceinline__ void prefill_teams_body(const FusedArgs& p,
                                                    const int chunk) {
+  // how much of the gate arithmetic runs at the end of phase M (with the
+  // join, phase G carries 17 more vector slots per element)
+  constexpr int kTailX = GELU ? kTailXJoined : kTailXPlain;
+  constexpr int kTailA = GELU ? kTailAJoined : kTailAPlain;
   extern __shared__ __align__(16) unsigned char lds_raw[];
   lds_byte* const lds3 = (lds_byte*)lds_raw;
 
@@ -260,6 +272,10 @@ __device__ __forceinline__ void prefill_teams_body(const FusedArgs& p,
       make_rsrc((const char*)p.x + (int64_t)b * seq_bytes, seq_bytes);
   const __amdgpu_buffer_rsrc_t ry = make_rsrc(
       (char*)p.y + (int64_t)b * seq_bytes, MODE == kChunkSummary ? 0 : seq_bytes);
+  // GELU: the block's other branch, read where y is written
+  const __amdgpu_buffer_rsrc_t rgate = make_rsrc(
+      (const char*)p.gate_branch + (int64_t)b * seq_bytes,
+      GELU && MODE != kChunkSummary ? seq_bytes : 0);
   const bool seg_is64 = p.seg_kind == kSegI64;
   const uint32_t seg_esize = seg_is64 ? 8u : 4u;
   const __amdgpu_buffer_rsrc_t rseg =
@@ -546,6 +562,15 @@ __device__ __forceinline__ void prefill_teams_body(const FusedArgs& p,
   auto phase_g_as = [&](int kb, auto GENERAL) {
     constexpr bool general = decltype(GENERAL)::value;
     const int t_blk = kb * kBT;
+    u32x4 g_pending[2];
+    if (GELU) {
+      // the gate-branch values at the positions of this block's outputs:
+      // asked for now, used at the end of the phase
+      g_pending[0] = __builtin_amdgcn_raw_buffer_load_b128(
+          rgate, y_lane_bytes + (uint32_t)t_blk * row_bytes, 0, 0);
+      g_pending[1] = __builtin_amdgcn_raw_buffer_load_b128(
+          rgate, y_lane_bytes + (uint32_t)(t_blk + 16) * row_bytes, 0, 0);
+    }
     gate_x(kTailX, 16);
     gate_a(kTailA, 16);
 #pragma unroll
@@ -619,6 +644,21 @@ __device__ __forceinline__ void prefill_teams_body(const FusedArgs& p,
         y_pending[g >> 1] = *reinterpret_cast<lds_u32x4*>(lds3 + patch_r_lane);
         asm volatile("" ::: "memory");
       }
+    }
+    if (GELU) {
+      // y * gelu(gate branch), each factor a bf16 tensor as in the reference:
+      // the arithmetic and roundings of the stand-alone gelu_mul pass
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const float lo = gelu_mul_bf16(__uint_as_float(y_pending[j][k] << 16),
+                                         __uint_as_float(g_pending[j][k] << 16));
+          const float hi =
+              gelu_mul_bf16(__uint_as_float(y_pending[j][k] & 0xffff0000u),
+                            __uint_as_float(g_pending[j][k] & 0xffff0000u));
+          y_pending[j][k] = pack_bf16x2(lo, hi);
+        }
     }
     y_pending_row = (uint32_t)t_blk * row_bytes;
   };
@@ -748,30 +788,37 @@ enum PrefillPass { kPassWholeRows = 0, kPassFirst = 1, kPassReplay = 2 };
 // blockIdx.x: (row, head); blockIdx.y: which chunk (kPassFirst: chunk 0 with
 // its outputs beside the summaries of chunks 1 .. n-2; kPassReplay: chunks
 // 1 .. n-1).
-template <int PASS>
+template <int PASS, bool GELU>
 __global__ void __launch_bounds__(kThreads) block_prefill_teams_bf16_kernel(
     FusedArgs p) {
   if (PASS == kPassWholeRows) {
-    prefill_teams_body<kWholeRow>(p, 0);
+    prefill_teams_body<kWholeRow, GELU>(p, 0);
   } else if (PASS == kPassReplay) {
-    prefill_teams_body<kChunkReplay>(p, (int)blockIdx.y + 1);
+    prefill_teams_body<kChunkReplay, GELU>(p, (int)blockIdx.y + 1);
   } else if (blockIdx.y == 0) {
-    prefill_teams_body<kChunkHead>(p, 0);
+    prefill_teams_body<kChunkHead, GELU>(p, 0);
   } else {
-    prefill_teams_body<kChunkSummary>(p, (int)blockIdx.y);
+    prefill_teams_body<kChunkSummary, false>(p, (int)blockIdx.y);
   }
+}
+
+template <int PASS, bool GELU>
+hipError_t launch_teams_pass_as(const FusedArgs& a, int grid_y, hipStream_t s) {
+  static OncePerDevice once;
+  hipError_t e = set_max_dynamic_lds(
+      once, (const void*)block_prefill_teams_bf16_kernel<PASS, GELU>,
+      kTeamsLdsBytes);
+  if (e != hipSuccess) return e;
+  block_prefill_teams_bf16_kernel<PASS, GELU>
+      <<<dim3((unsigned)(a.B * a.H), (unsigned)grid_y), kThreads, kTeamsLdsBytes,
+         s>>>(a);
+  return hipGetLastError();
 }
 
 template <int PASS>
 hipError_t launch_teams_pass(const FusedArgs& a, int grid_y, hipStream_t s) {
-  static OncePerDevice once;
-  hipError_t e = set_max_dynamic_lds(
-      once, (const void*)block_prefill_teams_bf16_kernel<PASS>, kTeamsLdsBytes);
-  if (e != hipSuccess) return e;
-  block_prefill_teams_bf16_kernel<PASS>
-      <<<dim3((unsigned)(a.B * a.H), (unsigned)grid_y), kThreads, kTeamsLdsBytes,
-         s>>>(a);
-  return hipGetLastError();
+  if (a.gate_branch) return launch_teams_pass_as<PASS, true>(a, grid_y, s);
+  return launch_teams_pass_as<PASS, false>(a, grid_y, s);
 }
 
 }  // namespace
@@ -779,7 +826,7 @@ hipError_t launch_teams_pass(const FusedArgs& a, int grid_y, hipStream_t s) {
 hipError_t launch_block_prefill_teams_bf16(const FusedArgs& a, hipStream_t s) {
   const int64_t blocks = (int64_t)a.B * a.H;
   if (blocks <= 0 || blocks > 0x7fffffff) return hipErrorInvalidValue;
-  if (a.gate_branch || !a.w_packed) return hipErrorInvalidValue;
+  if (!a.w_packed) return hipErrorInvalidValue;
   if (a.chunks <= 1) return launch_teams_pass<kPassWholeRows>(a, 1, s);
   if (a.chunks < 3 || a.chunks > 65535) return hipErrorInvalidValue;
   hipError_t e = launch_teams_pass<kPassFirst>(a, a.chunks - 1, s);

@@ -930,6 +930,38 @@ def test_recurrent_prefill_in_chunks_without_packed_weights(B, T, W, H,
   assert torch.equal(y1, y2) and torch.equal(h1, h2) and torch.equal(c1, c2)
 
 
+@pytest.mark.parametrize("B,T,W,H", [(3, 150, 512, 2), (1, 2048, 512, 2)])
+def test_recurrent_prefill_joined_without_packed_weights(B, T, W, H):
+  """The block's GELU join inside the kernel (rg_recurrent_prefill_gelu_mul),
+  whole rows and rows in chunks, through both kernel forms: same bits."""
+  lib = _lib.lib()
+  need = lib.rg_recurrent_prefill_split_workspace_bytes(B, T, W, H)
+  p = R.make_params(W, H, torch.bfloat16, seed=81, gate_bias_std=0.5)
+  P = {k: _dev(v) for k, v in p.items()}
+  g = torch.Generator().manual_seed(82)
+  x = _dev(torch.randn(B, T, W, generator=g).to(torch.bfloat16))
+  gate = _dev(torch.randn(B, T, W, generator=g).to(torch.bfloat16))
+  seg = _dev(helpers.document_positions(B, T, 60, seed=83))
+  y1, h1, c1 = ops.recurrent_prefill(x, seg, P["conv_w"], P["conv_b"],
+                                     P["w_x"], P["b_x"], P["w_a"], P["b_a"],
+                                     P["a_param"], gate_branch=gate)
+  y2 = torch.empty_like(x)
+  h2 = torch.empty(B, W, dtype=torch.float32, device=DEV)
+  c2 = x.new_empty(B, 3, W)
+  ws = torch.empty(max(need, 16), dtype=torch.uint8, device=DEV)
+  ptr = lambda t: t.data_ptr()
+  _lib.check(lib.rg_recurrent_prefill_gelu_mul(
+      ptr(x), ptr(gate), ptr(seg), 1, ptr(P["conv_w"]), ptr(P["conv_b"]),
+      ptr(P["w_x"]), ptr(P["b_x"]), ptr(P["w_a"]), ptr(P["b_a"]), None,
+      ptr(P["a_param"]), None, ptr(y2), ptr(h2), ptr(c2), ptr(ws), need, B, T,
+      W, H, 1, torch.cuda.current_stream().cuda_stream))
+  assert torch.equal(y1, y2) and torch.equal(h1, h2) and torch.equal(c1, c2)
+  # and against the plain kernel followed by the join as its own pass
+  y3, _, _ = ops.recurrent_prefill(x, seg, P["conv_w"], P["conv_b"], P["w_x"],
+                                   P["b_x"], P["w_a"], P["b_a"], P["a_param"])
+  assert torch.equal(y1, ops.gelu_mul(y3, gate))
+
+
 def test_recurrent_core_picks_single_launch():
   """With enough (row, head) pairs recurrent_core runs prefill as one launch
   and decode as one launch; both against the oracle, chained."""
