@@ -99,7 +99,7 @@ WORKLOADS = {
 MEASURED_TRAFFIC_BYTES = {
     ("9b_prefill", "single"): (2.162e9, "profiles/hbm_traffic_9b_prefill.txt"),
     ("9b_prefill", "scan"): (4.345e9, "profiles/hbm_traffic_9b_prefill.txt"),
-    ("2b_prefill", "single"): (0.476e9, "profiles/hbm_traffic_2b_prefill.txt"),
+    ("2b_prefill", "single"): (0.474e9, "profiles/hbm_traffic_2b_prefill.txt"),
     ("2b_prefill", "scan"): (0.681e9, "profiles/hbm_traffic_2b_prefill.txt"),
 }
 
