@@ -50,15 +50,20 @@ pack_gate_weights_kernel(const uint16_t* __restrict__ w_x,
 //
 // Replaces Conv1D.forward's decode branch (layers.py:469-474, 491-529) and
 // RGLRU.forward / rnn_scan with T == 1 (layers.py:313-365, 170-177).
-constexpr int kStepRows = 32;
-constexpr int kStepRowsPerThread = 4;  // 32 rows x 64 channel quads / 512
+// ROWS = 32 rows of a tile, or 16 where 32 would leave CUs without a
+// workgroup (the matrix instructions then run half empty, which costs
+// nothing here: a step is loads and stores).
 
 // GELU: y leaves as y * gelu(gate_branch), the join of the recurrent block's
 // two branches (recurrentgemma/torch/modules.py:627-628, 644) with the
 // arithmetic and roundings of the stand-alone gelu_mul pass.
-template <bool GELU>
+template <bool GELU, int ROWS>
 __global__ void __launch_bounds__(512) block_step_bf16_kernel(StepArgs p) {
-  __shared__ __align__(16) uint16_t stage[kStepRows * kLdsStride];
+  constexpr int kStepRows = ROWS;
+  constexpr int kStepRowsPerThread = ROWS / 8;  // rows x 64 channel quads / 512
+  constexpr int kRuns = ROWS / 2;  // of a lane's 16 accumulator rows: in use
+  // (32 rows staged whatever ROWS is: the matrix instructions read 32)
+  __shared__ __align__(16) uint16_t stage[32 * kLdsStride];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -155,9 +160,9 @@ __global__ void __launch_bounds__(512) block_step_bf16_kernel(StepArgs p) {
     seg_hi = __builtin_amdgcn_raw_buffer_load_b32(
         rseg, is64 ? off + 4u : kBufferOutOfRange, 0, 0);
   }
-  float hv[16];
+  float hv[kRuns];
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
+  for (int r = 0; r < kRuns; ++r) {
     // row 8 (r / 4) + r % 4 (+ 4 in the upper half-wave)
     hv[r] = __builtin_bit_cast(
         float,
@@ -167,11 +172,11 @@ __global__ void __launch_bounds__(512) block_step_bf16_kernel(StepArgs p) {
   }
 
   // GELU: the gate branch where this lane stores y (see the output stage)
-  uint32_t gate2[8];
+  uint32_t gate2[kRuns / 2];
   if (GELU) {
     const uint32_t lane_rows = ((lane & 1) ? 1u : 0u) + (upper ? 4u : 0u);
 #pragma unroll
-    for (int r = 0; r < 16; r += 2)
+    for (int r = 0; r < kRuns; r += 2)
       gate2[r >> 1] = __builtin_amdgcn_raw_buffer_load_b32(
           rgate, (uint32_t)(ch & ~1) * 2u + lane_rows * row_bytes,
           (uint32_t)(8 * (r >> 2) + (r & 3)) * row_bytes, 0);
@@ -257,7 +262,7 @@ __global__ void __launch_bounds__(512) block_step_bf16_kernel(StepArgs p) {
   const bool odd = lane & 1;
   const uint32_t pair_ch = (uint32_t)(ch & ~1);
 #pragma unroll
-  for (int r = 0; r < 16; r += 2) {
+  for (int r = 0; r < kRuns; r += 2) {
     // pre-activations are a bf16 module output in the reference
     const uint32_t px2 = pack_bf16x2(acc_x[r], acc_x[r + 1]);
     const uint32_t pa2 = pack_bf16x2(acc_a[r], acc_a[r + 1]);
@@ -320,13 +325,22 @@ hipError_t launch_pack_gate_weights(const void* w_x, const void* w_a,
 
 hipError_t launch_block_step_bf16(const StepArgs& a, hipStream_t s) {
   // needs head width 256 (checked by the caller)
-  const int tiles = (a.B + kStepRows - 1) / kStepRows;
-  if (tiles <= 0 || (int64_t)tiles * a.H > 0x7fffffff)
+  const int tiles32 = (a.B + 31) / 32;
+  if (tiles32 <= 0 || (int64_t)tiles32 * 2 * a.H > 0x7fffffff)
     return hipErrorInvalidValue;
-  if (a.gate_branch)
-    block_step_bf16_kernel<true><<<dim3((unsigned)(tiles * a.H)), 512, 0, s>>>(a);
-  else
-    block_step_bf16_kernel<false><<<dim3((unsigned)(tiles * a.H)), 512, 0, s>>>(a);
+  // tiles of 16 rows while 32 would give fewer workgroups than CUs (256 rows
+  // x 16 heads: 128 workgroups 10.2 us, 256 workgroups 9.0 us, 512 of 8 rows
+  // 13.6 us a step)
+  const bool half = (int64_t)tiles32 * a.H < 256 && a.B > 16;
+  const int tiles = half ? (a.B + 15) / 16 : tiles32;
+  const dim3 grid((unsigned)(tiles * a.H));
+  if (a.gate_branch) {
+    if (half) block_step_bf16_kernel<true, 16><<<grid, 512, 0, s>>>(a);
+    else block_step_bf16_kernel<true, 32><<<grid, 512, 0, s>>>(a);
+  } else {
+    if (half) block_step_bf16_kernel<false, 16><<<grid, 512, 0, s>>>(a);
+    else block_step_bf16_kernel<false, 32><<<grid, 512, 0, s>>>(a);
+  }
   return hipGetLastError();
 }
 

@@ -3,14 +3,19 @@
 // recurrence.  Neither the conv output nor the gate pre-activations ever go to
 // memory: per element the kernel reads x once and writes y once.
 //
-// One workgroup of FOUR waves -- one per SIMD, each with the SIMD's whole
-// register file -- per (sequence row b, head h), or per (b, h, chunk of the
-// sequence), walks its tokens in tiles of 64.  Wave w owns 64 channels of the
-// head for both gates; its 2 x 256 x 64 weights (256 registers) stay resident
-// for the whole kernel.  A wave that has a SIMD to itself issues in order at a
-// steady one instruction per four cycles; two waves per SIMD (half the
-// registers each) lost a quarter of the time to the issue arbiter, which
-// serves the older wave first, and to the barriers where that wave then waits.
+// The form with ONE wave per SIMD.  One workgroup of four waves -- each with
+// its SIMD's whole register file -- per (sequence row b, head h), or per (b, h,
+// chunk of the sequence), walks its tokens in tiles of 64.  Wave w owns 64
+// channels of the head for both gates; its 2 x 256 x 64 weights (256
+// registers) stay resident for the whole kernel, and the matrix instructions
+// of the next 32 tokens are pinned between the pieces of the gate arithmetic
+// of the current ones.  A lone wave issues in order, one instruction per four
+// cycles at best, and 68 % of the slots at that: the form with two waves per
+// SIMD that alternate between a matrix phase and a gate phase
+// (rg_prefill_teams.hip) is 10-20 % faster and is what callers with
+// re-laid-out weights get.  This form serves weights in the reference layout
+// (transposed through LDS in the prologue) and is the second implementation
+// that the bit-equality tests hold the other one against.
 //
 // Replaces the chain Conv1D.forward -> RGLRU.forward of
 // recurrentgemma/torch/modules.py:632-643 (layers.py:447-529, 313-365,
