@@ -937,6 +937,10 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras,
     step = step_core
   else:
     step = step_single if path == "single" else step_split
+  # float32, 256-wide heads, at most 32 (row, head) pairs: the library's
+  # one-launch float32 kernel (core_f32_small_serves in csrc/rg_core_f32.hip)
+  f32_single = (args.path == "auto" and esize == 4 and W // H == 256
+                and B * H <= 32)
 
   per_launch = {}
 
@@ -1011,6 +1015,19 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras,
         "launch_ms": per_launch["main"][0],
         "mfma_tflops": gemm_flops / (first_ms * 1e-3) / 1e12,
         "frac_of_bf16_mfma_peak": gemm_flops / (first_ms * 1e-3) / 2.5e15}
+  elif f32_single:
+    # float32 with few rows: rg_recurrent_core is ONE launch that does the
+    # conv, both gate projections (true float32 products on the float32
+    # matrix instruction), the gates and the recurrence
+    algo = single_algorithmic_bytes(B, T, W, H, 4, seg_bytes, has_h0=False)
+    tf = gemm_flops / (first_ms * 1e-3) / 1e12
+    roofline = {
+        "kernel": "core_f32_small_kernel (conv + gate GEMMs on "
+                  "v_mfma_f32_16x16x4_f32 + gates + scan, one launch)",
+        "bound": "mfma", "achieved": tf, "peak": 157.3, "unit": "TFLOP/s",
+        "frac": tf / 157.3, "traffic": None, "algorithmic_bytes": algo,
+        "avg_launch_ms": first_ms, "launch_ms": per_launch["main"][0],
+        "gbs": algo / (first_ms * 1e-3) / 1e9}
   else:
     if args.path == "auto":
       # per-kernel durations: the same two launches called one by one, with
@@ -1070,6 +1087,8 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras,
                    "chunks side by side)" if path == "single" and chunked
                    else "rg_recurrent_prefill (single launch)"
                    if path == "single"
+                   else "rg_recurrent_core: one float32 launch (conv + gate "
+                        "GEMMs + gates + scan)" if f32_single
                    else ("rg_recurrent_core: " if args.path == "auto" else "")
                         + "rg_gates_gemm(conv on load) + "
                         + ("rg_lru_scan_fused_split(conv): sequences in chunks "
@@ -1079,7 +1098,7 @@ def run_prefill(args, torch, rg, R, ops, workload, steps, warmup, extras,
   }
   if cold:
     result["cold_caches"] = cold
-  if path == "split":
+  if path == "split" and not f32_single:
     result["gate_gemm"] = figs["gate_gemm"]
   elif args.path == "auto":
     # the two-kernel form of the same step, measured after the timed region

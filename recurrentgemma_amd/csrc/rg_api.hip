@@ -543,12 +543,17 @@ int rg_recurrent_prefill_gelu_mul(
 // (one per row, head and time chunk) fill the GPU, else the gate GEMM and the
 // scan kernel with the pre-activations of both gates in the workspace.
 struct CorePlan {
+  bool small_f32;      // core_f32_small_kernel: everything in one launch
   bool single;         // block_prefill_bf16_kernel
   size_t split_bytes;  // chunk summaries of whichever form runs
   size_t gate_bytes;   // one gate's pre-activations (two-kernel form), padded
 };
 static CorePlan core_plan(int B, int T, int W, int H, int dtype) {
   CorePlan p{};
+  // float32 with few rows: one launch, no workspace (a short float32 call is
+  // three launches' worth of latency otherwise)
+  p.small_f32 = dtype == RG_DTYPE_F32 && rg::core_f32_small_serves(B, T, W, H);
+  if (p.small_f32) return p;
   const bool fits = dtype == RG_DTYPE_BF16 && W / H == 256 &&
                     (int64_t)T * W * 2 < (int64_t)0x7fffffff;
   const size_t chunk_bytes =
@@ -614,7 +619,44 @@ int rg_recurrent_core(const void* x, const void* gate_branch,
     return fail(RG_ERR_WORKSPACE,
                 "%s: workspace of %zu bytes (16-byte aligned) required, got %zu",
                 __func__, need, workspace ? workspace_bytes : (size_t)0);
-  if (p.single) {
+  if (p.small_f32) {
+    RG_CHECK_PTR(x);
+    RG_CHECK_PTR(segpos);
+    RG_CHECK_OPT_PTR(conv_w);
+    RG_CHECK_OPT_PTR(conv_b);
+    RG_CHECK_PTR(w_x);
+    RG_CHECK_PTR(b_x);
+    RG_CHECK_PTR(w_a);
+    RG_CHECK_PTR(b_a);
+    RG_CHECK_PTR(a_param);
+    RG_CHECK_PTR(out);
+    RG_CHECK_OPT_PTR(h0);
+    RG_CHECK_OPT_PTR(h_last);
+    RG_CHECK_OPT_PTR(conv_cache_out);
+    RG_REQUIRE(out != x, "%s: out must not alias x", __func__);
+    rg::FusedArgs a{};
+    a.x = x;
+    a.segpos = segpos;
+    a.seg_kind = segpos_is_i64 ? 1 : 0;
+    a.conv_w = conv_w;
+    a.conv_b = conv_b;
+    a.w[0] = w_x;
+    a.b[0] = b_x;
+    a.w[1] = w_a;
+    a.b[1] = b_a;
+    a.a_param = a_param;
+    a.h0 = (const float*)h0;
+    a.y = out;
+    a.h_last = (float*)h_last;
+    a.cache_out = conv_cache_out;
+    a.B = B;
+    a.T = T;
+    a.W = W;
+    a.H = H;
+    const int rc = launch_status(
+        __func__, rg::launch_core_f32_small(a, (hipStream_t)stream));
+    if (rc != RG_OK || gate_branch == nullptr) return rc;
+  } else if (p.single) {
     // rows in chunks write the plain output; the join follows as its own pass
     const bool join_inside = gate_branch != nullptr && p.split_bytes == 0;
     const int rc = recurrent_prefill_impl(

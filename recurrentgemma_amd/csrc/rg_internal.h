@@ -249,6 +249,10 @@ void scan_split_plan(int B, int T, int W, int granule, int* chunks,
 int scan_split_granule(int dtype, int W);
 hipError_t launch_block_prefill_bf16(const FusedArgs& a, hipStream_t s);
 hipError_t launch_block_prefill_teams_bf16(const FusedArgs& a, hipStream_t s);
+// float32, 256-wide heads, few rows: conv, gate projections, gates and
+// recurrence in one launch (rg_core_f32.hip)
+bool core_f32_small_serves(int B, int T, int W, int H);
+hipError_t launch_core_f32_small(const FusedArgs& a, hipStream_t s);
 void prefill_chunk_plan(int B, int H, int T, int* chunks, int* tiles_per_chunk);
 hipError_t launch_block_step_bf16(const StepArgs& a, hipStream_t s);
 // bf16 [H,256,256] x 2 -> one buffer of the same total size in MFMA operand

@@ -1025,7 +1025,8 @@ def test_recurrent_core_entry_equals_its_parts(dtype, B, T, W, H, joined):
         x, seg, P["conv_w"], P["conv_b"], P["w_x"], P["b_x"], P["w_a"],
         P["b_a"], P["a_param"], h0=h0)
   else:
-    assert need >= 2 * x.numel() * x.element_size()
+    small_f32 = dtype == torch.float32 and W // H == 256 and B * H <= 32
+    assert need >= 2 * x.numel() * x.element_size() or small_f32
     gx, ga = ops.gates_gemm(x, P["w_x"], P["b_x"], P["w_a"], P["b_a"],
                             conv=(seg, P["conv_w"], P["conv_b"]))
     y2, h2, c2 = ops.lru_scan_fused(x, gx, ga, P["a_param"], seg, h0=h0,
@@ -1033,6 +1034,13 @@ def test_recurrent_core_entry_equals_its_parts(dtype, B, T, W, H, joined):
                                     return_conv_cache=True)
   if joined:
     y2 = ops.gelu_mul(y2, gate)
+  if dtype == torch.float32 and W // H == 256 and B * H <= 32:
+    # the one-launch float32 kernel sums its products in another order than
+    # the gate GEMM: float32 agreement, not bit equality (conv state: exact)
+    assert need == 0
+    assert helpers.max_rel(y, y2) < 2e-6 and helpers.max_rel(h, h2) < 2e-6
+    assert torch.equal(c, c2)
+    return
   assert torch.equal(y, y2) and torch.equal(h, h2) and torch.equal(c, c2)
   # and against the oracle
   ref = R.recurrent_core if dtype == torch.float32 else R.widened_recurrent_core
@@ -1047,7 +1055,7 @@ def test_recurrent_core_entry_equals_its_parts(dtype, B, T, W, H, joined):
 
 
 def test_recurrent_core_entry_rejects_a_short_workspace():
-  B, T, W, H = 1, 512, 512, 2
+  B, T, W, H = 1, 512, 512, 4  # float32, 128-wide heads: the two-kernel form
   x = _dev(torch.zeros(B, T, W))
   seg = _dev(torch.arange(T).expand(B, T).contiguous())
   p = {k: _dev(v) for k, v in R.make_params(W, H, torch.float32, seed=1).items()}

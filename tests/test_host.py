@@ -164,7 +164,13 @@ def test_c_side_validation_without_launch():
   assert lib.rg_recurrent_core_workspace_bytes(16, 8192, 4096, 16, 1) == 0
   assert (lib.rg_recurrent_core_workspace_bytes(1, 8192, 2560, 10, 1) ==
           lib.rg_recurrent_prefill_split_workspace_bytes(1, 8192, 2560, 10))
-  assert (lib.rg_recurrent_core_workspace_bytes(1, 512, 2560, 10, 0) ==
+  # float32 with 256-wide heads and at most 32 (row, head) pairs: one launch,
+  # no workspace; more pairs or other head widths: the two-kernel form
+  assert lib.rg_recurrent_core_workspace_bytes(1, 512, 2560, 10, 0) == 0
+  assert lib.rg_recurrent_core_workspace_bytes(3, 512, 2560, 10, 0) == 0
+  assert (lib.rg_recurrent_core_workspace_bytes(4, 512, 2560, 10, 0) ==
+          2 * 4 * 512 * 2560 * 4 + lib.rg_scan_split_workspace_bytes(4, 512, 2560))
+  assert (lib.rg_recurrent_core_workspace_bytes(1, 512, 2560, 20, 0) ==
           2 * 512 * 2560 * 4 + lib.rg_scan_split_workspace_bytes(1, 512, 2560))
   # bf16 with 256-wide heads: the single kernel whatever the number of rows ...
   assert lib.rg_recurrent_core_workspace_bytes(2, 100, 512, 2, 1) == 0
