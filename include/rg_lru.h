@@ -285,7 +285,9 @@ int rg_recurrent_prefill_gelu_mul(
  * with the choice of kernels made here: the single prefill kernel
  * (rg_recurrent_prefill_split; bf16, 256-wide heads, enough (row, head) pairs
  * or rows long enough to be cut into chunks, but not more than 256 pairs of
- * fewer than 64 tokens), else rg_gates_gemm with the conv
+ * fewer than 64 tokens); for float32 with 256-wide heads and at most 32
+ * (row, head) pairs one launch that does the same in float32 (needs no
+ * workspace; no entry point of its own); else rg_gates_gemm with the conv
  * applied on load followed by rg_lru_scan_fused_split, the pre-activations of
  * both gates living in the workspace.  gate_branch (nullable, [B,T,W]): the
  * block's linear_y output; `out` is then rglru(conv1d(x)) * gelu_tanh(
