@@ -69,8 +69,9 @@ int rg_conv1d_prefill(const void* x, const void* segpos, int segpos_is_i64,
  * rg_conv1d_backward_workspace_bytes / ((temporal_width + 1) * W * 4)), per
  * chunk of rows the sums that add up to the gradient of w (planes 0 ..
  * temporal_width-1, laid out like w) and of b (last plane); the caller sums
- * over the chunks.  Taps cut by a document start carry no gradient, as in the
- * forward pass.  2 <= temporal_width <= RG_MAX_CONV_WIDTH. */
+ * over the chunks (chunks of 32 rows of [B*T] while that leaves at most 512 of
+ * them, of 64, 128 or 256 rows beyond).  Taps cut by a document start carry no
+ * gradient, as in the forward pass.  2 <= temporal_width <= RG_MAX_CONV_WIDTH. */
 size_t rg_conv1d_backward_workspace_bytes(int B, int T, int W,
                                           int temporal_width);
 int rg_conv1d_backward(const void* dout, const void* x, const void* segpos,

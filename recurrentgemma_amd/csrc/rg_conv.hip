@@ -59,11 +59,16 @@ conv1d_cache_tail_kernel(const T* __restrict__ x,
 //   out[t] = bias + sum_s w[K-1-s] x[t-s] keep_s[t]
 //   dx[u]      = sum_s w[K-1-s] dout[u+s] keep_s[u+s]        (u + s < T)
 //   dw[K-1-s] += x[t-s] keep_s[t] dout[t],   dbias += dout[t]
-// A thread owns one channel and a run of kConvBwdRows consecutive flattened
-// rows (b, t): it writes dx for them and leaves its sums of dw and dbias in
+// A thread owns one channel and a run of `rows` consecutive flattened rows
+// (b, t): it writes dx for them and leaves its sums of dw and dbias in
 // `partial` [row chunks][K + 1][W] (float32), which the caller adds up.  The
-// neighbouring rows it re-reads come from cache.
-constexpr int kConvBwdRows = 32;  // (the 16-byte kernels below share it)
+// neighbouring rows it re-reads come from cache.  `rows` is 32 while that
+// leaves at most 512 chunks and grows up to 256 beyond (conv1d_backward_rows):
+// a plane of partial sums is (K + 1) W floats written and read again, 16 %
+// of the pass's own traffic at 32 rows of bf16 and 2 % at 256.
+constexpr int kConvBwdRows = 32;
+constexpr int kConvBwdMaxRows = 256;
+constexpr int kConvBwdChunks = 512;
 
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -71,11 +76,11 @@ conv1d_backward_kernel(const T* __restrict__ dout, const T* __restrict__ x,
                        const void* __restrict__ segpos, int seg_kind,
                        const T* __restrict__ w, T* __restrict__ dx,
                        float* __restrict__ partial, int T_len, int W, int K,
-                       int64_t M) {
+                       int64_t M, int rows) {
   const int c = blockIdx.y * 256 + threadIdx.x;
   if (c >= W) return;
-  const int64_t m0 = (int64_t)blockIdx.x * kConvBwdRows;
-  const int64_t m1 = m0 + kConvBwdRows < M ? m0 + kConvBwdRows : M;
+  const int64_t m0 = (int64_t)blockIdx.x * rows;
+  const int64_t m1 = m0 + rows < M ? m0 + rows : M;
   constexpr int kMaxK = 16;  // widths above are refused by the caller
   float wk[kMaxK], dw[kMaxK], db = 0.0f;
 #pragma unroll
@@ -122,7 +127,7 @@ conv1d_backward_kernel(const T* __restrict__ dout, const T* __restrict__ x,
 // zeroes the history registers: later tokens then see zeros exactly where the
 // definition drops a tap.  Rows are requested eight at a time before the first
 // is used.
-constexpr int kConvRun = 32;    // rows per wave (= kConvBwdRows: the partial planes)
+constexpr int kConvRun = 32;    // rows per wave of the forward kernels
 constexpr int kConvBatch = 8;   // rows requested together
 
 template <typename T>
@@ -345,14 +350,14 @@ conv1d_backward_k4_kernel(const T* __restrict__ dout, const T* __restrict__ x,
                           const void* __restrict__ segpos, int seg_kind,
                           const T* __restrict__ w, T* __restrict__ dx,
                           float* __restrict__ partial, int T_len, int W,
-                          int64_t M) {
+                          int64_t M, int rows) {
   using V = Vec16<T>;
   constexpr int N = V::N;
   const int c = ((int)blockIdx.y * 64 + (int)threadIdx.x) * N;
   if (c >= W) return;
-  const int64_t m0 = (int64_t)blockIdx.x * kConvRun;
-  const int64_t m1 = m0 + kConvRun < M ? m0 + kConvRun : M;
-  const SeqStarts seq(m0 >= 3 ? m0 - 3 : 0, T_len, kConvRun + 6);
+  const int64_t m0 = (int64_t)blockIdx.x * rows;
+  const int64_t m1 = m0 + rows < M ? m0 + rows : M;
+  const SeqStarts seq(m0 >= 3 ? m0 - 3 : 0, T_len, rows + 6);
   auto row = [&](const T* base, int64_t m) {
     return *reinterpret_cast<const u32x4*>(base + m * W + c);
   };
@@ -580,14 +585,25 @@ hipError_t launch_conv1d_step(const ConvStepArgs& a, int dtype,
   return dtype == 0 ? conv_step_t<float>(a, s) : conv_step_t<uint16_t>(a, s);
 }
 
+// Rows per chunk of the backward pass (see kConvBwdRows above).
+static int conv1d_backward_rows(int64_t M) {
+  int rows = kConvBwdRows;
+  while (rows < kConvBwdMaxRows && (M + rows - 1) / rows > kConvBwdChunks)
+    rows *= 2;
+  return rows;
+}
+
 int conv1d_backward_chunks(int B, int T) {
-  return (int)(((int64_t)B * T + kConvBwdRows - 1) / kConvBwdRows);
+  const int64_t M = (int64_t)B * T;
+  const int rows = conv1d_backward_rows(M);
+  return (int)((M + rows - 1) / rows);
 }
 
 hipError_t launch_conv1d_backward(const ConvBwdArgs& a, int dtype,
                                   hipStream_t s) {
   const int64_t M = (int64_t)a.B * a.T;
   const int64_t chunks = conv1d_backward_chunks(a.B, a.T);
+  const int rows = conv1d_backward_rows(M);
   const int64_t cblocks = ((int64_t)a.W + 255) / 256;
   if (chunks <= 0 || chunks > 0x7fffffff || cblocks > 65535 || a.K < 2 ||
       a.K > 16)
@@ -598,24 +614,25 @@ hipError_t launch_conv1d_backward(const ConvBwdArgs& a, int dtype,
       conv1d_backward_k4_kernel<float>
           <<<dim3((unsigned)chunks, (unsigned)((a.W / 4 + 63) / 64)), 64, 0, s>>>(
               (const float*)a.dout, (const float*)a.x, a.segpos, a.seg_kind,
-              (const float*)a.w, (float*)a.dx, a.partial, a.T, a.W, M);
+              (const float*)a.w, (float*)a.dx, a.partial, a.T, a.W, M, rows);
     else
       conv1d_backward_k4_kernel<uint16_t>
           <<<dim3((unsigned)chunks, (unsigned)((a.W / 8 + 63) / 64)), 64, 0, s>>>(
               (const uint16_t*)a.dout, (const uint16_t*)a.x, a.segpos,
               a.seg_kind, (const uint16_t*)a.w, (uint16_t*)a.dx, a.partial, a.T,
-              a.W, M);
+              a.W, M, rows);
     return hipGetLastError();
   }
   const dim3 grid((unsigned)chunks, (unsigned)cblocks);
   if (dtype == 0)
     conv1d_backward_kernel<float><<<grid, 256, 0, s>>>(
         (const float*)a.dout, (const float*)a.x, a.segpos, a.seg_kind,
-        (const float*)a.w, (float*)a.dx, a.partial, a.T, a.W, a.K, M);
+        (const float*)a.w, (float*)a.dx, a.partial, a.T, a.W, a.K, M, rows);
   else
     conv1d_backward_kernel<uint16_t><<<grid, 256, 0, s>>>(
         (const uint16_t*)a.dout, (const uint16_t*)a.x, a.segpos, a.seg_kind,
-        (const uint16_t*)a.w, (uint16_t*)a.dx, a.partial, a.T, a.W, a.K, M);
+        (const uint16_t*)a.w, (uint16_t*)a.dx, a.partial, a.T, a.W, a.K, M,
+        rows);
   return hipGetLastError();
 }
 

@@ -375,3 +375,49 @@ def test_conv_backward_kernel(dtype, B, T, W, K):
   out2 = training.conv1d_tensor_ops(x2, seg.to(DEV), w2, b2)
   (out2.float() * r.to(DEV).float()).sum().backward()
   near(x2.grad, xd.grad, "dx (tensor ops)")
+
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,T,W,K", [(2, 40000, 64, 4), (3, 9000, 64, 4),
+                                     (1, 70000, 32, 2)])
+def test_conv_backward_kernel_many_rows(dtype, B, T, W, K):
+  """rg_conv1d_backward where a chunk of its partial sums covers more than 32
+  rows (64, 128 or 256: the kernel widens its chunks once there would be more
+  than 512 of them): dx, dw and db against autograd through the tensor-op
+  form of the same conv (training.conv1d_tensor_ops, which the test above
+  pins to the definition) evaluated in float64 on the same dtype-valued
+  inputs.  Tolerances as above; the number of planes is what the library
+  says."""
+  from tests import helpers
+  from recurrentgemma_amd import _lib
+  gen = torch.Generator().manual_seed(B + T + K)
+  x = torch.randn(B, T, W, generator=gen).to(dtype)
+  w = (torch.randn(K, W, generator=gen) * 0.5).to(dtype)
+  b = torch.randn(W, generator=gen).to(dtype)
+  r = (torch.randn(B, T, W, generator=gen) / (B * T) ** 0.5).to(dtype)
+  seg = helpers.document_positions(B, T, 300, seed=T)
+  seg[-1, T - 1] = 0
+
+  lib = _lib.lib()
+  planes = lib.rg_conv1d_backward_workspace_bytes(B, T, W, K) // ((K + 1) * W * 4)
+  assert planes <= 512 and planes * 32 < B * T <= planes * 256
+
+  x2, w2, b2 = (t.to(DEV).double().requires_grad_(True) for t in (x, w, b))
+  out2 = training.conv1d_tensor_ops(x2, seg.to(DEV), w2, b2)
+  (out2 * r.to(DEV).double()).sum().backward()
+
+  xg, wg, bg = (t.to(DEV).requires_grad_(True) for t in (x, w, b))
+  with training.differentiable():
+    out = training.conv1d(xg, seg.to(DEV), wg, bg)
+  (out.float() * r.to(DEV).float()).sum().backward()
+  tol = 1e-5 if dtype == torch.float32 else 1e-2
+
+  def near(got, want, what):
+    want = want.detach().double()
+    err = (got.detach().double() - want).abs().max().item()
+    assert err <= tol * max(want.abs().max().item(), 1e-12), (what, err)
+
+  near(xg.grad, x2.grad, "dx")
+  near(wg.grad, w2.grad, "dw")
+  near(bg.grad, b2.grad, "db")

@@ -118,6 +118,11 @@ def test_c_side_validation_without_launch():
                              ok, ok, None, 1, 4, 8, 0, None)
   assert rc == -1 and b"dy is null" in lib.rg_last_error()
   assert lib.rg_conv1d_backward_workspace_bytes(2, 100, 64, 4) == 7 * 5 * 64 * 4
+  # chunks of 32 rows while that leaves at most 512 of them, then 64, 128, 256
+  assert lib.rg_conv1d_backward_workspace_bytes(16, 1024, 64, 4) == 512 * 5 * 64 * 4
+  assert lib.rg_conv1d_backward_workspace_bytes(16, 1025, 64, 4) == 257 * 5 * 64 * 4
+  assert lib.rg_conv1d_backward_workspace_bytes(16, 8192, 64, 4) == 512 * 5 * 64 * 4
+  assert lib.rg_conv1d_backward_workspace_bytes(32, 8192, 64, 4) == 1024 * 5 * 64 * 4
   assert lib.rg_conv1d_backward_workspace_bytes(2, 100, 64, 1) == 0
   rc = lib.rg_conv1d_backward(ok, ok, ok, 1, ok, ctypes.c_void_p(512), None, 0,
                               2, 100, 64, 4, 0, None)
