@@ -292,9 +292,9 @@ int rg_recurrent_prefill_gelu_mul(
  * applied on load followed by rg_lru_scan_fused_split, the pre-activations of
  * both gates living in the workspace.  gate_branch (nullable, [B,T,W]): the
  * block's linear_y output; `out` is then rglru(conv1d(x)) * gelu_tanh(
- * gate_branch) (modules.py:627-628, 644: rg_recurrent_prefill_gelu_mul where
- * whole rows run in the single kernel, otherwise rg_gelu_mul over `out` as a
- * last launch), else the plain RG-LRU output.  `workspace` (16-byte aligned)
+ * gate_branch) (modules.py:627-628, 644: inside the single kernels, bf16 and
+ * float32, as in rg_recurrent_prefill_gelu_mul; after the two-kernel form
+ * rg_gelu_mul over `out` as a last launch), else the plain RG-LRU output.  `workspace` (16-byte aligned)
  * must hold rg_recurrent_core_workspace_bytes(B, T, W, H, dtype) bytes (0 for
  * whole rows in the single kernel: workspace may then be null).  Same values
  * as the calls it is made of; h0 / h_last / conv_cache_out / w_packed as in

@@ -649,22 +649,20 @@ int rg_recurrent_core(const void* x, const void* gate_branch,
     a.y = out;
     a.h_last = (float*)h_last;
     a.cache_out = conv_cache_out;
+    a.gate_branch = gate_branch;  // the join is in the kernel's y stores
     a.B = B;
     a.T = T;
     a.W = W;
     a.H = H;
-    const int rc = launch_status(
+    return launch_status(
         __func__, rg::launch_core_f32_small(a, (hipStream_t)stream));
-    if (rc != RG_OK || gate_branch == nullptr) return rc;
   } else if (p.single) {
-    // rows in chunks write the plain output; the join follows as its own pass
-    const bool join_inside = gate_branch != nullptr && p.split_bytes == 0;
-    const int rc = recurrent_prefill_impl(
+    // the join is part of the kernel's output stage, for rows in chunks too
+    // (the launches that write y apply it)
+    return recurrent_prefill_impl(
         __func__, x, segpos, segpos_is_i64, conv_w, conv_b, w_x, b_x, w_a, b_a,
-        w_packed, a_param, h0, join_inside ? gate_branch : nullptr, out, h_last,
-        conv_cache_out, workspace, workspace_bytes, true, B, T, W, H, dtype,
-        stream);
-    if (rc != RG_OK || gate_branch == nullptr || join_inside) return rc;
+        w_packed, a_param, h0, gate_branch, out, h_last, conv_cache_out,
+        workspace, workspace_bytes, true, B, T, W, H, dtype, stream);
   } else {
     char* const ws = (char*)workspace;
     void* const gx = ws + p.split_bytes;

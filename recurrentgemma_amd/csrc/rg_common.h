@@ -347,5 +347,18 @@ __device__ __forceinline__ float gelu_mul_bf16(float av, float gv) {
   return av * round_to_bf16(0.5f * gv * (1.0f + t));
 }
 
+// a * gelu_tanh(g) in float32 by the reference's own formula
+// (modules.py:289-291, :644), every step rounded as written (no fused
+// multiply-adds), so that every kernel that has it gives the same bits.
+__device__ __forceinline__ float gelu_mul_f32(float av, float gv) {
+  constexpr float c0 = 0.7978845608028654f;  // sqrt(2/pi)
+  constexpr float c1 = 0.044715f;
+  const float cube = __fmul_rn(__fmul_rn(__fmul_rn(c1, gv), gv), gv);
+  const float u = __fmul_rn(c0, __fadd_rn(gv, cube));
+  const float gelu =
+      __fmul_rn(__fmul_rn(0.5f, gv), __fadd_rn(1.0f, tanhf(u)));
+  return __fmul_rn(av, gelu);
+}
+
 }  // namespace rg
 #endif  // RG_COMMON_H_

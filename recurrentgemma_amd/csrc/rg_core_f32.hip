@@ -123,7 +123,9 @@ __device__ __forceinline__ void static_for(F&& f) {
   }
 }
 
-template <bool HAS_CONV>
+// GELU: y is written as y * gelu(gate_branch), the join of the recurrent
+// block's two branches (recurrentgemma/torch/modules.py:627-628, 644).
+template <bool HAS_CONV, bool GELU>
 __global__ void __launch_bounds__(kThreads) core_f32_small_kernel(FusedArgs p) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   CoreF32Lds& lds = *reinterpret_cast<CoreF32Lds*>(lds_raw);
@@ -486,13 +488,22 @@ __global__ void __launch_bounds__(kThreads) core_f32_small_kernel(FusedArgs p) {
       }
       __syncthreads();
       float hin = lds.chunk_h[chunk][ch];
-      float* y = (float*)p.y + ((int64_t)b * T + seg * kSeg + i0) * W + c0 + ch;
+      const int64_t y_at = ((int64_t)b * T + seg * kSeg + i0) * W + c0 + ch;
+      float* y = (float*)p.y + y_at;
       const int left = T - (seg * kSeg + i0);
+      float other[kChunk];  // GELU: the other branch at this thread's tokens
+      if (GELU) {
+        const float* gb = (const float*)p.gate_branch + y_at;
+#pragma unroll
+        for (int i = 0; i < kChunk; ++i)
+          other[i] = i < left ? gb[(int64_t)i * W] : 0.0f;
+      }
 #pragma unroll
       for (int i = 0; i < kChunk; ++i) {
         hin = __builtin_fmaf(lds.a[gate_slot(i0 + i)][ch], hin,
                              lds.xn[gate_slot(i0 + i)][ch]);
-        if (i < left) y[(int64_t)i * W] = hin;
+        if (i < left)
+          y[(int64_t)i * W] = GELU ? gelu_mul_f32(hin, other[i]) : hin;
       }
     }
     __syncthreads();  // a, xn and the chunk states are free again
@@ -527,23 +538,27 @@ bool core_f32_small_serves(int B, int T, int W, int H) {
          (int64_t)T * W * 4 < (int64_t)0x7fffffff;
 }
 
+template <bool HAS_CONV, bool GELU>
+static hipError_t launch_core_f32_small_as(const FusedArgs& a, dim3 grid,
+                                           hipStream_t s) {
+  static OncePerDevice once;
+  hipError_t e = set_max_dynamic_lds(
+      once, (const void*)core_f32_small_kernel<HAS_CONV, GELU>,
+      (int)sizeof(CoreF32Lds));
+  if (e != hipSuccess) return e;
+  core_f32_small_kernel<HAS_CONV, GELU>
+      <<<grid, kThreads, sizeof(CoreF32Lds), s>>>(a);
+  return hipGetLastError();
+}
+
 hipError_t launch_core_f32_small(const FusedArgs& a, hipStream_t s) {
   const int rounds = (a.B * a.H + 7) / 8;
   const dim3 grid((unsigned)(rounds * 8 * (kBW / kCh)));
-  if (a.conv_w) {
-    static OncePerDevice once;
-    hipError_t e = set_max_dynamic_lds(
-        once, (const void*)core_f32_small_kernel<true>, (int)sizeof(CoreF32Lds));
-    if (e != hipSuccess) return e;
-    core_f32_small_kernel<true><<<grid, kThreads, sizeof(CoreF32Lds), s>>>(a);
-  } else {
-    static OncePerDevice once;
-    hipError_t e = set_max_dynamic_lds(
-        once, (const void*)core_f32_small_kernel<false>, (int)sizeof(CoreF32Lds));
-    if (e != hipSuccess) return e;
-    core_f32_small_kernel<false><<<grid, kThreads, sizeof(CoreF32Lds), s>>>(a);
-  }
-  return hipGetLastError();
+  if (a.conv_w)
+    return a.gate_branch ? launch_core_f32_small_as<true, true>(a, grid, s)
+                         : launch_core_f32_small_as<true, false>(a, grid, s);
+  return a.gate_branch ? launch_core_f32_small_as<false, true>(a, grid, s)
+                       : launch_core_f32_small_as<false, false>(a, grid, s);
 }
 
 }  // namespace rg

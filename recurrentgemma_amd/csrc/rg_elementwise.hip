@@ -50,10 +50,7 @@ __global__ void __launch_bounds__(256)
 gelu_mul_f32_kernel(const f32x4* a, const f32x4* __restrict__ g, f32x4* out,
                     int64_t n4, const float* a_tail,
                     const float* g_tail, float* out_tail, int tail) {
-  auto one = [](float av, float gv) {
-    const float u = kGeluC0 * (gv + kGeluC1 * gv * gv * gv);
-    return av * (0.5f * gv * (1.0f + tanhf(u)));
-  };
+  auto one = [](float av, float gv) { return gelu_mul_f32(av, gv); };
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i < n4) {
     const f32x4 av = __builtin_nontemporal_load(a + i);

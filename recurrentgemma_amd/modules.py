@@ -81,11 +81,10 @@ def recurrent_core(conv_1d: layers.Conv1D, rg_lru: layers.RGLRU, x,
     # One call; the library picks the kernels (rg_recurrent_core): for bf16
     # and 256-wide heads the single-launch kernel, one workgroup per (row,
     # head) or -- rows of few pairs -- per chunk of one (many rows of a few
-    # tokens and every other dtype or head width: gate GEMM + scan), and the
-    # join with the gate branch inside that kernel for whole rows of at least
-    # 129 pairs (with rows in chunks it would lengthen the one workgroup per
-    # row that produces outputs in the first launch while the others only
-    # summarise, so there it stays a pass of its own).
+    # tokens and every other dtype or head width: gate GEMM + scan; float32
+    # with 256-wide heads and few pairs: a one-launch float32 kernel), and
+    # the join with the gate branch inside those kernels (after the two-kernel
+    # form it is a pass of its own).
     if compiled.tracing():
       y, h, conv_state = torch.ops.recurrentgemma_amd.recurrent_core(
           x, segment_pos, conv_1d.w, conv_1d.b, rg_lru.input_gate.w,
