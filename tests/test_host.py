@@ -266,6 +266,39 @@ def test_prefill_kernel_keeps_its_hand_numbered_registers():
                         stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
 
 
+def test_build_check_for_early_reads_of_matrix_results(tmp_path):
+  """check_mfma_wait.py (part of `make check-registers`): an instruction that
+  touches the result registers of a matrix instruction right behind it is
+  reported; the same instruction behind the kernel's own wait, a matrix
+  instruction that accumulates into the same registers, and instructions on
+  other registers are not."""
+  import subprocess
+  import sys
+  script = os.path.join(_lib.CSRC, "check_mfma_wait.py")
+  mfma = ("\tv_mfma_f32_16x16x4_f32 v[2:5], v17, a[63], v[2:5]\n"
+          "\tv_mfma_f32_16x16x4_f32 v[6:9], v17, a[0x7f], v[6:9]\n")
+  wait = "\ts_nop 15\n\ts_nop 3\n"
+  cases = {
+      "copy_before_wait": (mfma + "\ts_nop 0\n\tv_mov_b64_e32 v[16:17], v[8:9]\n"
+                           + wait, 1),
+      "copy_after_wait": (mfma + wait + "\tv_mov_b64_e32 v[16:17], v[8:9]\n", 0),
+      "other_registers": (mfma + "\tv_mul_f32_e32 v10, v11, v12\n"
+                          "\tds_read_b128 v[18:21], v83\n" + wait, 0),
+      "accumulating": (mfma + mfma + wait, 0),
+      "store_of_result": ("\tv_mfma_f32_32x32x16_bf16 v[2:17], v[100:103], "
+                          "a[31*4:31*4+3], v[2:17]\n"
+                          "\tds_write_b32 v40, v17\n" + wait, 1),
+      "far_enough": (mfma + "\ts_mov_b32 s0, s1\n" * 24
+                     + "\tv_mov_b32_e32 v20, v9\n", 0),
+  }
+  for name, (text, want) in cases.items():
+    path = tmp_path / (name + ".s")
+    path.write_text(text)
+    rc = subprocess.run([sys.executable, script, str(path)],
+                        stdout=subprocess.DEVNULL).returncode
+    assert rc == want, name
+
+
 def test_no_cpu_fallback():
   conv = rg.Conv1D(width=8, temporal_width=4)
   with pytest.raises(RuntimeError, match="GPU only"):
