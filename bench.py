@@ -410,6 +410,10 @@ def run_training(args, torch, rg, ops, wl):
         ("rg_gates_gemm (forward of both gate projections)",
          lambda: ops.gates_gemm(xc, lru.input_gate.w, lru.input_gate.b,
                                 lru.a_gate.w, lru.a_gate.b), 3),
+        ("rg_gates_weight_grads (weight and bias gradients of both gate "
+         "projections)",
+         lambda: ops.gates_weight_grads(xc, dy, dy, lru.input_gate.w.shape[0]),
+         3),
         ("rg_lru_scan_fused (forward of gating and recurrence)",
          lambda: ops.lru_scan_fused(xc, gx, ga, lru.a_param, seg), 4)):
       ms = events(fn)

@@ -94,6 +94,23 @@ int rg_conv1d_step(const void* x, const void* cache_in, const void* w,
 int rg_block_diag_linear(const void* x, const void* w, const void* b, void* y,
                          int64_t M, int H, int bw, int dtype, void* stream);
 
+/* Weight and bias gradients of the two gate projections of RGLRU.forward
+ * (what autograd forms for recurrentgemma/torch/layers.py:134-136, called at
+ * :338-339 on the same x) from the gradients of their outputs:
+ *   dw_g[h,i,j] = sum_m x[m, h*256 + i] * dy_g[m, h*256 + j]
+ *   db_g[h,j]   = sum_m dy_g[m, h*256 + j]            g = input gate, a gate
+ * x, dgx, dga [M, W] (M = B*T rows); dwx, dwa [H,256,256] laid out like the
+ * weights; dbx, dba [H,256] (both nullable, together).  bf16, W == 256 * H
+ * (RG_ERR_UNSUPPORTED otherwise: the caller keeps its own batched product);
+ * sums in float32 over row ranges whose partial results meet in `workspace`
+ * (rg_gates_weight_grads_workspace_bytes, 16-byte aligned) in a fixed order,
+ * one rounding: the same bits on every run. */
+size_t rg_gates_weight_grads_workspace_bytes(int64_t M, int W, int H);
+int rg_gates_weight_grads(const void* x, const void* dgx, const void* dga,
+                          void* dwx, void* dwa, void* dbx, void* dba,
+                          void* workspace, size_t workspace_bytes, int64_t M,
+                          int W, int H, int dtype, void* stream);
+
 /* The two gate projections of RGLRU.forward (layers.py:338-339, before the
  * sigmoid) in one pass over x:
  *   gx_pre = input_gate(xc), ga_pre = a_gate(xc), both [B,T,W] in `dtype`.

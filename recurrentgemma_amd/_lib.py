@@ -35,6 +35,8 @@ SIGNATURES = {
                                _i, _vp]),
     "rg_conv1d_step": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "rg_block_diag_linear": (_i, [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp]),
+    "rg_gates_weight_grads_workspace_bytes": (_sz, [_i64, _i, _i]),
+    "rg_gates_weight_grads": (_i, [_vp] * 8 + [_sz, _i64, _i, _i, _i, _vp]),
     "rg_gates_gemm": (_i, [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                            _vp, _i, _i, _i, _i, _i, _vp]),
     "rg_lru_scan_fused": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp,

@@ -223,6 +223,42 @@ int rg_block_diag_linear(const void* x, const void* w, const void* b, void* y,
                        rg::launch_gemm_generic(a, dtype, (hipStream_t)stream));
 }
 
+size_t rg_gates_weight_grads_workspace_bytes(int64_t M, int W, int H) {
+  return rg::gates_wgrad_workspace_bytes(M, W, H);
+}
+
+int rg_gates_weight_grads(const void* x, const void* dgx, const void* dga,
+                          void* dwx, void* dwa, void* dbx, void* dba,
+                          void* workspace, size_t workspace_bytes, int64_t M,
+                          int W, int H, int dtype, void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(M > 0 && W > 0 && H > 0, "%s: M=%lld W=%d H=%d must be positive",
+             __func__, (long long)M, W, H);
+  if (dtype != RG_DTYPE_BF16 || !rg::gates_wgrad_serves(M, W, H))
+    return fail(RG_ERR_UNSUPPORTED,
+                "%s: unsupported: bf16 with 256-wide heads only (W=%d H=%d)",
+                __func__, W, H);
+  RG_CHECK_PTR(x);
+  RG_CHECK_PTR(dgx);
+  RG_CHECK_PTR(dga);
+  RG_CHECK_PTR(dwx);
+  RG_CHECK_PTR(dwa);
+  RG_CHECK_OPT_PTR(dbx);
+  RG_CHECK_OPT_PTR(dba);
+  RG_REQUIRE((dbx == nullptr) == (dba == nullptr),
+             "%s: dbx and dba are given together or not at all", __func__);
+  RG_REQUIRE(aligned16(x) && aligned16(dgx) && aligned16(dga),
+             "%s: x, dgx and dga must be 16-byte aligned", __func__);
+  const size_t need = rg::gates_wgrad_workspace_bytes(M, W, H);
+  if (workspace == nullptr || workspace_bytes < need || !aligned16(workspace))
+    return fail(RG_ERR_WORKSPACE,
+                "%s: workspace of %zu bytes (16-byte aligned) required, got %zu",
+                __func__, need, workspace ? workspace_bytes : (size_t)0);
+  return launch_status(
+      __func__, rg::launch_gates_wgrad(x, dgx, dga, dwx, dwa, dbx, dba,
+                                       workspace, M, W, H, (hipStream_t)stream));
+}
+
 int rg_gates_gemm(const void* x, int apply_conv, const void* segpos,
                   int segpos_is_i64, const void* conv_w, const void* conv_b,
                   const void* w_x, const void* b_x, const void* w_a,

@@ -10,8 +10,6 @@
 namespace rg {
 namespace {
 
-constexpr float kGeluC0 = 0.7978845608028654f;  // sqrt(2/pi)
-constexpr float kGeluC1 = 0.044715f;
 
 // bf16: gelu_mul_bf16 per element, the product rounded once.
 // One 16-byte item (eight elements) per thread, streaming loads and stores, no

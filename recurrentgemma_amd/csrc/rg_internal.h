@@ -305,6 +305,13 @@ hipError_t launch_rms_norm_partial(const float* sums, int slices,
 // out[0] = shader cycles, out[1] = 10 ns ticks that `iters` rounds of a short
 // dependent instruction chain took (rg_elementwise.hip)
 hipError_t launch_clock_probe(uint64_t* out, int iters, hipStream_t s);
+// rg_gates_wgrad.hip: weight and bias gradients of both gate projections
+bool gates_wgrad_serves(int64_t M, int W, int H);
+size_t gates_wgrad_workspace_bytes(int64_t M, int W, int H);
+hipError_t launch_gates_wgrad(const void* x, const void* dgx, const void* dga,
+                              void* dwx, void* dwa, void* dbx, void* dba,
+                              void* workspace, int64_t M, int W, int H,
+                              hipStream_t s);
 hipError_t launch_pack_gate_weights(const void* w_x, const void* w_a,
                                     void* packed, int H, hipStream_t s);
 

@@ -218,6 +218,39 @@ def gates_gemm(x, w_x, b_x, w_a, b_a, conv=None):
   return gx, ga
 
 
+def gates_weight_grads_supported(x, num_heads) -> bool:
+  """bf16 with 256-wide heads: what rg_gates_weight_grads takes."""
+  return (x.dtype == torch.bfloat16 and x.shape[-1] == 256 * num_heads)
+
+
+def gates_weight_grads(x, dgx, dga, num_heads, with_bias=True):
+  """(dw_x, dw_a, db_x, db_a) of the two gate projections on x from the
+  gradients of their outputs (autograd of layers.py:134-136 with respect to
+  w and b): dw [H,256,256], db [H,256] or None; bf16, 256-wide heads."""
+  W = x.shape[-1]
+  assert dgx.shape == x.shape and dga.shape == x.shape
+  x = _dev(x, "x")
+  _same(x.dtype, x.device, dgx=dgx, dga=dga)
+  dgx, dga = _dev(dgx, "dgx"), _dev(dga, "dga")
+  M = x.numel() // W
+  H = num_heads
+  lib = _lib.lib()
+  need = lib.rg_gates_weight_grads_workspace_bytes(M, W, H)
+  if need == 0:
+    raise ValueError("gates_weight_grads: bf16 with 256-wide heads only")
+  ws = torch.empty(need, dtype=torch.uint8, device=x.device)
+  dwx = torch.empty(H, 256, 256, dtype=x.dtype, device=x.device)
+  dwa = torch.empty_like(dwx)
+  dbx = torch.empty(H, 256, dtype=x.dtype, device=x.device) if with_bias else None
+  dba = torch.empty_like(dbx) if with_bias else None
+  with _on(x.device):
+    _lib.check(lib.rg_gates_weight_grads(
+        _p(x), _p(dgx), _p(dga), _p(dwx), _p(dwa),
+        None if dbx is None else _p(dbx), None if dba is None else _p(dba),
+        _p(ws), need, M, W, H, _dtype_code(x), _stream(x)))
+  return dwx, dwa, dbx, dba
+
+
 def _scan_workspace(B, T, W, device, split):
   """Workspace for a scan whose sequences are cut into chunks that run side
   by side (few rows and channels, long sequences), or None for the one-pass

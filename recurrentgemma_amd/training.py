@@ -166,10 +166,19 @@ class _GateProjections(torch.autograd.Function):
   def backward(ctx, dgx, dga):
     x, w_x, w_a = ctx.saved_tensors
     need = ctx.needs_input_grad
-    dx1, dwx, dbx = _projection_grads(x, w_x, dgx.contiguous(),
-                                      (need[0], need[1], need[2]))
-    dx2, dwa, dba = _projection_grads(x, w_a, dga.contiguous(),
-                                      (need[0], need[3], need[4]))
+    dgx, dga = dgx.contiguous(), dga.contiguous()
+    if (need[1] and need[3] and need[2] == need[4] and
+        ops.gates_weight_grads_supported(x, w_x.shape[0])):
+      # weight and bias gradients of both projections in one pass over x and
+      # the two output gradients (rg_gates_weight_grads)
+      dwx, dwa, dbx, dba = ops.gates_weight_grads(x, dgx, dga, w_x.shape[0],
+                                                  with_bias=need[2])
+      dx1 = _projection_grads(x, w_x, dgx, (need[0], False, False))[0]
+      dx2 = _projection_grads(x, w_a, dga, (need[0], False, False))[0]
+      dx = dx1.add_(dx2) if need[0] else None
+      return dx, dwx, dbx, dwa, dba
+    dx1, dwx, dbx = _projection_grads(x, w_x, dgx, (need[0], need[1], need[2]))
+    dx2, dwa, dba = _projection_grads(x, w_a, dga, (need[0], need[3], need[4]))
     # (the sum autograd would form of the two layers' input gradients)
     dx = dx1.add_(dx2) if need[0] else None
     return dx, dwx, dbx, dwa, dba

@@ -164,7 +164,8 @@ def test_scan_backward_kernel(dtype, B, T, W):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("B,T,W,H", [(2, 1, 64, 2), (3, 19, 96, 3),
-                                     (1, 333, 130, 1), (2, 700, 256, 2)])
+                                     (1, 333, 130, 1), (2, 700, 256, 2),
+                                     (2, 150, 512, 2)])
 def test_rglru_backward_kernel(dtype, B, T, W, H):
   """training.rg_lru (forward and backward kernels from the gate
   pre-activations on) against autograd through the reference's formulas
@@ -172,7 +173,8 @@ def test_rglru_backward_kernel(dtype, B, T, W, H):
   in float64 on the CPU with a loop over time, on the same dtype-valued
   inputs: y, h_last and the gradients of x, both gate matrices and biases,
   a_param and h0; document starts, one and two channels per lane, sequences of
-  one token up to several rows per wave.  Tolerance relative to the largest
+  one token up to several rows per wave; the last shape has 256-wide heads
+  (bf16: the gate projections and all their gradients on the matrix kernels).  Tolerance relative to the largest
   magnitude of each tensor: 1e-4 float32 (sums in another order), 2e-2 bf16
   (the kernels round x, the pre-activations, y and each gradient to bf16)."""
   from oracle import torch_ref as R
@@ -421,3 +423,60 @@ def test_conv_backward_kernel_many_rows(dtype, B, T, W, K):
   near(xg.grad, x2.grad, "dx")
   near(wg.grad, w2.grad, "dw")
   near(bg.grad, b2.grad, "db")
+
+
+@pytest.mark.parametrize("M,H", [(1, 1), (64, 1), (100, 2), (257, 3),
+                                 (4099, 3), (8192, 10), (300, 16)])
+def test_gate_weight_gradients_kernel(M, H):
+  """rg_gates_weight_grads (both gate projections' dw and db in one pass,
+  bf16, 256-wide heads) against the definition
+  dw[h,i,j] = sum_m x[m,h,i] dy[m,h,j], db[h,j] = sum_m dy[m,h,j]
+  (autograd of layers.py:134-136) in float64 on the same bf16-valued inputs:
+  one row, row counts below, at and off the kernel's 64-row steps and its
+  splits of the rows, 1 to 16 heads.  Tolerance: the bf16 rounding of the
+  result (2^-8 of each tensor's largest magnitude); the same bits on a second
+  run (fixed summation order)."""
+  W = 256 * H
+  gen = torch.Generator().manual_seed(M * 31 + H)
+  x = torch.randn(M, W, generator=gen).to(torch.bfloat16).to(DEV)
+  d0 = torch.randn(M, W, generator=gen).to(torch.bfloat16).to(DEV)
+  d1 = (torch.randn(M, W, generator=gen) * 3).to(torch.bfloat16).to(DEV)
+  got = rg.ops.gates_weight_grads(x, d0, d1, H)
+  again = rg.ops.gates_weight_grads(x, d0, d1, H)
+  xh = x.double().view(M, H, 256)
+  for d, dw, db, dw2, db2 in ((d0, got[0], got[2], again[0], again[2]),
+                              (d1, got[1], got[3], again[1], again[3])):
+    dh = d.double().view(M, H, 256)
+    want_w = torch.einsum("mhi,mhj->hij", xh, dh)
+    want_b = dh.sum(0)
+    assert dw.shape == (H, 256, 256) and db.shape == (H, 256)
+    assert dw.dtype == torch.bfloat16 and db.dtype == torch.bfloat16
+    assert (dw.double() - want_w).abs().max() <= 2 ** -8 * want_w.abs().max()
+    assert (db.double() - want_b).abs().max() <= 2 ** -8 * want_b.abs().max()
+    assert torch.equal(dw, dw2) and torch.equal(db, db2)
+  # without the bias gradients
+  only_w = rg.ops.gates_weight_grads(x, d0, d1, H, with_bias=False)
+  assert only_w[2] is None and only_w[3] is None
+  assert torch.equal(only_w[0], got[0]) and torch.equal(only_w[1], got[1])
+
+
+def test_gate_weight_gradients_kernel_refuses_other_shapes():
+  x = torch.zeros(8, 384, dtype=torch.bfloat16, device=DEV)
+  with pytest.raises(ValueError, match="256-wide"):
+    rg.ops.gates_weight_grads(x, x, x, 3)
+  lib = rg._lib.lib()
+  assert lib.rg_gates_weight_grads_workspace_bytes(8, 384, 3) == 0
+  p = x.data_ptr()
+  rc = lib.rg_gates_weight_grads(p, p, p, p, p, None, None, p, 1 << 20, 8, 384,
+                                 3, 1, None)
+  assert rc == -2 and b"256-wide" in lib.rg_last_error()
+  x = torch.zeros(8, 256, dtype=torch.float32, device=DEV)
+  rc = lib.rg_gates_weight_grads(p, p, p, p, p, None, None, p, 1 << 20, 8, 256,
+                                 1, 0, None)
+  assert rc == -2
+  # a workspace that is too small
+  need = lib.rg_gates_weight_grads_workspace_bytes(8, 256, 1)
+  assert need > 0
+  rc = lib.rg_gates_weight_grads(p, p, p, p, p, None, None, p, need - 1, 8, 256,
+                                 1, 1, None)
+  assert rc == -4 and b"workspace" in lib.rg_last_error()
