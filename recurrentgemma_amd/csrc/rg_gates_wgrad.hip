@@ -11,21 +11,27 @@
 // 91 us per gate at M = 8192, W = 2560.
 //
 // Here a workgroup of eight waves owns a 128 x 128 tile of one head's dw for
-// one gate and a range of rows m.  Per step of 64 rows, threads 0-255 load the
-// 64 x 128 tile of x and threads 256-511 that of dy, each thread four
-// consecutive rows of eight channels (16 bytes per row); it turns its 4 x 8
-// values into eight 4 x 1 columns in registers (v_perm_b32) and writes them
-// into LDS as [channel][m] -- eight 8-byte writes --, 16-byte chunks of a
-// channel's 64 m placed so that neither those writes nor the operand reads
-// (16 bytes per lane: eight consecutive m of one channel) meet a bank more
-// than twice.  Wave (wi, wj) multiplies rows 32 wi .. +31 of the tile by
-// columns 64 wj .. +63: per 16 m one A and two B operand reads and two
-// v_mfma_f32_32x32x16_bf16.  The loads of the next step are in flight during
-// the products; two LDS buffers, one barrier a step.  The workgroups with the
-// tile's first rows also add up dy's columns for db.  Row ranges (splits of M,
-// enough of them to fill the chip) leave float32 partial sums in the
-// workspace; a second kernel adds them in a fixed order and rounds once:
-// results do not vary from run to run.
+// one gate and a range of rows m.  Per step of 64 rows, waves 0-3 load the
+// 64 x 128 tile of x and waves 4-7 that of dy, each thread four consecutive
+// rows of eight channels (16 bytes per row); it turns its 4 x 8 values into
+// eight 4 x 1 columns in registers (v_perm_b32) and writes them into LDS as
+// [channel][m] -- eight 8-byte writes --, the 16-byte chunks of a channel's
+// 64 m placed so that the operand reads (16 bytes per lane: eight consecutive
+// m of one channel) meet no bank twice and the writes spread evenly over the
+// banks.  Wave (wi, wj) multiplies rows 32 wi .. +31 of the tile by columns
+// 64 wj .. +63: per 16 m one A and two B operand reads and two
+// v_mfma_f32_32x32x16_bf16.  Rows are requested two steps before they go to
+// LDS; two LDS buffers, one barrier a step.  The workgroups with the tile's
+// first rows also add up dy's columns for db (dot products with 1.0).  Row
+// ranges (splits of M: as many as keep every workgroup resident at once, two
+// to a CU) leave float32 partial sums in the workspace; a second kernel adds
+// them in a fixed order and rounds once: results do not vary from run to run.
+//
+// Measured at M = 8192, W = 2560 (H = 10: 480 workgroups): 36 us + 6 us for
+// the second kernel, where the library's two batched products and two column
+// sums take 245 us.  Bound by the LDS round trip of the operands (every value
+// is written once and read 1.5 times per 2 matrix instructions), not by the
+// matrix pipe (0.6 PFLOP/s, a quarter of its peak) or by memory (126 MB in).
 #include "rg_common.h"
 #include "rg_internal.h"
 
