@@ -226,45 +226,6 @@ __device__ __forceinline__ void prefill_teams_body(const FusedArgs& p,
   const bool upper = lane >= 32;
   const int n0 = wave * 32;  // first channel of this wave in the head
 
-  // ---- this wave's weights: 32 channels of the head, both gates ------------
-  {
-    const f32x4* src = reinterpret_cast<const f32x4*>(p.w_packed) +
-                       ((int64_t)(h * 8 + wave) * 16 * 2) * 64 + lane;
-#pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      f32x4 w[16];
-#pragma unroll
-      for (int i = 0; i < 16; ++i) w[i] = src[(16 * half + i) * 64];
-      asm volatile("" ::"v"(w[0]), "v"(w[1]), "v"(w[2]), "v"(w[3]), "v"(w[4]),
-                   "v"(w[5]), "v"(w[6]), "v"(w[7]), "v"(w[8]), "v"(w[9]),
-                   "v"(w[10]), "v"(w[11]), "v"(w[12]), "v"(w[13]), "v"(w[14]),
-                   "v"(w[15]));
-#pragma unroll
-      for (int i = 0; i < 16; ++i) set_weight_frag(16 * half + i, w[i]);
-    }
-  }
-
-  // ---- conv table ---------------------------------------------------------
-  if (tid < 128) {
-    uint32_t u0 = 0, u1 = 0, u2 = 0, u3 = 0x3f803f80u, ub = 0;
-    if (p.conv_w != nullptr) {
-      const uint16_t* cw = (const uint16_t*)p.conv_w + h * kBW + tid * 2;
-      u0 = *reinterpret_cast<const uint32_t*>(cw);
-      u1 = *reinterpret_cast<const uint32_t*>(cw + W);
-      u2 = *reinterpret_cast<const uint32_t*>(cw + 2 * W);
-      u3 = *reinterpret_cast<const uint32_t*>(cw + 3 * W);
-      ub = *reinterpret_cast<const uint32_t*>(
-          (const uint16_t*)p.conv_b + h * kBW + tid * 2);
-    }
-    // w0 multiplies x[t-3], w3 multiplies x[t] (layers.py:514)
-    const u32x4 t0 = {(u0 & 0xffffu) | (u1 << 16), (u2 & 0xffffu) | (u3 << 16),
-                      (u0 >> 16) | (u1 & 0xffff0000u),
-                      (u2 >> 16) | (u3 & 0xffff0000u)};
-    const u32x4 t1 = {ub << 16, ub & 0xffff0000u, 0u, 0u};
-    *reinterpret_cast<u32x4*>(lds_raw + kConvTabOff + tid * 32) = t0;
-    *reinterpret_cast<u32x4*>(lds_raw + kConvTabOff + tid * 32 + 16) = t1;
-  }
-
   // ---- addressing -----------------------------------------------------------
   const uint32_t row_bytes = 2u * (uint32_t)p.W;
   const uint32_t seq_bytes = (uint32_t)T_len * row_bytes;  // < 2^31 (launcher)
@@ -677,17 +638,67 @@ __device__ __forceinline__ void prefill_teams_body(const FusedArgs& p,
   };
 
   // ---- prologue -------------------------------------------------------------
-  fetch_seg(tile_begin - 1);
-  m_prev = start_mask(tile_begin - 1);
-  fetch_seg(tile_begin);
-  m_cur = start_mask(tile_begin);
-  fetch_seg(tile_begin + 1);
-  m_next = start_mask(tile_begin + 1);
+  // Everything the first phases need is requested before anything waits: the
+  // raw rows of the first two tiles, the positions of three tiles, then the
+  // weights and the conv taps (one memory round trip after the other would
+  // cost a launch of short chunks a tenth of its time).
 #pragma unroll
   for (int j = 0; j < kRawLoadsPerWave; ++j) {
     dma_tile(tile_begin, j);
     dma_tile(tile_begin + 1, j);
   }
+  uint32_t first_lo[3], first_hi[3];
+#pragma unroll
+  for (int k = 0; k < 3; ++k) {
+    fetch_seg(tile_begin - 1 + k);
+    first_lo[k] = seg_lo;
+    first_hi[k] = seg_hi;
+  }
+  // ---- this wave's weights: 32 channels of the head, both gates ------------
+  {
+    const f32x4* src = reinterpret_cast<const f32x4*>(p.w_packed) +
+                       ((int64_t)(h * 8 + wave) * 16 * 2) * 64 + lane;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      f32x4 w[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) w[i] = src[(16 * half + i) * 64];
+      asm volatile("" ::"v"(w[0]), "v"(w[1]), "v"(w[2]), "v"(w[3]), "v"(w[4]),
+                   "v"(w[5]), "v"(w[6]), "v"(w[7]), "v"(w[8]), "v"(w[9]),
+                   "v"(w[10]), "v"(w[11]), "v"(w[12]), "v"(w[13]), "v"(w[14]),
+                   "v"(w[15]));
+#pragma unroll
+      for (int i = 0; i < 16; ++i) set_weight_frag(16 * half + i, w[i]);
+    }
+  }
+
+  // ---- conv table ---------------------------------------------------------
+  if (tid < 128) {
+    uint32_t u0 = 0, u1 = 0, u2 = 0, u3 = 0x3f803f80u, ub = 0;
+    if (p.conv_w != nullptr) {
+      const uint16_t* cw = (const uint16_t*)p.conv_w + h * kBW + tid * 2;
+      u0 = *reinterpret_cast<const uint32_t*>(cw);
+      u1 = *reinterpret_cast<const uint32_t*>(cw + W);
+      u2 = *reinterpret_cast<const uint32_t*>(cw + 2 * W);
+      u3 = *reinterpret_cast<const uint32_t*>(cw + 3 * W);
+      ub = *reinterpret_cast<const uint32_t*>(
+          (const uint16_t*)p.conv_b + h * kBW + tid * 2);
+    }
+    // w0 multiplies x[t-3], w3 multiplies x[t] (layers.py:514)
+    const u32x4 t0 = {(u0 & 0xffffu) | (u1 << 16), (u2 & 0xffffu) | (u3 << 16),
+                      (u0 >> 16) | (u1 & 0xffff0000u),
+                      (u2 >> 16) | (u3 & 0xffff0000u)};
+    const u32x4 t1 = {ub << 16, ub & 0xffff0000u, 0u, 0u};
+    *reinterpret_cast<u32x4*>(lds_raw + kConvTabOff + tid * 32) = t0;
+    *reinterpret_cast<u32x4*>(lds_raw + kConvTabOff + tid * 32 + 16) = t1;
+  }
+
+  seg_lo = first_lo[0]; seg_hi = first_hi[0];
+  m_prev = start_mask(tile_begin - 1);
+  seg_lo = first_lo[1]; seg_hi = first_hi[1];
+  m_cur = start_mask(tile_begin);
+  seg_lo = first_lo[2]; seg_hi = first_hi[2];
+  m_next = start_mask(tile_begin + 1);
   wait_vmcnt<0>();
   __syncthreads();  // conv table, raw tiles
   {
