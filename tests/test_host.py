@@ -299,6 +299,19 @@ def test_build_check_for_early_reads_of_matrix_results(tmp_path):
     assert rc == want, name
 
 
+def test_bench_refuses_more_than_one_gpu():
+  """bench.py measures one GPU; any other --gpus ends with a message, not a
+  number."""
+  import subprocess
+  import sys
+  root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+  r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus",
+                      "2"], capture_output=True, text=True)
+  assert r.returncode != 0
+  assert "one GPU" in (r.stderr + r.stdout)
+  assert "{" not in r.stdout
+
+
 def test_no_cpu_fallback():
   conv = rg.Conv1D(width=8, temporal_width=4)
   with pytest.raises(RuntimeError, match="GPU only"):
