@@ -415,7 +415,11 @@ def run_training(args, torch, rg, ops, wl):
          lambda: ops.gates_weight_grads(xc, dy, dy, lru.input_gate.w.shape[0]),
          3),
         ("rg_lru_scan_fused (forward of gating and recurrence)",
-         lambda: ops.lru_scan_fused(xc, gx, ga, lru.a_param, seg), 4)):
+         lambda: ops.lru_scan_fused(xc, gx, ga, lru.a_param, seg), 4),
+        ("rg_gelu_mul (the block's x * gelu(y) join)",
+         lambda: ops.gelu_mul(xc, gx), 3),
+        ("rg_gelu_mul_backward", lambda: ops.gelu_mul_backward(dy, xc, gx),
+         5)):
       ms = events(fn)
       nbytes = per_element * n * 2
       gbs = nbytes / (ms * 1e-3) / 1e9
@@ -432,8 +436,8 @@ def run_training(args, torch, rg, ops, wl):
                  "width": W, "lru_width": W, "heads": H,
                  "documents": "geometric mean %d" % wl["mean_doc"],
                  "path": "training.differentiable(): kernels for conv, gate "
-                         "projections, RG-LRU in both directions; linear "
-                         "layers torch autograd"},
+                         "projections, RG-LRU and the gelu join in both "
+                         "directions; linear layers torch autograd"},
       "forward_only_ms": forward_only * 1e3,
       "roofline": {"kernel": "rglru_backward_kernel (rg_rglru_backward)",
                    "bound": "hbm", "achieved": main["achieved_gbs"],

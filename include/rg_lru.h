@@ -381,6 +381,19 @@ int rg_recurrent_step_static(const void* x, const void* segpos,
 int rg_gelu_mul(const void* a, const void* g, void* out, int64_t n, int dtype,
                 void* stream);
 
+/* The backward pass of rg_gelu_mul, for autograd through
+ * recurrentgemma/torch/modules.py:627-628 and :644 (the reference leaves it to
+ * torch's gelu and multiply nodes), one pass:
+ *   d_a = dout * gelu(g),   d_g = dout * a * gelu'(g)
+ * with gelu the tanh approximation of modules.py:289-291.  dout, a, g, d_a,
+ * d_g: n elements each in `dtype`, 16-byte aligned.  bf16: gelu(g) and
+ * dout * a are rounded to bf16 before they are used (the tensors they are in
+ * the reference's graph), the derivative is evaluated in float32, each output
+ * rounded once.  The outputs alias neither each other nor an input. */
+int rg_gelu_mul_backward(const void* dout, const void* a, const void* g,
+                         void* d_a, void* d_g, int64_t n, int dtype,
+                         void* stream);
+
 /* RMSNorm of the residual stack around the recurrent block, one pass:
  * out[r, :] = x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * (scale + 1) for
  * recurrentgemma/torch/layers.py:65-73 (RMSNorm.forward; eps 1e-6 there).

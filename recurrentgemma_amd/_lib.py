@@ -72,6 +72,7 @@ SIGNATURES = {
                                       _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i,
                                       _i, _vp]),
     "rg_gelu_mul": (_i, [_vp, _vp, _vp, ctypes.c_int64, _i, _vp]),
+    "rg_gelu_mul_backward": (_i, [_vp] * 5 + [ctypes.c_int64, _i, _vp]),
     "rg_rms_norm": (_i, [_vp, _vp, _vp, ctypes.c_int64, _i, ctypes.c_float, _i,
                          _vp]),
     "rg_linear_packed_bytes": (ctypes.c_size_t, [_i, _i, _i]),

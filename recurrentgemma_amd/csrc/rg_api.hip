@@ -945,6 +945,28 @@ int rg_gelu_mul(const void* a, const void* g, void* out, int64_t n, int dtype,
       __func__, rg::launch_gelu_mul(a, g, out, n, dtype, (hipStream_t)stream));
 }
 
+int rg_gelu_mul_backward(const void* dout, const void* a, const void* g,
+                         void* d_a, void* d_g, int64_t n, int dtype,
+                         void* stream) {
+  RG_CHECK_DTYPE(dtype);
+  RG_REQUIRE(n > 0, "%s: n=%lld must be positive", __func__, (long long)n);
+  RG_CHECK_PTR(dout);
+  RG_CHECK_PTR(a);
+  RG_CHECK_PTR(g);
+  RG_CHECK_PTR(d_a);
+  RG_CHECK_PTR(d_g);
+  RG_REQUIRE((((uintptr_t)dout | (uintptr_t)a | (uintptr_t)g | (uintptr_t)d_a |
+               (uintptr_t)d_g) & 15) == 0,
+             "%s: every operand must be 16-byte aligned", __func__);
+  RG_REQUIRE(d_a != d_g && d_a != dout && d_a != a && d_a != g &&
+                 d_g != dout && d_g != a && d_g != g,
+             "%s: d_a and d_g must alias neither each other nor an input",
+             __func__);
+  return launch_status(__func__,
+                       rg::launch_gelu_mul_backward(dout, a, g, d_a, d_g, n,
+                                                    dtype, (hipStream_t)stream));
+}
+
 int rg_soft_cap(const void* x, void* out, int64_t n, float cap, int dtype,
                 void* stream) {
   RG_CHECK_DTYPE(dtype);

@@ -62,6 +62,103 @@ gelu_mul_f32_kernel(const f32x4* a, const f32x4* __restrict__ g, f32x4* out,
     out_tail[threadIdx.x] = one(a_tail[threadIdx.x], g_tail[threadIdx.x]);
 }
 
+// The backward pass of the join, out = a * gelu_tanh(g) (modules.py:289-291,
+// :627-628, :644), one pass over the three operands:
+//   d_a = dout * gelu(g)
+//   d_g = (dout * a) * gelu'(g),
+//   gelu'(g) = 0.5 (1 + t) + 0.5 g (1 - t^2) sqrt(2/pi) (1 + 3 c1 g^2),
+//   t = tanh(sqrt(2/pi) (g + c1 g^3)).
+// bf16: gelu(g) and dout * a are rounded to bf16 first, as the tensors they
+// are when autograd walks the reference's two ops; each output is rounded
+// once.
+template <bool BF16>
+__device__ __forceinline__ void gelu_mul_backward_one(float dv, float av,
+                                                      float gv, float& da,
+                                                      float& dg) {
+  constexpr float c0 = 0.7978845608028654f;  // sqrt(2/pi)
+  constexpr float c1 = 0.044715f;
+  const float g2 = gv * gv;
+  const float u = c0 * __builtin_fmaf(c1 * g2, gv, gv);
+  const float t = BF16 ? __builtin_fmaf(2.0f, sigmoid_fast(2.0f * u), -1.0f)
+                       : tanhf(u);
+  const float half_g = 0.5f * gv;
+  const float gelu = half_g * (1.0f + t);
+  const float slope = __builtin_fmaf(
+      half_g * __builtin_fmaf(-t, t, 1.0f),
+      c0 * __builtin_fmaf(3.0f * c1, g2, 1.0f), 0.5f * (1.0f + t));
+  da = dv * (BF16 ? round_to_bf16(gelu) : gelu);
+  dg = (BF16 ? round_to_bf16(dv * av) : dv * av) * slope;
+}
+
+__global__ void __launch_bounds__(256)
+gelu_mul_backward_bf16_kernel(const u32x4* __restrict__ dout,
+                              const u32x4* __restrict__ a,
+                              const u32x4* __restrict__ g, u32x4* d_a,
+                              u32x4* d_g, int64_t n8, const uint16_t* dout_tail,
+                              const uint16_t* a_tail, const uint16_t* g_tail,
+                              uint16_t* d_a_tail, uint16_t* d_g_tail,
+                              int tail) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n8) {
+    const u32x4 dv = __builtin_nontemporal_load(dout + i);
+    const u32x4 av = __builtin_nontemporal_load(a + i);
+    const u32x4 gv = __builtin_nontemporal_load(g + i);
+    u32x4 oa, og;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      float da_lo, dg_lo, da_hi, dg_hi;
+      gelu_mul_backward_one<true>(__uint_as_float(dv[k] << 16),
+                                  __uint_as_float(av[k] << 16),
+                                  __uint_as_float(gv[k] << 16), da_lo, dg_lo);
+      gelu_mul_backward_one<true>(__uint_as_float(dv[k] & 0xffff0000u),
+                                  __uint_as_float(av[k] & 0xffff0000u),
+                                  __uint_as_float(gv[k] & 0xffff0000u), da_hi,
+                                  dg_hi);
+      oa[k] = pack_bf16x2(da_lo, da_hi);
+      og[k] = pack_bf16x2(dg_lo, dg_hi);
+    }
+    __builtin_nontemporal_store(oa, d_a + i);
+    __builtin_nontemporal_store(og, d_g + i);
+  }
+  if (blockIdx.x == 0 && (int)threadIdx.x < tail) {
+    float da, dg;
+    gelu_mul_backward_one<true>(bf16_bits_to_f32(dout_tail[threadIdx.x]),
+                                bf16_bits_to_f32(a_tail[threadIdx.x]),
+                                bf16_bits_to_f32(g_tail[threadIdx.x]), da, dg);
+    d_a_tail[threadIdx.x] = f32_to_bf16_bits(da);
+    d_g_tail[threadIdx.x] = f32_to_bf16_bits(dg);
+  }
+}
+
+__global__ void __launch_bounds__(256)
+gelu_mul_backward_f32_kernel(const f32x4* __restrict__ dout,
+                             const f32x4* __restrict__ a,
+                             const f32x4* __restrict__ g, f32x4* d_a,
+                             f32x4* d_g, int64_t n4, const float* dout_tail,
+                             const float* a_tail, const float* g_tail,
+                             float* d_a_tail, float* d_g_tail, int tail) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n4) {
+    const f32x4 dv = __builtin_nontemporal_load(dout + i);
+    const f32x4 av = __builtin_nontemporal_load(a + i);
+    const f32x4 gv = __builtin_nontemporal_load(g + i);
+    f32x4 oa, og;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      float da, dg;
+      gelu_mul_backward_one<false>(dv[k], av[k], gv[k], da, dg);
+      oa[k] = da;
+      og[k] = dg;
+    }
+    __builtin_nontemporal_store(oa, d_a + i);
+    __builtin_nontemporal_store(og, d_g + i);
+  }
+  if (blockIdx.x == 0 && (int)threadIdx.x < tail)
+    gelu_mul_backward_one<false>(dout_tail[threadIdx.x], a_tail[threadIdx.x],
+                                 g_tail[threadIdx.x], d_a_tail[threadIdx.x],
+                                 d_g_tail[threadIdx.x]);
+}
+
 // RMSNorm of the residual stack (recurrentgemma/torch/layers.py:65-73):
 //   var = mean(x^2);  out = x * rsqrt(var + eps) * (scale + 1)
 // with every step rounded to the activation dtype like the reference's chain
@@ -341,6 +438,30 @@ hipError_t launch_gelu_mul(const void* a, const void* g, void* out, int64_t n,
         (const u32x4*)a, (const u32x4*)g, (u32x4*)out, items,
         (const uint16_t*)a + items * per, (const uint16_t*)g + items * per,
         (uint16_t*)out + items * per, tail);
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_gelu_mul_backward(const void* dout, const void* a,
+                                    const void* g, void* d_a, void* d_g,
+                                    int64_t n, int dtype, hipStream_t s) {
+  const int per = dtype == 0 ? 4 : 8;  // elements per 16-byte item
+  const int64_t items = n / per;
+  const int tail = (int)(n - items * per);
+  const int64_t blocks = items > 0 ? (items + 255) / 256 : 1;
+  if (blocks > 0x7fffffff) return hipErrorInvalidValue;
+  const int64_t done = items * per;
+  if (dtype == 0) {
+    gelu_mul_backward_f32_kernel<<<dim3((unsigned)blocks), 256, 0, s>>>(
+        (const f32x4*)dout, (const f32x4*)a, (const f32x4*)g, (f32x4*)d_a,
+        (f32x4*)d_g, items, (const float*)dout + done, (const float*)a + done,
+        (const float*)g + done, (float*)d_a + done, (float*)d_g + done, tail);
+  } else {
+    gelu_mul_backward_bf16_kernel<<<dim3((unsigned)blocks), 256, 0, s>>>(
+        (const u32x4*)dout, (const u32x4*)a, (const u32x4*)g, (u32x4*)d_a,
+        (u32x4*)d_g, items, (const uint16_t*)dout + done,
+        (const uint16_t*)a + done, (const uint16_t*)g + done,
+        (uint16_t*)d_a + done, (uint16_t*)d_g + done, tail);
   }
   return hipGetLastError();
 }

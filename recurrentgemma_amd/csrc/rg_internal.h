@@ -260,6 +260,9 @@ hipError_t launch_block_step_bf16(const StepArgs& a, hipStream_t s);
 // out[i] = a[i] * gelu_tanh(g[i]) over n elements (out may alias a or g).
 hipError_t launch_gelu_mul(const void* a, const void* g, void* out, int64_t n,
                            int dtype, hipStream_t s);
+hipError_t launch_gelu_mul_backward(const void* dout, const void* a,
+                                    const void* g, void* d_a, void* d_g,
+                                    int64_t n, int dtype, hipStream_t s);
 // out = tanh(x / cap) * cap, n elements; out[r] = argmax(x[r, :n])
 hipError_t launch_soft_cap(const void* x, void* out, int64_t n, float cap,
                            int dtype, hipStream_t s);

@@ -196,11 +196,11 @@ class RecurrentBlock(nn.Module):
     """The reference's op sequence (modules.py:605-655) under autograd."""
     if cache is not None:
       raise NotImplementedError("the differentiable path is prefill only")
-    y = gelu(self.linear_y(x))
+    y = self.linear_y(x)
     x = self.linear_x(x)
     x, conv_state = self.conv_1d(x, segment_pos, None, return_cache)
     x, h = self.rg_lru(x, segment_pos, None, return_cache)
-    x = self.linear_out(x * y)
+    x = self.linear_out(training.gelu_mul(x, y))  # x * gelu(y)
     if not return_cache:
       return x, None
     return x, RecurrentBlockCache(rg_lru_state=h, conv1d_state=conv_state)

@@ -520,6 +520,21 @@ def gelu_mul(a, g):
   return out
 
 
+def gelu_mul_backward(dout, a, g):
+  """(d_a, d_g) of out = a * gelu_tanh(g), one pass."""
+  assert dout.shape == a.shape == g.shape
+  a = _dev(a, "a")
+  _same(a.dtype, a.device, g=g, dout=dout)
+  g = _dev(g, "g")
+  dout = _dev(dout, "dout")
+  d_a, d_g = torch.empty_like(a), torch.empty_like(g)
+  with _on(a.device):
+    _lib.check(_lib.lib().rg_gelu_mul_backward(
+        _p(dout), _p(a), _p(g), _p(d_a), _p(d_g), a.numel(), _dtype_code(a),
+        _stream(a)))
+  return d_a, d_g
+
+
 def rms_norm(x, scale, eps=1e-6):
   """x * rsqrt(mean(x^2, -1) + eps) * (scale + 1), one pass."""
   x = _dev(x, "x")

@@ -8,7 +8,8 @@ reference's sequence of tensor ops (recurrentgemma/torch/layers.py:127-137,
 a Python loop over time there: the linear recurrence (layers.py:140-191),
 which is the scan kernel in both directions (and, for the RG-LRU, the gating
 around it: one forward and one backward kernel from the gate pre-activations
-on, rg_rglru_backward) --
+on, rg_rglru_backward; the block's x * gelu(y) join likewise, rg_gelu_mul and
+rg_gelu_mul_backward) --
 
   forward   h_t = a_t h_{t-1} + x_t
   backward  g_t = dy_t + a_{t+1} g_{t+1}     (the same recurrence, time
@@ -225,6 +226,28 @@ def conv1d_tensor_ops(x, segment_pos, w, b):
     term = xs * keep[..., None] * w[K - 1 - s]
     out = term if out is None else out + term
   return out + b
+
+
+class _GeluMul(torch.autograd.Function):
+  """a * gelu_tanh(g), the join of RecurrentBlock.forward's two branches
+  (modules.py:627-628, :644): one kernel each way, keeping the two inputs
+  and not the activation."""
+
+  @staticmethod
+  def forward(ctx, a, g):
+    a, g = a.contiguous(), g.contiguous()
+    ctx.save_for_backward(a, g)
+    return ops.gelu_mul(a, g)
+
+  @staticmethod
+  def backward(ctx, dout):
+    a, g = ctx.saved_tensors
+    return ops.gelu_mul_backward(dout.contiguous(), a, g)
+
+
+def gelu_mul(a, g):
+  """a * gelu_tanh(g) on kernels in both directions."""
+  return _GeluMul.apply(a, g)
 
 
 class _GatedScan(torch.autograd.Function):

@@ -480,3 +480,71 @@ def test_gate_weight_gradients_kernel_refuses_other_shapes():
   rc = lib.rg_gates_weight_grads(p, p, p, p, p, None, None, p, need - 1, 8, 256,
                                  1, 1, None)
   assert rc == -4 and b"workspace" in lib.rg_last_error()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(1, 1, 3), (1, 1, 7), (2, 17, 96),
+                                   (1, 343, 3), (3, 333, 130),
+                                   (4, 2048, 2560)])
+def test_gelu_join_backward_kernel(dtype, shape):
+  """rg_gelu_mul_backward against float64 autograd of torch's own
+  a * gelu(g, approximate="tanh") (modules.py:289-291, :644) on the same
+  inputs: element counts below, at and off the kernel's 16-byte items, g over
+  both tails of the activation.  Per element: float32 1e-5 of the value plus
+  the cancellation in 1 + tanh (1e-6 of |dout| max(1,|a|) max(1,|g|)); bf16 the
+  two roundings the reference's graph has as well (2^-7 of the value) plus the
+  same absolute term at 1e-5."""
+  gen = torch.Generator().manual_seed(sum(shape))
+  a = torch.randn(shape, generator=gen).to(dtype).to(DEV)
+  g = (torch.randn(shape, generator=gen) * 3).to(dtype).to(DEV)
+  dout = torch.randn(shape, generator=gen).to(dtype).to(DEV)
+  d_a, d_g = rg.ops.gelu_mul_backward(dout, a, g)
+  assert d_a.dtype == dtype and d_g.dtype == dtype
+  assert d_a.shape == a.shape and d_g.shape == g.shape
+  a64 = a.double().requires_grad_()
+  g64 = g.double().requires_grad_()
+  out = a64 * torch.nn.functional.gelu(g64, approximate="tanh")
+  out.backward(dout.double())
+  rel, floor = (1e-5, 1e-6) if dtype == torch.float32 else (2.0 ** -7, 1e-5)
+  slack = floor * dout.double().abs() * a64.detach().abs().clamp(min=1) * \
+      g64.detach().abs().clamp(min=1)
+  for got, want, what in ((d_a, a64.grad, "d_a"), (d_g, g64.grad, "d_g")):
+    over = (got.double() - want).abs() - (rel * want.abs() + slack)
+    assert over.max().item() <= 0, (what, over.max().item())
+
+
+def test_gelu_join_under_autograd_matches_tensor_ops():
+  """training.gelu_mul (kernels both ways) against the same join written as
+  tensor ops, values and both gradients, float32 (1e-5) and bf16 (1e-2 of the
+  largest magnitude)."""
+  for dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 1e-2)):
+    gen = torch.Generator().manual_seed(5)
+    a0 = torch.randn(2, 300, 512, generator=gen).to(dtype).to(DEV)
+    g0 = (torch.randn(2, 300, 512, generator=gen) * 2).to(dtype).to(DEV)
+    dout = torch.randn(2, 300, 512, generator=gen).to(dtype).to(DEV)
+    a1, g1 = a0.clone().requires_grad_(), g0.clone().requires_grad_()
+    a2, g2 = a0.clone().requires_grad_(), g0.clone().requires_grad_()
+    out1 = training.gelu_mul(a1, g1)
+    out1.backward(dout)
+    out2 = a2 * torch.nn.functional.gelu(g2, approximate="tanh")
+    out2.backward(dout)
+    for got, want, what in ((out1, out2, "out"), (a1.grad, a2.grad, "d_a"),
+                            (g1.grad, g2.grad, "d_g")):
+      err = (got.float() - want.float()).abs().max().item()
+      assert err <= tol * want.float().abs().max().item(), (dtype, what, err)
+
+
+def test_gelu_join_backward_entry_rejects_bad_arguments():
+  lib = rg._lib.lib()
+  x = torch.zeros(64, dtype=torch.float32, device=DEV)
+  y = torch.zeros(64, dtype=torch.float32, device=DEV)
+  z = torch.zeros(64, dtype=torch.float32, device=DEV)
+  p, q, r = x.data_ptr(), y.data_ptr(), z.data_ptr()
+  assert lib.rg_gelu_mul_backward(p, p, p, q, r, 0, 0, None) == -1
+  assert lib.rg_gelu_mul_backward(p, p, p, q, q, 64, 0, None) == -1
+  assert b"alias" in lib.rg_last_error()
+  assert lib.rg_gelu_mul_backward(p, p, p, p, r, 64, 0, None) == -1
+  assert lib.rg_gelu_mul_backward(p, p, p, q + 4, r, 32, 0, None) == -1
+  assert b"aligned" in lib.rg_last_error()
+  assert lib.rg_gelu_mul_backward(p, p, p, q, r, 64, 7, None) == -2
+  assert lib.rg_gelu_mul_backward(None, p, p, q, r, 64, 0, None) == -1
