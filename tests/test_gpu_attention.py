@@ -2,7 +2,8 @@
 op sequence (recurrentgemma/torch/modules.py:444-476: scores in the activation
 dtype, scaled, masked with the band of :86-127, softmax in float32,
 probabilities back in the activation dtype, weighted sum of the values)
-evaluated with float32 tensor ops on the same bf16-valued inputs."""
+evaluated with float32 tensor ops on the same bf16-valued inputs, and against
+the library's attention routine where the mask is one it can take."""
 
 import pytest
 import torch
@@ -84,6 +85,40 @@ def test_attention_prefill_left_padded_rows():
   for b, pad in enumerate((0, 37, 150)):  # the real tokens
     helpers.assert_close_elementwise(got[b, pad:], want[b, pad:], rtol=2e-2,
                                      atol_of_max=2e-2, what=f"row {b}")
+
+
+@pytest.mark.parametrize("B,T,H,window", [(2, 257, 10, 2048), (1, 700, 3, 2048),
+                                          (2, 400, 4, 96), (1, 1500, 2, 300)])
+def test_attention_prefill_against_library_attention(B, T, H, window):
+  """The same kernel against the library's own attention routine
+  (torch.nn.functional.scaled_dot_product_attention, float32 on the same
+  bf16-valued inputs): one document per row; a prompt no longer than the
+  window is plain causal attention (is_causal=True, no mask written here),
+  a longer one the band `t - window <= s <= t` of modules.py:86-127 as a
+  boolean mask.  Tolerance: the bf16 roundings of scores and probabilities
+  that the kernel keeps from the reference's op sequence and float32
+  attention does not have (2e-2 of the value plus 2e-2 of the largest)."""
+  hd = 256
+  g = torch.Generator().manual_seed(T + window)
+  q = torch.randn(B, T, H, hd, generator=g).to(torch.bfloat16).to(DEV)
+  k = torch.randn(B, T, 1, hd, generator=g).to(torch.bfloat16).to(DEV)
+  v = torch.randn(B, T, 1, hd, generator=g).to(torch.bfloat16).to(DEV)
+  seg = torch.arange(T).expand(B, T).contiguous().to(DEV)
+  got = ops.attention_prefill(q, k, v, band(seg, window), hd ** -0.5)
+  qf = q.float().transpose(1, 2)                       # [B, H, T, hd]
+  kf = k.float().transpose(1, 2).expand(-1, H, -1, -1)
+  vf = v.float().transpose(1, 2).expand(-1, H, -1, -1)
+  if T <= window + 1:
+    want = torch.nn.functional.scaled_dot_product_attention(
+        qf, kf, vf, is_causal=True, scale=hd ** -0.5)
+  else:
+    t = torch.arange(T, device=DEV)
+    visible = (t[None, :] <= t[:, None]) & (t[None, :] >= t[:, None] - window)
+    want = torch.nn.functional.scaled_dot_product_attention(
+        qf, kf, vf, attn_mask=visible, scale=hd ** -0.5)
+  want = want.transpose(1, 2)
+  helpers.assert_close_elementwise(got, want, rtol=2e-2, atol_of_max=2e-2,
+                                   what="attention vs library")
 
 
 def test_attention_prefill_refuses_other_shapes():
