@@ -426,14 +426,16 @@ def test_conv_backward_kernel_many_rows(dtype, B, T, W, K):
 
 
 @pytest.mark.parametrize("M,H", [(1, 1), (64, 1), (100, 2), (257, 3),
-                                 (4099, 3), (8192, 10), (300, 16)])
+                                 (4099, 3), (8192, 10), (300, 16),
+                                 (131072, 16)])
 def test_gate_weight_gradients_kernel(M, H):
   """rg_gates_weight_grads (both gate projections' dw and db in one pass,
   bf16, 256-wide heads) against the definition
   dw[h,i,j] = sum_m x[m,h,i] dy[m,h,j], db[h,j] = sum_m dy[m,h,j]
   (autograd of layers.py:134-136) in float64 on the same bf16-valued inputs:
   one row, row counts below, at and off the kernel's 64-row steps and its
-  splits of the rows, 1 to 16 heads.  Tolerance: the bf16 rounding of the
+  splits of the rows, 1 to 16 heads, up to the 16 x 8192 rows of the widest
+  configuration.  Tolerance: the bf16 rounding of the
   result (2^-8 of each tensor's largest magnitude); the same bits on a second
   run (fixed summation order)."""
   W = 256 * H
