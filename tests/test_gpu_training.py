@@ -162,21 +162,10 @@ def test_scan_backward_kernel(dtype, B, T, W):
       assert got_dh0 is None
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("B,T,W,H", [(2, 1, 64, 2), (3, 19, 96, 3),
-                                     (1, 333, 130, 1), (2, 700, 256, 2),
-                                     (2, 150, 512, 2)])
-def test_rglru_backward_kernel(dtype, B, T, W, H):
-  """training.rg_lru (forward and backward kernels from the gate
-  pre-activations on) against autograd through the reference's formulas
-  (layers.py:335-360, the sqrt with its clipped derivative :216-230) evaluated
-  in float64 on the CPU with a loop over time, on the same dtype-valued
-  inputs: y, h_last and the gradients of x, both gate matrices and biases,
-  a_param and h0; document starts, one and two channels per lane, sequences of
-  one token up to several rows per wave; the last shape has 256-wide heads
-  (bf16: the gate projections and all their gradients on the matrix kernels).  Tolerance relative to the largest
-  magnitude of each tensor: 1e-4 float32 (sums in another order), 2e-2 bf16
-  (the kernels round x, the pre-activations, y and each gradient to bf16)."""
+def _rglru_against_float64(dtype, B, T, W, H, where):
+  """Runs training.rg_lru forward and backward on the GPU and the reference's
+  formulas under float64 autograd with a loop over time on `where`, on the
+  same dtype-valued inputs; compares y, h_last and every gradient."""
   from oracle import torch_ref as R
   gen = torch.Generator().manual_seed(B * 1000 + T)
   p = R.make_params(W, H, dtype, seed=T + 5, gate_bias_std=0.3)
@@ -192,10 +181,11 @@ def test_rglru_backward_kernel(dtype, B, T, W, H):
   rh = torch.randn(B, W, generator=gen)
   names = ("a_param", "w_x", "b_x", "w_a", "b_a")
 
-  # float64 on the CPU
-  q = {k: p[k].double().requires_grad_(True) for k in names}
-  xd, hd = x.double().requires_grad_(True), h0.double().requires_grad_(True)
-  reset = seg == 0
+  # float64
+  q = {k: p[k].double().to(where).requires_grad_(True) for k in names}
+  xd = x.double().to(where).requires_grad_(True)
+  hd = h0.double().to(where).requires_grad_(True)
+  reset = (seg == 0).to(where)
 
   class BoundedSqrt(torch.autograd.Function):
     @staticmethod
@@ -227,7 +217,7 @@ def test_rglru_backward_kernel(dtype, B, T, W, H):
     h = a[:, t] * (~reset[:, t])[:, None] * h + xn[:, t]
     ys.append(h)
   yd = torch.stack(ys, 1)
-  ((yd * r).sum() + (h * rh).sum()).backward()
+  ((yd * r.to(where)).sum() + (h * rh.to(where)).sum()).backward()
 
   # the kernels
   qg = {k: p[k].to(DEV).requires_grad_(True) for k in names}
@@ -240,7 +230,7 @@ def test_rglru_backward_kernel(dtype, B, T, W, H):
   tol = 1e-4 if dtype == torch.float32 else 2e-2
 
   def near(got, want, what):
-    want = want.detach().double()
+    want = want.detach().double().cpu()
     err = (got.detach().double().cpu() - want).abs().max().item()
     scale = max(want.abs().max().item(), 1e-12)
     assert err <= tol * scale, (what, err, scale)
@@ -252,6 +242,36 @@ def test_rglru_backward_kernel(dtype, B, T, W, H):
   for k in names:
     assert qg[k].grad.dtype == dtype
     near(qg[k].grad, q[k].grad, "d" + k)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,T,W,H", [(2, 1, 64, 2), (3, 19, 96, 3),
+                                     (1, 333, 130, 1), (2, 700, 256, 2),
+                                     (2, 150, 512, 2)])
+def test_rglru_backward_kernel(dtype, B, T, W, H):
+  """training.rg_lru (forward and backward kernels from the gate
+  pre-activations on) against autograd through the reference's formulas
+  (layers.py:335-360, the sqrt with its clipped derivative :216-230) evaluated
+  in float64 on the CPU with a loop over time, on the same dtype-valued
+  inputs: y, h_last and the gradients of x, both gate matrices and biases,
+  a_param and h0; document starts, one and two channels per lane, sequences of
+  one token up to several rows per wave; the last shape has 256-wide heads
+  (bf16: the gate projections and all their gradients on the matrix kernels).  Tolerance relative to the largest
+  magnitude of each tensor: 1e-4 float32 (sums in another order), 2e-2 bf16
+  (the kernels round x, the pre-activations, y and each gradient to bf16)."""
+  _rglru_against_float64(dtype, B, T, W, H, "cpu")
+
+
+@pytest.mark.parametrize("dtype,B,T,W,H", [
+    (torch.bfloat16, 4, 2048, 2560, 10), (torch.float32, 4, 2048, 2560, 10),
+    (torch.bfloat16, 2, 8192, 4096, 16)])
+def test_rglru_backward_kernel_full_size_rows(dtype, B, T, W, H):
+  """The same comparison at the lengths and widths of the listed
+  configurations (2B: 2048 tokens x 2560, 10 heads; 9B: two rows of 8192
+  tokens x 4096, 16 heads), the float64 loop over time on the GPU: every
+  chunk boundary of a full-length row, the gate projections' kernels at their
+  real row counts.  Same tolerances."""
+  _rglru_against_float64(dtype, B, T, W, H, DEV)
 
 
 def test_rglru_forms_agree():
