@@ -1378,6 +1378,16 @@ def _full_size_properties(B, T, W, H, seg, seed):
   assert (y_row.float() - y[:1].float()).abs().max().item() <= 0.125
   assert helpers.max_rel(c_row.rg_lru_state, cache.rg_lru_state[:1]) < BF16_TOL
   assert torch.equal(c_row.conv1d_state, cache.conv1d_state[:1])
+  # (7) the block's join inside the call (the single kernels carry it in
+  #     their output stage, whole rows and rows in chunks) == the separate
+  #     pass over the call's plain output, bit for bit; states unchanged
+  gate = torch.randn(B, T, W, generator=g).to(dtype).to(DEV)
+  y_join, cache_join = rg.recurrent_core(blk.conv_1d, blk.rg_lru, x, segd,
+                                         gate_branch=gate)
+  assert torch.equal(y_join, ops.gelu_mul(y_core, gate))
+  assert torch.equal(cache_join.rg_lru_state, cache_core.rg_lru_state)
+  assert torch.equal(cache_join.conv1d_state, cache_core.conv1d_state)
+  del gate, y_join, cache_join
   # (6) parity against the oracle over the WHOLE sequence on two sampled rows
   #     (not row 0): y element by element, the final state and the conv state,
   #     for what recurrent_core ran at this grid (every chunk boundary of a
