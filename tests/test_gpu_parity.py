@@ -1054,6 +1054,73 @@ def test_recurrent_core_entry_equals_its_parts(dtype, B, T, W, H, joined):
   assert torch.equal(c3.cpu(), co.conv1d_state)
 
 
+@pytest.mark.parametrize("B,T,H,mean_doc,pad,with_h0,joined,with_conv,i32", [
+    (1, 1, 1, 0, 0, False, False, True, True),
+    (3, 2, 2, 0, 0, True, True, True, False),
+    (2, 15, 3, 5, 0, True, False, True, True),
+    (1, 16, 10, 0, 0, False, True, False, True),
+    (4, 17, 8, 2, 3, True, False, True, False),
+    (32, 33, 1, 17, 0, False, True, True, True),
+    (1, 63, 4, 0, 20, True, True, True, True),
+    (8, 64, 4, 60, 0, False, False, False, False),
+    (2, 65, 10, 5, 0, True, True, True, True),
+    (1, 255, 2, 300, 0, False, False, True, False),
+    (3, 256, 10, 17, 100, True, False, True, True),
+    (1, 257, 8, 0, 0, True, True, False, True),
+    (2, 511, 3, 60, 0, False, True, True, True),
+    (1, 513, 10, 2, 0, True, False, True, False),
+    (4, 527, 8, 300, 200, False, False, True, True),
+    (1, 1023, 1, 0, 0, True, True, True, True),
+    (1, 1025, 10, 300, 0, False, True, True, False),
+    (2, 1300, 4, 60, 7, True, False, False, True),
+    (1, 3001, 2, 1000, 0, True, True, True, True),
+])
+def test_float32_one_launch_sweep(B, T, H, mean_doc, pad, with_h0, joined,
+                                  with_conv, i32):
+  """The float32 chain in one launch (256-wide heads, at most 32 (row, head)
+  pairs) against the oracle: one token to several 512-token segments, lengths
+  below, at and off the kernel's 16-token tiles and chunks, documents of a few
+  tokens, left padding, int32 / int64 positions, with and without a carried-in
+  state, the block's join and the conv (without: RGLRU.forward alone).  y and
+  the state within 1e-5 of the largest magnitude, conv state exact."""
+  W = 256 * H
+  assert B * H <= 32
+  dtype = torch.float32
+  p = R.make_params(W, H, dtype, seed=T + H, gate_bias_std=0.3)
+  P = {k: _dev(v) for k, v in p.items()}
+  g = torch.Generator().manual_seed(1000 + T + B)
+  x = torch.randn(B, T, W, generator=g)
+  gate = torch.randn(B, T, W, generator=g) if joined else None
+  seg = (helpers.document_positions(B, T, mean_doc, seed=T + 2) if mean_doc
+         else torch.arange(T).repeat(B, 1))
+  if pad:
+    seg = torch.cat([torch.full((B, pad), -1), seg[:, :T - pad]], 1)
+  seg = seg.to(torch.int32 if i32 else torch.int64)
+  h0 = torch.randn(B, W, generator=g) if with_h0 else None
+  lib = _lib.lib()
+  assert lib.rg_recurrent_core_workspace_bytes(B, T, W, H, 0) == 0
+  _announce("float32 one launch", (B, T, H, mean_doc, pad, with_h0, joined,
+                                   with_conv, i32))
+  cw, cb = (P["conv_w"], P["conv_b"]) if with_conv else (None, None)
+  y, h, c = ops.recurrent_core(
+      _dev(x), _dev(seg), cw, cb, P["w_x"], P["b_x"], P["w_a"], P["b_a"],
+      P["a_param"], h0=None if h0 is None else _dev(h0),
+      gate_branch=None if gate is None else _dev(gate))
+  if with_conv:
+    xc, conv_state = R.conv1d_forward(x, seg, p["conv_w"], p["conv_b"])
+    assert torch.equal(c.cpu(), conv_state)
+  else:
+    xc = x
+    assert c is None
+  yo, ho = R.rglru_forward(xc, seg, p["a_param"], p["w_x"], p["b_x"], p["w_a"],
+                           p["b_a"], cache=h0)
+  if joined:
+    yo = yo * torch.nn.functional.gelu(gate, approximate="tanh")
+  assert torch.isfinite(y).all()
+  assert helpers.max_rel(y, yo) < F32_TOL
+  assert helpers.max_rel(h, ho) < F32_TOL
+
+
 def test_recurrent_core_entry_rejects_a_short_workspace():
   B, T, W, H = 1, 512, 512, 4  # float32, 128-wide heads: the two-kernel form
   x = _dev(torch.zeros(B, T, W))
