@@ -760,6 +760,11 @@ def test_recurrent_prefill_single_launch(B, T, W, H, mean_doc, seg_dtype,
     (1, 2048, 512, 2, 300),    # rows in chunks
     (3, 1600, 768, 3, None),
     (40, 130, 1024, 4, 50),    # 160 (row, head) pairs
+    (2, 449, 512, 2, 60),      # the shortest rows that are cut into chunks
+    (1, 513, 256, 1, None),
+    (1, 4096, 2560, 10, 1024), # chunks at the 2B width
+    (5, 3000, 2560, 10, 5),    # ... ragged, documents of a few tokens
+    (6, 1500, 768, 3, 300),
 ])
 def test_prefill_joined_with_gate_branch(B, T, W, H, mean_doc):
   """rg_recurrent_prefill_gelu_mul (the block's x * gelu(y) join applied where
